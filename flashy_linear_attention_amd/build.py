@@ -1,0 +1,79 @@
+"""Builds ``libfla_gfx950.so`` in-tree with hipcc (gfx950 only).
+
+Run as ``python -m flashy_linear_attention_amd.build``.  hipcc cross-compiles
+without a GPU.  One object per (dtype, DC, DO) kernel instantiation, compiled in
+parallel, then linked with the C ABI into the package directory.
+"""
+
+from __future__ import annotations
+
+import concurrent.futures
+import os
+import shutil
+import subprocess
+import sys
+from typing import List
+
+PKG_DIR = os.path.dirname(os.path.abspath(__file__))
+REPO_ROOT = os.path.dirname(PKG_DIR)
+CSRC = os.path.join(PKG_DIR, "csrc")
+INCLUDE = os.path.join(REPO_ROOT, "include")
+OBJ_DIR = os.path.join(PKG_DIR, "csrc", "_obj")
+LIB_NAME = "libfla_gfx950.so"
+LIB_PATH = os.path.join(PKG_DIR, LIB_NAME)
+
+DIMS = (32, 64, 128, 256)
+HIPCC_FLAGS = [
+    "--offload-arch=gfx950",
+    "-O3",
+    "-std=c++17",
+    "-fPIC",
+    # hipcc may not form packed fp32 VALU ops on this target
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+    "-I" + INCLUDE,
+    "-I" + CSRC,
+]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found; the HIP kernels cannot be built")
+    return exe
+
+
+def _run(cmd: List[str]) -> None:
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: " + " ".join(cmd) + "\n" + proc.stdout)
+
+
+def _compile_inst(args) -> str:
+    dtype, dc, do = args
+    obj = os.path.join(OBJ_DIR, f"inst_t{dtype}_c{dc}_o{do}.o")
+    _run([_hipcc(), *HIPCC_FLAGS, f"-DFLA_INST_DTYPE={dtype}", f"-DFLA_INST_DC={dc}", f"-DFLA_INST_DO={do}",
+          "-c", os.path.join(CSRC, "fla_inst.hip"), "-o", obj])
+    return obj
+
+
+def build(jobs: int | None = None, verbose: bool = True) -> str:
+    """Compile every kernel instantiation and link the shared library.  Always recompiles."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    work = [(t, dc, do) for t in (0, 1) for dc in DIMS for do in DIMS]
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = list(pool.map(_compile_inst, work))
+    capi = os.path.join(OBJ_DIR, "fla_capi.o")
+    _run([_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, "fla_capi.hip"), "-o", capi])
+    tmp = LIB_PATH + ".tmp"
+    _run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, capi, *objs])
+    os.replace(tmp, LIB_PATH)
+    if verbose:
+        print(f"built {LIB_PATH} ({os.path.getsize(LIB_PATH) / 1e6:.1f} MB, {len(objs)} kernel objects)")
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    build()
+    sys.exit(0)

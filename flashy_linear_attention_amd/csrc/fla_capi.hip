@@ -1,0 +1,173 @@
+// C ABI of libfla_gfx950.so (declared in include/fla.h): argument checks,
+// mapping of forward / gradients onto the one masked-product kernel, launch.
+#include "fla.h"
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fla_dispatch.h"
+
+namespace {
+
+using fla::TriParams;
+typedef hipError_t (*launch_fn)(const TriParams &, hipStream_t);
+
+int pad_index(int64_t d) { return d <= 32 ? 0 : d <= 64 ? 1 : d <= 128 ? 2 : 3; }
+
+launch_fn lookup(int dtype, int64_t dc, int64_t dout) {
+#define FLA_ENTRY(c, o) {fla::FLA_LAUNCH_NAME(0, c, o), fla::FLA_LAUNCH_NAME(1, c, o)},
+    static const launch_fn table[16][2] = {FLA_FOR_EACH_DIM_PAIR(FLA_ENTRY)};
+#undef FLA_ENTRY
+    return table[pad_index(dc) * 4 + pad_index(dout)][dtype];
+}
+
+int64_t next_pow2(int64_t x) {
+    int64_t p = 1;
+    while (p < x) p <<= 1;
+    return p;
+}
+
+struct View {
+    const void *ptr;
+    const int64_t *strides;
+};
+
+int check_view(const View &t) {
+    if (!t.ptr) return FLA_ERR_NULL_POINTER;
+    if (!t.strides) return FLA_ERR_STRIDE;
+    if (t.strides[3] != 1) return FLA_ERR_STRIDE;
+    if (t.strides[0] < 0 || t.strides[1] < 0 || t.strides[2] < 0) return FLA_ERR_STRIDE;
+    return FLA_OK;
+}
+
+// 16-byte vector loads are legal when every row starts 16-byte aligned and the
+// width is a whole number of 8-element chunks.
+int vec_ok(const View &t, int64_t width) {
+    return width % 8 == 0 && reinterpret_cast<uintptr_t>(t.ptr) % 16 == 0 && t.strides[0] % 8 == 0 &&
+           t.strides[1] % 8 == 0 && t.strides[2] % 8 == 0;
+}
+
+int check_common(int64_t B, int64_t H, int64_t N, int dtype) {
+    if (dtype != FLA_DTYPE_BF16 && dtype != FLA_DTYPE_F16) return FLA_ERR_DTYPE;
+    if (B < 0 || H < 0 || N < 0) return FLA_ERR_SHAPE;
+    if (N > (int64_t)1 << 30) return FLA_ERR_SHAPE;
+    if (H > 0 && B > ((int64_t)1 << 30) / H) return FLA_ERR_SHAPE;
+    return FLA_OK;
+}
+
+// Out = mask(X Y^T) Z; all arguments already validated.
+int run_tri(const View &x, const View &y, const View &z, const View &out, int64_t B, int64_t H, int64_t N,
+            int64_t dc, int64_t dout, int upper, int dtype, void *stream) {
+    if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    TriParams p;
+    p.x = x.ptr, p.y = y.ptr, p.z = z.ptr, p.out = const_cast<void *>(out.ptr);
+    p.xs_b = x.strides[0], p.xs_h = x.strides[1], p.xs_n = x.strides[2];
+    p.ys_b = y.strides[0], p.ys_h = y.strides[1], p.ys_n = y.strides[2];
+    p.zs_b = z.strides[0], p.zs_h = z.strides[1], p.zs_n = z.strides[2];
+    p.os_b = out.strides[0], p.os_h = out.strides[1], p.os_n = out.strides[2];
+    p.H = (int32_t)H, p.N = (int32_t)N, p.BH = (int32_t)(B * H);
+    p.dc = (int32_t)dc, p.dout = (int32_t)dout;
+    p.upper = upper ? 1 : 0;
+    p.n_tiles = 0;
+    p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout);
+    launch_fn fn = lookup(dtype, dc, dout);
+    if (!fn) return FLA_ERR_UNSUPPORTED;
+    return fn(p, static_cast<hipStream_t>(stream)) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+}
+
+int forward(const View &q, const View &k, const View &v, const View &o, int64_t B, int64_t H, int64_t N,
+            int64_t dqk, int64_t dv, int dtype, void *stream) {
+    const View all[] = {q, k, v, o};
+    for (const View &t : all)
+        if (int rc = check_view(t)) return rc;
+    return run_tri(q, k, v, o, B, H, N, dqk, dv, 0, dtype, stream);
+}
+
+int backward(const View &go, const View &q, const View &k, const View &v, const View &dq, const View &dk,
+             const View &dv, int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dvw, int dtype, void *stream) {
+    const View all[] = {go, q, k, v, dq, dk, dv};
+    for (const View &t : all)
+        if (int rc = check_view(t)) return rc;
+    // dQ = lower(dO V^T) K ; dV = upper(K Q^T) dO ; dK = upper(V dO^T) Q
+    if (int rc = run_tri(go, v, k, dq, B, H, N, dvw, dqk, 0, dtype, stream)) return rc;
+    if (int rc = run_tri(k, q, go, dv, B, H, N, dqk, dvw, 1, dtype, stream)) return rc;
+    return run_tri(v, go, q, dk, B, H, N, dvw, dqk, 1, dtype, stream);
+}
+
+}  // namespace
+
+extern "C" {
+
+int fla_abi_version(void) { return FLA_ABI_VERSION; }
+
+const char *fla_strerror(int status) {
+    switch (status) {
+        case FLA_OK: return "ok";
+        case FLA_ERR_NULL_POINTER: return "a required pointer is NULL";
+        case FLA_ERR_DTYPE: return "dtype must be FLA_DTYPE_BF16 or FLA_DTYPE_F16";
+        case FLA_ERR_HEAD_DIM: return "Only head_dims <= 256 are supported.";
+        case FLA_ERR_V_HEAD_DIM:
+            return "value head dimension must be a power of 2 no larger than the padded query/key head dimension";
+        case FLA_ERR_SHAPE: return "B, H and N must be non-negative and B*H, N at most 2^30";
+        case FLA_ERR_STRIDE: return "strides must be given, non-negative, with innermost stride 1";
+        case FLA_ERR_LAUNCH: return "the HIP runtime rejected the kernel launch";
+        case FLA_ERR_UNSUPPORTED: return "no kernel was built for this combination";
+        default: return "unknown fla status";
+    }
+}
+
+int fla_linear_attn_fwd(const void *q, const void *k, const void *v, void *o, int64_t B, int64_t H, int64_t N,
+                        int64_t D, const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
+                        const int64_t *o_strides, int dtype, void *stream) {
+    if (int rc = check_common(B, H, N, dtype)) return rc;
+    if (D < 1 || D > 256) return FLA_ERR_HEAD_DIM;
+    return forward({q, q_strides}, {k, k_strides}, {v, v_strides}, {o, o_strides}, B, H, N, D, D, dtype, stream);
+}
+
+int fla_linear_attn_bwd(const void *grad_out, const void *q, const void *k, const void *v, void *dq, void *dk,
+                        void *dv, int64_t B, int64_t H, int64_t N, int64_t D, const int64_t *go_strides,
+                        const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
+                        const int64_t *dq_strides, const int64_t *dk_strides, const int64_t *dv_strides, int dtype,
+                        void *stream) {
+    if (int rc = check_common(B, H, N, dtype)) return rc;
+    if (D < 1 || D > 256) return FLA_ERR_HEAD_DIM;
+    return backward({grad_out, go_strides}, {q, q_strides}, {k, k_strides}, {v, v_strides}, {dq, dq_strides},
+                    {dk, dk_strides}, {dv, dv_strides}, B, H, N, D, D, dtype, stream);
+}
+
+int fla_linear_attn_smallv_fwd(const void *q, const void *k, const void *v, void *o, int64_t B, int64_t H,
+                               int64_t N, int64_t D_qk, int64_t D_v, const int64_t *q_strides,
+                               const int64_t *k_strides, const int64_t *v_strides, const int64_t *o_strides,
+                               int dtype, void *stream) {
+    if (int rc = check_common(B, H, N, dtype)) return rc;
+    if (D_qk < 1 || D_qk > 256) return FLA_ERR_HEAD_DIM;
+    if (D_v < 1 || next_pow2(D_v) != D_v || D_v > next_pow2(D_qk)) return FLA_ERR_V_HEAD_DIM;
+    return forward({q, q_strides}, {k, k_strides}, {v, v_strides}, {o, o_strides}, B, H, N, D_qk, D_v, dtype,
+                   stream);
+}
+
+int fla_linear_attn_smallv_bwd(const void *grad_out, const void *q, const void *k, const void *v, void *dq,
+                               void *dk, void *dv, int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                               const int64_t *go_strides, const int64_t *q_strides, const int64_t *k_strides,
+                               const int64_t *v_strides, const int64_t *dq_strides, const int64_t *dk_strides,
+                               const int64_t *dv_strides, int dtype, void *stream) {
+    if (int rc = check_common(B, H, N, dtype)) return rc;
+    if (D_qk < 1 || D_qk > 256) return FLA_ERR_HEAD_DIM;
+    if (D_v < 1 || D_v > 256) return FLA_ERR_V_HEAD_DIM;
+    return backward({grad_out, go_strides}, {q, q_strides}, {k, k_strides}, {v, v_strides}, {dq, dq_strides},
+                    {dk, dk_strides}, {dv, dv_strides}, B, H, N, D_qk, D_v, dtype, stream);
+}
+
+int fla_tri_xyt_z(const void *x, const void *y, const void *z, void *out, int64_t B, int64_t H, int64_t N,
+                  int64_t D_c, int64_t D_o, const int64_t *x_strides, const int64_t *y_strides,
+                  const int64_t *z_strides, const int64_t *out_strides, int upper, int dtype, void *stream) {
+    if (int rc = check_common(B, H, N, dtype)) return rc;
+    if (D_c < 1 || D_c > 256 || D_o < 1 || D_o > 256) return FLA_ERR_HEAD_DIM;
+    const View vx{x, x_strides}, vy{y, y_strides}, vz{z, z_strides}, vo{out, out_strides};
+    const View all[] = {vx, vy, vz, vo};
+    for (const View &t : all)
+        if (int rc = check_view(t)) return rc;
+    return run_tri(vx, vy, vz, vo, B, H, N, D_c, D_o, upper, dtype, stream);
+}
+
+}  // extern "C"

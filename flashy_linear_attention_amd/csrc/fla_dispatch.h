@@ -1,0 +1,24 @@
+// Declarations shared by the per-instantiation translation units and the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "fla_tri_kernel.h"
+
+// Padded (DC, DO) pairs for which a kernel is built.  Widths are padded to the
+// next of 32/64/128/256, as the reference pads to the next power of two
+// (flashlinear/kernels/linear_attn_kernels.py:316).
+#define FLA_FOR_EACH_DIM_PAIR(X)                                                               \
+    X(32, 32) X(32, 64) X(32, 128) X(32, 256) X(64, 32) X(64, 64) X(64, 128) X(64, 256)        \
+    X(128, 32) X(128, 64) X(128, 128) X(128, 256) X(256, 32) X(256, 64) X(256, 128) X(256, 256)
+
+#define FLA_LAUNCH_NAME_(t, dc, dout) fla_launch_tri_t##t##_c##dc##_o##dout
+#define FLA_LAUNCH_NAME(t, dc, dout) FLA_LAUNCH_NAME_(t, dc, dout)
+
+namespace fla {
+#define FLA_DECLARE(dc, dout)                                                        \
+    hipError_t FLA_LAUNCH_NAME(0, dc, dout)(const TriParams &p, hipStream_t stream); \
+    hipError_t FLA_LAUNCH_NAME(1, dc, dout)(const TriParams &p, hipStream_t stream);
+FLA_FOR_EACH_DIM_PAIR(FLA_DECLARE)
+#undef FLA_DECLARE
+}  // namespace fla

@@ -1,0 +1,21 @@
+// One kernel instantiation per compilation: build with
+//   -DFLA_INST_DTYPE={0 bf16 | 1 f16} -DFLA_INST_DC=<32|64|128|256> -DFLA_INST_DO=<32|64|128|256>
+#include "fla_dispatch.h"
+
+#if !defined(FLA_INST_DTYPE) || !defined(FLA_INST_DC) || !defined(FLA_INST_DO)
+#error "define FLA_INST_DTYPE, FLA_INST_DC and FLA_INST_DO"
+#endif
+
+namespace fla {
+
+#if FLA_INST_DTYPE == 0
+using InstT = __bf16;
+#else
+using InstT = _Float16;
+#endif
+
+hipError_t FLA_LAUNCH_NAME(FLA_INST_DTYPE, FLA_INST_DC, FLA_INST_DO)(const TriParams &p, hipStream_t stream) {
+    return launch_tri<InstT, FLA_INST_DC, FLA_INST_DO>(p, stream);
+}
+
+}  // namespace fla

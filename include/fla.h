@@ -1,0 +1,125 @@
+/* fla.h -- C ABI of libfla_gfx950.so: causal linear attention O = tril(Q K^T) V,
+ * forward and backward, as hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * The reference has no native surface for this path: its four Python launch
+ * wrappers JIT-compile Triton kernels.  Each entry point below replaces one of
+ * those wrappers (cited per function); a Python binding passes
+ * `tensor.data_ptr()`, `tensor.stride()` and the current stream's handle.
+ *
+ * Conventions
+ *   - Every pointer is a device pointer on the current HIP device.
+ *   - Tensors are 4-D, logical shape (B, H, N, D); `strides` is an array of 4
+ *     element strides (b, h, n, d) and strides[3] must be 1.
+ *   - `dtype` selects 16-bit storage: FLA_DTYPE_BF16 or FLA_DTYPE_F16.  Products
+ *     run on bf16 / fp16 MFMA with fp32 accumulation; outputs are rounded once.
+ *   - `stream` is a hipStream_t (NULL = the null stream).  Calls only enqueue
+ *     work; they never synchronise, allocate or free.  Outputs must not alias
+ *     inputs.
+ *   - Re-entrant, no global mutable state (except the no-allocation variant
+ *     documented at its declaration, if present).
+ *   - Return value: FLA_OK or a negative FLA_ERR_* code; fla_strerror() names it.
+ *     Nothing is enqueued when an error is returned.
+ *   - N may be any non-negative value (the kernels bound-check rows).  The
+ *     reference's "N % 64 == 0" precondition is enforced by the Python layer
+ *     that mirrors the reference's asserts, not here.
+ */
+#ifndef FLA_H
+#define FLA_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FLA_ABI_VERSION 1
+
+enum fla_dtype { FLA_DTYPE_BF16 = 0, FLA_DTYPE_F16 = 1 };
+
+enum fla_status {
+    FLA_OK = 0,
+    FLA_ERR_NULL_POINTER = -1, /* a required pointer is NULL */
+    FLA_ERR_DTYPE = -2,        /* dtype is not one of enum fla_dtype */
+    FLA_ERR_HEAD_DIM = -3,     /* head dim < 1 or > 256 (linear_attn_kernels.py:322) */
+    FLA_ERR_V_HEAD_DIM = -4,   /* small-V: D_v not a power of two, or next_pow2(D_v) > next_pow2(D_qk)
+                                  (linear_attn_kernels_smallv_hd.py:336-337) */
+    FLA_ERR_SHAPE = -5,        /* negative B, H or N, or B*H*N too large */
+    FLA_ERR_STRIDE = -6,       /* strides[3] != 1, a NULL strides array, or a negative stride */
+    FLA_ERR_LAUNCH = -7,       /* the HIP runtime rejected the launch */
+    FLA_ERR_UNSUPPORTED = -8   /* no kernel was built for this combination */
+};
+
+/* ABI revision of the loaded library (== FLA_ABI_VERSION it was built with). */
+int fla_abi_version(void);
+
+/* Static, human-readable text for a status code. */
+const char *fla_strerror(int status);
+
+/* O = tril(Q K^T) V with equal head dims.
+ * Replaces linear_flash_wrapper_fwd (flashlinear/kernels/linear_attn_kernels.py:310-341)
+ * and the kernel it launches (linear_attn_kernels.py:11-100). */
+int fla_linear_attn_fwd(const void *q, const void *k, const void *v, void *o,
+                        int64_t B, int64_t H, int64_t N, int64_t D,
+                        const int64_t *q_strides, const int64_t *k_strides,
+                        const int64_t *v_strides, const int64_t *o_strides,
+                        int dtype, void *stream);
+
+/* dQ = tril(dO V^T) K,  dK = tril(dO V^T)^T Q,  dV = tril(Q K^T)^T dO, equal head dims.
+ * Replaces linear_flash_wrapper_bwd (linear_attn_kernels.py:345-384) and
+ * flash_attn_bwd (linear_attn_kernels.py:102-307).  Every element of dq, dk, dv
+ * is written; no pre-zeroing is needed. */
+int fla_linear_attn_bwd(const void *grad_out, const void *q, const void *k, const void *v,
+                        void *dq, void *dk, void *dv,
+                        int64_t B, int64_t H, int64_t N, int64_t D,
+                        const int64_t *go_strides, const int64_t *q_strides,
+                        const int64_t *k_strides, const int64_t *v_strides,
+                        const int64_t *dq_strides, const int64_t *dk_strides,
+                        const int64_t *dv_strides,
+                        int dtype, void *stream);
+
+/* Forward with q, k of width D_qk and v, o of width D_v (D_v a power of two,
+ * next_pow2(D_v) <= next_pow2(D_qk)).
+ * Replaces linear_flash_wrapper_fwd_smallv_hd
+ * (flashlinear/kernels/linear_attn_kernels_smallv_hd.py:320-359) and its
+ * kernel (linear_attn_kernels_smallv_hd.py:12-108). */
+int fla_linear_attn_smallv_fwd(const void *q, const void *k, const void *v, void *o,
+                               int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                               const int64_t *q_strides, const int64_t *k_strides,
+                               const int64_t *v_strides, const int64_t *o_strides,
+                               int dtype, void *stream);
+
+/* Backward of the above.  Replaces linear_flash_wrapper_bwd_smallv_hd
+ * (linear_attn_kernels_smallv_hd.py:363-405) and its kernel
+ * (linear_attn_kernels_smallv_hd.py:111-317).  Like the reference's backward
+ * wrapper it checks only D_qk <= 256 (linear_attn_kernels_smallv_hd.py:381). */
+int fla_linear_attn_smallv_bwd(const void *grad_out, const void *q, const void *k, const void *v,
+                               void *dq, void *dk, void *dv,
+                               int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                               const int64_t *go_strides, const int64_t *q_strides,
+                               const int64_t *k_strides, const int64_t *v_strides,
+                               const int64_t *dq_strides, const int64_t *dk_strides,
+                               const int64_t *dv_strides,
+                               int dtype, void *stream);
+
+/* The one primitive all four calls above are built from:
+ *
+ *     Out = mask(X Y^T) Z        X, Y : (B, H, N, D_c)    Z, Out : (B, H, N, D_o)
+ *
+ * mask = lower triangle incl. diagonal when upper == 0 (row >= col), upper
+ * triangle incl. diagonal when upper != 0 (row <= col).
+ *     O  = lower(Q  K^T)  V      dQ = lower(dO V^T)  K
+ *     dV = upper(K  Q^T)  dO     dK = upper(V  dO^T) Q
+ * No counterpart in the reference (its kernels inline these four products,
+ * linear_attn_kernels.py:74-82, 179-197, 291-299); exported for tests and
+ * for callers that want a single gradient. */
+int fla_tri_xyt_z(const void *x, const void *y, const void *z, void *out,
+                  int64_t B, int64_t H, int64_t N, int64_t D_c, int64_t D_o,
+                  const int64_t *x_strides, const int64_t *y_strides,
+                  const int64_t *z_strides, const int64_t *out_strides,
+                  int upper, int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* FLA_H */

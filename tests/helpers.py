@@ -1,0 +1,46 @@
+"""Shared helpers of the test-suite: error metrics and input builders."""
+
+from __future__ import annotations
+
+import math
+from typing import Tuple
+
+import torch
+
+# Tolerances against the fp32 oracle, for 16-bit storage with fp32 accumulation.
+# E1 is the reference's criterion (flashlinear/test_attn.py:17,24-25); E2 bounds
+# the worst element relative to the largest magnitude of the expected tensor.
+TOL_FRO = 1e-2
+TOL_MAX = 1e-2
+
+
+def rel_fro(x: torch.Tensor, y: torch.Tensor) -> float:
+    x, y = x.double().cpu(), y.double().cpu()
+    return float(torch.linalg.norm(x - y) / torch.linalg.norm(y).clamp_min(1e-300))
+
+
+def rel_max(x: torch.Tensor, y: torch.Tensor) -> float:
+    x, y = x.double().cpu(), y.double().cpu()
+    return float((x - y).abs().max() / y.abs().max().clamp_min(1e-300))
+
+
+def assert_close(name: str, got: torch.Tensor, want: torch.Tensor, tol_fro: float = TOL_FRO, tol_max: float = TOL_MAX):
+    assert got.shape == want.shape, f"{name}: shape {tuple(got.shape)} != {tuple(want.shape)}"
+    assert torch.isfinite(got.float()).all(), f"{name}: non-finite values"
+    e1, e2 = rel_fro(got, want), rel_max(got, want)
+    assert e1 <= tol_fro, f"{name}: Frobenius-relative error {e1:.3e} > {tol_fro}"
+    assert e2 <= tol_max, f"{name}: max-abs/max error {e2:.3e} > {tol_max}"
+
+
+def reference_style_inputs(
+    bs: int, nh: int, sq: int, hd_qk: int, hd_v: int, dtype: torch.dtype, seed: int
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Inputs distributed like the reference's tests draw them
+    (flashlinear/test_attn.py:28-46,105): q, k = softplus(randn), q scaled by
+    1/sqrt(hd); v = randn; upstream gradient 0.1 * randn.  Drawn on the CPU."""
+    g = torch.Generator().manual_seed(seed)
+    q = torch.nn.functional.softplus(torch.randn(bs, nh, sq, hd_qk, generator=g)) / math.sqrt(hd_qk)
+    k = torch.nn.functional.softplus(torch.randn(bs, nh, sq, hd_qk, generator=g))
+    v = torch.randn(bs, nh, sq, hd_v, generator=g)
+    dy = 0.1 * torch.randn(bs, nh, sq, hd_v, generator=g)
+    return tuple(t.to(dtype) for t in (q, k, v, dy))

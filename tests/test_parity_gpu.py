@@ -1,0 +1,189 @@
+"""GPU parity of the HIP path against the CPU oracle (``-m gpu``).
+
+Every case calls the operators through the package, i.e. through the C ABI of
+libfla_gfx950.so.  The oracle consumes the already rounded 16-bit inputs in
+fp32, so input quantisation is not charged as error.
+"""
+
+import pytest
+import torch
+
+from flashy_linear_attention_amd import LinearAttention, LinearAttentionSmallVHD
+from flashy_linear_attention_amd.kernels import (
+    linear_flash_wrapper_bwd,
+    linear_flash_wrapper_bwd_smallv_hd,
+    linear_flash_wrapper_fwd,
+    linear_flash_wrapper_fwd_smallv_hd,
+)
+from oracle import naive
+
+from helpers import assert_close, reference_style_inputs
+
+pytestmark = pytest.mark.gpu
+
+# (batch, heads, seq, head_dim): the first cases the reference's four equal-D
+# tests draw (flashlinear/test_attn.py:65-74,89-98,121-131,145-155 with numpy
+# seed 0), then edges: one tile, tile boundaries, every padded width, widths
+# that are not a multiple of 8 (scalar load path), head dims above 128.
+EQUAL_D_CASES = [
+    (1, 4, 512, 64),
+    (3, 3, 1984, 128),
+    (2, 21, 256, 25),
+    (1, 27, 1344, 91),
+    (1, 1, 64, 32),
+    (1, 2, 128, 16),
+    (2, 3, 192, 64),
+    (1, 2, 320, 128),
+    (1, 9, 576, 48),
+    (1, 2, 256, 256),
+    (1, 3, 448, 200),
+    (1, 1, 1024, 17),
+]
+
+# (batch, heads, seq, hd_qk, hd_v): reference small-V envelope
+# (flashlinear/test_attn_smallv_hd.py:69-79) plus the 256/64 Taylor-feature shape.
+SMALL_V_CASES = [
+    (1, 4, 512, 64, 16),
+    (2, 5, 1984, 128, 32),
+    (1, 7, 256, 37, 16),
+    (1, 3, 1344, 91, 32),
+    (1, 2, 64, 32, 32),
+    (1, 2, 384, 256, 64),
+    (1, 2, 320, 128, 128),
+    (1, 2, 192, 100, 8),
+]
+
+
+def _oracle_fwd(q, k, v):
+    return naive.causal_dot_product(q.float().cpu(), k.float().cpu(), v.float().cpu())
+
+
+def _oracle_bwd(q, k, v, dy):
+    return naive.causal_dot_product_grads_autograd(q.float().cpu(), k.float().cpu(), v.float().cpu(), dy.float().cpu())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("dims", EQUAL_D_CASES, ids=lambda d: "x".join(map(str, d)))
+def test_attn_fwd(dims, dtype, gpu_device):
+    bs, nh, sq, hd = dims
+    q, k, v, _ = reference_style_inputs(bs, nh, sq, hd, hd, dtype, seed=sum(dims))
+    want = _oracle_fwd(q, k, v)
+    with torch.no_grad():
+        got = LinearAttention.apply(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device))
+    assert got.dtype == dtype and got.shape == q.shape
+    assert_close("O", got, want)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("dims", EQUAL_D_CASES, ids=lambda d: "x".join(map(str, d)))
+def test_attn_bwd(dims, dtype, gpu_device):
+    bs, nh, sq, hd = dims
+    q, k, v, dy = reference_style_inputs(bs, nh, sq, hd, hd, dtype, seed=sum(dims) + 1)
+    dq_w, dk_w, dv_w = _oracle_bwd(q, k, v, dy)
+    qg, kg, vg = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v))
+    out = LinearAttention.apply(qg, kg, vg)
+    out.backward(dy.to(gpu_device))
+    for name, got, want, like in (("dQ", qg.grad, dq_w, q), ("dK", kg.grad, dk_w, k), ("dV", vg.grad, dv_w, v)):
+        assert got.dtype == dtype and got.shape == like.shape
+        assert_close(name, got, want)
+
+
+@pytest.mark.parametrize("dims", SMALL_V_CASES, ids=lambda d: "x".join(map(str, d)))
+def test_attn_smallv_fwd(dims, gpu_device):
+    bs, nh, sq, hd_qk, hd_v = dims
+    q, k, v, _ = reference_style_inputs(bs, nh, sq, hd_qk, hd_v, torch.bfloat16, seed=sum(dims))
+    want = _oracle_fwd(q, k, v)
+    with torch.no_grad():
+        got = LinearAttentionSmallVHD.apply(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device))
+    assert got.dtype == torch.bfloat16 and got.shape == v.shape
+    assert_close("O", got, want)
+
+
+@pytest.mark.parametrize("dims", SMALL_V_CASES, ids=lambda d: "x".join(map(str, d)))
+def test_attn_smallv_bwd(dims, gpu_device):
+    bs, nh, sq, hd_qk, hd_v = dims
+    q, k, v, dy = reference_style_inputs(bs, nh, sq, hd_qk, hd_v, torch.bfloat16, seed=sum(dims) + 1)
+    dq_w, dk_w, dv_w = _oracle_bwd(q, k, v, dy)
+    qg, kg, vg = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v))
+    LinearAttentionSmallVHD.apply(qg, kg, vg).backward(dy.to(gpu_device))
+    for name, got, want in (("dQ", qg.grad, dq_w), ("dK", kg.grad, dk_w), ("dV", vg.grad, dv_w)):
+        assert_close(name, got, want)
+
+
+def test_wrappers_return_fresh_contiguous_outputs(gpu_device):
+    q, k, v, dy = (t.to(gpu_device) for t in reference_style_inputs(1, 2, 128, 64, 64, torch.bfloat16, 5))
+    out = linear_flash_wrapper_fwd(q, k, v)
+    dq, dk, dv = linear_flash_wrapper_bwd(dy, q, k, v)
+    for t in (out, dq, dk, dv):
+        assert t.is_contiguous() and t.shape == q.shape and t.dtype == q.dtype
+    q2, k2, v2, dy2 = (t.to(gpu_device) for t in reference_style_inputs(1, 2, 128, 64, 32, torch.bfloat16, 6))
+    out2 = linear_flash_wrapper_fwd_smallv_hd(q2, k2, v2)
+    dq2, dk2, dv2 = linear_flash_wrapper_bwd_smallv_hd(dy2, q2, k2, v2)
+    assert out2.shape == v2.shape and dq2.shape == q2.shape and dk2.shape == k2.shape and dv2.shape == v2.shape
+
+
+def test_non_contiguous_layouts(gpu_device):
+    """(B, N, H, D) storage viewed as (B, H, N, D), and a sliced head dim."""
+    bs, nh, sq, hd = 2, 3, 256, 64
+    q, k, v, dy = reference_style_inputs(bs, nh, sq, hd, hd, torch.bfloat16, seed=11)
+    want = _oracle_fwd(q, k, v)
+    dq_w, dk_w, dv_w = _oracle_bwd(q, k, v, dy)
+
+    def bnhd(t):  # same values, sequence-major storage
+        return t.to(gpu_device).transpose(1, 2).contiguous().transpose(1, 2)
+
+    qg, kg, vg = (bnhd(t).requires_grad_(True) for t in (q, k, v))
+    assert not qg.is_contiguous()
+    out = LinearAttention.apply(qg, kg, vg)
+    assert_close("O", out, want)
+    out.backward(bnhd(dy))
+    assert_close("dQ", qg.grad, dq_w)
+    assert_close("dK", kg.grad, dk_w)
+    assert_close("dV", vg.grad, dv_w)
+
+    wide = torch.zeros(bs, nh, sq, 2 * hd, dtype=torch.bfloat16, device=gpu_device)
+    wide[..., ::2] = q.to(gpu_device)
+    strided_q = wide[..., ::2]  # innermost stride 2: the wrapper must densify it
+    with torch.no_grad():
+        out2 = LinearAttention.apply(strided_q, k.to(gpu_device), v.to(gpu_device))
+    assert torch.equal(out2, out.detach())
+
+
+def test_autocast_casts_to_bf16(gpu_device):
+    """Under autocast fp32 inputs are cast to bf16 (flashlinear/linear_attn.py:13)."""
+    q, k, v, _ = reference_style_inputs(1, 2, 128, 64, 64, torch.float32, seed=3)
+    with torch.autocast("cuda", dtype=torch.bfloat16), torch.no_grad():
+        got = LinearAttention.apply(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device))
+    assert got.dtype == torch.bfloat16
+    want = _oracle_fwd(q.bfloat16(), k.bfloat16(), v.bfloat16())
+    assert_close("O", got, want)
+
+
+def test_fp32_inputs_rejected(gpu_device):
+    q, k, v, _ = (t.to(gpu_device) for t in reference_style_inputs(1, 1, 64, 32, 32, torch.float32, seed=3))
+    with pytest.raises(TypeError):
+        LinearAttention.apply(q, k, v)
+
+
+def test_end_to_end_with_pytorch_denominator(gpu_device):
+    """The README recipe (README.md:27-30): kernel output divided by a PyTorch
+    denominator; gradients flow through both the kernel and the denominator."""
+    from flashy_linear_attention_amd.synthetic import WORKLOADS, make_inputs
+
+    w = WORKLOADS["C1"]
+    q, k, v, dy = make_inputs(w)  # fp32, B=1 H=2 N=256 D=64, elu+1 features
+    q16, k16, v16 = (t.bfloat16() for t in (q, k, v))
+
+    qo, ko, vo = (t.float().requires_grad_(True) for t in (q16, k16, v16))
+    want = naive.linear_attention_normalised(qo, ko, vo, eps=1e-5)
+    want.backward(dy)
+
+    qg, kg, vg = (t.to(gpu_device).requires_grad_(True) for t in (q16, k16, v16))
+    num = LinearAttention.apply(qg, kg, vg)
+    denom = (qg.float() * kg.float().cumsum(-2)).sum(dim=-1, keepdim=True) + 1e-5
+    got = num.float() / denom
+    got.backward(dy.to(gpu_device))
+    assert_close("out", got, want.detach())
+    assert_close("dQ", qg.grad, qo.grad)
+    assert_close("dK", kg.grad, ko.grad)
+    assert_close("dV", vg.grad, vo.grad)
