@@ -1,0 +1,194 @@
+#!/usr/bin/env python3
+"""Benchmark of the causal-linear-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C3]
+
+One step = one forward (``linear_flash_wrapper_fwd``) plus one backward
+(``linear_flash_wrapper_bwd``) over one synthetic batch of the workload, through
+the C ABI of libfla_gfx950.so, inputs resident in HBM.  The default workload is
+the one the headline metric is quoted on: bf16, B=4 H=32 N=4096 D_qk=D_v=128.
+
+Prints ONE JSON line.  ``value`` is causal-counted algorithmic TFLOP/s of the
+whole step, N^2 (4 D_qk + 3 D_v) per (b, h) (five products: S, dS, dV, dK, dQ
+in backward, two in forward).  ``roofline`` describes the one kernel every
+launch of the step runs (Out = mask(X Y^T) Z; forward is one launch, backward
+three): algorithmic FLOPs of one launch, N^2 (D_c + D_o) B H, over the average
+launch duration measured here with HIP events on the launch stream, against
+the dense bf16 MFMA peak.  ``cpu_baseline`` times the oracle's naive PyTorch
+formula on the host cores over a bounded sample (whole (b, h) slices at full N
+and D), in the same unit.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0}  # MI355X dense MFMA, published
+HBM_PEAK_GBS = 8000.0
+
+
+def _parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU oracle timing")
+    ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target seconds of CPU work for the baseline")
+    return ap.parse_args()
+
+
+def _time_region(torch, fn, steps):
+    """Milliseconds for `steps` calls of fn, HIP events on the current stream."""
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1)
+
+
+def _cpu_baseline(torch, w, target_seconds):
+    """The oracle's naive formula, fp32, on the host: whole (b, h) slices of the
+    workload at full N and D, forward (+ backward), until ~target_seconds."""
+    from flashy_linear_attention_amd.synthetic import make_inputs
+    from oracle import naive
+
+    q, k, v, do = (t.float() for t in make_inputs(w, seed=1, batch=1, heads=1))
+    flops_slice = (w.flops_fwd + (w.flops_bwd if w.backward else 0.0)) / (w.batch * w.heads)
+
+    def one():
+        naive.causal_dot_product_blocked(q, k, v, block=2048)
+        if w.backward:
+            naive.causal_dot_product_grads_blocked(q, k, v, do, block=2048)
+
+    one()  # warm-up (thread pool, allocator)
+    n, t0 = 0, time.perf_counter()
+    while True:
+        one()
+        n += 1
+        dt = time.perf_counter() - t0
+        if dt >= target_seconds or n >= 4 * w.batch * w.heads:
+            break
+    return {
+        "value": round(flops_slice * n / dt / 1e12, 4),
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"{n} of {w.batch * w.heads} (b,h) slices at full N={w.seq}, D_qk={w.d_qk}, D_v={w.d_v}, "
+                  f"fp32 naive PyTorch fwd{'+bwd' if w.backward else ''}, {dt:.1f} s; os.cpu_count()={os.cpu_count()}",
+        "ms_per_step_extrapolated": round(dt / n * w.batch * w.heads * 1e3, 1),
+    }
+
+
+def main() -> int:
+    args = _parse()
+    if args.gpus != 1:
+        print("bench.py: this build runs the hot path on ONE GPU only (every (batch, head) slice is independent; "
+              "no collective exists on this path). Re-run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from flashy_linear_attention_amd import _lib
+    from flashy_linear_attention_amd.kernels import (
+        linear_flash_wrapper_bwd,
+        linear_flash_wrapper_bwd_smallv_hd,
+        linear_flash_wrapper_fwd,
+        linear_flash_wrapper_fwd_smallv_hd,
+    )
+    from flashy_linear_attention_amd.synthetic import WORKLOADS, make_inputs
+
+    if not torch.cuda.is_available():
+        print("bench.py: no ROCm GPU visible", file=sys.stderr)
+        return 2
+    _lib.load()  # fails loudly if the HIP library is missing
+
+    w = WORKLOADS[args.workload]
+    dev = torch.device("cuda:0")
+    q, k, v, do = (t.to(dev) for t in make_inputs(w, seed=0))
+    fwd = linear_flash_wrapper_fwd_smallv_hd if w.small_v else linear_flash_wrapper_fwd
+    bwd = linear_flash_wrapper_bwd_smallv_hd if w.small_v else linear_flash_wrapper_bwd
+
+    def step():
+        fwd(q, k, v)
+        if w.backward:
+            bwd(do, q, k, v)
+
+    for _ in range(args.warmup):
+        step()
+    ms_total = _time_region(torch, step, args.steps)
+    ms_step = ms_total / args.steps
+
+    # secondary figures: each half alone (same event method)
+    ms_fwd = _time_region(torch, lambda: fwd(q, k, v), args.steps) / args.steps
+    ms_bwd = _time_region(torch, lambda: bwd(do, q, k, v), args.steps) / args.steps if w.backward else None
+
+    flops_step = w.flops_fwd + (w.flops_bwd if w.backward else 0.0)
+    dt_name = {torch.bfloat16: "bf16", torch.float16: "f16"}[w.dtype]
+    peak = PEAK_TFLOPS[dt_name]
+    tflops = flops_step / (ms_step * 1e-3) / 1e12
+
+    # dominant (only) kernel: launches per step and algorithmic FLOPs per launch
+    launches = 1 + (3 if w.backward else 0)
+    flops_launch = float(w.batch * w.heads) * w.seq * w.seq * (w.d_qk + w.d_v)
+    ms_launch = ms_step / launches
+    achieved = flops_launch / (ms_launch * 1e-3) / 1e12
+
+    result = {
+        "metric": f"causal linear attention {'fwd+bwd' if w.backward else 'fwd'} TFLOP/s "
+                  f"(causal-counted), B={w.batch} H={w.heads} N={w.seq} D_qk={w.d_qk} D_v={w.d_v}, 1 MI355X",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dt_name,
+        "data": "synthetic",
+        "config": {
+            "workload": f"{w.name}: LinearAttention{'SmallVHD' if w.small_v else ''} "
+                        f"{'fwd+bwd' if w.backward else 'fwd'}, {dt_name}, B={w.batch} H={w.heads} N={w.seq} "
+                        f"D_qk={w.d_qk} D_v={w.d_v}, q/k features {w.features}, v and dO randn, seed 0",
+            "flops_per_step": flops_step,
+            "fwd_ms": round(ms_fwd, 4),
+            "bwd_ms": None if ms_bwd is None else round(ms_bwd, 4),
+            "fwd_tflops": round(w.flops_fwd / (ms_fwd * 1e-3) / 1e12, 2),
+            "bwd_tflops": None if ms_bwd is None else round(w.flops_bwd / (ms_bwd * 1e-3) / 1e12, 2),
+            "pct_of_mfma_peak": round(100.0 * tflops / peak, 2),
+        },
+        "roofline": {
+            "bound": "mfma",
+            "kernel": "fla::tri_xyt_z_kernel (Out = mask(X Y^T) Z)",
+            "achieved": round(achieved, 2),
+            "peak": peak,
+            "unit": "TFLOP/s",
+            "frac": round(achieved / peak, 4),
+            "traffic": None,
+            "launches_per_step": launches,
+            "flops_per_launch": flops_launch,
+            "avg_launch_ms": round(ms_launch, 4),
+        },
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = _cpu_baseline(torch, w, args.cpu_seconds)
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

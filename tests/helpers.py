@@ -15,12 +15,12 @@ TOL_MAX = 1e-2
 
 
 def rel_fro(x: torch.Tensor, y: torch.Tensor) -> float:
-    x, y = x.double().cpu(), y.double().cpu()
+    x, y = x.detach().double().cpu(), y.detach().double().cpu()
     return float(torch.linalg.norm(x - y) / torch.linalg.norm(y).clamp_min(1e-300))
 
 
 def rel_max(x: torch.Tensor, y: torch.Tensor) -> float:
-    x, y = x.double().cpu(), y.double().cpu()
+    x, y = x.detach().double().cpu(), y.detach().double().cpu()
     return float((x - y).abs().max() / y.abs().max().clamp_min(1e-300))
 
 
@@ -44,3 +44,19 @@ def reference_style_inputs(
     v = torch.randn(bs, nh, sq, hd_v, generator=g)
     dy = 0.1 * torch.randn(bs, nh, sq, hd_v, generator=g)
     return tuple(t.to(dtype) for t in (q, k, v, dy))
+
+
+def load_golden(name: str):
+    """A fixture from tests/golden as torch tensors: bf16 inputs, fp32 expected outputs."""
+    import os
+
+    import numpy as np
+
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name + ".npz")
+    z = np.load(path, allow_pickle=False)
+    ins = {n: torch.from_numpy(z[n + "_bf16"].view(np.int16).copy()).view(torch.bfloat16) for n in ("q", "k", "v", "do")}
+    outs = {n: torch.from_numpy(z[n].copy()) for n in ("o", "dq", "dk", "dv")}
+    return ins, outs
+
+
+GOLDEN_CASES = ("equal_d_b1_h1_n128_d32", "small_v_b1_h1_n128_dqk64_dv16")

@@ -1,0 +1,142 @@
+"""Host-side checks that run without a GPU: the shared library loads and exports
+the declared ABI, argument validation in the C ABI and in the Python wrappers,
+and the oracle against the committed golden fixtures."""
+
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from flashy_linear_attention_amd import LinearAttention, LinearAttentionSmallVHD, _lib
+from flashy_linear_attention_amd import kernels
+from flashy_linear_attention_amd.synthetic import WORKLOADS, make_inputs
+from oracle import c_oracle, naive
+
+from helpers import GOLDEN_CASES, load_golden
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "fla.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(fla_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = _lib.load()
+    names = _declared_functions()
+    assert {"fla_linear_attn_fwd", "fla_linear_attn_bwd", "fla_linear_attn_smallv_fwd",
+            "fla_linear_attn_smallv_bwd", "fla_tri_xyt_z", "fla_abi_version", "fla_strerror"} <= set(names)
+    for n in names:
+        assert hasattr(lib, n), f"{n} is declared in include/fla.h but not exported"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature"
+    assert lib.fla_abi_version() == _lib.ABI_VERSION
+
+
+def test_package_surface_matches_reference_names():
+    """flashlinear/__init__.py:1-2 and flashlinear/kernels/__init__.py:1-5."""
+    assert issubclass(LinearAttention, torch.autograd.Function)
+    assert issubclass(LinearAttentionSmallVHD, torch.autograd.Function)
+    for n in ("linear_flash_wrapper_fwd", "linear_flash_wrapper_bwd",
+              "linear_flash_wrapper_fwd_smallv_hd", "linear_flash_wrapper_bwd_smallv_hd"):
+        assert callable(getattr(kernels, n))
+
+
+def _null_call(name, *tail):
+    fn = getattr(_lib.load(), name)
+    nptr = {"fla_linear_attn_fwd": 4, "fla_linear_attn_bwd": 7, "fla_linear_attn_smallv_fwd": 4,
+            "fla_linear_attn_smallv_bwd": 7, "fla_tri_xyt_z": 4}[name]
+    return fn, nptr
+
+
+S = (ctypes.c_int64 * 4)(4096, 2048, 32, 1)
+BAD_S = (ctypes.c_int64 * 4)(4096, 2048, 64, 2)
+P = ctypes.c_void_p(0x1000)  # never dereferenced: every call below fails validation first
+
+
+def test_c_abi_validation_codes():
+    lib = _lib.load()
+    f = lib.fla_linear_attn_fwd
+    assert f(P, P, P, P, 1, 2, 64, 32, S, S, S, S, 7, None) == -2          # dtype
+    assert f(P, P, P, P, 1, 2, 64, 257, S, S, S, S, 0, None) == -3         # head dim
+    assert f(P, P, P, P, 1, 2, 64, 0, S, S, S, S, 0, None) == -3
+    assert f(P, P, P, P, -1, 2, 64, 32, S, S, S, S, 0, None) == -5         # shape
+    assert f(None, P, P, P, 1, 2, 64, 32, S, S, S, S, 0, None) == -1       # null pointer
+    assert f(P, P, P, P, 1, 2, 64, 32, S, BAD_S, S, S, 0, None) == -6      # innermost stride
+    assert f(P, P, P, P, 1, 2, 64, 32, S, S, None, S, 0, None) == -6       # missing strides
+    assert f(P, P, P, P, 0, 2, 64, 32, S, S, S, S, 0, None) == 0           # empty problem: no-op
+    assert f(P, P, P, P, 1, 2, 0, 32, S, S, S, S, 1, None) == 0
+    b = lib.fla_linear_attn_bwd
+    assert b(P, P, P, P, P, P, P, 1, 2, 64, 300, S, S, S, S, S, S, S, 0, None) == -3
+    assert b(P, P, P, P, P, None, P, 1, 2, 64, 32, S, S, S, S, S, S, S, 0, None) == -1
+    sf = lib.fla_linear_attn_smallv_fwd
+    assert sf(P, P, P, P, 1, 2, 64, 64, 24, S, S, S, S, 0, None) == -4     # D_v not a power of two
+    assert sf(P, P, P, P, 1, 2, 64, 32, 64, S, S, S, S, 0, None) == -4     # D_v above padded D_qk
+    assert sf(P, P, P, P, 1, 2, 64, 300, 64, S, S, S, S, 0, None) == -3
+    assert sf(P, P, P, P, 1, 0, 64, 37, 64, S, S, S, S, 0, None) == 0      # 64 <= next_pow2(37): accepted
+    sb = lib.fla_linear_attn_smallv_bwd
+    assert sb(P, P, P, P, P, P, P, 1, 2, 64, 257, 16, S, S, S, S, S, S, S, 0, None) == -3
+    t = lib.fla_tri_xyt_z
+    assert t(P, P, P, P, 1, 2, 64, 32, 300, S, S, S, S, 0, 0, None) == -3
+    assert t(P, P, P, P, 1, 2, 64, 32, 32, S, S, S, S, 1, 5, None) == -2
+    for code in range(0, -9, -1):
+        assert lib.fla_strerror(code)
+    assert lib.fla_strerror(-3) == b"Only head_dims <= 256 are supported."
+
+
+def test_wrapper_assertions_match_reference():
+    """The reference raises AssertionError before launching
+    (linear_attn_kernels.py:322-325,361-364; linear_attn_kernels_smallv_hd.py:336-342,381-384)."""
+    z = lambda *s: torch.zeros(*s, dtype=torch.bfloat16)
+    with pytest.raises(AssertionError, match="Only head_dims <= 256"):
+        kernels.linear_flash_wrapper_fwd(z(1, 1, 64, 320), z(1, 1, 64, 320), z(1, 1, 64, 320))
+    with pytest.raises(AssertionError, match="multiple of 64"):
+        kernels.linear_flash_wrapper_fwd(z(1, 1, 96, 64), z(1, 1, 96, 64), z(1, 1, 96, 64))
+    with pytest.raises(AssertionError, match="multiple of 32"):
+        kernels.linear_flash_wrapper_fwd(z(1, 1, 48, 200), z(1, 1, 48, 200), z(1, 1, 48, 200))
+    with pytest.raises(AssertionError, match="multiple of 64"):
+        kernels.linear_flash_wrapper_bwd(z(1, 1, 100, 64), z(1, 1, 100, 64), z(1, 1, 100, 64), z(1, 1, 100, 64))
+    with pytest.raises(AssertionError, match="power of 2"):
+        kernels.linear_flash_wrapper_fwd_smallv_hd(z(1, 1, 64, 64), z(1, 1, 64, 64), z(1, 1, 64, 24))
+    with pytest.raises(AssertionError, match="less than Query/Key"):
+        kernels.linear_flash_wrapper_fwd_smallv_hd(z(1, 1, 64, 32), z(1, 1, 64, 32), z(1, 1, 64, 64))
+    with pytest.raises(AssertionError, match="Only head_dims <= 256"):
+        kernels.linear_flash_wrapper_bwd_smallv_hd(z(1, 1, 64, 16), z(1, 1, 64, 260), z(1, 1, 64, 260), z(1, 1, 64, 16))
+    with pytest.raises(AssertionError, match="multiple of 64"):
+        kernels.linear_flash_wrapper_bwd_smallv_hd(z(1, 1, 96, 16), z(1, 1, 96, 64), z(1, 1, 96, 64), z(1, 1, 96, 16))
+
+
+def test_cpu_tensors_fail_loudly_instead_of_falling_back():
+    q = torch.ones(1, 1, 64, 32, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="ROCm GPU"):
+        LinearAttention.apply(q, q, q)
+    with pytest.raises(RuntimeError, match="ROCm GPU"):
+        LinearAttentionSmallVHD.apply(q, q, q)
+
+
+@pytest.mark.parametrize("name", GOLDEN_CASES)
+def test_oracle_reproduces_golden_fixtures(name):
+    ins, outs = load_golden(name)
+    q, k, v, do = (ins[n].float() for n in ("q", "k", "v", "do"))
+    torch.testing.assert_close(naive.causal_dot_product(q, k, v), outs["o"], rtol=2e-5, atol=2e-4)
+    for got, n in zip(naive.causal_dot_product_grads(q, k, v, do), ("dq", "dk", "dv")):
+        torch.testing.assert_close(got, outs[n], rtol=2e-5, atol=2e-4)
+    np.testing.assert_allclose(c_oracle.fwd(q, k, v), outs["o"].numpy(), rtol=2e-6, atol=2e-5)
+    for got, n in zip(c_oracle.bwd(q, k, v, do), ("dq", "dk", "dv")):
+        np.testing.assert_allclose(got, outs[n].numpy(), rtol=2e-6, atol=2e-5)
+
+
+def test_synthetic_workloads_have_the_stated_shapes_and_features():
+    w = WORKLOADS["C3"]
+    assert (w.batch, w.heads, w.seq, w.d_qk, w.d_v, w.dtype) == (4, 32, 4096, 128, 128, torch.bfloat16)
+    assert abs(w.flops_fwd + w.flops_bwd - 1.924e12) < 1e9
+    q, k, v, do = make_inputs(WORKLOADS["C4"], batch=1, heads=1, seq=64)
+    assert q.shape == (1, 1, 64, 256) and v.shape == (1, 1, 64, 64) and q.dtype == torch.bfloat16
+    q1, k1, v1, _ = make_inputs(WORKLOADS["C2"], batch=1, heads=2, seq=64)
+    assert (q1 > 0).all() and (k1 > 0).all() and q1.dtype == torch.float16
+    q2, *_ = make_inputs(WORKLOADS["C2"], batch=1, heads=2, seq=64)
+    assert torch.equal(q1, q2)

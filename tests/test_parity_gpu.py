@@ -165,25 +165,63 @@ def test_fp32_inputs_rejected(gpu_device):
         LinearAttention.apply(q, k, v)
 
 
+class _RoundedOracleOp(torch.autograd.Function):
+    """The oracle's arithmetic with the operator's storage contract: output and
+    gradients are rounded to bf16 once, as LinearAttention stores them."""
+
+    @staticmethod
+    def forward(ctx, q, k, v):
+        ctx.save_for_backward(q, k, v)
+        return naive.causal_dot_product(q.float(), k.float(), v.float()).bfloat16()
+
+    @staticmethod
+    def backward(ctx, g):
+        q, k, v = ctx.saved_tensors
+        return tuple(t.bfloat16() for t in naive.causal_dot_product_grads(q.float(), k.float(), v.float(), g.float()))
+
+
 def test_end_to_end_with_pytorch_denominator(gpu_device):
-    """The README recipe (README.md:27-30): kernel output divided by a PyTorch
-    denominator; gradients flow through both the kernel and the denominator."""
+    """The README recipe (README.md:27-30) on the fp32 CPU-baseline workload
+    (B=1 H=2 N=256 D=64, elu+1 features): kernel output divided by a PyTorch
+    denominator; gradients flow through both the kernel and the denominator.
+
+    The gradient of a normalised average with respect to q is a small difference
+    of two terms of order 1, each of which passes through 16-bit storage (the
+    operator's output and its dQ).  In the first rows, where a single key
+    contributes, the exact gradient is ~1e-7 while one bf16 ulp of the cancelling
+    terms is 2^-8 = 3.9e-3, i.e. 2.9e-2 of the largest gradient magnitude
+    (0.137): any 16-bit implementation lands within an ulp or two of that, in
+    either direction.  So for the gradients the element bound is 5e-2 of the
+    largest magnitude (against both the fp32 recipe and the oracle with the same
+    storage roundings), while the Frobenius bound stays at 1e-2 and the output
+    itself keeps both 1e-2 bounds.
+    """
     from flashy_linear_attention_amd.synthetic import WORKLOADS, make_inputs
 
     w = WORKLOADS["C1"]
-    q, k, v, dy = make_inputs(w)  # fp32, B=1 H=2 N=256 D=64, elu+1 features
+    q, k, v, dy = make_inputs(w)
     q16, k16, v16 = (t.bfloat16() for t in (q, k, v))
+
+    def recipe(op, qq, kk, vv, grad):
+        num = op(qq, kk, vv)
+        denom = (qq.float() * kk.float().cumsum(-2)).sum(dim=-1, keepdim=True) + 1e-5
+        out = num.float() / denom
+        out.backward(grad)
+        return out.detach()
 
     qo, ko, vo = (t.float().requires_grad_(True) for t in (q16, k16, v16))
     want = naive.linear_attention_normalised(qo, ko, vo, eps=1e-5)
     want.backward(dy)
 
+    qr, kr, vr = (t.clone().requires_grad_(True) for t in (q16, k16, v16))
+    want_rounded = recipe(_RoundedOracleOp.apply, qr, kr, vr, dy)
+
     qg, kg, vg = (t.to(gpu_device).requires_grad_(True) for t in (q16, k16, v16))
-    num = LinearAttention.apply(qg, kg, vg)
-    denom = (qg.float() * kg.float().cumsum(-2)).sum(dim=-1, keepdim=True) + 1e-5
-    got = num.float() / denom
-    got.backward(dy.to(gpu_device))
+    got = recipe(LinearAttention.apply, qg, kg, vg, dy.to(gpu_device))
+
     assert_close("out", got, want.detach())
-    assert_close("dQ", qg.grad, qo.grad)
-    assert_close("dK", kg.grad, ko.grad)
-    assert_close("dV", vg.grad, vo.grad)
+    assert_close("out vs rounded oracle", got, want_rounded, tol_fro=4e-3, tol_max=8e-3)
+    for name, g, exact, rounded in (("dQ", qg.grad, qo.grad, qr.grad), ("dK", kg.grad, ko.grad, kr.grad),
+                                    ("dV", vg.grad, vo.grad, vr.grad)):
+        assert_close(name + " vs fp32 recipe", g, exact, tol_fro=1e-2, tol_max=5e-2)
+        assert_close(name + " vs rounded oracle", g, rounded, tol_fro=1e-2, tol_max=5e-2)
