@@ -1,6 +1,7 @@
 // One kernel instantiation per compilation: build with
 //   -DFLA_INST_DTYPE={0 bf16 | 1 f16} -DFLA_INST_DC=<32|64|128|256> -DFLA_INST_DO=<32|64|128|256>
 #include "fla_dispatch.h"
+#include "fla_tri_fast.h"
 
 #if !defined(FLA_INST_DTYPE) || !defined(FLA_INST_DC) || !defined(FLA_INST_DO)
 #error "define FLA_INST_DTYPE, FLA_INST_DC and FLA_INST_DO"
@@ -15,6 +16,11 @@ using InstT = _Float16;
 #endif
 
 hipError_t FLA_LAUNCH_NAME(FLA_INST_DTYPE, FLA_INST_DC, FLA_INST_DO)(const TriParams &p, hipStream_t stream) {
+    // aligned operands take the LDS-DMA pipelined kernel; anything else (odd
+    // widths, unaligned rows, slices beyond 1 GiB, tiles too big for three LDS
+    // stages) takes the bounds-checked generic kernel
+    if (FastConfig<FLA_INST_DC, FLA_INST_DO>::kSupported && fast_path_ok(p))
+        return launch_tri_fast<InstT, FLA_INST_DC, FLA_INST_DO>(p, stream);
     return launch_tri<InstT, FLA_INST_DC, FLA_INST_DO>(p, stream);
 }
 

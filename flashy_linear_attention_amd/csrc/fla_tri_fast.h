@@ -1,0 +1,401 @@
+// Fast path of Out = mask(X Y^T) Z for 16-byte aligned operands.
+//
+// Same mathematics and the same MFMA operand chaining as fla_tri_kernel.h (S^T
+// accumulators feed the second product straight from registers, Z is read with
+// ds_read_b64_tr_b16).  What differs is how data moves and how the loop is
+// pipelined:
+//
+//   * Y/Z tiles (BN = 64 rows) go HBM -> LDS with buffer_load_dwordx4 ... lds
+//     (no staging registers, no ds_write), into a ring of three LDS buffers.
+//     One wave instruction fills 1 KiB of LDS in lane order, so the bank
+//     spreading that padding would give is done by an XOR swizzle of the
+//     16-byte chunk index instead: a lane fetches the global chunk that belongs
+//     at its LDS slot.  Rows beyond N and chunks beyond the real width are
+//     pointed outside the buffer resource and arrive as zeros.
+//   * The walk over tiles that lie entirely inside the mask is software
+//     pipelined per 32-row sub-tile s, with no masking code at all:
+//         phase 1:  S_s = Y_s X^T       | fetch Z fragments of s-1 from LDS
+//         phase 2:  Out += P_{s-1} Z_{s-1} | fetch Y fragments of s+1, round S_s to P_s
+//     so every LDS read is issued about half an iteration (~500 cycles) before
+//     its MFMA and the two MFMA chains of a phase are independent.
+//     One barrier per tile, placed between the phases of the tile's second
+//     sub-tile: it publishes the next tile and retires the previous one.
+//   * The BM x BM block on the diagonal is handled afterwards by a plain
+//     S -> mask -> P -> PV sequence per sub-tile that skips the (block, sub-tile)
+//     pairs the mask removes entirely.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include <type_traits>
+
+#include "fla_tri_kernel.h"
+
+namespace fla {
+
+typedef __attribute__((address_space(3))) void *lds_void_ptr;
+typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+
+constexpr uint32_t kOobOffset = 0x40000000u;  // added to a buffer offset to force an out-of-range (zero) access
+constexpr int64_t kMaxFastExtent = 0x3fffffff;  // per-(b,h) byte extent the 32-bit buffer offsets can address
+
+template <int DC, int DO>
+struct FastConfig {
+    static constexpr int MW = TriConfig<DC, DO>::MW;
+    static constexpr int NW = 4;
+    static constexpr int BM = MW * NW;
+    static constexpr int BN = 64;
+    static constexpr int NBUF = 3;
+    static constexpr int RY = DC * 2, RZ = DO * 2;  // LDS row bytes (no padding)
+    static constexpr int CY = DC / 8, CZ = DO / 8;  // 16-byte chunks per row
+    static constexpr int Y_BYTES = BN * RY, Z_BYTES = BN * RZ;
+    static constexpr int STAGE_BYTES = Y_BYTES + Z_BYTES;
+    static constexpr int SMEM_BYTES = NBUF * STAGE_BYTES;
+    static constexpr bool kSupported = SMEM_BYTES <= 160 * 1024;
+    // wave-level 1 KiB DMA instructions per tile and wave
+    static constexpr int NIY = Y_BYTES / 4096, NIZ = Z_BYTES / 4096;
+    static_assert(Y_BYTES % 4096 == 0 && Z_BYTES % 4096 == 0, "tile must split into 1 KiB blocks over 4 waves");
+};
+
+// XOR applied to the chunk index of LDS row `row` (row counted inside the tile).
+template <int CY>
+__device__ __forceinline__ int swizzle_y(int row) {
+    if constexpr (CY == 4) return (row >> 1) & 3;   // 64-byte rows: two rows share 128 bytes
+    else if constexpr (CY == 8) return row & 7;
+    else return row & 15;
+}
+template <int CZ>
+__device__ __forceinline__ int swizzle_z(int row) {
+    if constexpr (CZ == 4) return ((row >> 1) & 1) << 1;
+    else return (row & 3) << 1;  // the 4 rows of one transposing read land in 4 different 32-byte slots
+}
+
+template <typename T, int DC, int DO>
+__global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) {
+    // The body is compiled in the device pass only: hipcc's host pass silently
+    // drops the launch stub of a kernel template whose body calls the LDS-DMA
+    // builtin from inside a lambda, and the host needs nothing but the stub.
+#if defined(__HIP_DEVICE_COMPILE__)
+    using Cfg = FastConfig<DC, DO>;
+    using M = Mma<T>;
+    using V8 = typename M::V8;
+    constexpr int MW = Cfg::MW, BM = Cfg::BM, BN = Cfg::BN;
+    constexpr int NIB = MW / 32, NBLK = BM / 32;
+    constexpr int KC = DC / 16, DB = DO / 32, NZF = 2 * DB;
+    constexpr int RY = Cfg::RY, RZ = Cfg::RZ, CY = Cfg::CY, CZ = Cfg::CZ;
+    constexpr int NIY = Cfg::NIY, NIZ = Cfg::NIZ;
+    constexpr int STAGE = Cfg::STAGE_BYTES, Y_BYTES = Cfg::Y_BYTES;
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, g = lane >> 5, lam = lane & 15;
+
+    const int wg = blockIdx.x, xcd = wg & 7, slot = wg >> 3;
+    const int hl = slot / p.n_tiles, rank = slot - hl * p.n_tiles;
+    const int bh = hl * 8 + xcd;
+    if (bh >= p.BH) return;
+    const bool upper = p.upper != 0;
+    const int tile = upper ? rank : (p.n_tiles - 1 - rank);
+    const int b = bh / p.H, h = bh - b * p.H;
+    const T *X = static_cast<const T *>(p.x) + b * p.xs_b + h * p.xs_h;
+    const T *Y = static_cast<const T *>(p.y) + b * p.ys_b + h * p.ys_h;
+    const T *Z = static_cast<const T *>(p.z) + b * p.zs_b + h * p.zs_h;
+    T *O = static_cast<T *>(p.out) + b * p.os_b + h * p.os_h;
+    const int N = p.N;
+    const int i0 = tile * BM;
+
+    // raw buffer resources covering exactly the valid rows of this (b, h)
+    const int xs2 = (int)p.xs_n * 2, ys2 = (int)p.ys_n * 2, zs2 = (int)p.zs_n * 2;
+    const __amdgpu_buffer_rsrc_t rx =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(X), 0, (N - 1) * xs2 + p.dc * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t ry =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(Y), 0, (N - 1) * ys2 + p.dc * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rz =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(Z), 0, (N - 1) * zs2 + p.dout * 2, 0x00020000);
+
+    int blk[NIB];
+    blk[0] = wave;
+    if constexpr (NIB == 2) blk[1] = NBLK - 1 - wave;
+
+    // ---- tile sequence: tiles fully inside the mask first, then the diagonal block
+    const int diag_rows = (N - i0 < BM) ? (N - i0) : BM;
+    const int n_diag = (diag_rows + BN - 1) / BN;
+    int n_full, full_row0;
+    if (upper) {
+        const int rest = N - (i0 + BM);
+        n_full = rest > 0 ? (rest + BN - 1) / BN : 0;
+        full_row0 = i0 + BM;
+    } else {
+        n_full = i0 / BN;
+        full_row0 = 0;
+    }
+    const int n_seq = n_full + n_diag;
+    auto seq_row0 = [&](int q) { return q < n_full ? full_row0 + q * BN : i0 + (q - n_full) * BN; };
+
+    // ---- HBM -> LDS: per-lane source offsets (constant over tiles)
+    uint32_t ydma[NIY], zdma[NIZ];
+#pragma unroll
+    for (int u = 0; u < NIY; ++u) {
+        const int row = (u * 4 + wave) * (1024 / RY) + lane / CY;
+        const int c = (lane % CY) ^ swizzle_y<CY>(row);
+        ydma[u] = (uint32_t)(row * ys2 + c * 16) + (c * 8 < p.dc ? 0u : kOobOffset);
+    }
+#pragma unroll
+    for (int u = 0; u < NIZ; ++u) {
+        const int row = (u * 4 + wave) * (1024 / RZ) + lane / CZ;
+        const int c = (lane % CZ) ^ swizzle_z<CZ>(row);
+        zdma[u] = (uint32_t)(row * zs2 + c * 16) + (c * 8 < p.dout ? 0u : kOobOffset);
+    }
+    auto issue_tile = [&](int q) {
+        if (q < n_seq) {
+            const int row0 = seq_row0(q);
+            unsigned char *yb = smem + (q % Cfg::NBUF) * STAGE;
+            unsigned char *zb = yb + Y_BYTES;
+#pragma unroll
+            for (int u = 0; u < NIY; ++u)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(ry, (lds_void_ptr)(yb + (u * 4 + wave) * 1024), 16, ydma[u],
+                                                         row0 * ys2, 0, 0);
+#pragma unroll
+            for (int u = 0; u < NIZ; ++u)
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(rz, (lds_void_ptr)(zb + (u * 4 + wave) * 1024), 16, zdma[u],
+                                                         row0 * zs2, 0, 0);
+        }
+    };
+
+    issue_tile(0);
+
+    // ---- resident X fragments
+    V8 xf[NIB][KC];
+#pragma unroll
+    for (int ib = 0; ib < NIB; ++ib) {
+        const int row = i0 + blk[ib] * 32 + l32;
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc) {
+            const int col = kc * 16 + 8 * g;
+            const uint32_t off = (uint32_t)(row * xs2 + col * 2) + (col < p.dc ? 0u : kOobOffset);
+            xf[ib][kc] = __builtin_bit_cast(V8, __builtin_amdgcn_raw_buffer_load_b128(rx, off, 0, 0));
+        }
+    }
+
+    f32x16 acc[NIB][DB];
+#pragma unroll
+    for (int ib = 0; ib < NIB; ++ib)
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[ib][db][v] = 0.f;
+
+    // ---- LDS read offsets inside a stage (per lane, constant over tiles)
+    int yoff[KC], zoff[DB];
+    {
+        const int sy = swizzle_y<CY>(l32);
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc) yoff[kc] = l32 * RY + (((2 * kc + g) ^ sy) << 4);
+        const int zrow = 4 * g + (lam >> 2);
+        const int sz = swizzle_z<CZ>(zrow);
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+            zoff[db] = Y_BYTES + zrow * RZ + (((4 * db + 2 * ((lane >> 4) & 1) + ((lam & 3) >> 1)) ^ sz) << 4) + 8 * (lam & 1);
+    }
+    auto y_read = [&](const unsigned char *stage, int sub, int kc) -> V8 {
+        return __builtin_bit_cast(V8, *reinterpret_cast<const u32x4 *>(stage + sub * 32 * RY + yoff[kc]));
+    };
+    // fragment f = (t, db): rows 16t + {4g..4g+3, 8+4g..} of sub-tile `sub`, column 32 db + l32
+    auto z_read = [&](const unsigned char *stage, int sub, int f) -> V8 {
+        const int t = f / DB, db = f % DB;
+        const unsigned char *zp = stage + (sub * 32 + 16 * t) * RZ + zoff[db];
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(zp));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(zp + 8 * RZ));
+        return __builtin_bit_cast(V8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+    auto round_p = [&](const f32x16 (&s)[NIB], V8 (&pf)[NIB][2]) {
+#pragma unroll
+        for (int ib = 0; ib < NIB; ++ib)
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) pf[ib][t][e] = static_cast<T>(s[ib][8 * t + e]);
+    };
+
+    __syncthreads();  // tile 0 is in LDS
+    issue_tile(1);
+
+    // ================= tiles fully inside the mask: pipelined, no masking =================
+    if (n_full > 0) {
+        V8 yf[KC], zf[NZF], pfa[NIB][2], pfb[NIB][2];
+        f32x16 s[NIB];
+        const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kc = 0; kc < KC; ++kc) yf[kc] = y_read(smem, 0, kc);
+
+        // phase 1 of sub-tile s: S = Y_s X^T, interleaved with the Z fragment reads of the previous sub-tile
+        auto phase1 = [&](auto with_z, const unsigned char *zstage, int zsub) {
+#pragma unroll
+            for (int kc = 0; kc < KC; ++kc) {
+#pragma unroll
+                for (int ib = 0; ib < NIB; ++ib) s[ib] = M::mma(yf[kc], xf[ib][kc], kc == 0 ? zero : s[ib]);
+                if constexpr (decltype(with_z)::value) {
+#pragma unroll
+                    for (int f = 0; f < NZF; ++f)
+                        if (f * KC / NZF == kc) zf[f] = z_read(zstage, zsub, f);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        // phase 2: Out += P_prev Z_prev, interleaved with the Y fragment reads of the next sub-tile
+        // and the rounding of S into `pcur`
+        auto phase2 = [&](auto with_pv, V8 (&pprev)[NIB][2], V8 (&pcur)[NIB][2], const unsigned char *ystage, int ysub) {
+#pragma unroll
+            for (int f = 0; f < NZF; ++f) {
+                if constexpr (decltype(with_pv)::value) {
+                    const int t = f / DB, db = f % DB;
+#pragma unroll
+                    for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(pprev[ib][t], zf[f], acc[ib][db]);
+                }
+#pragma unroll
+                for (int kc = 0; kc < KC; ++kc)
+                    if (kc * NZF / KC == f) yf[kc] = y_read(ystage, ysub, kc);
+                if (f == NZF / 2) round_p(s, pcur);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        auto tile_body = [&](auto first, int q) {
+            constexpr bool kFirst = decltype(first)::value;
+            const unsigned char *cur = smem + (q % Cfg::NBUF) * STAGE;
+            const unsigned char *prev = smem + ((q + Cfg::NBUF - 1) % Cfg::NBUF) * STAGE;
+            const unsigned char *next = smem + ((q + 1) % Cfg::NBUF) * STAGE;
+            // first sub-tile of tile q
+            phase1(std::integral_constant<bool, !kFirst>{}, prev, 1);
+            phase2(std::integral_constant<bool, !kFirst>{}, pfb, pfa, cur, 1);
+            // second sub-tile
+            phase1(std::true_type{}, cur, 0);
+            __syncthreads();  // tile q+1 has landed; nobody reads tile q-1 any more
+            issue_tile(q + 2);
+            phase2(std::true_type{}, pfa, pfb, next, 0);
+        };
+        tile_body(std::true_type{}, 0);
+        for (int q = 1; q < n_full; ++q) tile_body(std::false_type{}, q);
+        // drain: the last sub-tile's P still has to meet its Z
+        {
+            const unsigned char *last = smem + ((n_full - 1) % Cfg::NBUF) * STAGE;
+#pragma unroll
+            for (int f = 0; f < NZF; ++f) zf[f] = z_read(last, 1, f);
+#pragma unroll
+            for (int f = 0; f < NZF; ++f) {
+                const int t = f / DB, db = f % DB;
+#pragma unroll
+                for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(pfb[ib][t], zf[f], acc[ib][db]);
+            }
+        }
+    }
+
+    // ================= the diagonal block =================
+    for (int q = n_full; q < n_seq; ++q) {
+        const unsigned char *cur = smem + (q % Cfg::NBUF) * STAGE;
+        const int row0 = i0 + (q - n_full) * BN;
+#pragma unroll
+        for (int sub = 0; sub < BN / 32; ++sub) {
+            const int j0 = row0 + sub * 32;
+            // 0: fully masked, 1: fully kept, 2: straddles the diagonal
+            int st[NIB];
+            bool any = false;
+#pragma unroll
+            for (int ib = 0; ib < NIB; ++ib) {
+                const int ib0 = i0 + blk[ib] * 32;
+                if (upper)
+                    st[ib] = (j0 < ib0) ? 0 : (j0 == ib0 ? 2 : 1);
+                else
+                    st[ib] = (j0 > ib0) ? 0 : (j0 == ib0 ? 2 : 1);
+                any = any || st[ib] != 0;
+            }
+            if (!any || j0 >= N) continue;
+
+            V8 yf[KC];
+#pragma unroll
+            for (int kc = 0; kc < KC; ++kc) yf[kc] = y_read(cur, sub, kc);
+            V8 zf[NZF];
+#pragma unroll
+            for (int f = 0; f < NZF; ++f) zf[f] = z_read(cur, sub, f);
+
+#pragma unroll
+            for (int ib = 0; ib < NIB; ++ib) {
+                if (st[ib] == 0) continue;
+                f32x16 s;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) s[v] = 0.f;
+#pragma unroll
+                for (int kc = 0; kc < KC; ++kc) s = M::mma(yf[kc], xf[ib][kc], s);
+                if (st[ib] == 2) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int jl = 8 * (v / 4) + 4 * g + (v % 4);
+                        const bool keep = upper ? l32 <= jl : l32 >= jl;
+                        s[v] = keep ? s[v] : 0.f;
+                    }
+                }
+                V8 pf[2];
+#pragma unroll
+                for (int t = 0; t < 2; ++t)
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) pf[t][e] = static_cast<T>(s[8 * t + e]);
+#pragma unroll
+                for (int f = 0; f < NZF; ++f) acc[ib][f % DB] = M::mma(pf[f / DB], zf[f], acc[ib][f % DB]);
+            }
+        }
+        __syncthreads();  // tile q+1 has landed; tile q is retired
+        issue_tile(q + 2);
+    }
+
+    // ---- epilogue: acc[ib][db][v] is Out[row = 8(v/4) + 4g + v%4][col = 32 db + l32] of block ib
+#pragma unroll
+    for (int ib = 0; ib < NIB; ++ib) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int row = i0 + blk[ib] * 32 + 8 * (v / 4) + 4 * g + (v % 4);
+            if (row < N) {
+                T *rp = O + (int64_t)row * p.os_n;
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                    const int col = db * 32 + l32;
+                    if (col < p.dout) rp[col] = static_cast<T>(acc[ib][db][v]);
+                }
+            }
+        }
+    }
+#else
+    (void)p;
+#endif
+}
+
+// True when the fast kernel can take this problem: every operand 16-byte
+// aligned with widths in whole chunks, and each (b, h) slice addressable with
+// 32-bit byte offsets.
+inline bool fast_path_ok(const TriParams &p) {
+    if (!(p.vec_x && p.vec_y && p.vec_z)) return false;
+    const int64_t n = p.N;
+    return n * p.xs_n * 2 <= kMaxFastExtent && n * p.ys_n * 2 <= kMaxFastExtent && n * p.zs_n * 2 <= kMaxFastExtent;
+}
+
+template <typename T, int DC, int DO>
+hipError_t launch_tri_fast(TriParams p, hipStream_t stream) {
+    using Cfg = FastConfig<DC, DO>;
+    if constexpr (!Cfg::kSupported) {
+        return hipErrorNotSupported;
+    } else {
+        p.n_tiles = (p.N + Cfg::BM - 1) / Cfg::BM;
+        const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_tiles;
+        if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+        auto kern = tri_xyt_z_fast_kernel<T, DC, DO>;
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM_BYTES);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), Cfg::SMEM_BYTES, stream, p);
+        return hipGetLastError();
+    }
+}
+
+}  // namespace fla
