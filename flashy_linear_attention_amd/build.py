@@ -30,6 +30,9 @@ HIPCC_FLAGS = [
     "-fPIC",
     # hipcc may not form packed fp32 VALU ops on this target
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results in architectural VGPRs (operands may still sit in AGPRs): the S
+    # accumulators are read by VALU right away, and the AGPR form costs 32 copies per sub-tile
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
     "-Wno-unused-command-line-argument",
     "-I" + INCLUDE,
     "-I" + CSRC,

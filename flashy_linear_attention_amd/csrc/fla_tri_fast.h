@@ -38,6 +38,25 @@ typedef __attribute__((address_space(3))) void *lds_void_ptr;
 typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
 typedef short s16x8 __attribute__((ext_vector_type(8)));
 
+// One wave-wide HBM -> LDS copy of 64 x 16 bytes: lane l's 16 bytes land at lds_addr + 16 l.
+// Issued through inline assembly so that the compiler's wait-count insertion does not
+// serialise later LDS reads of *other* ring slots against it; completion is awaited
+// explicitly (wait_dma) before the barrier that publishes the slot.
+__device__ __forceinline__ void dma_16B_per_lane(u32x4 rsrc, uint32_t lds_addr, uint32_t voffset, uint32_t soffset) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
+                 : "memory", "m0");
+}
+// s_waitcnt vmcnt(0) only (expcnt and lgkmcnt fields left at their maxima)
+__device__ __forceinline__ void wait_dma() { __builtin_amdgcn_s_waitcnt(0x0f70); }
+
+__device__ __forceinline__ u32x4 make_rsrc(const void *base, uint32_t bytes) {
+    const uint64_t a = reinterpret_cast<uint64_t>(base);
+    u32x4 r = {(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, bytes, 0x00020000u};
+    return r;
+}
+
 constexpr uint32_t kOobOffset = 0x40000000u;  // added to a buffer offset to force an out-of-range (zero) access
 constexpr int64_t kMaxFastExtent = 0x3fffffff;  // per-(b,h) byte extent the 32-bit buffer offsets can address
 
@@ -62,9 +81,8 @@ struct FastConfig {
 // XOR applied to the chunk index of LDS row `row` (row counted inside the tile).
 template <int CY>
 __device__ __forceinline__ int swizzle_y(int row) {
-    if constexpr (CY == 4) return (row >> 1) & 3;   // 64-byte rows: two rows share 128 bytes
-    else if constexpr (CY == 8) return row & 7;
-    else return row & 15;
+    if constexpr (CY == 4) return (row >> 1) & 3;  // 64-byte rows: two rows share 128 bytes
+    else return row & 7;  // 8 consecutive rows hit 8 different 16-byte slots of a 128-byte window
 }
 template <int CZ>
 __device__ __forceinline__ int swizzle_z(int row) {
@@ -87,8 +105,11 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
     constexpr int RY = Cfg::RY, RZ = Cfg::RZ, CY = Cfg::CY, CZ = Cfg::CZ;
     constexpr int NIY = Cfg::NIY, NIZ = Cfg::NIZ;
     constexpr int STAGE = Cfg::STAGE_BYTES, Y_BYTES = Cfg::Y_BYTES;
+    constexpr int YQ = KC < 4 ? KC : 4;  // Y read addresses that differ by more than an immediate
+    constexpr int ZQ = DB < 2 ? DB : 2;  // same for Z
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -112,10 +133,8 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
     const int xs2 = (int)p.xs_n * 2, ys2 = (int)p.ys_n * 2, zs2 = (int)p.zs_n * 2;
     const __amdgpu_buffer_rsrc_t rx =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(X), 0, (N - 1) * xs2 + p.dc * 2, 0x00020000);
-    const __amdgpu_buffer_rsrc_t ry =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(Y), 0, (N - 1) * ys2 + p.dc * 2, 0x00020000);
-    const __amdgpu_buffer_rsrc_t rz =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(Z), 0, (N - 1) * zs2 + p.dout * 2, 0x00020000);
+    const u32x4 ry = make_rsrc(Y, (uint32_t)((N - 1) * ys2 + p.dc * 2));
+    const u32x4 rz = make_rsrc(Z, (uint32_t)((N - 1) * zs2 + p.dout * 2));
 
     int blk[NIB];
     blk[0] = wave;
@@ -134,7 +153,6 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
         full_row0 = 0;
     }
     const int n_seq = n_full + n_diag;
-    auto seq_row0 = [&](int q) { return q < n_full ? full_row0 + q * BN : i0 + (q - n_full) * BN; };
 
     // ---- HBM -> LDS: per-lane source offsets (constant over tiles)
     uint32_t ydma[NIY], zdma[NIZ];
@@ -150,23 +168,20 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
         const int c = (lane % CZ) ^ swizzle_z<CZ>(row);
         zdma[u] = (uint32_t)(row * zs2 + c * 16) + (c * 8 < p.dout ? 0u : kOobOffset);
     }
-    auto issue_tile = [&](int q) {
+    // tile q of the sequence -> ring slot q % 3, tracked incrementally
+    auto issue_tile = [&](int q, int slot_off) {
         if (q < n_seq) {
-            const int row0 = seq_row0(q);
-            unsigned char *yb = smem + (q % Cfg::NBUF) * STAGE;
-            unsigned char *zb = yb + Y_BYTES;
+            const int row0 = q < n_full ? full_row0 + q * BN : i0 + (q - n_full) * BN;
+            const uint32_t yb = lds0 + slot_off + wave * 1024, zb = yb + Y_BYTES;
 #pragma unroll
-            for (int u = 0; u < NIY; ++u)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(ry, (lds_void_ptr)(yb + (u * 4 + wave) * 1024), 16, ydma[u],
-                                                         row0 * ys2, 0, 0);
+            for (int u = 0; u < NIY; ++u) dma_16B_per_lane(ry, yb + u * 4096, ydma[u], row0 * ys2);
 #pragma unroll
-            for (int u = 0; u < NIZ; ++u)
-                __builtin_amdgcn_raw_ptr_buffer_load_lds(rz, (lds_void_ptr)(zb + (u * 4 + wave) * 1024), 16, zdma[u],
-                                                         row0 * zs2, 0, 0);
+            for (int u = 0; u < NIZ; ++u) dma_16B_per_lane(rz, zb + u * 4096, zdma[u], row0 * zs2);
         }
     };
+    auto next_slot = [](int off) { return off + STAGE == Cfg::NBUF * STAGE ? 0 : off + STAGE; };
 
-    issue_tile(0);
+    issue_tile(0, 0);
 
     // ---- resident X fragments
     V8 xf[NIB][KC];
@@ -189,28 +204,37 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[ib][db][v] = 0.f;
 
-    // ---- LDS read offsets inside a stage (per lane, constant over tiles)
-    int yoff[KC], zoff[DB];
+    // ---- LDS read offsets inside a stage.  Only the chunk bits the swizzle touches need a
+    // register; the rest of (sub-tile, kc / t, db) is an immediate offset of the DS instruction.
+    int ylane[YQ], zlane[ZQ];
     {
         const int sy = swizzle_y<CY>(l32);
 #pragma unroll
-        for (int kc = 0; kc < KC; ++kc) yoff[kc] = l32 * RY + (((2 * kc + g) ^ sy) << 4);
+        for (int j = 0; j < YQ; ++j) ylane[j] = l32 * RY + (((2 * j + g) ^ sy) << 4);
         const int zrow = 4 * g + (lam >> 2);
         const int sz = swizzle_z<CZ>(zrow);
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
-            zoff[db] = Y_BYTES + zrow * RZ + (((4 * db + 2 * ((lane >> 4) & 1) + ((lam & 3) >> 1)) ^ sz) << 4) + 8 * (lam & 1);
+        for (int j = 0; j < ZQ; ++j)
+            zlane[j] = Y_BYTES + zrow * RZ + (((4 * j + 2 * ((lane >> 4) & 1) + ((lam & 3) >> 1)) ^ sz) << 4) + 8 * (lam & 1);
     }
-    auto y_read = [&](const unsigned char *stage, int sub, int kc) -> V8 {
-        return __builtin_bit_cast(V8, *reinterpret_cast<const u32x4 *>(stage + sub * 32 * RY + yoff[kc]));
+    // `ya` / `za`: ylane / zlane plus the byte offset of a ring slot
+    auto y_read = [&](const int (&ya)[YQ], int sub, int kc) -> V8 {
+        const unsigned char *ptr = smem + ya[kc % YQ] + (sub * 32 * RY + (kc / YQ) * (YQ * 32));
+        return __builtin_bit_cast(V8, *reinterpret_cast<const u32x4 *>(ptr));
     };
     // fragment f = (t, db): rows 16t + {4g..4g+3, 8+4g..} of sub-tile `sub`, column 32 db + l32
-    auto z_read = [&](const unsigned char *stage, int sub, int f) -> V8 {
+    auto z_read = [&](const int (&za)[ZQ], int sub, int f) -> V8 {
         const int t = f / DB, db = f % DB;
-        const unsigned char *zp = stage + (sub * 32 + 16 * t) * RZ + zoff[db];
+        const unsigned char *zp = smem + za[db % ZQ] + ((sub * 32 + 16 * t) * RZ + (db / ZQ) * (ZQ * 64));
         const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(zp));
         const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(zp + 8 * RZ));
         return __builtin_bit_cast(V8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+    auto slot_addrs = [&](int slot_off, int (&ya)[YQ], int (&za)[ZQ]) {
+#pragma unroll
+        for (int j = 0; j < YQ; ++j) ya[j] = ylane[j] + slot_off;
+#pragma unroll
+        for (int j = 0; j < ZQ; ++j) za[j] = zlane[j] + slot_off;
     };
     auto round_p = [&](const f32x16 (&s)[NIB], V8 (&pf)[NIB][2]) {
 #pragma unroll
@@ -221,19 +245,32 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
                 for (int e = 0; e < 8; ++e) pf[ib][t][e] = static_cast<T>(s[ib][8 * t + e]);
     };
 
-    __syncthreads();  // tile 0 is in LDS
-    issue_tile(1);
+    wait_dma();
+    __builtin_amdgcn_s_barrier();  // tile 0 is in LDS
+    issue_tile(1, STAGE);
+
+    int prev_off = 2 * STAGE, cur_off = 0, next_off = STAGE;  // ring slots (byte offsets) around the tile being consumed
+    auto advance = [&]() {
+        prev_off = cur_off;
+        cur_off = next_off;
+        next_off = next_slot(next_off);
+    };
+    int q = 0;
 
     // ================= tiles fully inside the mask: pipelined, no masking =================
     if (n_full > 0) {
         V8 yf[KC], zf[NZF], pfa[NIB][2], pfb[NIB][2];
         f32x16 s[NIB];
         const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        {
+            int ya0[YQ], za0[ZQ];
+            slot_addrs(0, ya0, za0);
 #pragma unroll
-        for (int kc = 0; kc < KC; ++kc) yf[kc] = y_read(smem, 0, kc);
+            for (int kc = 0; kc < KC; ++kc) yf[kc] = y_read(ya0, 0, kc);
+        }
 
         // phase 1 of sub-tile s: S = Y_s X^T, interleaved with the Z fragment reads of the previous sub-tile
-        auto phase1 = [&](auto with_z, const unsigned char *zstage, int zsub) {
+        auto phase1 = [&](auto with_z, const int (&za)[ZQ], int zsub) {
 #pragma unroll
             for (int kc = 0; kc < KC; ++kc) {
 #pragma unroll
@@ -241,14 +278,14 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
                 if constexpr (decltype(with_z)::value) {
 #pragma unroll
                     for (int f = 0; f < NZF; ++f)
-                        if (f * KC / NZF == kc) zf[f] = z_read(zstage, zsub, f);
+                        if (f * KC / NZF == kc) zf[f] = z_read(za, zsub, f);
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
         // phase 2: Out += P_prev Z_prev, interleaved with the Y fragment reads of the next sub-tile
         // and the rounding of S into `pcur`
-        auto phase2 = [&](auto with_pv, V8 (&pprev)[NIB][2], V8 (&pcur)[NIB][2], const unsigned char *ystage, int ysub) {
+        auto phase2 = [&](auto with_pv, V8 (&pprev)[NIB][2], V8 (&pcur)[NIB][2], const int (&ya)[YQ], int ysub) {
 #pragma unroll
             for (int f = 0; f < NZF; ++f) {
                 if constexpr (decltype(with_pv)::value) {
@@ -258,32 +295,37 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
                 }
 #pragma unroll
                 for (int kc = 0; kc < KC; ++kc)
-                    if (kc * NZF / KC == f) yf[kc] = y_read(ystage, ysub, kc);
+                    if (kc * NZF / KC == f) yf[kc] = y_read(ya, ysub, kc);
                 if (f == NZF / 2) round_p(s, pcur);
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
-        auto tile_body = [&](auto first, int q) {
+        auto tile_body = [&](auto first) {
             constexpr bool kFirst = decltype(first)::value;
-            const unsigned char *cur = smem + (q % Cfg::NBUF) * STAGE;
-            const unsigned char *prev = smem + ((q + Cfg::NBUF - 1) % Cfg::NBUF) * STAGE;
-            const unsigned char *next = smem + ((q + 1) % Cfg::NBUF) * STAGE;
-            // first sub-tile of tile q
-            phase1(std::integral_constant<bool, !kFirst>{}, prev, 1);
-            phase2(std::integral_constant<bool, !kFirst>{}, pfb, pfa, cur, 1);
+            int ya_cur[YQ], za_cur[ZQ], ya_next[YQ], za_prev[ZQ], unused_y[YQ], unused_z[ZQ];
+            slot_addrs(cur_off, ya_cur, za_cur);
+            slot_addrs(prev_off, unused_y, za_prev);
+            slot_addrs(next_off, ya_next, unused_z);
+            // first sub-tile: Z of the previous tile's second sub-tile, then Y of this tile's second
+            phase1(std::integral_constant<bool, !kFirst>{}, za_prev, 1);
+            phase2(std::integral_constant<bool, !kFirst>{}, pfb, pfa, ya_cur, 1);
             // second sub-tile
-            phase1(std::true_type{}, cur, 0);
-            __syncthreads();  // tile q+1 has landed; nobody reads tile q-1 any more
-            issue_tile(q + 2);
-            phase2(std::true_type{}, pfa, pfb, next, 0);
+            phase1(std::true_type{}, za_cur, 0);
+            wait_dma();
+            __builtin_amdgcn_s_barrier();  // tile q+1 has landed; nobody reads tile q-1 any more
+            issue_tile(q + 2, prev_off);
+            phase2(std::true_type{}, pfa, pfb, ya_next, 0);
+            advance();
+            ++q;
         };
-        tile_body(std::true_type{}, 0);
-        for (int q = 1; q < n_full; ++q) tile_body(std::false_type{}, q);
-        // drain: the last sub-tile's P still has to meet its Z
+        tile_body(std::true_type{});
+        while (q < n_full) tile_body(std::false_type{});
+        // drain: the last sub-tile's P still has to meet its Z (second half of the previous slot)
         {
-            const unsigned char *last = smem + ((n_full - 1) % Cfg::NBUF) * STAGE;
+            int unused_y[YQ], za_prev[ZQ];
+            slot_addrs(prev_off, unused_y, za_prev);
 #pragma unroll
-            for (int f = 0; f < NZF; ++f) zf[f] = z_read(last, 1, f);
+            for (int f = 0; f < NZF; ++f) zf[f] = z_read(za_prev, 1, f);
 #pragma unroll
             for (int f = 0; f < NZF; ++f) {
                 const int t = f / DB, db = f % DB;
@@ -294,9 +336,10 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
     }
 
     // ================= the diagonal block =================
-    for (int q = n_full; q < n_seq; ++q) {
-        const unsigned char *cur = smem + (q % Cfg::NBUF) * STAGE;
+    for (; q < n_seq; ++q) {
         const int row0 = i0 + (q - n_full) * BN;
+        int ya_cur[YQ], za_cur[ZQ];
+        slot_addrs(cur_off, ya_cur, za_cur);
 #pragma unroll
         for (int sub = 0; sub < BN / 32; ++sub) {
             const int j0 = row0 + sub * 32;
@@ -316,10 +359,10 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
 
             V8 yf[KC];
 #pragma unroll
-            for (int kc = 0; kc < KC; ++kc) yf[kc] = y_read(cur, sub, kc);
+            for (int kc = 0; kc < KC; ++kc) yf[kc] = y_read(ya_cur, sub, kc);
             V8 zf[NZF];
 #pragma unroll
-            for (int f = 0; f < NZF; ++f) zf[f] = z_read(cur, sub, f);
+            for (int f = 0; f < NZF; ++f) zf[f] = z_read(za_cur, sub, f);
 
 #pragma unroll
             for (int ib = 0; ib < NIB; ++ib) {
@@ -346,8 +389,10 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
                 for (int f = 0; f < NZF; ++f) acc[ib][f % DB] = M::mma(pf[f / DB], zf[f], acc[ib][f % DB]);
             }
         }
-        __syncthreads();  // tile q+1 has landed; tile q is retired
-        issue_tile(q + 2);
+        wait_dma();
+        __builtin_amdgcn_s_barrier();  // tile q+1 has landed; tile q is retired (and q-1 long before)
+        issue_tile(q + 2, prev_off);
+        advance();
     }
 
     // ---- epilogue: acc[ib][db][v] is Out[row = 8(v/4) + 4g + v%4][col = 32 db + l32] of block ib
