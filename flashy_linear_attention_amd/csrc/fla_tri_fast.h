@@ -48,12 +48,36 @@ __device__ __forceinline__ void dma_16B_per_lane(u32x4 rsrc, uint32_t lds_addr, 
                  : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
                  : "memory", "m0");
 }
-// s_waitcnt vmcnt(0) only (expcnt and lgkmcnt fields left at their maxima)
-__device__ __forceinline__ void wait_dma() { __builtin_amdgcn_s_waitcnt(0x0f70); }
+// s_waitcnt vmcnt(N) only (expcnt and lgkmcnt fields left at their maxima): returns once at
+// most N of this wave's buffer loads, the most recently issued ones, are still in flight.
+template <int N>
+__device__ __forceinline__ void wait_vm() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (N & 15) | ((N >> 4) << 14));
+}
 
 __device__ __forceinline__ u32x4 make_rsrc(const void *base, uint32_t bytes) {
     const uint64_t a = reinterpret_cast<uint64_t>(base);
     u32x4 r = {(uint32_t)a, (uint32_t)(a >> 32) & 0xffffu, bytes, 0x00020000u};
+    return r;
+}
+
+// Two fp32 values rounded (nearest even) and packed into one 16-bit pair, pinned to this
+// point of the instruction stream.  As a plain conversion the compiler sinks all sixteen of a
+// sub-tile to just before the first MFMA that reads the result, where they leave the matrix
+// pipe idle.  The empty volatile asm statement demands the result right here, and the
+// scheduling barriers around the caller keep it from moving up; the conversion itself stays
+// a compiler-generated instruction, so that the hazard recogniser still sees it next to the
+// MFMAs that produce and consume these registers (hand-written conversion instructions in
+// inline assembly gave wrong results: the required wait states were missing).
+template <typename T>
+__device__ __forceinline__ uint32_t round_pack_pinned(float lo, float hi) {
+    typedef T pair_t __attribute__((ext_vector_type(2)));
+    pair_t pr;
+    pr[0] = static_cast<T>(lo);
+    pr[1] = static_cast<T>(hi);
+    uint32_t r = __builtin_bit_cast(uint32_t, pr);
+    asm volatile("" : "+v"(r));
     return r;
 }
 
@@ -66,7 +90,9 @@ struct FastConfig {
     static constexpr int NW = 4;
     static constexpr int BM = MW * NW;
     static constexpr int BN = 64;
-    static constexpr int NBUF = 3;
+    // LDS ring depth: the tile being consumed, the one before it (its second half is still
+    // being read for a while) and NBUF-2 tiles landed or in flight.  Four slots when they fit.
+    static constexpr int NBUF = 4 * (BN * (DC + DO) * 2) <= 160 * 1024 ? 4 : 3;
     static constexpr int RY = DC * 2, RZ = DO * 2;  // LDS row bytes (no padding)
     static constexpr int CY = DC / 8, CZ = DO / 8;  // 16-byte chunks per row
     static constexpr int Y_BYTES = BN * RY, Z_BYTES = BN * RZ;
@@ -75,6 +101,7 @@ struct FastConfig {
     static constexpr bool kSupported = SMEM_BYTES <= 160 * 1024;
     // wave-level 1 KiB DMA instructions per tile and wave
     static constexpr int NIY = Y_BYTES / 4096, NIZ = Z_BYTES / 4096;
+    static constexpr int NT = NIY + NIZ;  // buffer loads per wave and tile
     static_assert(Y_BYTES % 4096 == 0 && Z_BYTES % 4096 == 0, "tile must split into 1 KiB blocks over 4 waves");
 };
 
@@ -116,18 +143,19 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
     const int l32 = lane & 31, g = lane >> 5, lam = lane & 15;
 
     const int wg = blockIdx.x, xcd = wg & 7, slot = wg >> 3;
-    const int hl = slot / p.n_tiles, rank = slot - hl * p.n_tiles;
+    // Each workgroup takes two row tiles of one head, r and n_tiles-1-r: under a triangular
+    // mask their work adds up to the same amount for every r, so all workgroups are equal.
+    const int n_pairs = (p.n_tiles + 1) >> 1;
+    const int hl = slot / n_pairs, rank = slot - hl * n_pairs;
     const int bh = hl * 8 + xcd;
     if (bh >= p.BH) return;
     const bool upper = p.upper != 0;
-    const int tile = upper ? rank : (p.n_tiles - 1 - rank);
     const int b = bh / p.H, h = bh - b * p.H;
     const T *X = static_cast<const T *>(p.x) + b * p.xs_b + h * p.xs_h;
     const T *Y = static_cast<const T *>(p.y) + b * p.ys_b + h * p.ys_h;
     const T *Z = static_cast<const T *>(p.z) + b * p.zs_b + h * p.zs_h;
     T *O = static_cast<T *>(p.out) + b * p.os_b + h * p.os_h;
     const int N = p.N;
-    const int i0 = tile * BM;
 
     // raw buffer resources covering exactly the valid rows of this (b, h)
     const int xs2 = (int)p.xs_n * 2, ys2 = (int)p.ys_n * 2, zs2 = (int)p.zs_n * 2;
@@ -139,6 +167,11 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
     int blk[NIB];
     blk[0] = wave;
     if constexpr (NIB == 2) blk[1] = NBLK - 1 - wave;
+
+    for (int pass = 0; pass < 2; ++pass) {
+    const int tile = pass == 0 ? p.n_tiles - 1 - rank : rank;
+    if (pass == 1 && tile == p.n_tiles - 1 - rank) break;  // odd tile count: the middle tile has no partner
+    const int i0 = tile * BM;
 
     // ---- tile sequence: tiles fully inside the mask first, then the diagonal block
     const int diag_rows = (N - i0 < BM) ? (N - i0) : BM;
@@ -180,6 +213,14 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
         }
     };
     auto next_slot = [](int off) { return off + STAGE == Cfg::NBUF * STAGE ? 0 : off + STAGE; };
+    // Wait until tile `q` has landed, given that every tile up to q + NBUF - 3 has been issued:
+    // the loads of later tiles (at most one tile's worth with four slots) may stay in flight.
+    auto wait_tile = [&](int q) {
+        if (Cfg::NBUF == 4 && q + 1 < n_seq)
+            wait_vm<Cfg::NT>();
+        else
+            wait_vm<0>();
+    };
 
     issue_tile(0, 0);
 
@@ -245,15 +286,22 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
                 for (int e = 0; e < 8; ++e) pf[ib][t][e] = static_cast<T>(s[ib][8 * t + e]);
     };
 
-    wait_dma();
-    __builtin_amdgcn_s_barrier();  // tile 0 is in LDS
-    issue_tile(1, STAGE);
-
-    int prev_off = 2 * STAGE, cur_off = 0, next_off = STAGE;  // ring slots (byte offsets) around the tile being consumed
+    // ring state: byte offsets of the slots of tile q-1, q, q+1 and of the next tile to issue
+    int prev_off = (Cfg::NBUF - 1) * STAGE, cur_off = 0, next_off = STAGE, issue_off = STAGE;
+    if constexpr (Cfg::NBUF == 4) {
+        issue_tile(1, STAGE);
+        issue_off = 2 * STAGE;
+    }
+    wait_tile(0);
+    __builtin_amdgcn_s_barrier();  // tile 0 (and the X fragments) have landed
+    issue_tile(Cfg::NBUF - 2, issue_off);
+    issue_off = next_slot(issue_off);
+    // from here on: tiles up to q + NBUF - 2 are issued while tile q is consumed
     auto advance = [&]() {
         prev_off = cur_off;
         cur_off = next_off;
         next_off = next_slot(next_off);
+        issue_off = next_slot(issue_off);
     };
     int q = 0;
 
@@ -276,9 +324,15 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
 #pragma unroll
                 for (int ib = 0; ib < NIB; ++ib) s[ib] = M::mma(yf[kc], xf[ib][kc], kc == 0 ? zero : s[ib]);
                 if constexpr (decltype(with_z)::value) {
+#ifndef FLA_DBG_NO_ZREAD
 #pragma unroll
                     for (int f = 0; f < NZF; ++f)
                         if (f * KC / NZF == kc) zf[f] = z_read(za, zsub, f);
+#else
+#pragma unroll
+                    for (int f = 0; f < NZF; ++f)
+                        if (f * KC / NZF == kc) asm volatile("" : "+v"(zf[f]));
+#endif
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -286,6 +340,8 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
         // phase 2: Out += P_prev Z_prev, interleaved with the Y fragment reads of the next sub-tile
         // and the rounding of S into `pcur`
         auto phase2 = [&](auto with_pv, V8 (&pprev)[NIB][2], V8 (&pcur)[NIB][2], const int (&ya)[YQ], int ysub) {
+            constexpr int NPK = NIB * 8;  // packed pairs that make up P of one sub-tile
+            u32x4 pk[NIB][2];
 #pragma unroll
             for (int f = 0; f < NZF; ++f) {
                 if constexpr (decltype(with_pv)::value) {
@@ -293,12 +349,30 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
 #pragma unroll
                     for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(pprev[ib][t], zf[f], acc[ib][db]);
                 }
+#ifndef FLA_DBG_NO_YREAD
 #pragma unroll
                 for (int kc = 0; kc < KC; ++kc)
                     if (kc * NZF / KC == f) yf[kc] = y_read(ya, ysub, kc);
-                if (f == NZF / 2) round_p(s, pcur);
+#else
+#pragma unroll
+                for (int kc = 0; kc < KC; ++kc)
+                    if (kc * NZF / KC == f) asm volatile("" : "+v"(yf[kc]));
+#endif
+                // S of this sub-tile is complete once a couple of the independent MFMAs above have
+                // issued; its rounding is spread over the second half of the phase
+#pragma unroll
+                for (int c = 0; c < NPK; ++c) {
+                    if (NZF / 2 + (c * (NZF - NZF / 2)) / NPK == f) {
+                        const int ib = c / 8, t = (c / 4) % 2, w = c % 4;
+                        pk[ib][t][w] = round_pack_pinned<T>(s[ib][8 * t + 2 * w], s[ib][8 * t + 2 * w + 1]);
+                    }
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
+#pragma unroll
+            for (int ib = 0; ib < NIB; ++ib)
+#pragma unroll
+                for (int t = 0; t < 2; ++t) pcur[ib][t] = __builtin_bit_cast(V8, pk[ib][t]);
         };
         auto tile_body = [&](auto first) {
             constexpr bool kFirst = decltype(first)::value;
@@ -311,9 +385,15 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
             phase2(std::integral_constant<bool, !kFirst>{}, pfb, pfa, ya_cur, 1);
             // second sub-tile
             phase1(std::true_type{}, za_cur, 0);
-            wait_dma();
+#ifndef FLA_DBG_NO_WAIT
+            wait_tile(q + 1);
+#endif
+#ifndef FLA_DBG_NO_BARRIER
             __builtin_amdgcn_s_barrier();  // tile q+1 has landed; nobody reads tile q-1 any more
-            issue_tile(q + 2, prev_off);
+#endif
+#ifndef FLA_DBG_NO_DMA
+            issue_tile(q + Cfg::NBUF - 1, issue_off);
+#endif
             phase2(std::true_type{}, pfa, pfb, ya_next, 0);
             advance();
             ++q;
@@ -389,9 +469,9 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
                 for (int f = 0; f < NZF; ++f) acc[ib][f % DB] = M::mma(pf[f / DB], zf[f], acc[ib][f % DB]);
             }
         }
-        wait_dma();
-        __builtin_amdgcn_s_barrier();  // tile q+1 has landed; tile q is retired (and q-1 long before)
-        issue_tile(q + 2, prev_off);
+        wait_tile(q + 1);
+        __builtin_amdgcn_s_barrier();  // tile q+1 has landed; tile q-1 is long retired
+        issue_tile(q + Cfg::NBUF - 1, issue_off);
         advance();
     }
 
@@ -411,6 +491,7 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
             }
         }
     }
+    }  // pass
 #else
     (void)p;
 #endif
@@ -432,7 +513,7 @@ hipError_t launch_tri_fast(TriParams p, hipStream_t stream) {
         return hipErrorNotSupported;
     } else {
         p.n_tiles = (p.N + Cfg::BM - 1) / Cfg::BM;
-        const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_tiles;
+        const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * ((p.n_tiles + 1) / 2);
         if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
         auto kern = tri_xyt_z_fast_kernel<T, DC, DO>;
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
