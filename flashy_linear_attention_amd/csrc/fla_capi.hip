@@ -4,6 +4,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "fla_dispatch.h"
 
@@ -69,7 +70,13 @@ int run_tri(const View &x, const View &y, const View &z, const View &out, int64_
     p.dc = (int32_t)dc, p.dout = (int32_t)dout;
     p.upper = upper ? 1 : 0;
     p.n_tiles = 0;
-    p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout);
+    p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout), p.vec_out = vec_ok(out, dout);
+#ifdef FLA_DBG_TIMING
+    {
+        const char *e = getenv("FLA_DBG_TIMING_PTR");
+        p.dbg = e ? reinterpret_cast<unsigned long long *>(strtoull(e, nullptr, 16)) : nullptr;
+    }
+#endif
     launch_fn fn = lookup(dtype, dc, dout);
     if (!fn) return FLA_ERR_UNSUPPORTED;
     return fn(p, static_cast<hipStream_t>(stream)) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;

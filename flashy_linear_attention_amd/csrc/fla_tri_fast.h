@@ -102,6 +102,9 @@ struct FastConfig {
     // wave-level 1 KiB DMA instructions per tile and wave
     static constexpr int NIY = Y_BYTES / 4096, NIZ = Z_BYTES / 4096;
     static constexpr int NT = NIY + NIZ;  // buffer loads per wave and tile
+    // output staging in LDS: BM rows of DO 16-bit values, 16 bytes of padding per row
+    static constexpr int RO = DO * 2 + 16;
+    static_assert(BM * RO <= SMEM_BYTES, "output staging must fit in the ring");
     static_assert(Y_BYTES % 4096 == 0 && Z_BYTES % 4096 == 0, "tile must split into 1 KiB blocks over 4 waves");
 };
 
@@ -168,7 +171,19 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
     blk[0] = wave;
     if constexpr (NIB == 2) blk[1] = NBLK - 1 - wave;
 
+    // FLA_DBG_TIMING builds record the shader clock at the phase boundaries of every workgroup
+#ifdef FLA_DBG_TIMING
+#define FLA_STAMP(k)                                                                                           \
+    do {                                                                                                       \
+        if (p.dbg && tid == 0) p.dbg[(size_t)blockIdx.x * 16 + pass * 8 + (k)] = __builtin_readcyclecounter(); \
+    } while (0)
+#else
+#define FLA_STAMP(k) \
+    do {             \
+    } while (0)
+#endif
     for (int pass = 0; pass < 2; ++pass) {
+    FLA_STAMP(0);
     const int tile = pass == 0 ? p.n_tiles - 1 - rank : rank;
     if (pass == 1 && tile == p.n_tiles - 1 - rank) break;  // odd tile count: the middle tile has no partner
     const int i0 = tile * BM;
@@ -252,18 +267,25 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
         const int sy = swizzle_y<CY>(l32);
 #pragma unroll
         for (int j = 0; j < YQ; ++j) ylane[j] = l32 * RY + (((2 * j + g) ^ sy) << 4);
+        // Transposing read: source lane `lam` of a 16-lane group supplies row lam/4 and the
+        // 4-column chunk c = lam%4; destination lane 4c + x receives column x of that chunk.
+        // Chunk c of group beta = (lane/16)%2 is taken from columns 16 (c&1) + 8 beta + 4 (c>>1)
+        // of the 32-column block, which makes MFMA row m = 8a + 4g' + b of the fragment hold
+        // column 16 g' + 4 a + b: the accumulator registers of one lane then cover 16
+        // consecutive output columns (see the epilogue).
         const int zrow = 4 * g + (lam >> 2);
         const int sz = swizzle_z<CZ>(zrow);
+        const int zc = lam & 3, beta = (lane >> 4) & 1;
 #pragma unroll
         for (int j = 0; j < ZQ; ++j)
-            zlane[j] = Y_BYTES + zrow * RZ + (((4 * j + 2 * ((lane >> 4) & 1) + ((lam & 3) >> 1)) ^ sz) << 4) + 8 * (lam & 1);
+            zlane[j] = Y_BYTES + zrow * RZ + (((4 * j + 2 * (zc & 1) + beta) ^ sz) << 4) + 8 * (zc >> 1);
     }
     // `ya` / `za`: ylane / zlane plus the byte offset of a ring slot
     auto y_read = [&](const int (&ya)[YQ], int sub, int kc) -> V8 {
         const unsigned char *ptr = smem + ya[kc % YQ] + (sub * 32 * RY + (kc / YQ) * (YQ * 32));
         return __builtin_bit_cast(V8, *reinterpret_cast<const u32x4 *>(ptr));
     };
-    // fragment f = (t, db): rows 16t + {4g..4g+3, 8+4g..} of sub-tile `sub`, column 32 db + l32
+    // fragment f = (t, db): rows 16t + {4g..4g+3, 8+4g..} of sub-tile `sub`, columns of block db
     auto z_read = [&](const int (&za)[ZQ], int sub, int f) -> V8 {
         const int t = f / DB, db = f % DB;
         const unsigned char *zp = smem + za[db % ZQ] + ((sub * 32 + 16 * t) * RZ + (db / ZQ) * (ZQ * 64));
@@ -294,6 +316,7 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
     }
     wait_tile(0);
     __builtin_amdgcn_s_barrier();  // tile 0 (and the X fragments) have landed
+    FLA_STAMP(1);
     issue_tile(Cfg::NBUF - 2, issue_off);
     issue_off = next_slot(issue_off);
     // from here on: tiles up to q + NBUF - 2 are issued while tile q is consumed
@@ -347,7 +370,7 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
                 if constexpr (decltype(with_pv)::value) {
                     const int t = f / DB, db = f % DB;
 #pragma unroll
-                    for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(pprev[ib][t], zf[f], acc[ib][db]);
+                    for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(zf[f], pprev[ib][t], acc[ib][db]);
                 }
 #ifndef FLA_DBG_NO_YREAD
 #pragma unroll
@@ -410,11 +433,12 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
             for (int f = 0; f < NZF; ++f) {
                 const int t = f / DB, db = f % DB;
 #pragma unroll
-                for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(pfb[ib][t], zf[f], acc[ib][db]);
+                for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(zf[f], pfb[ib][t], acc[ib][db]);
             }
         }
     }
 
+    FLA_STAMP(2);
     // ================= the diagonal block =================
     for (; q < n_seq; ++q) {
         const int row0 = i0 + (q - n_full) * BN;
@@ -466,7 +490,7 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
 #pragma unroll
                     for (int e = 0; e < 8; ++e) pf[t][e] = static_cast<T>(s[8 * t + e]);
 #pragma unroll
-                for (int f = 0; f < NZF; ++f) acc[ib][f % DB] = M::mma(pf[f / DB], zf[f], acc[ib][f % DB]);
+                for (int f = 0; f < NZF; ++f) acc[ib][f % DB] = M::mma(zf[f], pf[f / DB], acc[ib][f % DB]);
             }
         }
         wait_tile(q + 1);
@@ -475,22 +499,42 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
         advance();
     }
 
-    // ---- epilogue: acc[ib][db][v] is Out[row = 8(v/4) + 4g + v%4][col = 32 db + l32] of block ib
+    FLA_STAMP(3);
+    // ---- epilogue.  The second product is issued as Out^T += Z^T P^T (the two register
+    // operands swapped), and with the column permutation of the Z fragments acc[ib][db][v] is
+    // Out[row l32 of block ib][column 32 db + 16 g + v]: 16 consecutive columns per lane.
+    // They go to LDS as two 16-byte writes (the ring is idle: every wave has passed the last
+    // barrier of the walk), and the tile leaves as whole rows, 16 bytes per lane.
+    {
+        constexpr int RO = Cfg::RO;
 #pragma unroll
-    for (int ib = 0; ib < NIB; ++ib) {
+        for (int ib = 0; ib < NIB; ++ib) {
+            unsigned char *rowp = smem + (blk[ib] * 32 + l32) * RO + 32 * g;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int row = i0 + blk[ib] * 32 + 8 * (v / 4) + 4 * g + (v % 4);
-            if (row < N) {
-                T *rp = O + (int64_t)row * p.os_n;
+            for (int db = 0; db < DB; ++db) {
 #pragma unroll
-                for (int db = 0; db < DB; ++db) {
-                    const int col = db * 32 + l32;
-                    if (col < p.dout) rp[col] = static_cast<T>(acc[ib][db][v]);
+                for (int hq = 0; hq < 2; ++hq) {
+                    V8 o8;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) o8[e] = static_cast<T>(acc[ib][db][8 * hq + e]);
+                    *reinterpret_cast<u32x4 *>(rowp + 64 * db + 16 * hq) = __builtin_bit_cast(u32x4, o8);
                 }
             }
         }
+        __syncthreads();
+        constexpr int CO = DO / 8;  // 16-byte chunks per output row
+#pragma unroll
+        for (int u = 0; u < BM * CO / 256; ++u) {
+            const int c = tid + 256 * u, r = c / CO, cc = c - r * CO;
+            const int row = i0 + r;
+            if (row < N && cc * 8 < p.dout) {
+                const u32x4 val = *reinterpret_cast<const u32x4 *>(smem + r * RO + cc * 16);
+                *reinterpret_cast<u32x4 *>(O + (int64_t)row * p.os_n + cc * 8) = val;
+            }
+        }
+        __syncthreads();  // the staging area is ring space again
     }
+    FLA_STAMP(4);
     }  // pass
 #else
     (void)p;
@@ -501,7 +545,7 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
 // aligned with widths in whole chunks, and each (b, h) slice addressable with
 // 32-bit byte offsets.
 inline bool fast_path_ok(const TriParams &p) {
-    if (!(p.vec_x && p.vec_y && p.vec_z)) return false;
+    if (!(p.vec_x && p.vec_y && p.vec_z && p.vec_out)) return false;
     const int64_t n = p.N;
     return n * p.xs_n * 2 <= kMaxFastExtent && n * p.ys_n * 2 <= kMaxFastExtent && n * p.zs_n * 2 <= kMaxFastExtent;
 }

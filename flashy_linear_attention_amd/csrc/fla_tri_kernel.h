@@ -47,6 +47,10 @@ struct TriParams {
     int32_t upper;     // 0: keep row >= col, 1: keep row <= col
     int32_t n_tiles;   // ceil(N / BM), filled by the launcher
     int32_t vec_x, vec_y, vec_z;  // 1: rows are 16-byte aligned and width % 8 == 0
+    int32_t vec_out;              // same for the output
+#ifdef FLA_DBG_TIMING
+    unsigned long long *dbg;      // 16 clock stamps per workgroup (experimental builds only)
+#endif
 };
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
