@@ -33,6 +33,10 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0}  # MI355X dense MFMA, published
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per kernel launch (mean over the launches of one step), measured with
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`, each scaled by what the same counter
+# reads for a 256 MiB device copy (fetch x2.0, write x1.0); see profiles/*_pmc.md.
+MEASURED_TRAFFIC_BYTES = {"C3": 796e6}
 
 
 def _parse():
@@ -43,6 +47,9 @@ def _parse():
     ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU oracle timing")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target seconds of CPU work for the baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one plain device copy of 256 MiB (a known-size reference for scaling "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     return ap.parse_args()
 
 
@@ -126,6 +133,13 @@ def main() -> int:
         if w.backward:
             bwd(do, q, k, v)
 
+    if args.calibrate_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
+
     for _ in range(args.warmup):
         step()
     ms_total = _time_region(torch, step, args.steps)
@@ -178,7 +192,7 @@ def main() -> int:
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": round(achieved / peak, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
             "launches_per_step": launches,
             "flops_per_launch": flops_launch,
             "avg_launch_ms": round(ms_launch, 4),
