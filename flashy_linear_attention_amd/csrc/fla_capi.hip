@@ -60,6 +60,17 @@ int check_common(int64_t B, int64_t H, int64_t N, int dtype) {
 int run_tri(const View &x, const View &y, const View &z, const View &out, int64_t B, int64_t H, int64_t N,
             int64_t dc, int64_t dout, int upper, int dtype, void *stream) {
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    // Output wider than 128 columns with a narrow (<= 64) or a 256-wide contraction: run the two
+    // 128-column halves of Z / Out as separate launches.  The 64-rows-per-wave kernels that
+    // this selects beat the single 256-wide launch (which needs the 32-row layout, or the
+    // generic kernel for 256 x 256) although S is formed twice; results are bit-identical
+    // because every output column is an independent sum.
+    if (dout > 128 && (dc <= 64 || dc > 128)) {
+        const View z_hi{static_cast<const char *>(z.ptr) + 128 * 2, z.strides};
+        const View out_hi{static_cast<const char *>(out.ptr) + 128 * 2, out.strides};
+        if (int rc = run_tri(x, y, z, out, B, H, N, dc, 128, upper, dtype, stream)) return rc;
+        return run_tri(x, y, z_hi, out_hi, B, H, N, dc, dout - 128, upper, dtype, stream);
+    }
     TriParams p;
     p.x = x.ptr, p.y = y.ptr, p.z = z.ptr, p.out = const_cast<void *>(out.ptr);
     p.xs_b = x.strides[0], p.xs_h = x.strides[1], p.xs_n = x.strides[2];
