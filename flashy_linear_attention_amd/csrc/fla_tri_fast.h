@@ -440,63 +440,94 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
 
     FLA_STAMP(2);
     // ================= the diagonal block =================
-    for (; q < n_seq; ++q) {
-        const int row0 = i0 + (q - n_full) * BN;
-        int ya_cur[YQ], za_cur[ZQ];
-        slot_addrs(cur_off, ya_cur, za_cur);
+    // Its tiles (BM / BN of them, never more than the ring holds) are all made resident first;
+    // then every wave walks the 32-row sub-tiles its two row blocks touch, without barriers,
+    // fetching the fragments of the next sub-tile while the MFMAs of the current one run.
+    {
+        static_assert(BM / BN <= Cfg::NBUF, "the diagonal block must fit in the LDS ring");
+        if (n_full > 0) __builtin_amdgcn_s_barrier();  // every wave is done with the last full tile
+        issue_tile(q + Cfg::NBUF - 1, issue_off);      // the one tile not yet requested (if any)
+        wait_vm<0>();
+        __builtin_amdgcn_s_barrier();
+        FLA_STAMP(5);
+
+        constexpr int RING = Cfg::NBUF * STAGE;
+        const int nsub = (diag_rows + 31) >> 5;  // sub-tiles with at least one valid row
+        int blk_min = blk[0], blk_max = blk[0];
+        if constexpr (NIB == 2) {
+            blk_min = blk[0] < blk[1] ? blk[0] : blk[1];
+            blk_max = blk[0] < blk[1] ? blk[1] : blk[0];
+        }
+        const int s_lo = upper ? blk_min : 0;
+        const int s_hi = upper ? nsub - 1 : (blk_max < nsub - 1 ? blk_max : nsub - 1);
+
+        auto load_sub = [&](int s8, V8 (&yf)[KC], V8 (&zf)[NZF]) {
+            int so = cur_off + (s8 >> 1) * STAGE;
+            if (so >= RING) so -= RING;
+            int ya[YQ], za[ZQ];
 #pragma unroll
-        for (int sub = 0; sub < BN / 32; ++sub) {
-            const int j0 = row0 + sub * 32;
-            // 0: fully masked, 1: fully kept, 2: straddles the diagonal
-            int st[NIB];
-            bool any = false;
+            for (int j = 0; j < YQ; ++j) ya[j] = ylane[j] + so + (s8 & 1) * (32 * RY);
+#pragma unroll
+            for (int j = 0; j < ZQ; ++j) za[j] = zlane[j] + so + (s8 & 1) * (32 * RZ);
+#pragma unroll
+            for (int kc = 0; kc < KC; ++kc) yf[kc] = y_read(ya, 0, kc);
+#pragma unroll
+            for (int f = 0; f < NZF; ++f) zf[f] = z_read(za, 0, f);
+        };
+        auto compute_sub = [&](int s8, const V8 (&yf)[KC], const V8 (&zf)[NZF]) {
+            bool act[NIB];
+            f32x16 sd[NIB];
 #pragma unroll
             for (int ib = 0; ib < NIB; ++ib) {
-                const int ib0 = i0 + blk[ib] * 32;
-                if (upper)
-                    st[ib] = (j0 < ib0) ? 0 : (j0 == ib0 ? 2 : 1);
-                else
-                    st[ib] = (j0 > ib0) ? 0 : (j0 == ib0 ? 2 : 1);
-                any = any || st[ib] != 0;
+                act[ib] = upper ? s8 >= blk[ib] : s8 <= blk[ib];
+                if (act[ib]) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) sd[ib][v] = 0.f;
+#pragma unroll
+                    for (int kc = 0; kc < KC; ++kc) sd[ib] = M::mma(yf[kc], xf[ib][kc], sd[ib]);
+                }
             }
-            if (!any || j0 >= N) continue;
-
-            V8 yf[KC];
-#pragma unroll
-            for (int kc = 0; kc < KC; ++kc) yf[kc] = y_read(ya_cur, sub, kc);
-            V8 zf[NZF];
-#pragma unroll
-            for (int f = 0; f < NZF; ++f) zf[f] = z_read(za_cur, sub, f);
-
 #pragma unroll
             for (int ib = 0; ib < NIB; ++ib) {
-                if (st[ib] == 0) continue;
-                f32x16 s;
-#pragma unroll
-                for (int v = 0; v < 16; ++v) s[v] = 0.f;
-#pragma unroll
-                for (int kc = 0; kc < KC; ++kc) s = M::mma(yf[kc], xf[ib][kc], s);
-                if (st[ib] == 2) {
+                if (!act[ib]) continue;
+                if (s8 == blk[ib]) {  // the 32 x 32 block on the diagonal itself
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int jl = 8 * (v / 4) + 4 * g + (v % 4);
                         const bool keep = upper ? l32 <= jl : l32 >= jl;
-                        s[v] = keep ? s[v] : 0.f;
+                        sd[ib][v] = keep ? sd[ib][v] : 0.f;
                     }
                 }
                 V8 pf[2];
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) pf[t][e] = static_cast<T>(s[8 * t + e]);
+                    for (int e = 0; e < 8; ++e) pf[t][e] = static_cast<T>(sd[ib][8 * t + e]);
 #pragma unroll
                 for (int f = 0; f < NZF; ++f) acc[ib][f % DB] = M::mma(zf[f], pf[f / DB], acc[ib][f % DB]);
             }
+        };
+#ifndef FLA_DBG_NO_DIAG
+        if (s_lo <= s_hi) {
+            V8 yfa[KC], zfa[NZF], yfb[KC], zfb[NZF];
+            load_sub(s_lo, yfa, zfa);
+            for (int s8 = s_lo; s8 <= s_hi; s8 += 2) {
+                // the scheduling barriers keep the compiler from sinking the prefetch next to its use
+                if (s8 + 1 <= s_hi) load_sub(s8 + 1, yfb, zfb);
+                __builtin_amdgcn_sched_barrier(0);
+                compute_sub(s8, yfa, zfa);
+                __builtin_amdgcn_sched_barrier(0);
+                if (s8 + 1 <= s_hi) {
+                    if (s8 + 2 <= s_hi) load_sub(s8 + 2, yfa, zfa);
+                    __builtin_amdgcn_sched_barrier(0);
+                    compute_sub(s8 + 1, yfb, zfb);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
         }
-        wait_tile(q + 1);
-        __builtin_amdgcn_s_barrier();  // tile q+1 has landed; tile q-1 is long retired
-        issue_tile(q + Cfg::NBUF - 1, issue_off);
-        advance();
+#endif
+        FLA_STAMP(6);
+        __builtin_amdgcn_s_barrier();  // all LDS reads of the walk are done: the ring can be reused
     }
 
     FLA_STAMP(3);
