@@ -1,7 +1,8 @@
 """Causal linear attention for MI355X (gfx950): hand-written HIP kernels behind
 the Python surface of ``flashlinear`` (flashlinear/__init__.py:1-2)."""
 
+from .chunked import LinearAttentionChunked
 from .linear_attn import LinearAttention
 from .linear_attn_smallv_hd import LinearAttentionSmallVHD
 
-__all__ = ["LinearAttention", "LinearAttentionSmallVHD"]
+__all__ = ["LinearAttention", "LinearAttentionSmallVHD", "LinearAttentionChunked"]

@@ -31,6 +31,9 @@ SIGNATURES = {
     "fla_linear_attn_smallv_fwd": ([_ptr] * 4 + [_i64] * 5 + [_strides] * 4 + [ctypes.c_int, _ptr], ctypes.c_int),
     "fla_linear_attn_smallv_bwd": ([_ptr] * 7 + [_i64] * 5 + [_strides] * 7 + [ctypes.c_int, _ptr], ctypes.c_int),
     "fla_tri_xyt_z": ([_ptr] * 4 + [_i64] * 5 + [_strides] * 4 + [ctypes.c_int, ctypes.c_int, _ptr], ctypes.c_int),
+    "fla_chunked_workspace_bytes": ([_i64] * 5, ctypes.c_int64),
+    "fla_tri_xyt_z_chunked": ([_ptr] * 4 + [_i64] * 5 + [_strides] * 4 + [ctypes.c_int, ctypes.c_int, _ptr, _i64, _ptr],
+                              ctypes.c_int),
 }
 
 _lock = threading.Lock()

@@ -22,6 +22,25 @@ launch_fn lookup(int dtype, int64_t dc, int64_t dout) {
     return table[pad_index(dc) * 4 + pad_index(dout)][dtype];
 }
 
+typedef hipError_t (*state_fn)(const fla::ChunkStateParams &, hipStream_t);
+
+state_fn lookup_state(int dtype, int64_t dc, int64_t dout) {
+#define FLA_ENTRY(c, o) {fla::FLA_STATE_NAME(0, c, o), fla::FLA_STATE_NAME(1, c, o)},
+    static const state_fn table[16][2] = {FLA_FOR_EACH_DIM_PAIR(FLA_ENTRY)};
+#undef FLA_ENTRY
+    return table[pad_index(dc) * 4 + pad_index(dout)][dtype];
+}
+
+// rows per chunk of the chunked evaluation for this pair of widths (0: none available)
+int chunk_rows(int64_t dc, int64_t dout) {
+#define FLA_ENTRY(c, o) fla::fla_chunk_rows_c##c##_o##o,
+    static int (*const table[16])() = {FLA_FOR_EACH_DIM_PAIR(FLA_ENTRY)};
+#undef FLA_ENTRY
+    return table[pad_index(dc) * 4 + pad_index(dout)]();
+}
+
+int64_t padded(int64_t d) { return d <= 32 ? 32 : d <= 64 ? 64 : d <= 128 ? 128 : 256; }
+
 int64_t next_pow2(int64_t x) {
     int64_t p = 1;
     while (p < x) p <<= 1;
@@ -81,6 +100,7 @@ int run_tri(const View &x, const View &y, const View &z, const View &out, int64_
     p.dc = (int32_t)dc, p.dout = (int32_t)dout;
     p.upper = upper ? 1 : 0;
     p.n_tiles = 0;
+    p.state = nullptr;
     p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout), p.vec_out = vec_ok(out, dout);
 #ifdef FLA_DBG_TIMING
     {
@@ -91,6 +111,72 @@ int run_tri(const View &x, const View &y, const View &z, const View &out, int64_
     launch_fn fn = lookup(dtype, dc, dout);
     if (!fn) return FLA_ERR_UNSUPPORTED;
     return fn(p, static_cast<hipStream_t>(stream)) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+}
+
+// bytes of workspace the chunked evaluation of one product needs: fp32 chunk states plus
+// their 16-bit running sums, [BH][chunks][DO][DC] each with padded widths
+int64_t chunked_bytes(int64_t B, int64_t H, int64_t N, int64_t dc, int64_t dout) {
+    if (dout > 128 && (dc <= 64 || dc > 128)) dout = 128;  // evaluated as two 128-column halves
+    const int rows = chunk_rows(dc, dout);
+    if (rows == 0 || N <= rows) return 0;
+    const int64_t chunks = (N + rows - 1) / rows;
+    return B * H * chunks * padded(dc) * padded(dout) * 6;
+}
+
+// Out = mask(X Y^T) Z evaluated chunk-wise; same arguments as run_tri plus the workspace.
+// Falls back to the quadratic kernels when the operands do not qualify for the fast path
+// or the sequence is a single chunk.
+int run_tri_chunked(const View &x, const View &y, const View &z, const View &out, int64_t B, int64_t H, int64_t N,
+                    int64_t dc, int64_t dout, int upper, int dtype, void *workspace, int64_t workspace_bytes,
+                    void *stream) {
+    if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    if (dout > 128 && (dc <= 64 || dc > 128)) {
+        const View z_hi{static_cast<const char *>(z.ptr) + 128 * 2, z.strides};
+        const View out_hi{static_cast<const char *>(out.ptr) + 128 * 2, out.strides};
+        if (int rc = run_tri_chunked(x, y, z, out, B, H, N, dc, 128, upper, dtype, workspace, workspace_bytes, stream))
+            return rc;
+        return run_tri_chunked(x, y, z_hi, out_hi, B, H, N, dc, dout - 128, upper, dtype, workspace, workspace_bytes,
+                               stream);
+    }
+    const int rows = chunk_rows(dc, dout);
+    TriParams p;
+    p.x = x.ptr, p.y = y.ptr, p.z = z.ptr, p.out = const_cast<void *>(out.ptr);
+    p.xs_b = x.strides[0], p.xs_h = x.strides[1], p.xs_n = x.strides[2];
+    p.ys_b = y.strides[0], p.ys_h = y.strides[1], p.ys_n = y.strides[2];
+    p.zs_b = z.strides[0], p.zs_h = z.strides[1], p.zs_n = z.strides[2];
+    p.os_b = out.strides[0], p.os_h = out.strides[1], p.os_n = out.strides[2];
+    p.H = (int32_t)H, p.N = (int32_t)N, p.BH = (int32_t)(B * H);
+    p.dc = (int32_t)dc, p.dout = (int32_t)dout;
+    p.upper = upper ? 1 : 0;
+    p.n_tiles = 0;
+    p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout), p.vec_out = vec_ok(out, dout);
+    p.state = nullptr;
+#ifdef FLA_DBG_TIMING
+    p.dbg = nullptr;
+#endif
+    if (rows == 0 || N <= rows || !fla::fast_path_ok(p))
+        return run_tri(x, y, z, out, B, H, N, dc, dout, upper, dtype, stream);
+
+    const int64_t chunks = (N + rows - 1) / rows, E = padded(dc) * padded(dout), BH = B * H;
+    if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < BH * chunks * E * 6)
+        return FLA_ERR_WORKSPACE;
+    float *w = static_cast<float *>(workspace);
+    void *state = static_cast<char *>(workspace) + BH * chunks * E * 4;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+
+    fla::ChunkStateParams cp;
+    cp.y = y.ptr, cp.z = z.ptr, cp.w = w;
+    cp.ys_b = p.ys_b, cp.ys_h = p.ys_h, cp.ys_n = p.ys_n;
+    cp.zs_b = p.zs_b, cp.zs_h = p.zs_h, cp.zs_n = p.zs_n;
+    cp.H = p.H, cp.N = p.N, cp.BH = p.BH, cp.dc = p.dc, cp.dout = p.dout;
+    cp.n_chunks = (int32_t)chunks;
+    if (lookup_state(dtype, dc, dout)(cp, s) != hipSuccess) return FLA_ERR_LAUNCH;
+    const hipError_t e = dtype == FLA_DTYPE_BF16
+                             ? fla::launch_chunk_scan<__bf16>(w, state, BH, (int)chunks, E, upper ? 1 : 0, s)
+                             : fla::launch_chunk_scan<_Float16>(w, state, BH, (int)chunks, E, upper ? 1 : 0, s);
+    if (e != hipSuccess) return FLA_ERR_LAUNCH;
+    p.state = state;
+    return lookup(dtype, dc, dout)(p, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
 }
 
 int forward(const View &q, const View &k, const View &v, const View &o, int64_t B, int64_t H, int64_t N,
@@ -130,6 +216,7 @@ const char *fla_strerror(int status) {
         case FLA_ERR_STRIDE: return "strides must be given, non-negative, with innermost stride 1";
         case FLA_ERR_LAUNCH: return "the HIP runtime rejected the kernel launch";
         case FLA_ERR_UNSUPPORTED: return "no kernel was built for this combination";
+        case FLA_ERR_WORKSPACE: return "workspace is NULL, not 16-byte aligned, or smaller than fla_chunked_workspace_bytes()";
         default: return "unknown fla status";
     }
 }
@@ -186,6 +273,24 @@ int fla_tri_xyt_z(const void *x, const void *y, const void *z, void *out, int64_
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
     return run_tri(vx, vy, vz, vo, B, H, N, D_c, D_o, upper, dtype, stream);
+}
+
+int64_t fla_chunked_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t D_c, int64_t D_o) {
+    if (B < 0 || H < 0 || N < 0 || D_c < 1 || D_c > 256 || D_o < 1 || D_o > 256) return 0;
+    return chunked_bytes(B, H, N, D_c, D_o);
+}
+
+int fla_tri_xyt_z_chunked(const void *x, const void *y, const void *z, void *out, int64_t B, int64_t H, int64_t N,
+                          int64_t D_c, int64_t D_o, const int64_t *x_strides, const int64_t *y_strides,
+                          const int64_t *z_strides, const int64_t *out_strides, int upper, int dtype,
+                          void *workspace, int64_t workspace_bytes, void *stream) {
+    if (int rc = check_common(B, H, N, dtype)) return rc;
+    if (D_c < 1 || D_c > 256 || D_o < 1 || D_o > 256) return FLA_ERR_HEAD_DIM;
+    const View vx{x, x_strides}, vy{y, y_strides}, vz{z, z_strides}, vo{out, out_strides};
+    const View all[] = {vx, vy, vz, vo};
+    for (const View &t : all)
+        if (int rc = check_view(t)) return rc;
+    return run_tri_chunked(vx, vy, vz, vo, B, H, N, D_c, D_o, upper, dtype, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -1,0 +1,198 @@
+// Chunk states for the chunked evaluation of Out = mask(X Y^T) Z.
+//
+// With the rows cut into chunks of BM rows (the row tile of the main kernel),
+//
+//     Out_c = mask(X_c Y_c^T) Z_c  +  X_c . S_c ,    S_c = sum over chunks c' before c (lower mask)
+//                                                         or after c (upper mask) of Y_c'^T Z_c'
+//
+// so everything off the diagonal blocks collapses into a D_c x D_o state per chunk:
+// O(N BM D + N D_c D_o) work instead of O(N^2 D).  Two kernels prepare the states:
+//
+//   chunk_state_kernel : W_c^T = Z_c^T Y_c for every chunk, fp32, [BH][chunks][DO][DC]
+//                        (both MFMA operands are column reads of row-major LDS tiles, i.e.
+//                        ds_read_b64_tr_b16; the kernel reads Y and Z once and is HBM-bound)
+//   chunk_scan_kernel  : exclusive prefix (lower) or suffix (upper) sum over the chunks in fp32,
+//                        rounded once to the 16-bit storage type the main kernel multiplies with
+//
+// The main kernel (fla_tri_fast.h, TriParams::state) then adds X_c . S_c after its diagonal block.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fla_tri_fast.h"
+
+namespace fla {
+
+struct ChunkStateParams {
+    const void *y, *z;
+    float *w;  // [BH][n_chunks][DO][DC] fp32, padded widths
+    int64_t ys_b, ys_h, ys_n;
+    int64_t zs_b, zs_h, zs_n;
+    int32_t H, N, BH;
+    int32_t dc, dout;
+    int32_t n_chunks;
+};
+
+template <typename T, int DC, int DO>
+__global__ __launch_bounds__(256) void chunk_state_kernel(const ChunkStateParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    using Cfg = FastConfig<DC, DO>;
+    using M = Mma<T>;
+    using V8 = typename M::V8;
+    constexpr int BM = Cfg::BM, BN = Cfg::BN;
+    constexpr int RY = Cfg::RY, RZ = Cfg::RZ, CY = Cfg::CY, CZ = Cfg::CZ;
+    constexpr int NIY = Cfg::NIY, NIZ = Cfg::NIZ;
+    constexpr int STAGE = Cfg::STAGE_BYTES, Y_BYTES = Cfg::Y_BYTES;
+    constexpr int NTILE = BM / BN;  // 64-row tiles per chunk, all resident in LDS at once
+    static_assert(NTILE <= Cfg::NBUF, "a chunk must fit in the LDS ring");
+    constexpr int EB = DO / 32, DBK = DC / 32;     // 32 x 32 output blocks
+    constexpr int NBW = (EB * DBK + 3) / 4;        // blocks per wave (block b goes to wave b % 4)
+
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int g = lane >> 5, lam = lane & 15, l32 = lane & 31, beta = (lane >> 4) & 1;
+
+    const int wg = blockIdx.x, xcd = wg & 7, slot = wg >> 3;
+    const int hl = slot / p.n_chunks, chunk = slot - hl * p.n_chunks;
+    const int bh = hl * 8 + xcd;
+    if (bh >= p.BH) return;
+    const int b = bh / p.H, h = bh - b * p.H;
+    const T *Y = static_cast<const T *>(p.y) + b * p.ys_b + h * p.ys_h;
+    const T *Z = static_cast<const T *>(p.z) + b * p.zs_b + h * p.zs_h;
+    const int N = p.N, r0 = chunk * BM;
+    const int ys2 = (int)p.ys_n * 2, zs2 = (int)p.zs_n * 2;
+    const u32x4 ry = make_rsrc(Y, (uint32_t)((N - 1) * ys2 + p.dc * 2));
+    const u32x4 rz = make_rsrc(Z, (uint32_t)((N - 1) * zs2 + p.dout * 2));
+
+    // whole chunk -> LDS (rows beyond N and columns beyond the true widths arrive as zeros)
+#pragma unroll
+    for (int t = 0; t < NTILE; ++t) {
+        const uint32_t yb = lds0 + t * STAGE + wave * 1024, zb = yb + Y_BYTES;
+        const int row0 = r0 + t * BN;
+#pragma unroll
+        for (int u = 0; u < NIY; ++u) {
+            const int row = (u * 4 + wave) * (1024 / RY) + lane / CY;
+            const int c = (lane % CY) ^ swizzle_y<CY>(row);
+            const uint32_t off = (uint32_t)(row * ys2 + c * 16) + (c * 8 < p.dc ? 0u : kOobOffset);
+            dma_16B_per_lane(ry, yb + u * 4096, off, row0 * ys2);
+        }
+#pragma unroll
+        for (int u = 0; u < NIZ; ++u) {
+            const int row = (u * 4 + wave) * (1024 / RZ) + lane / CZ;
+            const int c = (lane % CZ) ^ swizzle_z<CZ>(row);
+            const uint32_t off = (uint32_t)(row * zs2 + c * 16) + (c * 8 < p.dout ? 0u : kOobOffset);
+            dma_16B_per_lane(rz, zb + u * 4096, off, row0 * zs2);
+        }
+    }
+    wait_vm<0>();
+    __builtin_amdgcn_s_barrier();
+
+    // Column fragment of a row-major tile: rows R0 + {4g..4g+3, 8+4g..8+4g+3}, column 32 cb + l32.
+    // Source lane `lam` of a 16-lane group addresses row lam/4, chunk lam%4 of the 16 columns
+    // 32 cb + 16 beta .. +15 (plain, unpermuted mapping: destination lane i gets column i).
+    auto col_frag = [&](const unsigned char *tile, int rowbytes, int cb, int R0, auto swz) -> V8 {
+        const int row_lo = R0 + 4 * g + (lam >> 2), row_hi = row_lo + 8;
+        const int chunk16 = 4 * cb + 2 * beta + ((lam & 3) >> 1), sub = 8 * (lam & 1);
+        const unsigned char *plo = tile + row_lo * rowbytes + ((chunk16 ^ swz(row_lo)) << 4) + sub;
+        const unsigned char *phi = tile + row_hi * rowbytes + ((chunk16 ^ swz(row_hi)) << 4) + sub;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(plo));
+        const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(phi));
+        return __builtin_bit_cast(V8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+    };
+
+    f32x16 acc[NBW];
+#pragma unroll
+    for (int i = 0; i < NBW; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+
+#pragma unroll 1
+    for (int t = 0; t < NTILE; ++t) {
+        const unsigned char *ytile = smem + t * STAGE, *ztile = ytile + Y_BYTES;
+#pragma unroll
+        for (int ks = 0; ks < BN / 16; ++ks) {
+#pragma unroll
+            for (int i = 0; i < NBW; ++i) {
+                const int blk = wave + 4 * i;  // = eb * DBK + dbk
+                if (blk < EB * DBK) {
+                    const int eb = blk / DBK, dbk = blk % DBK;
+                    const V8 a = col_frag(ztile, RZ, eb, 16 * ks, [](int r) { return swizzle_z<CZ>(r); });
+                    const V8 bfr = col_frag(ytile, RY, dbk, 16 * ks, [](int r) { return swizzle_y<CY>(r); });
+                    acc[i] = M::mma(a, bfr, acc[i]);
+                }
+            }
+        }
+    }
+
+    // acc[i][v] = W^T[e = 32 eb + 8(v/4) + 4g + v%4][d = 32 dbk + l32]
+    float *W = p.w + ((int64_t)bh * p.n_chunks + chunk) * (DO * DC);
+#pragma unroll
+    for (int i = 0; i < NBW; ++i) {
+        const int blk = wave + 4 * i;
+        if (blk < EB * DBK) {
+            const int eb = blk / DBK, dbk = blk % DBK;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) W[(32 * eb + 8 * (v / 4) + 4 * g + (v % 4)) * DC + 32 * dbk + l32] = acc[i][v];
+        }
+    }
+#else
+    (void)p;
+#endif
+}
+
+// Exclusive running sum over the chunk axis of w[bh][chunk][E] (fp32), rounded to T.
+// reverse == 0: state[c] = sum_{c' < c} w[c'];  reverse != 0: state[c] = sum_{c' > c} w[c'].
+template <typename T>
+__global__ __launch_bounds__(256) void chunk_scan_kernel(const float *w, T *state, int n_chunks, int64_t E,
+                                                        int64_t total4, int reverse) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));
+    typedef T t4 __attribute__((ext_vector_type(4)));
+    const int64_t i4 = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index of a group of 4 elements within [BH][E]
+    if (i4 >= total4) return;
+    const int64_t bh = (i4 * 4) / E, e = (i4 * 4) - bh * E;
+    const float *wp = w + bh * n_chunks * E + e;
+    T *sp = state + bh * n_chunks * E + e;
+    f32x4 run = {0.f, 0.f, 0.f, 0.f};
+    for (int k = 0; k < n_chunks; ++k) {
+        const int c = reverse ? n_chunks - 1 - k : k;
+        t4 o;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) o[x] = static_cast<T>(run[x]);
+        *reinterpret_cast<t4 *>(sp + (int64_t)c * E) = o;
+        run += *reinterpret_cast<const f32x4 *>(wp + (int64_t)c * E);
+    }
+}
+
+template <typename T, int DC, int DO>
+hipError_t launch_chunk_state(ChunkStateParams p, hipStream_t stream) {
+    using Cfg = FastConfig<DC, DO>;
+    if constexpr (!Cfg::kSupported) {
+        return hipErrorNotSupported;
+    } else {
+        const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_chunks;
+        if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+        auto kern = chunk_state_kernel<T, DC, DO>;
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM_BYTES);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), Cfg::SMEM_BYTES, stream, p);
+        return hipGetLastError();
+    }
+}
+
+template <typename T>
+hipError_t launch_chunk_scan(const float *w, void *state, int64_t BH, int n_chunks, int64_t E, int reverse,
+                             hipStream_t stream) {
+    const int64_t total4 = BH * E / 4;
+    const int64_t grid = (total4 + 255) / 256;
+    if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    hipLaunchKernelGGL(chunk_scan_kernel<T>, dim3((unsigned)grid), dim3(256), 0, stream, w, static_cast<T *>(state),
+                       n_chunks, E, total4, reverse);
+    return hipGetLastError();
+}
+
+}  // namespace fla

@@ -3,6 +3,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include "fla_chunk_state.h"
 #include "fla_tri_kernel.h"
 
 // Padded (DC, DO) pairs for which a kernel is built.  Widths are padded to the
@@ -14,11 +15,16 @@
 
 #define FLA_LAUNCH_NAME_(t, dc, dout) fla_launch_tri_t##t##_c##dc##_o##dout
 #define FLA_LAUNCH_NAME(t, dc, dout) FLA_LAUNCH_NAME_(t, dc, dout)
+#define FLA_STATE_NAME_(t, dc, dout) fla_launch_state_t##t##_c##dc##_o##dout
+#define FLA_STATE_NAME(t, dc, dout) FLA_STATE_NAME_(t, dc, dout)
 
 namespace fla {
-#define FLA_DECLARE(dc, dout)                                                        \
-    hipError_t FLA_LAUNCH_NAME(0, dc, dout)(const TriParams &p, hipStream_t stream); \
-    hipError_t FLA_LAUNCH_NAME(1, dc, dout)(const TriParams &p, hipStream_t stream);
+#define FLA_DECLARE(dc, dout)                                                               \
+    hipError_t FLA_LAUNCH_NAME(0, dc, dout)(const TriParams &p, hipStream_t stream);        \
+    hipError_t FLA_LAUNCH_NAME(1, dc, dout)(const TriParams &p, hipStream_t stream);        \
+    hipError_t FLA_STATE_NAME(0, dc, dout)(const ChunkStateParams &p, hipStream_t stream);  \
+    hipError_t FLA_STATE_NAME(1, dc, dout)(const ChunkStateParams &p, hipStream_t stream);  \
+    int fla_chunk_rows_c##dc##_o##dout();
 FLA_FOR_EACH_DIM_PAIR(FLA_DECLARE)
 #undef FLA_DECLARE
 }  // namespace fla

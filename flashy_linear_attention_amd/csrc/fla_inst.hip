@@ -24,4 +24,17 @@ hipError_t FLA_LAUNCH_NAME(FLA_INST_DTYPE, FLA_INST_DC, FLA_INST_DO)(const TriPa
     return launch_tri<InstT, FLA_INST_DC, FLA_INST_DO>(p, stream);
 }
 
+hipError_t FLA_STATE_NAME(FLA_INST_DTYPE, FLA_INST_DC, FLA_INST_DO)(const ChunkStateParams &p, hipStream_t stream) {
+    return launch_chunk_state<InstT, FLA_INST_DC, FLA_INST_DO>(p, stream);
+}
+
+#if FLA_INST_DTYPE == 0
+// rows per chunk of the chunked evaluation = row tile of the fast kernel (0: no fast kernel)
+#define FLA_CHUNK_ROWS_NAME_(dc, dout) fla_chunk_rows_c##dc##_o##dout
+#define FLA_CHUNK_ROWS_NAME(dc, dout) FLA_CHUNK_ROWS_NAME_(dc, dout)
+int FLA_CHUNK_ROWS_NAME(FLA_INST_DC, FLA_INST_DO)() {
+    return FastConfig<FLA_INST_DC, FLA_INST_DO>::kSupported ? FastConfig<FLA_INST_DC, FLA_INST_DO>::BM : 0;
+}
+#endif
+
 }  // namespace fla

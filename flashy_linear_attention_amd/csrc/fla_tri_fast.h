@@ -148,7 +148,9 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
     const int wg = blockIdx.x, xcd = wg & 7, slot = wg >> 3;
     // Each workgroup takes two row tiles of one head, r and n_tiles-1-r: under a triangular
     // mask their work adds up to the same amount for every r, so all workgroups are equal.
-    const int n_pairs = (p.n_tiles + 1) >> 1;
+    // (Chunked evaluation: one row tile per workgroup, all of equal work already.)
+    const bool chunked = p.state != nullptr;
+    const int n_pairs = chunked ? p.n_tiles : (p.n_tiles + 1) >> 1;
     const int hl = slot / n_pairs, rank = slot - hl * n_pairs;
     const int bh = hl * 8 + xcd;
     if (bh >= p.BH) return;
@@ -184,8 +186,9 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
 #endif
     for (int pass = 0; pass < 2; ++pass) {
     FLA_STAMP(0);
-    const int tile = pass == 0 ? p.n_tiles - 1 - rank : rank;
-    if (pass == 1 && tile == p.n_tiles - 1 - rank) break;  // odd tile count: the middle tile has no partner
+    const int tile = chunked ? rank : (pass == 0 ? p.n_tiles - 1 - rank : rank);
+    // odd tile count: the middle tile has no partner; chunked: a single tile per workgroup
+    if (pass == 1 && (chunked || tile == p.n_tiles - 1 - rank)) break;
     const int i0 = tile * BM;
 
     // ---- tile sequence: tiles fully inside the mask first, then the diagonal block
@@ -200,6 +203,7 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
         n_full = i0 / BN;
         full_row0 = 0;
     }
+    if (chunked) n_full = 0;  // everything off the diagonal block arrives through the state
     const int n_seq = n_full + n_diag;
 
     // ---- HBM -> LDS: per-lane source offsets (constant over tiles)
@@ -530,6 +534,28 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
         __builtin_amdgcn_s_barrier();  // all LDS reads of the walk are done: the ring can be reused
     }
 
+    // ---- chunked evaluation: Out_tile += X_tile . S with S^T[e][d] read straight from global
+    // memory as A operand (row = output column as permuted in the accumulators, k = d) and the
+    // resident X fragments as B operand.
+    if (chunked && (upper ? tile + 1 < p.n_tiles : tile > 0)) {
+        const T *st = static_cast<const T *>(p.state) + ((int64_t)bh * p.n_tiles + tile) * (DO * DC);
+        // accumulator register v of lane (l32, g) is column 16 g + v of its block; MFMA row
+        // m = 8a + 4g' + b of the A operand lands in register 4a + b of the lanes with g = g'
+        const int e_lane = 16 * ((l32 >> 2) & 1) + 4 * (l32 >> 3) + (l32 & 3);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            V8 sf[KC];
+#pragma unroll
+            for (int kc = 0; kc < KC; ++kc)
+                sf[kc] = __builtin_bit_cast(
+                    V8, *reinterpret_cast<const u32x4 *>(st + (32 * db + e_lane) * DC + 16 * kc + 8 * g));
+#pragma unroll
+            for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+                for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(sf[kc], xf[ib][kc], acc[ib][db]);
+        }
+    }
+
     FLA_STAMP(3);
     // ---- epilogue.  The second product is issued as Out^T += Z^T P^T (the two register
     // operands swapped), and with the column permutation of the Z fragments acc[ib][db][v] is
@@ -588,7 +614,7 @@ hipError_t launch_tri_fast(TriParams p, hipStream_t stream) {
         return hipErrorNotSupported;
     } else {
         p.n_tiles = (p.N + Cfg::BM - 1) / Cfg::BM;
-        const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * ((p.n_tiles + 1) / 2);
+        const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * (p.state ? p.n_tiles : (p.n_tiles + 1) / 2);
         if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
         auto kern = tri_xyt_z_fast_kernel<T, DC, DO>;
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),

@@ -48,6 +48,11 @@ struct TriParams {
     int32_t n_tiles;   // ceil(N / BM), filled by the launcher
     int32_t vec_x, vec_y, vec_z;  // 1: rows are 16-byte aligned and width % 8 == 0
     int32_t vec_out;              // same for the output
+    // Chunked evaluation (fast path only): when non-null, each workgroup computes only the
+    // diagonal BM x BM block of its row tile and adds X_tile . S, where S is the 16-bit sum of
+    // Y_c^T Z_c over the chunks before (lower) / after (upper) the tile, stored transposed as
+    // state[(bh * n_tiles + tile)][DO][DC] with the padded DO, DC of the instantiation.
+    const void *state;
 #ifdef FLA_DBG_TIMING
     unsigned long long *dbg;      // 16 clock stamps per workgroup (experimental builds only)
 #endif

@@ -46,7 +46,8 @@ enum fla_status {
     FLA_ERR_SHAPE = -5,        /* negative B, H or N, or B*H*N too large */
     FLA_ERR_STRIDE = -6,       /* strides[3] != 1, a NULL strides array, or a negative stride */
     FLA_ERR_LAUNCH = -7,       /* the HIP runtime rejected the launch */
-    FLA_ERR_UNSUPPORTED = -8   /* no kernel was built for this combination */
+    FLA_ERR_UNSUPPORTED = -8,  /* no kernel was built for this combination */
+    FLA_ERR_WORKSPACE = -9     /* chunked call: workspace missing, misaligned or too small */
 };
 
 /* ABI revision of the loaded library (== FLA_ABI_VERSION it was built with). */
@@ -117,6 +118,26 @@ int fla_tri_xyt_z(const void *x, const void *y, const void *z, void *out,
                   const int64_t *x_strides, const int64_t *y_strides,
                   const int64_t *z_strides, const int64_t *out_strides,
                   int upper, int dtype, void *stream);
+
+/* The same product evaluated chunk-wise: rows are cut into chunks of the kernel's row tile
+ * (256 or 128 rows); each chunk's diagonal block is computed as above and everything off the
+ * diagonal arrives through the running sum S of the per-chunk states Y_c^T Z_c (fp32,
+ * rounded once to the storage dtype before X_c . S).  O(N (tile) D + N D_c D_o) work instead
+ * of O(N^2 D): the algorithm of choice for long sequences.  Results differ from
+ * fla_tri_xyt_z only by rounding.
+ *
+ * `workspace` is caller-owned device memory of at least fla_chunked_workspace_bytes() bytes,
+ * 16-byte aligned; it is scratch (no need to clear it) and may be reused by the next call on
+ * the same stream.  Operands that do not meet the fast-path alignment rules, and sequences
+ * of a single chunk, are evaluated by fla_tri_xyt_z instead (workspace unused).
+ * No counterpart in the reference: its kernels are quadratic in N
+ * (linear_attn_kernels.py:63, 166-171). */
+int64_t fla_chunked_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t D_c, int64_t D_o);
+int fla_tri_xyt_z_chunked(const void *x, const void *y, const void *z, void *out,
+                          int64_t B, int64_t H, int64_t N, int64_t D_c, int64_t D_o,
+                          const int64_t *x_strides, const int64_t *y_strides,
+                          const int64_t *z_strides, const int64_t *out_strides,
+                          int upper, int dtype, void *workspace, int64_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

@@ -1,0 +1,103 @@
+"""Chunk-wise evaluation (fla_tri_xyt_z_chunked) against the CPU oracle and against the
+quadratic kernels (``-m gpu``)."""
+
+import pytest
+import torch
+
+from flashy_linear_attention_amd import LinearAttention, LinearAttentionChunked, LinearAttentionSmallVHD
+from flashy_linear_attention_amd.chunked import tri_xyt_z_chunked
+from flashy_linear_attention_amd.synthetic import WORKLOADS, make_inputs
+from oracle import naive
+
+from helpers import assert_close, reference_style_inputs
+
+pytestmark = pytest.mark.gpu
+
+# (batch, heads, seq, d_qk, d_v): one chunk (falls through to the quadratic kernel), exact
+# multiples of the 256- and 128-row chunks, ragged last chunks, both chunk sizes, wide outputs
+CASES = [
+    (1, 2, 256, 64, 64),
+    (1, 3, 512, 64, 64),
+    (2, 2, 1024, 128, 128),
+    (1, 2, 1984, 128, 128),
+    (1, 2, 832, 64, 32),
+    (1, 2, 768, 256, 64),
+    (1, 2, 640, 64, 256),
+    (1, 1, 512, 128, 256),
+    (1, 2, 576, 48, 48),
+    (1, 1, 1024, 32, 32),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("dims", CASES, ids=lambda d: "x".join(map(str, d)))
+def test_chunked_fwd_bwd_vs_oracle(dims, dtype, gpu_device):
+    bs, nh, sq, dqk, dv = dims
+    q, k, v, dy = reference_style_inputs(bs, nh, sq, dqk, dv, dtype, seed=sum(dims))
+    want_o = naive.causal_dot_product(q.float(), k.float(), v.float())
+    want_g = naive.causal_dot_product_grads(q.float(), k.float(), v.float(), dy.float())
+    qg, kg, vg = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v))
+    out = LinearAttentionChunked.apply(qg, kg, vg)
+    assert out.dtype == dtype and out.shape == v.shape
+    out.backward(dy.to(gpu_device))
+    assert_close("O", out, want_o)
+    for name, got, want in (("dQ", qg.grad, want_g[0]), ("dK", kg.grad, want_g[1]), ("dV", vg.grad, want_g[2])):
+        assert_close(name, got, want)
+
+
+def test_chunked_matches_quadratic_closely(gpu_device):
+    """Same inputs through both algorithms: they differ only by the rounding of the running
+    state, far inside the tolerance against the oracle."""
+    q, k, v, dy = (t.to(gpu_device) for t in reference_style_inputs(2, 4, 2048, 128, 128, torch.bfloat16, seed=21))
+    a = LinearAttention.apply(q, k, v)
+    b = LinearAttentionChunked.apply(q, k, v)
+    assert_close("chunked vs quadratic", b, a.float(), tol_fro=5e-3, tol_max=1e-2)
+    q2, k2, v2, _ = (t.to(gpu_device) for t in reference_style_inputs(1, 2, 1024, 256, 64, torch.bfloat16, seed=22))
+    assert_close("small-V", LinearAttentionChunked.apply(q2, k2, v2), LinearAttentionSmallVHD.apply(q2, k2, v2).float(),
+                 tol_fro=5e-3, tol_max=1e-2)
+
+
+def test_chunked_upper_mask_and_unaligned_fallback(gpu_device):
+    x, y, z, _ = (t.to(gpu_device) for t in reference_style_inputs(1, 2, 768, 64, 64, torch.bfloat16, seed=23))
+    want = torch.matmul(torch.triu(torch.matmul(x.float().cpu(), y.float().cpu().transpose(-1, -2))), z.float().cpu())
+    assert_close("upper", tri_xyt_z_chunked(x, y, z, upper=True), want)
+    # width 50 is not a multiple of 8: evaluated by the quadratic generic kernel, same answer
+    x2, y2, z2, _ = (t.to(gpu_device) for t in reference_style_inputs(1, 2, 512, 50, 50, torch.bfloat16, seed=24))
+    want2 = naive.causal_dot_product(x2.float().cpu(), y2.float().cpu(), z2.float().cpu())
+    assert_close("unaligned", tri_xyt_z_chunked(x2, y2, z2, upper=False), want2)
+
+
+def test_chunked_long_context_workload(gpu_device):
+    """C5 (N = 32768, D = 64, bf16) forward + backward through the chunked path; four heads
+    against the oracle formula in fp32 on the GPU."""
+    w = WORKLOADS["C5"]
+    q, k, v, do = (t.to(gpu_device) for t in make_inputs(w, heads=4))
+    qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
+    out = LinearAttentionChunked.apply(qg, kg, vg)
+    out.backward(do)
+    for hh in range(4):
+        sl = (slice(0, 1), slice(hh, hh + 1))
+        qs, ks, vs, ds = (t[sl].float() for t in (q, k, v, do))
+        assert_close(f"O head {hh}", out[sl], naive.causal_dot_product_blocked(qs, ks, vs, block=2048))
+        for name, got, want in zip(("dQ", "dK", "dV"), (qg.grad, kg.grad, vg.grad),
+                                   naive.causal_dot_product_grads_blocked(qs, ks, vs, ds, block=2048)):
+            assert_close(f"{name} head {hh}", got[sl], want)
+
+
+def test_chunked_workspace_errors(gpu_device):
+    from flashy_linear_attention_amd import _lib
+
+    lib = _lib.load()
+    x = torch.zeros(1, 1, 1024, 64, dtype=torch.bfloat16, device=gpu_device)
+    out = torch.empty_like(x)
+    need = lib.fla_chunked_workspace_bytes(1, 1, 1024, 64, 64)
+    assert need == 1 * 1 * 4 * 64 * 64 * 6
+    assert lib.fla_chunked_workspace_bytes(1, 1, 256, 64, 64) == 0  # a single chunk needs none
+    st = _lib.strides_arg(x)
+    small = torch.empty(need - 16, dtype=torch.uint8, device=gpu_device)
+    rc = lib.fla_tri_xyt_z_chunked(x.data_ptr(), x.data_ptr(), x.data_ptr(), out.data_ptr(), 1, 1, 1024, 64, 64,
+                                   st, st, st, st, 0, 0, small.data_ptr(), need - 16, None)
+    assert rc == -9 and b"workspace" in lib.fla_strerror(rc)
+    rc = lib.fla_tri_xyt_z_chunked(x.data_ptr(), x.data_ptr(), x.data_ptr(), out.data_ptr(), 1, 1, 1024, 64, 64,
+                                   st, st, st, st, 0, 0, None, 0, None)
+    assert rc == -9
