@@ -47,6 +47,9 @@ def _parse():
     ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU oracle timing")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target seconds of CPU work for the baseline")
+    ap.add_argument("--algo", default="quadratic", choices=["quadratic", "chunked"],
+                    help="quadratic: the tiled O(N^2 D) kernels the headline metric is defined on (default); "
+                         "chunked: the O(N) chunk-state path, reported with its own FLOP count and an HBM roofline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain device copy of 256 MiB (a known-size reference for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -127,6 +130,10 @@ def main() -> int:
     q, k, v, do = (t.to(dev) for t in make_inputs(w, seed=0))
     fwd = linear_flash_wrapper_fwd_smallv_hd if w.small_v else linear_flash_wrapper_fwd
     bwd = linear_flash_wrapper_bwd_smallv_hd if w.small_v else linear_flash_wrapper_bwd
+    if args.algo == "chunked":
+        from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
+
+        fwd, bwd = linear_attention_chunked_fwd, linear_attention_chunked_bwd
 
     def step():
         fwd(q, k, v)
@@ -155,8 +162,16 @@ def main() -> int:
     tflops = flops_step / (ms_step * 1e-3) / 1e12
 
     # dominant (only) kernel: launches per step and algorithmic FLOPs per launch
-    launches = 1 + (3 if w.backward else 0)
-    flops_launch = float(w.batch * w.heads) * w.seq * w.seq * (w.d_qk + w.d_v)
+    # (a product whose output is wider than 128 columns with a <=64- or 256-wide contraction runs
+    # as two launches, one per 128-column half; flops_per_launch is then the mean over launches)
+    def n_launches(dc, dout):
+        return 2 if dout > 128 and (dc <= 64 or dc > 128) else 1
+
+    launches = n_launches(w.d_qk, w.d_v)
+    if w.backward:
+        launches += n_launches(w.d_v, w.d_qk) * 2 + n_launches(w.d_qk, w.d_v)
+    products = 1 + (3 if w.backward else 0)
+    flops_launch = float(w.batch * w.heads) * w.seq * w.seq * (w.d_qk + w.d_v) * products / launches
     ms_launch = ms_step / launches
     achieved = flops_launch / (ms_launch * 1e-3) / 1e12
 
@@ -198,6 +213,34 @@ def main() -> int:
             "avg_launch_ms": round(ms_launch, 4),
         },
     }
+    if args.algo == "chunked":
+        # The chunked path does different (far less) arithmetic, so it is never priced in the
+        # quadratic algorithm's FLOPs: its own count, and the HBM roofline that bounds it.
+        chunk = 256 if (w.d_qk // 2 + w.d_v <= 192 and w.d_v // 2 + w.d_qk <= 192) else 128
+        bh, n = w.batch * w.heads, w.seq
+        f_intra = float(bh) * n * chunk * (w.d_qk + w.d_v)          # causal-counted diagonal blocks
+        f_state = 4.0 * bh * n * w.d_qk * w.d_v                     # Y^T Z per chunk + X . S
+        flops_fwd = f_intra + f_state
+        flops_bwd = 3.0 * flops_fwd if w.backward else 0.0          # three products of the same shape
+        bytes_step = w.bytes_fwd + (w.bytes_bwd if w.backward else 0.0)
+        result["metric"] = result["metric"].replace("TFLOP/s (causal-counted)", "TFLOP/s (chunked algorithm's own FLOPs)")
+        result["value"] = round((flops_fwd + flops_bwd) / (ms_step * 1e-3) / 1e12, 2)
+        result["config"]["workload"] += f"; chunk-wise evaluation, {chunk}-row chunks"
+        result["config"]["flops_per_step"] = flops_fwd + flops_bwd
+        result["config"]["fwd_tflops"] = round(flops_fwd / (ms_fwd * 1e-3) / 1e12, 2)
+        result["config"]["bwd_tflops"] = None if ms_bwd is None else round(flops_bwd / (ms_bwd * 1e-3) / 1e12, 2)
+        result["config"]["pct_of_mfma_peak"] = round(100.0 * result["value"] / peak, 2)
+        gbs = bytes_step / (ms_step * 1e-3) / 1e9
+        result["roofline"] = {
+            "bound": "hbm",
+            "kernel": "chunk_state + chunk_scan + tri_xyt_z_fast (chunked) per product",
+            "achieved": round(gbs, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(gbs / HBM_PEAK_GBS, 4),
+            "traffic": None,
+            "algorithmic_bytes_per_step": bytes_step,
+        }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = _cpu_baseline(torch, w, args.cpu_seconds)
     print(json.dumps(result))
