@@ -146,24 +146,49 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(const ChunkStateParams
 
 // Exclusive running sum over the chunk axis of w[bh][chunk][E] (fp32), rounded to T.
 // reverse == 0: state[c] = sum_{c' < c} w[c'];  reverse != 0: state[c] = sum_{c' > c} w[c'].
+// One thread per pair of elements (many sequences have few (b, h) pairs, so parallelism has to
+// come from the state elements); the chunk loop is unrolled by 8 so that eight independent
+// loads are in flight per thread.
 template <typename T>
 __global__ __launch_bounds__(256) void chunk_scan_kernel(const float *w, T *state, int n_chunks, int64_t E,
-                                                        int64_t total4, int reverse) {
-    typedef float f32x4 __attribute__((ext_vector_type(4)));
-    typedef T t4 __attribute__((ext_vector_type(4)));
-    const int64_t i4 = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index of a group of 4 elements within [BH][E]
-    if (i4 >= total4) return;
-    const int64_t bh = (i4 * 4) / E, e = (i4 * 4) - bh * E;
+                                                        int64_t total2, int reverse) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    typedef T t2 __attribute__((ext_vector_type(2)));
+    const int64_t i2 = (int64_t)blockIdx.x * 256 + threadIdx.x;  // index of a pair of elements within [BH][E]
+    if (i2 >= total2) return;
+    const int64_t bh = (i2 * 2) / E, e = (i2 * 2) - bh * E;
     const float *wp = w + bh * n_chunks * E + e;
     T *sp = state + bh * n_chunks * E + e;
-    f32x4 run = {0.f, 0.f, 0.f, 0.f};
-    for (int k = 0; k < n_chunks; ++k) {
-        const int c = reverse ? n_chunks - 1 - k : k;
-        t4 o;
+    const int64_t step = reverse ? -E : E;
+    if (reverse) {
+        wp += (int64_t)(n_chunks - 1) * E;
+        sp += (int64_t)(n_chunks - 1) * E;
+    }
+    f32x2 run = {0.f, 0.f};
+    int k = 0;
+    for (; k + 8 <= n_chunks; k += 8) {
+        f32x2 v[8];
 #pragma unroll
-        for (int x = 0; x < 4; ++x) o[x] = static_cast<T>(run[x]);
-        *reinterpret_cast<t4 *>(sp + (int64_t)c * E) = o;
-        run += *reinterpret_cast<const f32x4 *>(wp + (int64_t)c * E);
+        for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const f32x2 *>(wp + u * step);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            t2 o;
+            o[0] = static_cast<T>(run[0]);
+            o[1] = static_cast<T>(run[1]);
+            *reinterpret_cast<t2 *>(sp + u * step) = o;
+            run += v[u];
+        }
+        wp += 8 * step;
+        sp += 8 * step;
+    }
+    for (; k < n_chunks; ++k) {
+        t2 o;
+        o[0] = static_cast<T>(run[0]);
+        o[1] = static_cast<T>(run[1]);
+        *reinterpret_cast<t2 *>(sp) = o;
+        run += *reinterpret_cast<const f32x2 *>(wp);
+        wp += step;
+        sp += step;
     }
 }
 
@@ -187,11 +212,11 @@ hipError_t launch_chunk_state(ChunkStateParams p, hipStream_t stream) {
 template <typename T>
 hipError_t launch_chunk_scan(const float *w, void *state, int64_t BH, int n_chunks, int64_t E, int reverse,
                              hipStream_t stream) {
-    const int64_t total4 = BH * E / 4;
-    const int64_t grid = (total4 + 255) / 256;
+    const int64_t total2 = BH * E / 2;
+    const int64_t grid = (total2 + 255) / 256;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     hipLaunchKernelGGL(chunk_scan_kernel<T>, dim3((unsigned)grid), dim3(256), 0, stream, w, static_cast<T *>(state),
-                       n_chunks, E, total4, reverse);
+                       n_chunks, E, total2, reverse);
     return hipGetLastError();
 }
 

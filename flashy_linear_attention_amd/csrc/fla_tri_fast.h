@@ -542,17 +542,22 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
         // accumulator register v of lane (l32, g) is column 16 g + v of its block; MFMA row
         // m = 8a + 4g' + b of the A operand lands in register 4a + b of the lanes with g = g'
         const int e_lane = 16 * ((l32 >> 2) & 1) + 4 * (l32 >> 3) + (l32 & 3);
+        // two column blocks of fragments in flight: the loads of block db+1 overlap the MFMAs of db
+        V8 sf[2][KC];
+        auto load_block = [&](int db, V8 (&dst)[KC]) {
+#pragma unroll
+            for (int kc = 0; kc < KC; ++kc)
+                dst[kc] = __builtin_bit_cast(
+                    V8, *reinterpret_cast<const u32x4 *>(st + (32 * db + e_lane) * DC + 16 * kc + 8 * g));
+        };
+        load_block(0, sf[0]);
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-            V8 sf[KC];
-#pragma unroll
-            for (int kc = 0; kc < KC; ++kc)
-                sf[kc] = __builtin_bit_cast(
-                    V8, *reinterpret_cast<const u32x4 *>(st + (32 * db + e_lane) * DC + 16 * kc + 8 * g));
+            if (db + 1 < DB) load_block(db + 1, sf[(db + 1) & 1]);
 #pragma unroll
             for (int kc = 0; kc < KC; ++kc)
 #pragma unroll
-                for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(sf[kc], xf[ib][kc], acc[ib][db]);
+                for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(sf[db & 1][kc], xf[ib][kc], acc[ib][db]);
         }
     }
 
