@@ -100,6 +100,7 @@ int run_tri(const View &x, const View &y, const View &z, const View &out, int64_
     p.dc = (int32_t)dc, p.dout = (int32_t)dout;
     p.upper = upper ? 1 : 0;
     p.n_tiles = 0;
+    p.single = 0;
     p.state = nullptr;
     p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout), p.vec_out = vec_ok(out, dout);
 #ifdef FLA_DBG_TIMING
@@ -149,6 +150,7 @@ int run_tri_chunked(const View &x, const View &y, const View &z, const View &out
     p.dc = (int32_t)dc, p.dout = (int32_t)dout;
     p.upper = upper ? 1 : 0;
     p.n_tiles = 0;
+    p.single = 0;
     p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout), p.vec_out = vec_ok(out, dout);
     p.state = nullptr;
 #ifdef FLA_DBG_TIMING

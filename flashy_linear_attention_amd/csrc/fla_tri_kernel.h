@@ -46,6 +46,7 @@ struct TriParams {
     int32_t dc, dout;  // actual widths (<= DC, DO of the instantiation)
     int32_t upper;     // 0: keep row >= col, 1: keep row <= col
     int32_t n_tiles;   // ceil(N / BM), filled by the launcher
+    int32_t single;    // fast path: one row tile per workgroup instead of a balanced pair (launcher's choice)
     int32_t vec_x, vec_y, vec_z;  // 1: rows are 16-byte aligned and width % 8 == 0
     int32_t vec_out;              // same for the output
     // Chunked evaluation (fast path only): when non-null, each workgroup computes only the
