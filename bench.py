@@ -8,6 +8,10 @@ One step = one forward (``linear_flash_wrapper_fwd``) plus one backward
 the C ABI of libfla_gfx950.so, inputs resident in HBM.  The default workload is
 the one the headline metric is quoted on: bf16, B=4 H=32 N=4096 D_qk=D_v=128.
 
+Before the W warm-up steps the same step runs untimed for ``--settle-seconds``
+(default 0.3 s) so that the shader clock has left its idle state; the timed
+region is exactly K steps between two synchronisations.
+
 Prints ONE JSON line.  ``value`` is causal-counted algorithmic TFLOP/s of the
 whole step, N^2 (4 D_qk + 3 D_v) per (b, h) (five products: S, dS, dV, dK, dQ
 in backward, two in forward).  ``roofline`` describes the one kernel every
@@ -42,8 +46,12 @@ MEASURED_TRAFFIC_BYTES = {"C3": 796e6}
 def _parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=300)
+    ap.add_argument("--warmup", type=int, default=100)
+    ap.add_argument("--settle-seconds", type=float, default=0.3,
+                    help="run untimed steps for this long before the warm-up steps: an idle MI355X sits at a "
+                         "95 MHz shader clock and needs about 50 ms of load to reach its sustained clock "
+                         "(a 10 ms idle gap is enough to drop it again)")
     ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU oracle timing")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target seconds of CPU work for the baseline")
@@ -147,6 +155,13 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
 
+    settle_steps = 0
+    t_settle = time.perf_counter()
+    while time.perf_counter() - t_settle < args.settle_seconds:
+        for _ in range(8):
+            step()
+        settle_steps += 8
+        torch.cuda.synchronize()
     for _ in range(args.warmup):
         step()
     ms_total = _time_region(torch, step, args.steps)
@@ -194,6 +209,7 @@ def main() -> int:
                         f"{'fwd+bwd' if w.backward else 'fwd'}, {dt_name}, B={w.batch} H={w.heads} N={w.seq} "
                         f"D_qk={w.d_qk} D_v={w.d_v}, q/k features {w.features}, v and dO randn, seed 0",
             "flops_per_step": flops_step,
+            "clock_settle_steps": settle_steps,
             "fwd_ms": round(ms_fwd, 4),
             "bwd_ms": None if ms_bwd is None else round(ms_bwd, 4),
             "fwd_tflops": round(w.flops_fwd / (ms_fwd * 1e-3) / 1e12, 2),

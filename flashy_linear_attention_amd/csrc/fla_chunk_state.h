@@ -68,26 +68,33 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(const ChunkStateParams
     const u32x4 ry = make_rsrc(Y, (uint32_t)((N - 1) * ys2 + p.dc * 2));
     const u32x4 rz = make_rsrc(Z, (uint32_t)((N - 1) * zs2 + p.dout * 2));
 
-    // whole chunk -> LDS (rows beyond N and columns beyond the true widths arrive as zeros)
-#pragma unroll
-    for (int t = 0; t < NTILE; ++t) {
-        const uint32_t yb = lds0 + t * STAGE + wave * 1024, zb = yb + Y_BYTES;
-        const int row0 = r0 + t * BN;
-#pragma unroll
-        for (int u = 0; u < NIY; ++u) {
-            const int row = (u * 4 + wave) * (1024 / RY) + lane / CY;
-            const int c = (lane % CY) ^ swizzle_y<CY>(row);
-            const uint32_t off = (uint32_t)(row * ys2 + c * 16) + (c * 8 < p.dc ? 0u : kOobOffset);
-            dma_16B_per_lane(ry, yb + u * 4096, off, row0 * ys2);
-        }
-#pragma unroll
-        for (int u = 0; u < NIZ; ++u) {
-            const int row = (u * 4 + wave) * (1024 / RZ) + lane / CZ;
-            const int c = (lane % CZ) ^ swizzle_z<CZ>(row);
-            const uint32_t off = (uint32_t)(row * zs2 + c * 16) + (c * 8 < p.dout ? 0u : kOobOffset);
-            dma_16B_per_lane(rz, zb + u * 4096, off, row0 * zs2);
-        }
+    // whole chunk -> LDS (rows beyond N and columns beyond the true widths arrive as zeros);
+    // same lane -> chunk assignment as the main kernel's tile loads
+    constexpr int YSTEP = 4 * (1024 / RY), ZSTEP = 4 * (1024 / RZ);
+    uint32_t ydma, zdma;
+    {
+        const int row = wave * (1024 / RY) + lane / CY;
+        const int c = (lane % CY) ^ swizzle_y<CY>(row);
+        ydma = (uint32_t)(row * ys2 + c * 16) + (c * 8 < p.dc ? 0u : kOobOffset);
     }
+    {
+        const int row = wave * (1024 / RZ) + lane / CZ;
+        const int c = (lane % CZ) ^ swizzle_z<CZ>(row);
+        zdma = (uint32_t)(row * zs2 + c * 16) + (c * 8 < p.dout ? 0u : kOobOffset);
+    }
+    const uint32_t lds_wave = lds0 + wave * 1024;
+    static_for<0, NTILE>([&](auto tt) {
+        constexpr int t = decltype(tt)::value;
+        const int row0 = r0 + t * BN;
+        static_for<0, NIY>([&](auto u) {
+            constexpr int U = decltype(u)::value;
+            dma_16B_per_lane<t * STAGE + U * 4096>(ry, lds_wave, ydma, (uint32_t)((row0 + U * YSTEP) * ys2));
+        });
+        static_for<0, NIZ>([&](auto u) {
+            constexpr int U = decltype(u)::value;
+            dma_16B_per_lane<t * STAGE + Y_BYTES + U * 4096>(rz, lds_wave, zdma, (uint32_t)((row0 + U * ZSTEP) * zs2));
+        });
+    });
     wait_vm<0>();
     __builtin_amdgcn_s_barrier();
 

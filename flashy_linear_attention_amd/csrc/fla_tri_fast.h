@@ -42,14 +42,25 @@ typedef short s16x8 __attribute__((ext_vector_type(8)));
 // Issued through inline assembly so that the compiler's wait-count insertion does not
 // serialise later LDS reads of *other* ring slots against it; completion is awaited
 // explicitly (wait_dma) before the barrier that publishes the slot.
-__device__ __forceinline__ void dma_16B_per_lane(u32x4 rsrc, uint32_t lds_addr, uint32_t voffset, uint32_t soffset) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+// The LDS address is lds_base + LDS_IMM with LDS_IMM a compile-time constant, added while M0 is
+// written: the loads of one tile then need a single scalar base between them.
+template <int LDS_IMM>
+__device__ __forceinline__ void dma_16B_per_lane(u32x4 rsrc, uint32_t lds_base, uint32_t voffset, uint32_t soffset) {
+    asm volatile("s_add_u32 m0, %0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
-                 : "s"(lds_addr), "v"(voffset), "s"(rsrc), "s"(soffset)
-                 : "memory", "m0");
+                 : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset), "n"(LDS_IMM)
+                 : "memory", "m0", "scc");
 }
 // s_waitcnt vmcnt(N) only (expcnt and lgkmcnt fields left at their maxima): returns once at
 // most N of this wave's buffer loads, the most recently issued ones, are still in flight.
+// f(integral_constant<int, I>) for I = BEGIN .. END-1, unrolled at compile time
+template <int BEGIN, int END, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (BEGIN < END) {
+        f(std::integral_constant<int, BEGIN>{});
+        static_for<BEGIN + 1, END>(f);
+    }
+}
 template <int N>
 __device__ __forceinline__ void wait_vm() {
     static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
@@ -208,29 +219,38 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
     if (chunked) n_full = 0;  // everything off the diagonal block arrives through the state
     const int n_seq = n_full + n_diag;
 
-    // ---- HBM -> LDS: per-lane source offsets (constant over tiles)
-    uint32_t ydma[NIY], zdma[NIZ];
-#pragma unroll
-    for (int u = 0; u < NIY; ++u) {
-        const int row = (u * 4 + wave) * (1024 / RY) + lane / CY;
+    // ---- HBM -> LDS: per-lane source offsets (constant over tiles).  Load u of a wave covers
+    // rows u * YSTEP + wave * (1024 / RY) + lane / CY of the tile; YSTEP is a multiple of the
+    // swizzle period, so the lane's chunk is the same for every u and the row advance goes into
+    // the scalar offset: one address register per operand, no vector work per load.
+    constexpr int YSTEP = 4 * (1024 / RY), ZSTEP = 4 * (1024 / RZ);
+    static_assert(NIY == 1 || YSTEP % 8 == 0, "Y swizzle must not depend on the load index");
+    static_assert(NIZ == 1 || ZSTEP % 4 == 0, "Z swizzle must not depend on the load index");
+    uint32_t ydma, zdma;
+    {
+        const int row = wave * (1024 / RY) + lane / CY;
         const int c = (lane % CY) ^ swizzle_y<CY>(row);
-        ydma[u] = (uint32_t)(row * ys2 + c * 16) + (c * 8 < p.dc ? 0u : kOobOffset);
+        ydma = (uint32_t)(row * ys2 + c * 16) + (c * 8 < p.dc ? 0u : kOobOffset);
     }
-#pragma unroll
-    for (int u = 0; u < NIZ; ++u) {
-        const int row = (u * 4 + wave) * (1024 / RZ) + lane / CZ;
+    {
+        const int row = wave * (1024 / RZ) + lane / CZ;
         const int c = (lane % CZ) ^ swizzle_z<CZ>(row);
-        zdma[u] = (uint32_t)(row * zs2 + c * 16) + (c * 8 < p.dout ? 0u : kOobOffset);
+        zdma = (uint32_t)(row * zs2 + c * 16) + (c * 8 < p.dout ? 0u : kOobOffset);
     }
-    // tile q of the sequence -> ring slot q % 3, tracked incrementally
+    const uint32_t lds_wave = lds0 + wave * 1024;
+    // tile q of the sequence -> ring slot q % NBUF, tracked incrementally by the caller
     auto issue_tile = [&](int q, int slot_off) {
         if (q < n_seq) {
             const int row0 = q < n_full ? full_row0 + q * BN : i0 + (q - n_full) * BN;
-            const uint32_t yb = lds0 + slot_off + wave * 1024, zb = yb + Y_BYTES;
-#pragma unroll
-            for (int u = 0; u < NIY; ++u) dma_16B_per_lane(ry, yb + u * 4096, ydma[u], row0 * ys2);
-#pragma unroll
-            for (int u = 0; u < NIZ; ++u) dma_16B_per_lane(rz, zb + u * 4096, zdma[u], row0 * zs2);
+            const uint32_t yb = lds_wave + slot_off;
+            static_for<0, NIY>([&](auto u) {
+                constexpr int U = decltype(u)::value;
+                dma_16B_per_lane<U * 4096>(ry, yb, ydma, (uint32_t)((row0 + U * YSTEP) * ys2));
+            });
+            static_for<0, NIZ>([&](auto u) {
+                constexpr int U = decltype(u)::value;
+                dma_16B_per_lane<Y_BYTES + U * 4096>(rz, yb, zdma, (uint32_t)((row0 + U * ZSTEP) * zs2));
+            });
         }
     };
     auto next_slot = [](int off) { return off + STAGE == Cfg::NBUF * STAGE ? 0 : off + STAGE; };
@@ -368,7 +388,8 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
         };
         // phase 2: Out += P_prev Z_prev, interleaved with the Y fragment reads of the next sub-tile
         // and the rounding of S into `pcur`
-        auto phase2 = [&](auto with_pv, V8 (&pprev)[NIB][2], V8 (&pcur)[NIB][2], const int (&ya)[YQ], int ysub) {
+        auto phase2 = [&](auto with_pv, V8 (&pprev)[NIB][2], V8 (&pcur)[NIB][2], const int (&ya)[YQ], int ysub,
+                          auto &&after_first_group) {
             constexpr int NPK = NIB * 8;  // packed pairs that make up P of one sub-tile
             u32x4 pk[NIB][2];
 #pragma unroll
@@ -396,6 +417,7 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
                         pk[ib][t][w] = round_pack_pinned<T>(s[ib][8 * t + 2 * w], s[ib][8 * t + 2 * w + 1]);
                     }
                 }
+                if (f == 0) after_first_group();
                 __builtin_amdgcn_sched_barrier(0);
             }
 #pragma unroll
@@ -411,7 +433,7 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
             slot_addrs(next_off, ya_next, unused_z);
             // first sub-tile: Z of the previous tile's second sub-tile, then Y of this tile's second
             phase1(std::integral_constant<bool, !kFirst>{}, za_prev, 1);
-            phase2(std::integral_constant<bool, !kFirst>{}, pfb, pfa, ya_cur, 1);
+            phase2(std::integral_constant<bool, !kFirst>{}, pfb, pfa, ya_cur, 1, [] {});
             // second sub-tile
             phase1(std::true_type{}, za_cur, 0);
 #ifndef FLA_DBG_NO_WAIT
@@ -420,10 +442,12 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
 #ifndef FLA_DBG_NO_BARRIER
             __builtin_amdgcn_s_barrier();  // tile q+1 has landed; nobody reads tile q-1 any more
 #endif
-#ifndef FLA_DBG_NO_DMA
+#ifdef FLA_DMA_LATE
+            phase2(std::true_type{}, pfa, pfb, ya_next, 0, [&] { issue_tile(q + Cfg::NBUF - 1, issue_off); });
+#else
             issue_tile(q + Cfg::NBUF - 1, issue_off);
+            phase2(std::true_type{}, pfa, pfb, ya_next, 0, [] {});
 #endif
-            phase2(std::true_type{}, pfa, pfb, ya_next, 0);
             advance();
             ++q;
         };
