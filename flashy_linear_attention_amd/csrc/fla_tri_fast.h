@@ -468,6 +468,39 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
         }
     }
 
+    // (placed before the diagonal block: its global loads overlap the wait for the block's tiles)
+    // ---- chunked evaluation: Out_tile += X_tile . S with S^T[e][d] read straight from global
+    // memory as A operand (row = output column as permuted in the accumulators, k = d) and the
+    // resident X fragments as B operand.
+    if (chunked && (upper ? tile + 1 < p.n_tiles : tile > 0)) {
+        const T *st = static_cast<const T *>(p.state) + ((int64_t)bh * p.n_tiles + tile) * (DO * DC);
+        // accumulator register v of lane (l32, g) is column 16 g + v of its block; MFMA row
+        // m = 8a + 4g' + b of the A operand lands in register 4a + b of the lanes with g = g'
+        const int e_lane = 16 * ((l32 >> 2) & 1) + 4 * (l32 >> 3) + (l32 & 3);
+        // two column blocks of fragments in flight: the loads of block db+1 overlap the MFMAs of db
+        V8 sf[2][KC];
+        // one lane offset for all fragments: column block and k chunk go into the scalar offset
+        const __amdgpu_buffer_rsrc_t rs =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(st), 0, DO * DC * 2, 0x00020000);
+        uint32_t st_lane = (uint32_t)((e_lane * DC + 8 * g) * 2);
+        asm volatile("" : "+v"(st_lane));  // keeps derived addresses from being hoisted out of the pass loop
+        auto load_block = [&](int db, V8 (&dst)[KC]) {
+#pragma unroll
+            for (int kc = 0; kc < KC; ++kc)
+                dst[kc] = __builtin_bit_cast(
+                    V8, __builtin_amdgcn_raw_buffer_load_b128(rs, st_lane, 32 * db * DC * 2 + 32 * kc, 0));
+        };
+        load_block(0, sf[0]);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            if (db + 1 < DB) load_block(db + 1, sf[(db + 1) & 1]);
+#pragma unroll
+            for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+                for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(sf[db & 1][kc], xf[ib][kc], acc[ib][db]);
+        }
+    }
+
     FLA_STAMP(2);
     // ================= the diagonal block =================
     // Its tiles (BM / BN of them, never more than the ring holds) are all made resident first;
@@ -558,33 +591,6 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
 #endif
         FLA_STAMP(6);
         __builtin_amdgcn_s_barrier();  // all LDS reads of the walk are done: the ring can be reused
-    }
-
-    // ---- chunked evaluation: Out_tile += X_tile . S with S^T[e][d] read straight from global
-    // memory as A operand (row = output column as permuted in the accumulators, k = d) and the
-    // resident X fragments as B operand.
-    if (chunked && (upper ? tile + 1 < p.n_tiles : tile > 0)) {
-        const T *st = static_cast<const T *>(p.state) + ((int64_t)bh * p.n_tiles + tile) * (DO * DC);
-        // accumulator register v of lane (l32, g) is column 16 g + v of its block; MFMA row
-        // m = 8a + 4g' + b of the A operand lands in register 4a + b of the lanes with g = g'
-        const int e_lane = 16 * ((l32 >> 2) & 1) + 4 * (l32 >> 3) + (l32 & 3);
-        // two column blocks of fragments in flight: the loads of block db+1 overlap the MFMAs of db
-        V8 sf[2][KC];
-        auto load_block = [&](int db, V8 (&dst)[KC]) {
-#pragma unroll
-            for (int kc = 0; kc < KC; ++kc)
-                dst[kc] = __builtin_bit_cast(
-                    V8, *reinterpret_cast<const u32x4 *>(st + (32 * db + e_lane) * DC + 16 * kc + 8 * g));
-        };
-        load_block(0, sf[0]);
-#pragma unroll
-        for (int db = 0; db < DB; ++db) {
-            if (db + 1 < DB) load_block(db + 1, sf[(db + 1) & 1]);
-#pragma unroll
-            for (int kc = 0; kc < KC; ++kc)
-#pragma unroll
-                for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(sf[db & 1][kc], xf[ib][kc], acc[ib][db]);
-        }
     }
 
     FLA_STAMP(3);
