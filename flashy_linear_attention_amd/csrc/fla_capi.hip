@@ -154,7 +154,10 @@ int run_tri_chunked(const View &x, const View &y, const View &z, const View &out
     p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout), p.vec_out = vec_ok(out, dout);
     p.state = nullptr;
 #ifdef FLA_DBG_TIMING
-    p.dbg = nullptr;
+    {
+        const char *e = getenv("FLA_DBG_TIMING_PTR");
+        p.dbg = e ? reinterpret_cast<unsigned long long *>(strtoull(e, nullptr, 16)) : nullptr;
+    }
 #endif
     if (rows == 0 || N <= rows || !fla::fast_path_ok(p))
         return run_tri(x, y, z, out, B, H, N, dc, dout, upper, dtype, stream);

@@ -110,6 +110,13 @@ struct FastConfig {
     static constexpr int STAGE_BYTES = Y_BYTES + Z_BYTES;
     static constexpr int SMEM_BYTES = NBUF * STAGE_BYTES;
     static constexpr bool kSupported = SMEM_BYTES <= 160 * 1024;
+    // chunked evaluation: the running state S^T, [DO rows][DC] 16-bit, sits behind the ring in
+    // whole 64-row units of the Y tile layout when the 160 KiB allow it
+    static constexpr int STATE_BYTES = ((DO + 63) / 64) * Y_BYTES;
+    static constexpr bool kStateInLds = SMEM_BYTES + STATE_BYTES <= 160 * 1024;
+    // Narrow shapes need half the LDS and about half the registers: holding the kernel to 256
+    // registers lets two workgroups share a CU, which hides each other's prologue and epilogue.
+    static constexpr int kMinWavesPerSimd = (DC <= 64 && DO <= 64) ? 2 : 1;
     // wave-level 1 KiB DMA instructions per tile and wave
     static constexpr int NIY = Y_BYTES / 4096, NIZ = Z_BYTES / 4096;
     static constexpr int NT = NIY + NIZ;  // buffer loads per wave and tile
@@ -132,7 +139,7 @@ __device__ __forceinline__ int swizzle_z(int row) {
 }
 
 template <typename T, int DC, int DO>
-__global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) {
+__global__ __launch_bounds__(256, (FastConfig<DC, DO>::kMinWavesPerSimd)) void tri_xyt_z_fast_kernel(const TriParams p) {
     // The body is compiled in the device pass only: hipcc's host pass silently
     // drops the launch stub of a kernel template whose body calls the LDS-DMA
     // builtin from inside a lambda, and the host needs nothing but the stub.
@@ -336,15 +343,41 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
 
     // ring state: byte offsets of the slots of tile q-1, q, q+1 and of the next tile to issue
     int prev_off = (Cfg::NBUF - 1) * STAGE, cur_off = 0, next_off = STAGE, issue_off = STAGE;
-    if constexpr (Cfg::NBUF == 4) {
-        issue_tile(1, STAGE);
-        issue_off = 2 * STAGE;
+    const bool has_state = chunked && (upper ? tile + 1 < p.n_tiles : tile > 0);
+    const T *st = has_state ? static_cast<const T *>(p.state) + ((int64_t)bh * p.n_tiles + tile) * (DO * DC) : nullptr;
+    if (chunked) {
+        // everything this workgroup will ever read is requested at once: the rest of the diagonal
+        // block's tiles and the running state (the kernel is latency-bound in this mode)
+        static_for<1, BM / BN>([&](auto qq) { issue_tile(decltype(qq)::value, decltype(qq)::value * STAGE); });
+        if constexpr (Cfg::kStateInLds) {
+            if (has_state) {
+                const u32x4 rs = make_rsrc(st, DO * DC * 2);
+                const int row = wave * (1024 / RY) + lane / CY;
+                const uint32_t sdma = (uint32_t)(row * RY + (((lane % CY) ^ swizzle_y<CY>(row)) << 4));
+                static_for<0, Cfg::STATE_BYTES / Y_BYTES>([&](auto uu) {
+                    constexpr int UNIT = decltype(uu)::value;
+                    static_for<0, NIY>([&](auto u) {
+                        constexpr int U = decltype(u)::value;
+                        dma_16B_per_lane<Cfg::SMEM_BYTES + UNIT * Y_BYTES + U * 4096>(
+                            rs, lds_wave, sdma, (uint32_t)((UNIT * 64 + U * YSTEP) * RY));
+                    });
+                });
+            }
+        }
+        wait_vm<0>();
+        __builtin_amdgcn_s_barrier();
+        FLA_STAMP(1);
+    } else {
+        if constexpr (Cfg::NBUF == 4) {
+            issue_tile(1, STAGE);
+            issue_off = 2 * STAGE;
+        }
+        wait_tile(0);
+        __builtin_amdgcn_s_barrier();  // tile 0 (and the X fragments) have landed
+        FLA_STAMP(1);
+        issue_tile(Cfg::NBUF - 2, issue_off);
+        issue_off = next_slot(issue_off);
     }
-    wait_tile(0);
-    __builtin_amdgcn_s_barrier();  // tile 0 (and the X fragments) have landed
-    FLA_STAMP(1);
-    issue_tile(Cfg::NBUF - 2, issue_off);
-    issue_off = next_slot(issue_off);
     // from here on: tiles up to q + NBUF - 2 are issued while tile q is consumed
     auto advance = [&]() {
         prev_off = cur_off;
@@ -468,36 +501,60 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
         }
     }
 
-    // (placed before the diagonal block: its global loads overlap the wait for the block's tiles)
-    // ---- chunked evaluation: Out_tile += X_tile . S with S^T[e][d] read straight from global
-    // memory as A operand (row = output column as permuted in the accumulators, k = d) and the
-    // resident X fragments as B operand.
-    if (chunked && (upper ? tile + 1 < p.n_tiles : tile > 0)) {
-        const T *st = static_cast<const T *>(p.state) + ((int64_t)bh * p.n_tiles + tile) * (DO * DC);
+    // ---- chunked evaluation: Out_tile += X_tile . S with S^T[e][d] as A operand (row = output
+    // column as permuted in the accumulators, k = d) and the resident X fragments as B operand.
+    if (has_state) {
         // accumulator register v of lane (l32, g) is column 16 g + v of its block; MFMA row
         // m = 8a + 4g' + b of the A operand lands in register 4a + b of the lanes with g = g'
         const int e_lane = 16 * ((l32 >> 2) & 1) + 4 * (l32 >> 3) + (l32 & 3);
         // two column blocks of fragments in flight: the loads of block db+1 overlap the MFMAs of db
         V8 sf[2][KC];
-        // one lane offset for all fragments: column block and k chunk go into the scalar offset
-        const __amdgpu_buffer_rsrc_t rs =
-            __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(st), 0, DO * DC * 2, 0x00020000);
-        uint32_t st_lane = (uint32_t)((e_lane * DC + 8 * g) * 2);
-        asm volatile("" : "+v"(st_lane));  // keeps derived addresses from being hoisted out of the pass loop
-        auto load_block = [&](int db, V8 (&dst)[KC]) {
+        if constexpr (Cfg::kStateInLds) {
+            // from LDS, in the Y tile layout (row e, chunk index XOR swizzle(e))
+            int sl[YQ];
+            const int sw = swizzle_y<CY>(e_lane);
 #pragma unroll
-            for (int kc = 0; kc < KC; ++kc)
-                dst[kc] = __builtin_bit_cast(
-                    V8, __builtin_amdgcn_raw_buffer_load_b128(rs, st_lane, 32 * db * DC * 2 + 32 * kc, 0));
-        };
-        load_block(0, sf[0]);
+            for (int j = 0; j < YQ; ++j) {
+                sl[j] = Cfg::SMEM_BYTES + e_lane * RY + (((2 * j + g) ^ sw) << 4);
+                asm volatile("" : "+v"(sl[j]));  // computed here, not once per kernel
+            }
+            auto load_block = [&](int db, V8 (&dst)[KC]) {
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-            if (db + 1 < DB) load_block(db + 1, sf[(db + 1) & 1]);
+                for (int kc = 0; kc < KC; ++kc)
+                    dst[kc] = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4 *>(
+                                                         smem + sl[kc % YQ] + (db * 32 * RY + (kc / YQ) * (YQ * 32))));
+            };
+            load_block(0, sf[0]);
 #pragma unroll
-            for (int kc = 0; kc < KC; ++kc)
+            for (int db = 0; db < DB; ++db) {
+                if (db + 1 < DB) load_block(db + 1, sf[(db + 1) & 1]);
 #pragma unroll
-                for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(sf[db & 1][kc], xf[ib][kc], acc[ib][db]);
+                for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+                    for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(sf[db & 1][kc], xf[ib][kc], acc[ib][db]);
+            }
+        } else {
+            // straight from global memory: one lane offset for all fragments, column block and
+            // k chunk go into the scalar offset
+            const __amdgpu_buffer_rsrc_t rs =
+                __builtin_amdgcn_make_buffer_rsrc(const_cast<T *>(st), 0, DO * DC * 2, 0x00020000);
+            uint32_t st_lane = (uint32_t)((e_lane * DC + 8 * g) * 2);
+            asm volatile("" : "+v"(st_lane));  // keeps derived addresses from being hoisted out of the pass loop
+            auto load_block = [&](int db, V8 (&dst)[KC]) {
+#pragma unroll
+                for (int kc = 0; kc < KC; ++kc)
+                    dst[kc] = __builtin_bit_cast(
+                        V8, __builtin_amdgcn_raw_buffer_load_b128(rs, st_lane, 32 * db * DC * 2 + 32 * kc, 0));
+            };
+            load_block(0, sf[0]);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                if (db + 1 < DB) load_block(db + 1, sf[(db + 1) & 1]);
+#pragma unroll
+                for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+                    for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(sf[db & 1][kc], xf[ib][kc], acc[ib][db]);
+            }
         }
     }
 
@@ -509,9 +566,11 @@ __global__ __launch_bounds__(256) void tri_xyt_z_fast_kernel(const TriParams p) 
     {
         static_assert(BM / BN <= Cfg::NBUF, "the diagonal block must fit in the LDS ring");
         if (n_full > 0) __builtin_amdgcn_s_barrier();  // every wave is done with the last full tile
-        issue_tile(q + Cfg::NBUF - 1, issue_off);      // the one tile not yet requested (if any)
-        wait_vm<0>();
-        __builtin_amdgcn_s_barrier();
+        if (!chunked) {
+            issue_tile(q + Cfg::NBUF - 1, issue_off);  // the one tile not yet requested (if any)
+            wait_vm<0>();
+            __builtin_amdgcn_s_barrier();
+        }
         FLA_STAMP(5);
 
         constexpr int RING = Cfg::NBUF * STAGE;
@@ -658,10 +717,11 @@ hipError_t launch_tri_fast(TriParams p, hipStream_t stream) {
         const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * ((p.state || p.single) ? p.n_tiles : (p.n_tiles + 1) / 2);
         if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
         auto kern = tri_xyt_z_fast_kernel<T, DC, DO>;
+        const int smem = Cfg::SMEM_BYTES + (p.state && Cfg::kStateInLds ? Cfg::STATE_BYTES : 0);
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM_BYTES);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), Cfg::SMEM_BYTES, stream, p);
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
         return hipGetLastError();
     }
 }
