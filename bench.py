@@ -55,9 +55,11 @@ def _parse():
     ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU oracle timing")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target seconds of CPU work for the baseline")
-    ap.add_argument("--algo", default="quadratic", choices=["quadratic", "chunked"],
+    ap.add_argument("--algo", default="quadratic", choices=["quadratic", "chunked", "normalised"],
                     help="quadratic: the tiled O(N^2 D) kernels the headline metric is defined on (default); "
-                         "chunked: the O(N) chunk-state path, reported with its own FLOP count and an HBM roofline")
+                         "chunked: the O(N) chunk-state path, reported with its own FLOP count and an HBM roofline; "
+                         "normalised: the quadratic kernels plus the fused normaliser (out / (q . cumsum(k) + eps)), "
+                         "with the normaliser's own time, bytes and the PyTorch recipe's time beside it")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain device copy of 256 MiB (a known-size reference for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -142,6 +144,20 @@ def main() -> int:
         from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
 
         fwd, bwd = linear_attention_chunked_fwd, linear_attention_chunked_bwd
+    plain_fwd, plain_bwd = fwd, bwd
+    if args.algo == "normalised":
+        from flashy_linear_attention_amd.normalised import (
+            linear_attention_normalised_bwd,
+            linear_attention_normalised_fwd,
+        )
+
+        norm_out, norm_denom = linear_attention_normalised_fwd(q, k, v, 1e-5)
+
+        def fwd(q_, k_, v_):
+            return linear_attention_normalised_fwd(q_, k_, v_, 1e-5)
+
+        def bwd(do_, q_, k_, v_):
+            return linear_attention_normalised_bwd(do_, q_, k_, v_, norm_out, norm_denom)
 
     def step():
         fwd(q, k, v)
@@ -256,6 +272,48 @@ def main() -> int:
             "frac": round(gbs / HBM_PEAK_GBS, 4),
             "traffic": None,
             "algorithmic_bytes_per_step": bytes_step,
+        }
+    if args.algo == "normalised":
+        # The product kernels are unchanged; what is new are the memory-bound passes around them.
+        # Their time is the difference to the plain step in this same run, their algorithmic bytes:
+        # forward reads q, k, O and writes out (+ n); backward reads g, out (pre-pass, writes dO) and
+        # q, k, dq, dk (post-pass, writes dq, dk); 2 bytes per element, fp32 vectors of length N aside.
+        def plain_step():
+            plain_fwd(q, k, v)
+            if w.backward:
+                plain_bwd(do, q, k, v)
+
+        ms_plain = _time_region(torch, plain_step, args.steps) / args.steps
+        e = float(w.batch * w.heads * w.seq)
+        nbytes = 2.0 * e * (2 * w.d_qk + 2 * w.d_v)
+        if w.backward:
+            nbytes += 2.0 * e * (3 * w.d_v + 6 * w.d_qk)
+        extra_ms = ms_step - ms_plain
+
+        def recipe_step():
+            qa, ka, va = (t.detach().requires_grad_(w.backward) for t in (q, k, v))
+            op = LinearAttentionSmallVHD if w.small_v else LinearAttention
+            num = op.apply(qa, ka, va)
+            den = (qa * ka.cumsum(-2)).sum(dim=-1, keepdim=True) + 1e-5
+            out = num / den
+            if w.backward:
+                out.backward(do)
+
+        from flashy_linear_attention_amd import LinearAttention, LinearAttentionSmallVHD
+
+        for _ in range(10):
+            recipe_step()
+        ms_recipe = _time_region(torch, recipe_step, max(10, args.steps // 5)) / max(10, args.steps // 5)
+        result["metric"] = result["metric"].replace("causal linear attention", "normalised causal linear attention")
+        result["config"]["workload"] += "; fused normaliser out / (q . cumsum(k) + 1e-5)"
+        result["config"]["normaliser"] = {
+            "plain_step_ms": round(ms_plain, 4),
+            "extra_ms": round(extra_ms, 4),
+            "algorithmic_bytes": nbytes,
+            "gbps": round(nbytes / (extra_ms * 1e-3) / 1e9, 1) if extra_ms > 0 else None,
+            "frac_of_hbm_peak": round(nbytes / (extra_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4) if extra_ms > 0 else None,
+            "pytorch_recipe_step_ms": round(ms_recipe, 4),
+            "speedup_vs_pytorch_recipe": round(ms_recipe / ms_step, 2),
         }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = _cpu_baseline(torch, w, args.cpu_seconds)

@@ -4,5 +4,6 @@ the Python surface of ``flashlinear`` (flashlinear/__init__.py:1-2)."""
 from .chunked import LinearAttentionChunked
 from .linear_attn import LinearAttention
 from .linear_attn_smallv_hd import LinearAttentionSmallVHD
+from .normalised import LinearAttentionNormalised
 
-__all__ = ["LinearAttention", "LinearAttentionSmallVHD", "LinearAttentionChunked"]
+__all__ = ["LinearAttention", "LinearAttentionSmallVHD", "LinearAttentionChunked", "LinearAttentionNormalised"]

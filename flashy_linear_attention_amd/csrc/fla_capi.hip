@@ -7,6 +7,7 @@
 #include <stdlib.h>
 
 #include "fla_dispatch.h"
+#include "fla_norm.h"
 
 namespace {
 
@@ -203,6 +204,113 @@ int backward(const View &go, const View &q, const View &k, const View &v, const 
     return run_tri(v, go, q, dk, B, H, N, dvw, dqk, 1, dtype, stream);
 }
 
+// ---- normalised linear attention: out = tril(Q K^T) V / (q . cumsum(k) + eps)
+
+struct NormLayout {
+    int lpr;
+    int64_t chunks, sums_bytes, do_bytes, dn_bytes;
+};
+
+NormLayout norm_layout(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
+    NormLayout l;
+    l.lpr = fla::norm_lanes_per_row((int)(dqk > dv ? dqk : dv));
+    const int64_t rows = fla::norm_chunk_rows(l.lpr);
+    l.chunks = (N + rows - 1) / rows;
+    l.sums_bytes = B * H * l.chunks * (l.lpr * 8) * 4;
+    l.do_bytes = (B * H * N * dv * 2 + 15) / 16 * 16;
+    l.dn_bytes = (B * H * N * 4 + 15) / 16 * 16;
+    return l;
+}
+
+void norm_common(fla::NormParams &p, const View &q, const View &k, int64_t B, int64_t H, int64_t N, int64_t dqk,
+                 int64_t dv, const NormLayout &l) {
+    p = fla::NormParams{};
+    p.q = q.ptr, p.k = k.ptr;
+    p.qs_b = q.strides[0], p.qs_h = q.strides[1], p.qs_n = q.strides[2];
+    p.ks_b = k.strides[0], p.ks_h = k.strides[1], p.ks_n = k.strides[2];
+    p.H = (int32_t)H, p.N = (int32_t)N, p.BH = (int32_t)(B * H), p.dqk = (int32_t)dqk, p.dv = (int32_t)dv;
+    p.n_chunks = (int32_t)l.chunks;
+    p.vec_q = vec_ok(q, dqk), p.vec_k = vec_ok(k, dqk);
+}
+
+hipError_t norm_launch(int which, int dtype, int lpr, const fla::NormParams &p, void *stream) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return dtype == FLA_DTYPE_BF16 ? fla::launch_norm<__bf16>(which, lpr, p, s)
+                                   : fla::launch_norm<_Float16>(which, lpr, p, s);
+}
+
+int check_norm_args(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv, int dtype) {
+    if (int rc = check_common(B, H, N, dtype)) return rc;
+    if (dqk < 1 || dqk > 256) return FLA_ERR_HEAD_DIM;
+    if (dv < 1 || dv > 256) return FLA_ERR_V_HEAD_DIM;
+    // the grid's second dimension is the (batch, head) index
+    if (B * H > 65535) return FLA_ERR_SHAPE;
+    return FLA_OK;
+}
+
+int normalised_forward(const View &q, const View &k, const View &v, const View &o, float *denom, int64_t B, int64_t H,
+                       int64_t N, int64_t dqk, int64_t dv, float eps, int dtype, void *workspace,
+                       int64_t workspace_bytes, void *stream) {
+    const View all[] = {q, k, v, o};
+    for (const View &t : all)
+        if (int rc = check_view(t)) return rc;
+    if (!denom) return FLA_ERR_NULL_POINTER;
+    if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    const NormLayout l = norm_layout(B, H, N, dqk, dv);
+    if (l.chunks > 1 && (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < l.sums_bytes))
+        return FLA_ERR_WORKSPACE;
+    if (int rc = run_tri(q, k, v, o, B, H, N, dqk, dv, 0, dtype, stream)) return rc;
+    fla::NormParams p;
+    norm_common(p, q, k, B, H, N, dqk, dv, l);
+    p.a = o.ptr, p.out = const_cast<void *>(o.ptr);  // normalised in place
+    p.as_b = p.os_b = o.strides[0], p.as_h = p.os_h = o.strides[1], p.as_n = p.os_n = o.strides[2];
+    p.vec_a = p.vec_out = vec_ok(o, dv);
+    p.denom = denom;
+    p.ksum = static_cast<float *>(workspace);
+    p.eps = eps;
+    return norm_launch(0, dtype, l.lpr, p, stream) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+}
+
+int normalised_backward(const View &go, const View &q, const View &k, const View &v, const View &o,
+                        const float *denom, const View &dq, const View &dk, const View &dvv, int64_t B, int64_t H,
+                        int64_t N, int64_t dqk, int64_t dv, int dtype, void *workspace, int64_t workspace_bytes,
+                        void *stream) {
+    const View all[] = {go, q, k, v, o, dq, dk, dvv};
+    for (const View &t : all)
+        if (int rc = check_view(t)) return rc;
+    if (!denom) return FLA_ERR_NULL_POINTER;
+    if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    const NormLayout l = norm_layout(B, H, N, dqk, dv);
+    if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 ||
+        workspace_bytes < l.do_bytes + l.dn_bytes + 2 * l.sums_bytes)
+        return FLA_ERR_WORKSPACE;
+    char *ws = static_cast<char *>(workspace);
+    void *dO = ws;
+    float *dn = reinterpret_cast<float *>(ws + l.do_bytes);
+    float *ksum = reinterpret_cast<float *>(ws + l.do_bytes + l.dn_bytes);
+    float *wsum = reinterpret_cast<float *>(ws + l.do_bytes + l.dn_bytes + l.sums_bytes);
+    const int64_t do_strides[4] = {H * N * dv, N * dv, dv, 1};
+    const View dOv{dO, do_strides};
+
+    fla::NormParams p;
+    norm_common(p, q, k, B, H, N, dqk, dv, l);
+    p.denom = const_cast<float *>(denom), p.dn = dn, p.ksum = ksum, p.wsum = wsum;
+    // dO = g / n, dn = -(g . out) / n
+    p.a = go.ptr, p.as_b = go.strides[0], p.as_h = go.strides[1], p.as_n = go.strides[2], p.vec_a = vec_ok(go, dv);
+    p.b = o.ptr, p.bs_b = o.strides[0], p.bs_h = o.strides[1], p.bs_n = o.strides[2], p.vec_b = vec_ok(o, dv);
+    p.out = dO, p.os_b = do_strides[0], p.os_h = do_strides[1], p.os_n = do_strides[2], p.vec_out = vec_ok(dOv, dv);
+    if (norm_launch(1, dtype, l.lpr, p, stream) != hipSuccess) return FLA_ERR_LAUNCH;
+    // gradients of the unnormalised product
+    if (int rc = run_tri(dOv, v, k, dq, B, H, N, dv, dqk, 0, dtype, stream)) return rc;
+    if (int rc = run_tri(k, q, dOv, dvv, B, H, N, dqk, dv, 1, dtype, stream)) return rc;
+    if (int rc = run_tri(v, dOv, q, dk, B, H, N, dv, dqk, 1, dtype, stream)) return rc;
+    // the normaliser's own terms
+    p.dq = const_cast<void *>(dq.ptr), p.dqs_b = dq.strides[0], p.dqs_h = dq.strides[1], p.dqs_n = dq.strides[2];
+    p.dk = const_cast<void *>(dk.ptr), p.dks_b = dk.strides[0], p.dks_h = dk.strides[1], p.dks_n = dk.strides[2];
+    p.vec_dq = vec_ok(dq, dqk), p.vec_dk = vec_ok(dk, dqk);
+    return norm_launch(2, dtype, l.lpr, p, stream) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+}
+
 }  // namespace
 
 extern "C" {
@@ -296,6 +404,34 @@ int fla_tri_xyt_z_chunked(const void *x, const void *y, const void *z, void *out
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
     return run_tri_chunked(vx, vy, vz, vo, B, H, N, D_c, D_o, upper, dtype, workspace, workspace_bytes, stream);
+}
+
+int64_t fla_normalised_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v) {
+    if (B < 0 || H < 0 || N < 0 || D_qk < 1 || D_qk > 256 || D_v < 1 || D_v > 256) return 0;
+    const NormLayout l = norm_layout(B, H, N, D_qk, D_v);
+    return l.do_bytes + l.dn_bytes + 2 * l.sums_bytes;
+}
+
+int fla_linear_attn_normalised_fwd(const void *q, const void *k, const void *v, void *o, float *denom, int64_t B,
+                                   int64_t H, int64_t N, int64_t D_qk, int64_t D_v, const int64_t *q_strides,
+                                   const int64_t *k_strides, const int64_t *v_strides, const int64_t *o_strides,
+                                   float eps, int dtype, void *workspace, int64_t workspace_bytes, void *stream) {
+    if (int rc = check_norm_args(B, H, N, D_qk, D_v, dtype)) return rc;
+    return normalised_forward({q, q_strides}, {k, k_strides}, {v, v_strides}, {o, o_strides}, denom, B, H, N, D_qk,
+                              D_v, eps, dtype, workspace, workspace_bytes, stream);
+}
+
+int fla_linear_attn_normalised_bwd(const void *grad_out, const void *q, const void *k, const void *v, const void *o,
+                                   const float *denom, void *dq, void *dk, void *dv, int64_t B, int64_t H,
+                                   int64_t N, int64_t D_qk, int64_t D_v, const int64_t *go_strides,
+                                   const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
+                                   const int64_t *o_strides, const int64_t *dq_strides, const int64_t *dk_strides,
+                                   const int64_t *dv_strides, int dtype, void *workspace, int64_t workspace_bytes,
+                                   void *stream) {
+    if (int rc = check_norm_args(B, H, N, D_qk, D_v, dtype)) return rc;
+    return normalised_backward({grad_out, go_strides}, {q, q_strides}, {k, k_strides}, {v, v_strides},
+                               {o, o_strides}, denom, {dq, dq_strides}, {dk, dk_strides}, {dv, dv_strides}, B, H, N,
+                               D_qk, D_v, dtype, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

@@ -1,0 +1,375 @@
+// The normaliser of causal linear attention, fused into four memory-bound kernels:
+//
+//     n_i   = q_i . (k_0 + ... + k_i) + eps          out_i = O_i / n_i
+//
+// (the recipe the reference leaves to the caller in PyTorch, README.md:27-30: a cumsum over k,
+// an elementwise product with q, a row sum, an add and a division) and its backward.  With
+// g = d(out), the unnormalised product's gradient and the normaliser's own terms are
+//
+//     dO_i = g_i / n_i        dn_i = -(g_i . out_i) / n_i
+//     dq_i += dn_i (k_0 + ... + k_i)        dk_j += dn_j q_j + ... + dn_{N-1} q_{N-1}
+//
+// Everything is a running sum along the sequence, so a (batch, head) slice is cut into chunks
+// of R rows: one kernel writes per-chunk column sums, the consumer adds the sums of the chunks
+// before (after) its own and scans its own rows.  Inside a chunk every group of LPR lanes owns
+// a segment of 16 consecutive rows (8 columns per lane, kept in registers), segment totals are
+// exchanged through LDS, and each row is visited once more with the right offset.  Arithmetic
+// is fp32 throughout; inputs and outputs are the 16-bit storage type.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fla_tri_kernel.h"
+
+namespace fla {
+
+constexpr int kNormSegRows = 16;  // rows per segment (kept packed in registers)
+
+struct NormParams {
+    const void *q, *k;       // (B, H, N, dqk)
+    const void *a;           // fwd: unnormalised O; bwd-pre: grad of the normalised output; (B, H, N, dv)
+    const void *b;           // bwd-pre: the normalised output saved by forward; (B, H, N, dv)
+    void *out;               // fwd: normalised output; bwd-pre: dO = g / n (contiguous); (B, H, N, dv)
+    void *dq, *dk;           // bwd-post: gradients, updated in place; (B, H, N, dqk)
+    float *denom;            // n, fp32, contiguous (B H, N)
+    float *dn;               // bwd: dn, fp32, contiguous (B H, N)
+    float *ksum, *wsum;      // per-chunk column sums of k and of dn q: fp32 [B H][chunks][DP]
+    int64_t qs_b, qs_h, qs_n, ks_b, ks_h, ks_n;
+    int64_t as_b, as_h, as_n, bs_b, bs_h, bs_n, os_b, os_h, os_n;
+    int64_t dqs_b, dqs_h, dqs_n, dks_b, dks_h, dks_n;
+    int32_t H, N, BH, dqk, dv, n_chunks;
+    int32_t vec_q, vec_k, vec_a, vec_b, vec_out, vec_dq, vec_dk;
+    float eps;
+};
+
+template <typename T>
+__device__ __forceinline__ void unpack8(u32x4 w, float (&f)[8]) {
+    typedef T v8 __attribute__((ext_vector_type(8)));
+    const v8 x = __builtin_bit_cast(v8, w);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) f[e] = static_cast<float>(x[e]);
+}
+template <typename T>
+__device__ __forceinline__ u32x4 pack8(const float (&f)[8]) {
+    typedef T v8 __attribute__((ext_vector_type(8)));
+    v8 x;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) x[e] = static_cast<T>(f[e]);
+    return __builtin_bit_cast(u32x4, x);
+}
+template <typename T>
+__device__ __forceinline__ void store8(T *row, int col, int dlim, bool vec, u32x4 w) {
+    if (col >= dlim) return;
+    if (vec) {
+        *reinterpret_cast<u32x4 *>(row + col) = w;
+    } else {
+        unsigned short *e = reinterpret_cast<unsigned short *>(row);
+#pragma unroll
+        for (int x = 0; x < 8; ++x)
+            if (col + x < dlim) e[col + x] = (unsigned short)(w[x >> 1] >> (16 * (x & 1)));
+    }
+}
+// sum over the LPR lanes that share a row (LPR a power of two, lanes contiguous)
+template <int LPR>
+__device__ __forceinline__ float row_sum(float v) {
+#pragma unroll
+    for (int m = 1; m < LPR; m <<= 1) v += __shfl_xor(v, m, 64);
+    return v;
+}
+
+// Geometry shared by the kernels: 256 threads, LPR lanes per row, 64 / LPR row slots per wave,
+// 4 waves -> NSEG segments of kNormSegRows rows each.
+template <int LPR>
+struct NormGeom {
+    static constexpr int RPS = 64 / LPR;
+    static constexpr int NSEG = 4 * RPS;
+    static constexpr int R = NSEG * kNormSegRows;  // rows per chunk
+    static constexpr int DP = LPR * 8;             // padded width
+};
+
+// ---- per-chunk column sums: ksum = sum k_r, and (WITH_W) wsum = sum dn_r q_r
+template <typename T, int LPR, bool WITH_W>
+__global__ __launch_bounds__(256) void norm_chunk_sums_kernel(const NormParams p) {
+    using G = NormGeom<LPR>;
+    __shared__ float red[(WITH_W ? 2 : 1) * G::NSEG * G::DP];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane % LPR, seg = wave * G::RPS + lane / LPR;
+    const int chunk = blockIdx.x, bh = blockIdx.y;
+    const int b = bh / p.H, h = bh - b * p.H;
+    const T *K = static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h;
+    const T *Q = static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h;
+    const int row0 = chunk * G::R + seg * kNormSegRows, col = 8 * li;
+    float sk[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, sw[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int r = 0; r < kNormSegRows; ++r) {
+        const int row = row0 + r;
+        const bool ok = row < p.N;
+        float kf[8];
+        unpack8<T>(load8(K + (int64_t)row * p.ks_n, ok, col, p.dqk, p.vec_k != 0), kf);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sk[e] += kf[e];
+        if constexpr (WITH_W) {
+            float qf[8];
+            unpack8<T>(load8(Q + (int64_t)row * p.qs_n, ok, col, p.dqk, p.vec_q != 0), qf);
+            const float dn = ok ? p.dn[(int64_t)bh * p.N + row] : 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) sw[e] += dn * qf[e];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        red[seg * G::DP + col + e] = sk[e];
+        if constexpr (WITH_W) red[(G::NSEG + seg) * G::DP + col + e] = sw[e];
+    }
+    __syncthreads();
+    for (int c = tid; c < (WITH_W ? 2 : 1) * G::DP; c += 256) {
+        const int which = c / G::DP, cc = c - which * G::DP;
+        float t = 0.f;
+#pragma unroll
+        for (int s = 0; s < G::NSEG; ++s) t += red[(which * G::NSEG + s) * G::DP + cc];
+        float *dst = which ? p.wsum : p.ksum;
+        dst[((int64_t)bh * p.n_chunks + chunk) * G::DP + cc] = t;
+    }
+}
+
+// ---- forward: n_i = q_i . cumsum(k)_i + eps, out_i = a_i / n_i (a = unnormalised O; may alias out)
+template <typename T, int LPR>
+__global__ __launch_bounds__(256) void norm_fwd_kernel(const NormParams p) {
+    using G = NormGeom<LPR>;
+    __shared__ float tot[G::NSEG * G::DP];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane % LPR, seg = wave * G::RPS + lane / LPR;
+    const int chunk = blockIdx.x, bh = blockIdx.y;
+    const int b = bh / p.H, h = bh - b * p.H;
+    const T *K = static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h;
+    const T *Q = static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h;
+    const T *A = static_cast<const T *>(p.a) + b * p.as_b + h * p.as_h;
+    T *O = static_cast<T *>(p.out) + b * p.os_b + h * p.os_h;
+    const int row0 = chunk * G::R + seg * kNormSegRows, col = 8 * li;
+
+    // this segment's rows of k, packed, and their total
+    u32x4 kr[kNormSegRows];
+    float run[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < kNormSegRows; ++r) {
+        kr[r] = load8(K + (int64_t)(row0 + r) * p.ks_n, row0 + r < p.N, col, p.dqk, p.vec_k != 0);
+        float kf[8];
+        unpack8<T>(kr[r], kf);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) run[e] += kf[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) tot[seg * G::DP + col + e] = run[e];
+    // sums of the chunks before this one (while the LDS exchange settles)
+#pragma unroll
+    for (int e = 0; e < 8; ++e) run[e] = 0.f;
+    for (int c = 0; c < chunk; ++c) {
+        const float *src = p.ksum + ((int64_t)bh * p.n_chunks + c) * G::DP + col;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) run[e] += src[e];
+    }
+    __syncthreads();
+    for (int s = 0; s < seg; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) run[e] += tot[s * G::DP + col + e];
+
+#pragma unroll
+    for (int r = 0; r < kNormSegRows; ++r) {
+        const int row = row0 + r;
+        const bool ok = row < p.N;
+        float kf[8], qf[8];
+        unpack8<T>(kr[r], kf);
+        unpack8<T>(load8(Q + (int64_t)row * p.qs_n, ok, col, p.dqk, p.vec_q != 0), qf);
+        float part = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            run[e] += kf[e];
+            part += qf[e] * run[e];
+        }
+        const float n = row_sum<LPR>(part) + p.eps;
+        if (ok) {
+            const float inv = 1.0f / n;
+            if (col < p.dv) {
+                float af[8];
+                unpack8<T>(load8(A + (int64_t)row * p.as_n, true, col, p.dv, p.vec_a != 0), af);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) af[e] *= inv;
+                store8<T>(O + (int64_t)row * p.os_n, col, p.dv, p.vec_out != 0, pack8<T>(af));
+            }
+            if (li == 0) p.denom[(int64_t)bh * p.N + row] = n;
+        }
+    }
+}
+
+// ---- backward, before the main gradient kernels: dO = g / n (contiguous), dn = -(g . out) / n
+template <typename T, int LPR>
+__global__ __launch_bounds__(256) void norm_bwd_pre_kernel(const NormParams p) {
+    using G = NormGeom<LPR>;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane % LPR, slot = wave * G::RPS + lane / LPR;
+    const int bh = blockIdx.y;
+    const int b = bh / p.H, h = bh - b * p.H;
+    const T *Gr = static_cast<const T *>(p.a) + b * p.as_b + h * p.as_h;
+    const T *Ou = static_cast<const T *>(p.b) + b * p.bs_b + h * p.bs_h;
+    T *dO = static_cast<T *>(p.out) + b * p.os_b + h * p.os_h;
+    const int col = 8 * li;
+#pragma unroll 4
+    for (int r = 0; r < kNormSegRows; ++r) {
+        const int row = (blockIdx.x * kNormSegRows + r) * G::NSEG + slot;  // consecutive rows across the workgroup
+        const bool ok = row < p.N;
+        float gf[8], of[8];
+        unpack8<T>(load8(Gr + (int64_t)row * p.as_n, ok, col, p.dv, p.vec_a != 0), gf);
+        unpack8<T>(load8(Ou + (int64_t)row * p.bs_n, ok, col, p.dv, p.vec_b != 0), of);
+        float part = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) part += gf[e] * of[e];
+        const float dot = row_sum<LPR>(part);
+        if (ok) {
+            const float inv = 1.0f / p.denom[(int64_t)bh * p.N + row];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) gf[e] *= inv;
+            store8<T>(dO + (int64_t)row * p.os_n, col, p.dv, p.vec_out != 0, pack8<T>(gf));
+            if (li == 0) p.dn[(int64_t)bh * p.N + row] = -dot * inv;
+        }
+    }
+}
+
+// ---- backward, after the main gradient kernels: dq_i += dn_i cumsum(k)_i, dk_j += revcumsum(dn q)_j
+template <typename T, int LPR>
+__global__ __launch_bounds__(256) void norm_bwd_post_kernel(const NormParams p) {
+    using G = NormGeom<LPR>;
+    __shared__ float tot[2 * G::NSEG * G::DP];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int li = lane % LPR, seg = wave * G::RPS + lane / LPR;
+    const int chunk = blockIdx.x, bh = blockIdx.y;
+    const int b = bh / p.H, h = bh - b * p.H;
+    const T *K = static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h;
+    const T *Q = static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h;
+    T *DQ = static_cast<T *>(p.dq) + b * p.dqs_b + h * p.dqs_h;
+    T *DK = static_cast<T *>(p.dk) + b * p.dks_b + h * p.dks_h;
+    const int row0 = chunk * G::R + seg * kNormSegRows, col = 8 * li;
+
+    u32x4 kr[kNormSegRows], qr[kNormSegRows];
+    float dn[kNormSegRows];
+    float rk[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, rw[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < kNormSegRows; ++r) {
+        const int row = row0 + r;
+        const bool ok = row < p.N;
+        kr[r] = load8(K + (int64_t)row * p.ks_n, ok, col, p.dqk, p.vec_k != 0);
+        qr[r] = load8(Q + (int64_t)row * p.qs_n, ok, col, p.dqk, p.vec_q != 0);
+        dn[r] = ok ? p.dn[(int64_t)bh * p.N + row] : 0.f;
+        float kf[8], qf[8];
+        unpack8<T>(kr[r], kf);
+        unpack8<T>(qr[r], qf);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            rk[e] += kf[e];
+            rw[e] += dn[r] * qf[e];
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        tot[seg * G::DP + col + e] = rk[e];
+        tot[(G::NSEG + seg) * G::DP + col + e] = rw[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) rk[e] = rw[e] = 0.f;
+    for (int c = 0; c < chunk; ++c) {
+        const float *src = p.ksum + ((int64_t)bh * p.n_chunks + c) * G::DP + col;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) rk[e] += src[e];
+    }
+    for (int c = chunk + 1; c < p.n_chunks; ++c) {
+        const float *src = p.wsum + ((int64_t)bh * p.n_chunks + c) * G::DP + col;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) rw[e] += src[e];
+    }
+    __syncthreads();
+    for (int s = 0; s < seg; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) rk[e] += tot[s * G::DP + col + e];
+    for (int s = seg + 1; s < G::NSEG; ++s)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) rw[e] += tot[(G::NSEG + s) * G::DP + col + e];
+
+    if (col >= p.dqk) return;
+    // dq: rows in ascending order with the inclusive prefix of k
+#pragma unroll
+    for (int r = 0; r < kNormSegRows; ++r) {
+        const int row = row0 + r;
+        float kf[8], g[8];
+        unpack8<T>(kr[r], kf);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) rk[e] += kf[e];
+        if (row < p.N) {
+            T *dst = DQ + (int64_t)row * p.dqs_n;
+            unpack8<T>(load8(dst, true, col, p.dqk, p.vec_dq != 0), g);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) g[e] += dn[r] * rk[e];
+            store8<T>(dst, col, p.dqk, p.vec_dq != 0, pack8<T>(g));
+        }
+    }
+    // dk: rows in descending order with the inclusive suffix of dn q
+#pragma unroll
+    for (int r = kNormSegRows - 1; r >= 0; --r) {
+        const int row = row0 + r;
+        float qf[8], g[8];
+        unpack8<T>(qr[r], qf);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) rw[e] += dn[r] * qf[e];
+        if (row < p.N) {
+            T *dst = DK + (int64_t)row * p.dks_n;
+            unpack8<T>(load8(dst, true, col, p.dqk, p.vec_dk != 0), g);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) g[e] += rw[e];
+            store8<T>(dst, col, p.dqk, p.vec_dk != 0, pack8<T>(g));
+        }
+    }
+}
+
+// lanes per row for a width: the smallest of 4, 8, 16, 32 with 8 LPR >= width
+inline int norm_lanes_per_row(int width) { return width <= 32 ? 4 : width <= 64 ? 8 : width <= 128 ? 16 : 32; }
+inline int norm_chunk_rows(int lpr) { return 4 * (64 / lpr) * kNormSegRows; }
+
+template <typename T, int LPR>
+hipError_t launch_norm_fwd_lpr(const NormParams &p, hipStream_t s) {
+    const dim3 grid((unsigned)p.n_chunks, (unsigned)p.BH);
+    if (p.n_chunks > 1) hipLaunchKernelGGL((norm_chunk_sums_kernel<T, LPR, false>), grid, dim3(256), 0, s, p);
+    hipLaunchKernelGGL((norm_fwd_kernel<T, LPR>), grid, dim3(256), 0, s, p);
+    return hipGetLastError();
+}
+template <typename T, int LPR>
+hipError_t launch_norm_bwd_pre_lpr(const NormParams &p, hipStream_t s) {
+    const dim3 grid((unsigned)p.n_chunks, (unsigned)p.BH);  // R rows per workgroup here too
+    hipLaunchKernelGGL((norm_bwd_pre_kernel<T, LPR>), grid, dim3(256), 0, s, p);
+    return hipGetLastError();
+}
+template <typename T, int LPR>
+hipError_t launch_norm_bwd_post_lpr(const NormParams &p, hipStream_t s) {
+    const dim3 grid((unsigned)p.n_chunks, (unsigned)p.BH);
+    if (p.n_chunks > 1) hipLaunchKernelGGL((norm_chunk_sums_kernel<T, LPR, true>), grid, dim3(256), 0, s, p);
+    hipLaunchKernelGGL((norm_bwd_post_kernel<T, LPR>), grid, dim3(256), 0, s, p);
+    return hipGetLastError();
+}
+
+// which: 0 forward, 1 backward-pre, 2 backward-post; lpr from norm_lanes_per_row
+template <typename T>
+hipError_t launch_norm(int which, int lpr, const NormParams &p, hipStream_t s) {
+#define FLA_NORM_CASE(L)                                                 \
+    case L:                                                              \
+        return which == 0   ? launch_norm_fwd_lpr<T, L>(p, s)            \
+               : which == 1 ? launch_norm_bwd_pre_lpr<T, L>(p, s)        \
+                            : launch_norm_bwd_post_lpr<T, L>(p, s);
+    switch (lpr) {
+        FLA_NORM_CASE(4)
+        FLA_NORM_CASE(8)
+        FLA_NORM_CASE(16)
+        FLA_NORM_CASE(32)
+        default: return hipErrorInvalidValue;
+    }
+#undef FLA_NORM_CASE
+}
+
+}  // namespace fla
