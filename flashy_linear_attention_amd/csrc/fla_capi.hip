@@ -235,8 +235,12 @@ void norm_common(fla::NormParams &p, const View &q, const View &k, int64_t B, in
 
 hipError_t norm_launch(int which, int dtype, int lpr, const fla::NormParams &p, void *stream) {
     hipStream_t s = static_cast<hipStream_t>(stream);
-    return dtype == FLA_DTYPE_BF16 ? fla::launch_norm<__bf16>(which, lpr, p, s)
-                                   : fla::launch_norm<_Float16>(which, lpr, p, s);
+    // the operands this pass touches all allow 16-byte accesses?
+    const bool vec = which == 0   ? (p.vec_q && p.vec_k && p.vec_a && p.vec_out)
+                     : which == 1 ? (p.vec_a && p.vec_b && p.vec_out)
+                                  : (p.vec_q && p.vec_k && p.vec_dq && p.vec_dk);
+    return dtype == FLA_DTYPE_BF16 ? fla::launch_norm<__bf16>(which, lpr, vec, p, s)
+                                   : fla::launch_norm<_Float16>(which, lpr, vec, p, s);
 }
 
 int check_norm_args(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv, int dtype) {

@@ -10,11 +10,13 @@
 //     dq_i += dn_i (k_0 + ... + k_i)        dk_j += dn_j q_j + ... + dn_{N-1} q_{N-1}
 //
 // Everything is a running sum along the sequence, so a (batch, head) slice is cut into chunks
-// of R rows: one kernel writes per-chunk column sums, the consumer adds the sums of the chunks
-// before (after) its own and scans its own rows.  Inside a chunk every group of LPR lanes owns
-// a segment of 16 consecutive rows (8 columns per lane, kept in registers), segment totals are
-// exchanged through LDS, and each row is visited once more with the right offset.  Arithmetic
-// is fp32 throughout; inputs and outputs are the 16-bit storage type.
+// of R rows: one kernel writes per-chunk column sums, a tiny kernel turns them into exclusive
+// prefix (suffix) sums over the chunks, and the consumer scans its own rows starting from its
+// chunk's entry.  Inside a chunk every group of LPR lanes owns a segment of 16 consecutive rows
+// (8 columns per lane, kept packed in registers), segment totals are exchanged through LDS, and
+// each row is visited once more with the right offset.  All loads of a workgroup are issued
+// before the first use.  Arithmetic is fp32 throughout; inputs and outputs are the 16-bit
+// storage type.  VEC = true instantiations assume every operand qualifies for 16-byte accesses.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -89,7 +91,7 @@ struct NormGeom {
 };
 
 // ---- per-chunk column sums: ksum = sum k_r, and (WITH_W) wsum = sum dn_r q_r
-template <typename T, int LPR, bool WITH_W>
+template <typename T, int LPR, bool VEC, bool WITH_W>
 __global__ __launch_bounds__(256) void norm_chunk_sums_kernel(const NormParams p) {
     using G = NormGeom<LPR>;
     __shared__ float red[(WITH_W ? 2 : 1) * G::NSEG * G::DP];
@@ -100,21 +102,30 @@ __global__ __launch_bounds__(256) void norm_chunk_sums_kernel(const NormParams p
     const T *K = static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h;
     const T *Q = static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h;
     const int row0 = chunk * G::R + seg * kNormSegRows, col = 8 * li;
-    float sk[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, sw[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
+    u32x4 kr[kNormSegRows], qr[WITH_W ? kNormSegRows : 1];
+    float dn[WITH_W ? kNormSegRows : 1];
+#pragma unroll
     for (int r = 0; r < kNormSegRows; ++r) {
         const int row = row0 + r;
         const bool ok = row < p.N;
+        kr[r] = load8(K + (int64_t)row * p.ks_n, ok, col, p.dqk, VEC || p.vec_k != 0);
+        if constexpr (WITH_W) {
+            qr[r] = load8(Q + (int64_t)row * p.qs_n, ok, col, p.dqk, VEC || p.vec_q != 0);
+            dn[r] = ok ? p.dn[(int64_t)bh * p.N + row] : 0.f;
+        }
+    }
+    float sk[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, sw[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < kNormSegRows; ++r) {
         float kf[8];
-        unpack8<T>(load8(K + (int64_t)row * p.ks_n, ok, col, p.dqk, p.vec_k != 0), kf);
+        unpack8<T>(kr[r], kf);
 #pragma unroll
         for (int e = 0; e < 8; ++e) sk[e] += kf[e];
         if constexpr (WITH_W) {
             float qf[8];
-            unpack8<T>(load8(Q + (int64_t)row * p.qs_n, ok, col, p.dqk, p.vec_q != 0), qf);
-            const float dn = ok ? p.dn[(int64_t)bh * p.N + row] : 0.f;
+            unpack8<T>(qr[r], qf);
 #pragma unroll
-            for (int e = 0; e < 8; ++e) sw[e] += dn * qf[e];
+            for (int e = 0; e < 8; ++e) sw[e] += dn[r] * qf[e];
         }
     }
 #pragma unroll
@@ -133,9 +144,33 @@ __global__ __launch_bounds__(256) void norm_chunk_sums_kernel(const NormParams p
     }
 }
 
+// ---- chunk sums -> exclusive prefix sums over the chunks (ksum) and exclusive suffix sums
+// (wsum, when given), in place.  One thread per (batch-head, column).
+__global__ __launch_bounds__(256) void norm_scan_kernel(float *ksum, float *wsum, int BH, int chunks, int DP) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= (int64_t)BH * DP) return;
+    const int64_t bh = t / DP, c0 = t - bh * DP;
+    float *ks = ksum + bh * chunks * DP + c0;
+    float run = 0.f;
+    for (int c = 0; c < chunks; ++c) {
+        const float v = ks[(int64_t)c * DP];
+        ks[(int64_t)c * DP] = run;
+        run += v;
+    }
+    if (wsum) {
+        float *ws = wsum + bh * chunks * DP + c0;
+        run = 0.f;
+        for (int c = chunks - 1; c >= 0; --c) {
+            const float v = ws[(int64_t)c * DP];
+            ws[(int64_t)c * DP] = run;
+            run += v;
+        }
+    }
+}
+
 // ---- forward: n_i = q_i . cumsum(k)_i + eps, out_i = a_i / n_i (a = unnormalised O; may alias out)
-template <typename T, int LPR>
-__global__ __launch_bounds__(256) void norm_fwd_kernel(const NormParams p) {
+template <typename T, int LPR, bool VEC>
+__global__ __launch_bounds__(256, 2) void norm_fwd_kernel(const NormParams p) {
     using G = NormGeom<LPR>;
     __shared__ float tot[G::NSEG * G::DP];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -148,39 +183,47 @@ __global__ __launch_bounds__(256) void norm_fwd_kernel(const NormParams p) {
     T *O = static_cast<T *>(p.out) + b * p.os_b + h * p.os_h;
     const int row0 = chunk * G::R + seg * kNormSegRows, col = 8 * li;
 
-    // this segment's rows of k, packed, and their total
-    u32x4 kr[kNormSegRows];
-    float run[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // this segment's rows of k and q, packed; all requested before anything is used
+    u32x4 kr[kNormSegRows], qr[kNormSegRows];
 #pragma unroll
-    for (int r = 0; r < kNormSegRows; ++r) {
-        kr[r] = load8(K + (int64_t)(row0 + r) * p.ks_n, row0 + r < p.N, col, p.dqk, p.vec_k != 0);
-        float kf[8];
-        unpack8<T>(kr[r], kf);
+    for (int r = 0; r < kNormSegRows; ++r)
+        kr[r] = load8(K + (int64_t)(row0 + r) * p.ks_n, row0 + r < p.N, col, p.dqk, VEC || p.vec_k != 0);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) run[e] += kf[e];
+    for (int r = 0; r < kNormSegRows; ++r)
+        qr[r] = load8(Q + (int64_t)(row0 + r) * p.qs_n, row0 + r < p.N, col, p.dqk, VEC || p.vec_q != 0);
+    float run[8];
+    if (chunk > 0) {
+        const float *src = p.ksum + ((int64_t)bh * p.n_chunks + chunk) * G::DP + col;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) run[e] = src[e];
+    } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) run[e] = 0.f;
     }
+    {
+        float t[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int e = 0; e < 8; ++e) tot[seg * G::DP + col + e] = run[e];
-    // sums of the chunks before this one (while the LDS exchange settles)
+        for (int r = 0; r < kNormSegRows; ++r) {
+            float kf[8];
+            unpack8<T>(kr[r], kf);
 #pragma unroll
-    for (int e = 0; e < 8; ++e) run[e] = 0.f;
-    for (int c = 0; c < chunk; ++c) {
-        const float *src = p.ksum + ((int64_t)bh * p.n_chunks + c) * G::DP + col;
+            for (int e = 0; e < 8; ++e) t[e] += kf[e];
+        }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) run[e] += src[e];
+        for (int e = 0; e < 8; ++e) tot[seg * G::DP + col + e] = t[e];
     }
     __syncthreads();
     for (int s = 0; s < seg; ++s)
 #pragma unroll
         for (int e = 0; e < 8; ++e) run[e] += tot[s * G::DP + col + e];
 
+    // normalisers of the segment's rows, then the division row by row
+    float inv[kNormSegRows];
 #pragma unroll
     for (int r = 0; r < kNormSegRows; ++r) {
-        const int row = row0 + r;
-        const bool ok = row < p.N;
         float kf[8], qf[8];
         unpack8<T>(kr[r], kf);
-        unpack8<T>(load8(Q + (int64_t)row * p.qs_n, ok, col, p.dqk, p.vec_q != 0), qf);
+        unpack8<T>(qr[r], qf);
         float part = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
@@ -188,22 +231,35 @@ __global__ __launch_bounds__(256) void norm_fwd_kernel(const NormParams p) {
             part += qf[e] * run[e];
         }
         const float n = row_sum<LPR>(part) + p.eps;
-        if (ok) {
-            const float inv = 1.0f / n;
-            if (col < p.dv) {
-                float af[8];
-                unpack8<T>(load8(A + (int64_t)row * p.as_n, true, col, p.dv, p.vec_a != 0), af);
+        inv[r] = 1.0f / n;
+        if (li == 0 && row0 + r < p.N) p.denom[(int64_t)bh * p.N + row0 + r] = n;
+    }
+    if (col >= p.dv) return;
+    constexpr int HALF = kNormSegRows / 2;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) af[e] *= inv;
-                store8<T>(O + (int64_t)row * p.os_n, col, p.dv, p.vec_out != 0, pack8<T>(af));
+    for (int half = 0; half < 2; ++half) {
+        u32x4 ar[HALF];
+#pragma unroll
+        for (int r = 0; r < HALF; ++r) {
+            const int row = row0 + half * HALF + r;
+            ar[r] = load8(A + (int64_t)row * p.as_n, row < p.N, col, p.dv, VEC || p.vec_a != 0);
+        }
+#pragma unroll
+        for (int r = 0; r < HALF; ++r) {
+            const int row = row0 + half * HALF + r;
+            if (row < p.N) {
+                float af[8];
+                unpack8<T>(ar[r], af);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) af[e] *= inv[half * HALF + r];
+                store8<T>(O + (int64_t)row * p.os_n, col, p.dv, VEC || p.vec_out != 0, pack8<T>(af));
             }
-            if (li == 0) p.denom[(int64_t)bh * p.N + row] = n;
         }
     }
 }
 
 // ---- backward, before the main gradient kernels: dO = g / n (contiguous), dn = -(g . out) / n
-template <typename T, int LPR>
+template <typename T, int LPR, bool VEC>
 __global__ __launch_bounds__(256) void norm_bwd_pre_kernel(const NormParams p) {
     using G = NormGeom<LPR>;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -219,8 +275,8 @@ __global__ __launch_bounds__(256) void norm_bwd_pre_kernel(const NormParams p) {
         const int row = (blockIdx.x * kNormSegRows + r) * G::NSEG + slot;  // consecutive rows across the workgroup
         const bool ok = row < p.N;
         float gf[8], of[8];
-        unpack8<T>(load8(Gr + (int64_t)row * p.as_n, ok, col, p.dv, p.vec_a != 0), gf);
-        unpack8<T>(load8(Ou + (int64_t)row * p.bs_n, ok, col, p.dv, p.vec_b != 0), of);
+        unpack8<T>(load8(Gr + (int64_t)row * p.as_n, ok, col, p.dv, VEC || p.vec_a != 0), gf);
+        unpack8<T>(load8(Ou + (int64_t)row * p.bs_n, ok, col, p.dv, VEC || p.vec_b != 0), of);
         float part = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) part += gf[e] * of[e];
@@ -229,103 +285,92 @@ __global__ __launch_bounds__(256) void norm_bwd_pre_kernel(const NormParams p) {
             const float inv = 1.0f / p.denom[(int64_t)bh * p.N + row];
 #pragma unroll
             for (int e = 0; e < 8; ++e) gf[e] *= inv;
-            store8<T>(dO + (int64_t)row * p.os_n, col, p.dv, p.vec_out != 0, pack8<T>(gf));
+            store8<T>(dO + (int64_t)row * p.os_n, col, p.dv, VEC || p.vec_out != 0, pack8<T>(gf));
             if (li == 0) p.dn[(int64_t)bh * p.N + row] = -dot * inv;
         }
     }
 }
 
-// ---- backward, after the main gradient kernels: dq_i += dn_i cumsum(k)_i, dk_j += revcumsum(dn q)_j
-template <typename T, int LPR>
-__global__ __launch_bounds__(256) void norm_bwd_post_kernel(const NormParams p) {
+// ---- backward, after the main gradient kernels.  blockIdx.z = 0: dq_i += dn_i cumsum(k)_i;
+// blockIdx.z = 1: dk_j += revcumsum(dn q)_j.  The two halves are independent.
+template <typename T, int LPR, bool VEC>
+__global__ __launch_bounds__(256, 2) void norm_bwd_post_kernel(const NormParams p) {
     using G = NormGeom<LPR>;
-    __shared__ float tot[2 * G::NSEG * G::DP];
+    __shared__ float tot[G::NSEG * G::DP];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane % LPR, seg = wave * G::RPS + lane / LPR;
     const int chunk = blockIdx.x, bh = blockIdx.y;
+    const bool part_dk = blockIdx.z != 0;
     const int b = bh / p.H, h = bh - b * p.H;
-    const T *K = static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h;
-    const T *Q = static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h;
-    T *DQ = static_cast<T *>(p.dq) + b * p.dqs_b + h * p.dqs_h;
-    T *DK = static_cast<T *>(p.dk) + b * p.dks_b + h * p.dks_h;
+    // the scanned operand (k for dq, q for dk) and the gradient that is updated
+    const T *S = part_dk ? static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h
+                         : static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h;
+    const int64_t ss_n = part_dk ? p.qs_n : p.ks_n;
+    const bool vec_s = VEC || (part_dk ? p.vec_q : p.vec_k) != 0;
+    T *D = part_dk ? static_cast<T *>(p.dk) + b * p.dks_b + h * p.dks_h
+                   : static_cast<T *>(p.dq) + b * p.dqs_b + h * p.dqs_h;
+    const int64_t ds_n = part_dk ? p.dks_n : p.dqs_n;
+    const bool vec_d = VEC || (part_dk ? p.vec_dk : p.vec_dq) != 0;
     const int row0 = chunk * G::R + seg * kNormSegRows, col = 8 * li;
 
-    u32x4 kr[kNormSegRows], qr[kNormSegRows];
+    u32x4 sr[kNormSegRows], dr[kNormSegRows];
     float dn[kNormSegRows];
-    float rk[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, rw[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int r = 0; r < kNormSegRows; ++r) {
         const int row = row0 + r;
-        const bool ok = row < p.N;
-        kr[r] = load8(K + (int64_t)row * p.ks_n, ok, col, p.dqk, p.vec_k != 0);
-        qr[r] = load8(Q + (int64_t)row * p.qs_n, ok, col, p.dqk, p.vec_q != 0);
-        dn[r] = ok ? p.dn[(int64_t)bh * p.N + row] : 0.f;
-        float kf[8], qf[8];
-        unpack8<T>(kr[r], kf);
-        unpack8<T>(qr[r], qf);
+        sr[r] = load8(S + (int64_t)row * ss_n, row < p.N, col, p.dqk, vec_s);
+        dn[r] = row < p.N ? p.dn[(int64_t)bh * p.N + row] : 0.f;
+    }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-            rk[e] += kf[e];
-            rw[e] += dn[r] * qf[e];
+    for (int r = 0; r < kNormSegRows; ++r)
+        dr[r] = load8(D + (int64_t)(row0 + r) * ds_n, row0 + r < p.N, col, p.dqk, vec_d);
+    // running sum at the entry of this chunk: chunks before it (k) or after it (dn q)
+    float run[8];
+    {
+        const float *src = (part_dk ? p.wsum : p.ksum) + ((int64_t)bh * p.n_chunks + chunk) * G::DP + col;
+        const bool have = p.n_chunks > 1;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) run[e] = have ? src[e] : 0.f;
+    }
+    {
+        float t[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int r = 0; r < kNormSegRows; ++r) {
+            float sf[8];
+            unpack8<T>(sr[r], sf);
+            const float w = part_dk ? dn[r] : 1.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) t[e] += w * sf[e];
         }
-    }
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        tot[seg * G::DP + col + e] = rk[e];
-        tot[(G::NSEG + seg) * G::DP + col + e] = rw[e];
-    }
-#pragma unroll
-    for (int e = 0; e < 8; ++e) rk[e] = rw[e] = 0.f;
-    for (int c = 0; c < chunk; ++c) {
-        const float *src = p.ksum + ((int64_t)bh * p.n_chunks + c) * G::DP + col;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) rk[e] += src[e];
-    }
-    for (int c = chunk + 1; c < p.n_chunks; ++c) {
-        const float *src = p.wsum + ((int64_t)bh * p.n_chunks + c) * G::DP + col;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) rw[e] += src[e];
+        for (int e = 0; e < 8; ++e) tot[seg * G::DP + col + e] = t[e];
     }
     __syncthreads();
-    for (int s = 0; s < seg; ++s)
+    if (part_dk) {
+        for (int s = seg + 1; s < G::NSEG; ++s)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) rk[e] += tot[s * G::DP + col + e];
-    for (int s = seg + 1; s < G::NSEG; ++s)
+            for (int e = 0; e < 8; ++e) run[e] += tot[s * G::DP + col + e];
+    } else {
+        for (int s = 0; s < seg; ++s)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) rw[e] += tot[(G::NSEG + s) * G::DP + col + e];
-
-    if (col >= p.dqk) return;
-    // dq: rows in ascending order with the inclusive prefix of k
-#pragma unroll
-    for (int r = 0; r < kNormSegRows; ++r) {
-        const int row = row0 + r;
-        float kf[8], g[8];
-        unpack8<T>(kr[r], kf);
-#pragma unroll
-        for (int e = 0; e < 8; ++e) rk[e] += kf[e];
-        if (row < p.N) {
-            T *dst = DQ + (int64_t)row * p.dqs_n;
-            unpack8<T>(load8(dst, true, col, p.dqk, p.vec_dq != 0), g);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) g[e] += dn[r] * rk[e];
-            store8<T>(dst, col, p.dqk, p.vec_dq != 0, pack8<T>(g));
-        }
+            for (int e = 0; e < 8; ++e) run[e] += tot[s * G::DP + col + e];
     }
-    // dk: rows in descending order with the inclusive suffix of dn q
+    if (col >= p.dqk) return;
+    // inclusive scan over the segment's rows: ascending for dq, descending for dk
 #pragma unroll
-    for (int r = kNormSegRows - 1; r >= 0; --r) {
-        const int row = row0 + r;
-        float qf[8], g[8];
-        unpack8<T>(qr[r], qf);
+    for (int i = 0; i < kNormSegRows; ++i) {
+        // register arrays are indexed by compile-time constants only: both candidates, then select
+        float sf[8], g[8];
+        unpack8<T>(part_dk ? sr[kNormSegRows - 1 - i] : sr[i], sf);
+        unpack8<T>(part_dk ? dr[kNormSegRows - 1 - i] : dr[i], g);
+        const float dnr = part_dk ? dn[kNormSegRows - 1 - i] : dn[i];
+        const int row = row0 + (part_dk ? kNormSegRows - 1 - i : i);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) rw[e] += dn[r] * qf[e];
-        if (row < p.N) {
-            T *dst = DK + (int64_t)row * p.dks_n;
-            unpack8<T>(load8(dst, true, col, p.dqk, p.vec_dk != 0), g);
-#pragma unroll
-            for (int e = 0; e < 8; ++e) g[e] += rw[e];
-            store8<T>(dst, col, p.dqk, p.vec_dk != 0, pack8<T>(g));
+        for (int e = 0; e < 8; ++e) {
+            run[e] += (part_dk ? dnr : 1.0f) * sf[e];
+            g[e] += (part_dk ? 1.0f : dnr) * run[e];
         }
+        if (row < p.N) store8<T>(D + (int64_t)row * ds_n, col, p.dqk, vec_d, pack8<T>(g));
     }
 }
 
@@ -333,35 +378,40 @@ __global__ __launch_bounds__(256) void norm_bwd_post_kernel(const NormParams p) 
 inline int norm_lanes_per_row(int width) { return width <= 32 ? 4 : width <= 64 ? 8 : width <= 128 ? 16 : 32; }
 inline int norm_chunk_rows(int lpr) { return 4 * (64 / lpr) * kNormSegRows; }
 
-template <typename T, int LPR>
-hipError_t launch_norm_fwd_lpr(const NormParams &p, hipStream_t s) {
-    const dim3 grid((unsigned)p.n_chunks, (unsigned)p.BH);
-    if (p.n_chunks > 1) hipLaunchKernelGGL((norm_chunk_sums_kernel<T, LPR, false>), grid, dim3(256), 0, s, p);
-    hipLaunchKernelGGL((norm_fwd_kernel<T, LPR>), grid, dim3(256), 0, s, p);
-    return hipGetLastError();
-}
-template <typename T, int LPR>
-hipError_t launch_norm_bwd_pre_lpr(const NormParams &p, hipStream_t s) {
-    const dim3 grid((unsigned)p.n_chunks, (unsigned)p.BH);  // R rows per workgroup here too
-    hipLaunchKernelGGL((norm_bwd_pre_kernel<T, LPR>), grid, dim3(256), 0, s, p);
-    return hipGetLastError();
-}
-template <typename T, int LPR>
-hipError_t launch_norm_bwd_post_lpr(const NormParams &p, hipStream_t s) {
-    const dim3 grid((unsigned)p.n_chunks, (unsigned)p.BH);
-    if (p.n_chunks > 1) hipLaunchKernelGGL((norm_chunk_sums_kernel<T, LPR, true>), grid, dim3(256), 0, s, p);
-    hipLaunchKernelGGL((norm_bwd_post_kernel<T, LPR>), grid, dim3(256), 0, s, p);
+inline hipError_t launch_norm_scan(const NormParams &p, int dp, bool with_w, hipStream_t s) {
+    const int64_t threads = (int64_t)p.BH * dp;
+    hipLaunchKernelGGL(norm_scan_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, p.ksum,
+                       with_w ? p.wsum : nullptr, p.BH, p.n_chunks, dp);
     return hipGetLastError();
 }
 
-// which: 0 forward, 1 backward-pre, 2 backward-post; lpr from norm_lanes_per_row
+// which: 0 forward, 1 backward-pre, 2 backward-post
+template <typename T, int LPR, bool VEC>
+hipError_t launch_norm_lpr(int which, const NormParams &p, hipStream_t s) {
+    const dim3 grid((unsigned)p.n_chunks, (unsigned)p.BH);
+    if (which == 0) {
+        if (p.n_chunks > 1) {
+            hipLaunchKernelGGL((norm_chunk_sums_kernel<T, LPR, VEC, false>), grid, dim3(256), 0, s, p);
+            launch_norm_scan(p, LPR * 8, false, s);
+        }
+        hipLaunchKernelGGL((norm_fwd_kernel<T, LPR, VEC>), grid, dim3(256), 0, s, p);
+    } else if (which == 1) {
+        hipLaunchKernelGGL((norm_bwd_pre_kernel<T, LPR, VEC>), grid, dim3(256), 0, s, p);
+    } else {
+        if (p.n_chunks > 1) {
+            hipLaunchKernelGGL((norm_chunk_sums_kernel<T, LPR, VEC, true>), grid, dim3(256), 0, s, p);
+            launch_norm_scan(p, LPR * 8, true, s);
+        }
+        hipLaunchKernelGGL((norm_bwd_post_kernel<T, LPR, VEC>), dim3(grid.x, grid.y, 2), dim3(256), 0, s, p);
+    }
+    return hipGetLastError();
+}
+
+// lpr from norm_lanes_per_row; vec: every operand of this call qualifies for 16-byte accesses
 template <typename T>
-hipError_t launch_norm(int which, int lpr, const NormParams &p, hipStream_t s) {
-#define FLA_NORM_CASE(L)                                                 \
-    case L:                                                              \
-        return which == 0   ? launch_norm_fwd_lpr<T, L>(p, s)            \
-               : which == 1 ? launch_norm_bwd_pre_lpr<T, L>(p, s)        \
-                            : launch_norm_bwd_post_lpr<T, L>(p, s);
+hipError_t launch_norm(int which, int lpr, bool vec, const NormParams &p, hipStream_t s) {
+#define FLA_NORM_CASE(L) \
+    case L: return vec ? launch_norm_lpr<T, L, true>(which, p, s) : launch_norm_lpr<T, L, false>(which, p, s);
     switch (lpr) {
         FLA_NORM_CASE(4)
         FLA_NORM_CASE(8)
