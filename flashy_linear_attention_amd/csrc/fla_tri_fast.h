@@ -95,25 +95,30 @@ __device__ __forceinline__ uint32_t round_pack_pinned(float lo, float hi) {
 constexpr uint32_t kOobOffset = 0x40000000u;  // added to a buffer offset to force an out-of-range (zero) access
 constexpr int64_t kMaxFastExtent = 0x3fffffff;  // per-(b,h) byte extent the 32-bit buffer offsets can address
 
-template <int DC, int DO>
+// CHUNKED = false: the quadratic walk over all tiles under the mask; true: chunk-wise evaluation
+// (diagonal block plus running state), compiled as a kernel of its own.
+template <int DC, int DO, bool CHUNKED = false>
 struct FastConfig {
     static constexpr int MW = TriConfig<DC, DO>::MW;
     static constexpr int NW = 4;
     static constexpr int BM = MW * NW;
     static constexpr int BN = 64;
-    // LDS ring depth: the tile being consumed, the one before it (its second half is still
-    // being read for a while) and NBUF-2 tiles landed or in flight.  Four slots when they fit.
-    static constexpr int NBUF = 4 * (BN * (DC + DO) * 2) <= 160 * 1024 ? 4 : 3;
     static constexpr int RY = DC * 2, RZ = DO * 2;  // LDS row bytes (no padding)
     static constexpr int CY = DC / 8, CZ = DO / 8;  // 16-byte chunks per row
     static constexpr int Y_BYTES = BN * RY, Z_BYTES = BN * RZ;
     static constexpr int STAGE_BYTES = Y_BYTES + Z_BYTES;
+    // LDS ring depth.  Quadratic walk: the tile being consumed, the one before it (its second
+    // half is still being read for a while) and NBUF-2 tiles landed or in flight: as many as
+    // fit, up to five (with five, the whole diagonal block is on its way when the walk over the
+    // full tiles ends).  Chunked: exactly the tiles of the diagonal block, nothing cycles.
+    static constexpr int kMaxSlots = (160 * 1024) / STAGE_BYTES;
+    static constexpr int NBUF = CHUNKED ? BM / BN : (kMaxSlots >= 5 ? 5 : kMaxSlots);
     static constexpr int SMEM_BYTES = NBUF * STAGE_BYTES;
-    static constexpr bool kSupported = SMEM_BYTES <= 160 * 1024;
-    // chunked evaluation: the running state S^T, [DO rows][DC] 16-bit, sits behind the ring in
+    static constexpr bool kSupported = kMaxSlots >= 3 && BM / BN <= kMaxSlots;
+    // chunked evaluation: the running state S^T, [DO rows][DC] 16-bit, sits behind the tiles in
     // whole 64-row units of the Y tile layout when the 160 KiB allow it
     static constexpr int STATE_BYTES = ((DO + 63) / 64) * Y_BYTES;
-    static constexpr bool kStateInLds = SMEM_BYTES + STATE_BYTES <= 160 * 1024;
+    static constexpr bool kStateInLds = CHUNKED && SMEM_BYTES + STATE_BYTES <= 160 * 1024;
     // Narrow shapes need half the LDS and about half the registers: holding the kernel to 256
     // registers lets two workgroups share a CU, which hides each other's prologue and epilogue.
     static constexpr int kMinWavesPerSimd = (DC <= 64 && DO <= 64) ? 2 : 1;
@@ -138,13 +143,14 @@ __device__ __forceinline__ int swizzle_z(int row) {
     else return (row & 3) << 1;  // the 4 rows of one transposing read land in 4 different 32-byte slots
 }
 
-template <typename T, int DC, int DO>
-__global__ __launch_bounds__(256, (FastConfig<DC, DO>::kMinWavesPerSimd)) void tri_xyt_z_fast_kernel(const TriParams p) {
+template <typename T, int DC, int DO, bool CHUNKED>
+__global__ __launch_bounds__(256, (FastConfig<DC, DO, CHUNKED>::kMinWavesPerSimd)) void tri_xyt_z_fast_kernel(
+    const TriParams p) {
     // The body is compiled in the device pass only: hipcc's host pass silently
     // drops the launch stub of a kernel template whose body calls the LDS-DMA
     // builtin from inside a lambda, and the host needs nothing but the stub.
 #if defined(__HIP_DEVICE_COMPILE__)
-    using Cfg = FastConfig<DC, DO>;
+    using Cfg = FastConfig<DC, DO, CHUNKED>;
     using M = Mma<T>;
     using V8 = typename M::V8;
     constexpr int MW = Cfg::MW, BM = Cfg::BM, BN = Cfg::BN;
@@ -167,7 +173,7 @@ __global__ __launch_bounds__(256, (FastConfig<DC, DO>::kMinWavesPerSimd)) void t
     // Each workgroup takes two row tiles of one head, r and n_tiles-1-r: under a triangular
     // mask their work adds up to the same amount for every r, so all workgroups are equal.
     // (Chunked evaluation: one row tile per workgroup, all of equal work already.)
-    const bool chunked = p.state != nullptr;
+    constexpr bool chunked = CHUNKED;
     const bool single = chunked || p.single != 0;
     const int n_pairs = single ? p.n_tiles : (p.n_tiles + 1) >> 1;
     const int hl = slot / n_pairs, rank = slot - hl * n_pairs;
@@ -262,10 +268,12 @@ __global__ __launch_bounds__(256, (FastConfig<DC, DO>::kMinWavesPerSimd)) void t
     };
     auto next_slot = [](int off) { return off + STAGE == Cfg::NBUF * STAGE ? 0 : off + STAGE; };
     // Wait until tile `q` has landed, given that every tile up to q + NBUF - 3 has been issued:
-    // the loads of later tiles (at most one tile's worth with four slots) may stay in flight.
+    // the loads of the NBUF - 3 tiles after it may stay in flight (when all of them exist).
     auto wait_tile = [&](int q) {
-        if (Cfg::NBUF == 4 && q + 1 < n_seq)
-            wait_vm<Cfg::NT>();
+        constexpr int AHEAD = Cfg::NBUF > 3 ? Cfg::NBUF - 3 : 0;
+        static_assert(AHEAD * Cfg::NT < 64, "vmcnt is a 6-bit field");
+        if (AHEAD > 0 && q + AHEAD < n_seq)
+            wait_vm<AHEAD * Cfg::NT>();
         else
             wait_vm<0>();
     };
@@ -345,7 +353,7 @@ __global__ __launch_bounds__(256, (FastConfig<DC, DO>::kMinWavesPerSimd)) void t
     int prev_off = (Cfg::NBUF - 1) * STAGE, cur_off = 0, next_off = STAGE, issue_off = STAGE;
     const bool has_state = chunked && (upper ? tile + 1 < p.n_tiles : tile > 0);
     const T *st = has_state ? static_cast<const T *>(p.state) + ((int64_t)bh * p.n_tiles + tile) * (DO * DC) : nullptr;
-    if (chunked) {
+    if constexpr (chunked) {
         // everything this workgroup will ever read is requested at once: the rest of the diagonal
         // block's tiles and the running state (the kernel is latency-bound in this mode)
         static_for<1, BM / BN>([&](auto qq) { issue_tile(decltype(qq)::value, decltype(qq)::value * STAGE); });
@@ -368,10 +376,9 @@ __global__ __launch_bounds__(256, (FastConfig<DC, DO>::kMinWavesPerSimd)) void t
         __builtin_amdgcn_s_barrier();
         FLA_STAMP(1);
     } else {
-        if constexpr (Cfg::NBUF == 4) {
-            issue_tile(1, STAGE);
-            issue_off = 2 * STAGE;
-        }
+        // tiles 1 .. NBUF-3 before the first wait, tile NBUF-2 right after it
+        static_for<1, Cfg::NBUF - 2>([&](auto qq) { issue_tile(decltype(qq)::value, decltype(qq)::value * STAGE); });
+        issue_off = (Cfg::NBUF - 2) * STAGE;
         wait_tile(0);
         __builtin_amdgcn_s_barrier();  // tile 0 (and the X fragments) have landed
         FLA_STAMP(1);
@@ -566,7 +573,7 @@ __global__ __launch_bounds__(256, (FastConfig<DC, DO>::kMinWavesPerSimd)) void t
     {
         static_assert(BM / BN <= Cfg::NBUF, "the diagonal block must fit in the LDS ring");
         if (n_full > 0) __builtin_amdgcn_s_barrier();  // every wave is done with the last full tile
-        if (!chunked) {
+        if constexpr (!chunked) {
             issue_tile(q + Cfg::NBUF - 1, issue_off);  // the one tile not yet requested (if any)
             wait_vm<0>();
             __builtin_amdgcn_s_barrier();
@@ -703,9 +710,18 @@ inline bool fast_path_ok(const TriParams &p) {
     return n * p.xs_n * 2 <= kMaxFastExtent && n * p.ys_n * 2 <= kMaxFastExtent && n * p.zs_n * 2 <= kMaxFastExtent;
 }
 
+template <typename T, int DC, int DO, bool CHUNKED>
+hipError_t launch_tri_fast_variant(TriParams p, hipStream_t stream);
+
 template <typename T, int DC, int DO>
-hipError_t launch_tri_fast(TriParams p, hipStream_t stream) {
-    using Cfg = FastConfig<DC, DO>;
+hipError_t launch_tri_fast(const TriParams &p, hipStream_t stream) {
+    return p.state ? launch_tri_fast_variant<T, DC, DO, true>(p, stream)
+                   : launch_tri_fast_variant<T, DC, DO, false>(p, stream);
+}
+
+template <typename T, int DC, int DO, bool CHUNKED>
+hipError_t launch_tri_fast_variant(TriParams p, hipStream_t stream) {
+    using Cfg = FastConfig<DC, DO, CHUNKED>;
     if constexpr (!Cfg::kSupported) {
         return hipErrorNotSupported;
     } else {
@@ -713,11 +729,11 @@ hipError_t launch_tri_fast(TriParams p, hipStream_t stream) {
         // Pairs of row tiles make all workgroups equal; a problem with fewer pairs than the chip has
         // CUs (256) would leave CUs idle and runs as single tiles instead (measured 10-20 % faster
         // there, while at exactly one pair per CU the equal pairs still win).
-        p.single = (p.state == nullptr && (int64_t)p.BH * ((p.n_tiles + 1) / 2) < 256) ? 1 : 0;
-        const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * ((p.state || p.single) ? p.n_tiles : (p.n_tiles + 1) / 2);
+        p.single = (!CHUNKED && (int64_t)p.BH * ((p.n_tiles + 1) / 2) < 256) ? 1 : 0;
+        const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * ((CHUNKED || p.single) ? p.n_tiles : (p.n_tiles + 1) / 2);
         if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-        auto kern = tri_xyt_z_fast_kernel<T, DC, DO>;
-        const int smem = Cfg::SMEM_BYTES + (p.state && Cfg::kStateInLds ? Cfg::STATE_BYTES : 0);
+        auto kern = tri_xyt_z_fast_kernel<T, DC, DO, CHUNKED>;
+        const int smem = Cfg::SMEM_BYTES + (Cfg::kStateInLds ? Cfg::STATE_BYTES : 0);
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return e;
