@@ -14,13 +14,15 @@ region is exactly K steps between two synchronisations.
 
 Prints ONE JSON line.  ``value`` is causal-counted algorithmic TFLOP/s of the
 whole step, N^2 (4 D_qk + 3 D_v) per (b, h) (five products: S, dS, dV, dK, dQ
-in backward, two in forward).  ``roofline`` describes the one kernel every
-launch of the step runs (Out = mask(X Y^T) Z; forward is one launch, backward
-three): algorithmic FLOPs of one launch, N^2 (D_c + D_o) B H, over the average
-launch duration measured here with HIP events on the launch stream, against
-the dense bf16 MFMA peak.  ``cpu_baseline`` times the oracle's naive PyTorch
-formula on the host cores over a bounded sample (whole (b, h) slices at full N
-and D), in the same unit.
+in backward, two in forward).  ``roofline`` describes the dominant kernel.  All
+launches evaluate products Out = mask(X Y^T) Z of N^2 (D_c + D_o) B H algorithmic
+FLOPs each; forward is one such launch, and with equal head dims up to 128 the
+three backward products are ONE launch of the batched kernel, which is then the
+dominant one: its FLOPs (three products) over the duration of the backward-only
+region timed here with HIP events on the launch stream, against the dense bf16
+MFMA peak.  ``cpu_baseline`` times the oracle's naive PyTorch formula on the
+host cores over a bounded sample (whole (b, h) slices at full N and D), in the
+same unit.
 """
 
 from __future__ import annotations
@@ -192,18 +194,34 @@ def main() -> int:
     peak = PEAK_TFLOPS[dt_name]
     tflops = flops_step / (ms_step * 1e-3) / 1e12
 
-    # dominant (only) kernel: launches per step and algorithmic FLOPs per launch
-    # (a product whose output is wider than 128 columns with a <=64- or 256-wide contraction runs
-    # as two launches, one per 128-column half; flops_per_launch is then the mean over launches)
+    # The dominant kernel and its launches.  Every launch evaluates products Out = mask(X Y^T) Z of
+    # N^2 (D_c + D_o) B H algorithmic FLOPs each.  With equal padded widths up to 128 the three
+    # backward products go out as ONE launch of fla::tri_xyt_z_fast_batch_kernel (the dominant
+    # kernel: three quarters of the step); its duration is the backward-only region timed above.
+    # Otherwise every product is a launch of its own (two when an output wider than 128 columns
+    # meets a <=64- or 256-wide contraction: one per 128-column half) and the figures are means
+    # over the launches of a step.
     def n_launches(dc, dout):
         return 2 if dout > 128 and (dc <= 64 or dc > 128) else 1
 
-    launches = n_launches(w.d_qk, w.d_v)
-    if w.backward:
-        launches += n_launches(w.d_v, w.d_qk) * 2 + n_launches(w.d_qk, w.d_v)
-    products = 1 + (3 if w.backward else 0)
-    flops_launch = float(w.batch * w.heads) * w.seq * w.seq * (w.d_qk + w.d_v) * products / launches
-    ms_launch = ms_step / launches
+    def pad(d):
+        return 32 if d <= 32 else 64 if d <= 64 else 128 if d <= 128 else 256
+
+    flops_product = float(w.batch * w.heads) * w.seq * w.seq * (w.d_qk + w.d_v)
+    batched_bwd = w.backward and pad(w.d_qk) == pad(w.d_v) and pad(w.d_qk) <= 128
+    if batched_bwd:
+        launches = 2
+        kernel_name = "fla::tri_xyt_z_fast_batch_kernel (dQ, dV, dK: three products Out = mask(X Y^T) Z in one launch)"
+        flops_launch = 3.0 * flops_product
+        ms_launch = ms_bwd
+    else:
+        launches = n_launches(w.d_qk, w.d_v)
+        if w.backward:
+            launches += n_launches(w.d_v, w.d_qk) * 2 + n_launches(w.d_qk, w.d_v)
+        products = 1 + (3 if w.backward else 0)
+        kernel_name = "fla::tri_xyt_z_fast_kernel (Out = mask(X Y^T) Z)"
+        flops_launch = flops_product * products / launches
+        ms_launch = ms_step / launches
     achieved = flops_launch / (ms_launch * 1e-3) / 1e12
 
     result = {
@@ -234,12 +252,13 @@ def main() -> int:
         },
         "roofline": {
             "bound": "mfma",
-            "kernel": "fla::tri_xyt_z_kernel (Out = mask(X Y^T) Z)",
+            "kernel": kernel_name,
             "achieved": round(achieved, 2),
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": round(achieved / peak, 4),
             "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
+            "traffic_note": "HBM bytes per launch of the dominant kernel, rocprofv3 FETCH_SIZE/WRITE_SIZE (profiles/)",
             "launches_per_step": launches,
             "flops_per_launch": flops_launch,
             "avg_launch_ms": round(ms_launch, 4),
@@ -305,8 +324,11 @@ def main() -> int:
             recipe_step()
         ms_recipe = _time_region(torch, recipe_step, max(10, args.steps // 5)) / max(10, args.steps // 5)
         # the dominant kernel is still the product kernel: its per-launch figures come from the plain step
+        plain_flops = flops_product * (4 if w.backward else 1)
+        result["roofline"]["kernel"] = "fla::tri_xyt_z_fast_kernel / _batch_kernel (all product launches of the plain step)"
         result["roofline"]["avg_launch_ms"] = round(ms_plain / launches, 4)
-        result["roofline"]["achieved"] = round(flops_launch / (ms_plain / launches * 1e-3) / 1e12, 2)
+        result["roofline"]["flops_per_launch"] = plain_flops / launches
+        result["roofline"]["achieved"] = round(plain_flops / (ms_plain * 1e-3) / 1e12, 2)
         result["roofline"]["frac"] = round(result["roofline"]["achieved"] / peak, 4)
         result["metric"] = result["metric"].replace("causal linear attention", "normalised causal linear attention")
         result["config"]["workload"] += "; fused normaliser out / (q . cumsum(k) + 1e-5)"

@@ -76,21 +76,8 @@ int check_common(int64_t B, int64_t H, int64_t N, int dtype) {
     return FLA_OK;
 }
 
-// Out = mask(X Y^T) Z; all arguments already validated.
-int run_tri(const View &x, const View &y, const View &z, const View &out, int64_t B, int64_t H, int64_t N,
-            int64_t dc, int64_t dout, int upper, int dtype, void *stream) {
-    if (B == 0 || H == 0 || N == 0) return FLA_OK;
-    // Output wider than 128 columns with a narrow (<= 64) or a 256-wide contraction: run the two
-    // 128-column halves of Z / Out as separate launches.  The 64-rows-per-wave kernels that
-    // this selects beat the single 256-wide launch (which needs the 32-row layout, or the
-    // generic kernel for 256 x 256) although S is formed twice; results are bit-identical
-    // because every output column is an independent sum.
-    if (dout > 128 && (dc <= 64 || dc > 128)) {
-        const View z_hi{static_cast<const char *>(z.ptr) + 128 * 2, z.strides};
-        const View out_hi{static_cast<const char *>(out.ptr) + 128 * 2, out.strides};
-        if (int rc = run_tri(x, y, z, out, B, H, N, dc, 128, upper, dtype, stream)) return rc;
-        return run_tri(x, y, z_hi, out_hi, B, H, N, dc, dout - 128, upper, dtype, stream);
-    }
+TriParams make_params(const View &x, const View &y, const View &z, const View &out, int64_t B, int64_t H, int64_t N,
+                      int64_t dc, int64_t dout, int upper) {
     TriParams p;
     p.x = x.ptr, p.y = y.ptr, p.z = z.ptr, p.out = const_cast<void *>(out.ptr);
     p.xs_b = x.strides[0], p.xs_h = x.strides[1], p.xs_n = x.strides[2];
@@ -110,6 +97,35 @@ int run_tri(const View &x, const View &y, const View &z, const View &out, int64_
         p.dbg = e ? reinterpret_cast<unsigned long long *>(strtoull(e, nullptr, 16)) : nullptr;
     }
 #endif
+    return p;
+}
+
+typedef hipError_t (*batch_fn)(const fla::TriBatch &, int, hipStream_t);
+
+batch_fn lookup_batch(int dtype, int64_t d) {
+    static const batch_fn table[4][2] = {{fla::FLA_BATCH_NAME(0, 32), fla::FLA_BATCH_NAME(1, 32)},
+                                         {fla::FLA_BATCH_NAME(0, 64), fla::FLA_BATCH_NAME(1, 64)},
+                                         {fla::FLA_BATCH_NAME(0, 128), fla::FLA_BATCH_NAME(1, 128)},
+                                         {fla::FLA_BATCH_NAME(0, 256), fla::FLA_BATCH_NAME(1, 256)}};
+    return table[pad_index(d)][dtype];
+}
+
+// Out = mask(X Y^T) Z; all arguments already validated.
+int run_tri(const View &x, const View &y, const View &z, const View &out, int64_t B, int64_t H, int64_t N,
+            int64_t dc, int64_t dout, int upper, int dtype, void *stream) {
+    if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    // Output wider than 128 columns with a narrow (<= 64) or a 256-wide contraction: run the two
+    // 128-column halves of Z / Out as separate launches.  The 64-rows-per-wave kernels that
+    // this selects beat the single 256-wide launch (which needs the 32-row layout, or the
+    // generic kernel for 256 x 256) although S is formed twice; results are bit-identical
+    // because every output column is an independent sum.
+    if (dout > 128 && (dc <= 64 || dc > 128)) {
+        const View z_hi{static_cast<const char *>(z.ptr) + 128 * 2, z.strides};
+        const View out_hi{static_cast<const char *>(out.ptr) + 128 * 2, out.strides};
+        if (int rc = run_tri(x, y, z, out, B, H, N, dc, 128, upper, dtype, stream)) return rc;
+        return run_tri(x, y, z_hi, out_hi, B, H, N, dc, dout - 128, upper, dtype, stream);
+    }
+    const TriParams p = make_params(x, y, z, out, B, H, N, dc, dout, upper);
     launch_fn fn = lookup(dtype, dc, dout);
     if (!fn) return FLA_ERR_UNSUPPORTED;
     return fn(p, static_cast<hipStream_t>(stream)) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
@@ -193,15 +209,36 @@ int forward(const View &q, const View &k, const View &v, const View &o, int64_t 
     return run_tri(q, k, v, o, B, H, N, dqk, dv, 0, dtype, stream);
 }
 
+// The three gradient products for validated views.
+int backward_products(const View &go, const View &q, const View &k, const View &v, const View &dq, const View &dk,
+                      const View &dv, int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dvw, int dtype,
+                      void *stream) {
+    // dQ = lower(dO V^T) K ; dV = upper(K Q^T) dO ; dK = upper(V dO^T) Q
+    if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    // Equal padded widths up to 128: all three products run the same kernel, so they go out as
+    // one launch (workgroups of the next product fill the previous one's tail).
+    if (pad_index(dqk) == pad_index(dvw) && padded(dqk) <= 128) {
+        fla::TriBatch b;
+        b.p[0] = make_params(go, v, k, dq, B, H, N, dvw, dqk, 0);
+        b.p[1] = make_params(k, q, go, dv, B, H, N, dqk, dvw, 1);
+        b.p[2] = make_params(v, go, q, dk, B, H, N, dvw, dqk, 1);
+        if (fla::fast_path_ok(b.p[0]) && fla::fast_path_ok(b.p[1]) && fla::fast_path_ok(b.p[2])) {
+            const hipError_t e = lookup_batch(dtype, dqk)(b, 3, static_cast<hipStream_t>(stream));
+            if (e == hipSuccess) return FLA_OK;
+            if (e != hipErrorNotSupported) return FLA_ERR_LAUNCH;
+        }
+    }
+    if (int rc = run_tri(go, v, k, dq, B, H, N, dvw, dqk, 0, dtype, stream)) return rc;
+    if (int rc = run_tri(k, q, go, dv, B, H, N, dqk, dvw, 1, dtype, stream)) return rc;
+    return run_tri(v, go, q, dk, B, H, N, dvw, dqk, 1, dtype, stream);
+}
+
 int backward(const View &go, const View &q, const View &k, const View &v, const View &dq, const View &dk,
              const View &dv, int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dvw, int dtype, void *stream) {
     const View all[] = {go, q, k, v, dq, dk, dv};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
-    // dQ = lower(dO V^T) K ; dV = upper(K Q^T) dO ; dK = upper(V dO^T) Q
-    if (int rc = run_tri(go, v, k, dq, B, H, N, dvw, dqk, 0, dtype, stream)) return rc;
-    if (int rc = run_tri(k, q, go, dv, B, H, N, dqk, dvw, 1, dtype, stream)) return rc;
-    return run_tri(v, go, q, dk, B, H, N, dvw, dqk, 1, dtype, stream);
+    return backward_products(go, q, k, v, dq, dk, dv, B, H, N, dqk, dvw, dtype, stream);
 }
 
 // ---- normalised linear attention: out = tril(Q K^T) V / (q . cumsum(k) + eps)
@@ -305,9 +342,7 @@ int normalised_backward(const View &go, const View &q, const View &k, const View
     p.out = dO, p.os_b = do_strides[0], p.os_h = do_strides[1], p.os_n = do_strides[2], p.vec_out = vec_ok(dOv, dv);
     if (norm_launch(1, dtype, l.lpr, p, stream) != hipSuccess) return FLA_ERR_LAUNCH;
     // gradients of the unnormalised product
-    if (int rc = run_tri(dOv, v, k, dq, B, H, N, dv, dqk, 0, dtype, stream)) return rc;
-    if (int rc = run_tri(k, q, dOv, dvv, B, H, N, dqk, dv, 1, dtype, stream)) return rc;
-    if (int rc = run_tri(v, dOv, q, dk, B, H, N, dv, dqk, 1, dtype, stream)) return rc;
+    if (int rc = backward_products(dOv, q, k, v, dq, dk, dvv, B, H, N, dqk, dv, dtype, stream)) return rc;
     // the normaliser's own terms
     p.dq = const_cast<void *>(dq.ptr), p.dqs_b = dq.strides[0], p.dqs_h = dq.strides[1], p.dqs_n = dq.strides[2];
     p.dk = const_cast<void *>(dk.ptr), p.dks_b = dk.strides[0], p.dks_h = dk.strides[1], p.dks_n = dk.strides[2];

@@ -28,6 +28,13 @@ hipError_t FLA_STATE_NAME(FLA_INST_DTYPE, FLA_INST_DC, FLA_INST_DO)(const ChunkS
     return launch_chunk_state<InstT, FLA_INST_DC, FLA_INST_DO>(p, stream);
 }
 
+#if FLA_INST_DC == FLA_INST_DO
+hipError_t FLA_BATCH_NAME(FLA_INST_DTYPE, FLA_INST_DC)(const TriBatch &b, int count, hipStream_t stream) {
+    if (!FastConfig<FLA_INST_DC, FLA_INST_DO>::kSupported) return hipErrorNotSupported;
+    return launch_tri_fast_batch<InstT, FLA_INST_DC, FLA_INST_DO>(b, count, stream);
+}
+#endif
+
 #if FLA_INST_DTYPE == 0
 // rows per chunk of the chunked evaluation = row tile of the fast kernel (0: no fast kernel)
 #define FLA_CHUNK_ROWS_NAME_(dc, dout) fla_chunk_rows_c##dc##_o##dout

@@ -143,9 +143,9 @@ __device__ __forceinline__ int swizzle_z(int row) {
     else return (row & 3) << 1;  // the 4 rows of one transposing read land in 4 different 32-byte slots
 }
 
+// The work of one workgroup; `wg_index` is its index within one product's grid.
 template <typename T, int DC, int DO, bool CHUNKED>
-__global__ __launch_bounds__(256, (FastConfig<DC, DO, CHUNKED>::kMinWavesPerSimd)) void tri_xyt_z_fast_kernel(
-    const TriParams p) {
+__device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_index) {
     // The body is compiled in the device pass only: hipcc's host pass silently
     // drops the launch stub of a kernel template whose body calls the LDS-DMA
     // builtin from inside a lambda, and the host needs nothing but the stub.
@@ -169,7 +169,7 @@ __global__ __launch_bounds__(256, (FastConfig<DC, DO, CHUNKED>::kMinWavesPerSimd
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, g = lane >> 5, lam = lane & 15;
 
-    const int wg = blockIdx.x, xcd = wg & 7, slot = wg >> 3;
+    const int wg = wg_index, xcd = wg & 7, slot = wg >> 3;
     // Each workgroup takes two row tiles of one head, r and n_tiles-1-r: under a triangular
     // mask their work adds up to the same amount for every r, so all workgroups are equal.
     // (Chunked evaluation: one row tile per workgroup, all of equal work already.)
@@ -202,12 +202,18 @@ __global__ __launch_bounds__(256, (FastConfig<DC, DO, CHUNKED>::kMinWavesPerSimd
 #ifdef FLA_DBG_TIMING
 #define FLA_STAMP(k)                                                                                           \
     do {                                                                                                       \
-        if (p.dbg && tid == 0) p.dbg[(size_t)blockIdx.x * 16 + pass * 8 + (k)] = __builtin_readcyclecounter(); \
+        if (p.dbg && tid == 0) p.dbg[(size_t)wg_index * 16 + pass * 8 + (k)] = __builtin_readcyclecounter(); \
     } while (0)
 #else
 #define FLA_STAMP(k) \
     do {             \
     } while (0)
+#endif
+#ifdef FLA_DBG_TIMING
+    // slot 7: constant-rate (100 MHz) clock at workgroup start, hardware id in the top bits; slot 15: at the end
+    if (p.dbg && tid == 0)
+        p.dbg[(size_t)wg_index * 16 + 7] = (__builtin_amdgcn_s_memrealtime() & 0xffffffffffull) |
+                                             ((unsigned long long)__builtin_amdgcn_s_getreg(63492) << 40);
 #endif
     for (int pass = 0; pass < 2; ++pass) {
     FLA_STAMP(0);
@@ -696,9 +702,26 @@ __global__ __launch_bounds__(256, (FastConfig<DC, DO, CHUNKED>::kMinWavesPerSimd
     }
     FLA_STAMP(4);
     }  // pass
+#ifdef FLA_DBG_TIMING
+    if (p.dbg && tid == 0) p.dbg[(size_t)wg_index * 16 + 15] = __builtin_amdgcn_s_memrealtime() & 0xffffffffffull;
+#endif
 #else
     (void)p;
+    (void)wg_index;
 #endif
+}
+
+template <typename T, int DC, int DO, bool CHUNKED>
+__global__ __launch_bounds__(256, (FastConfig<DC, DO, CHUNKED>::kMinWavesPerSimd)) void tri_xyt_z_fast_kernel(
+    const TriParams p) {
+    tri_fast_body<T, DC, DO, CHUNKED>(p, blockIdx.x);
+}
+
+// grid y = product index
+template <typename T, int DC, int DO>
+__global__ __launch_bounds__(256, (FastConfig<DC, DO, false>::kMinWavesPerSimd)) void tri_xyt_z_fast_batch_kernel(
+    const TriBatch b) {
+    tri_fast_body<T, DC, DO, false>(b.p[blockIdx.y], blockIdx.x);
 }
 
 // True when the fast kernel can take this problem: every operand 16-byte
@@ -738,6 +761,27 @@ hipError_t launch_tri_fast_variant(TriParams p, hipStream_t stream) {
                                            hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return e;
         hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+        return hipGetLastError();
+    }
+}
+
+// `count` products of the same shape (same N, B H, instantiation) in one launch.
+template <typename T, int DC, int DO>
+hipError_t launch_tri_fast_batch(TriBatch b, int count, hipStream_t stream) {
+    using Cfg = FastConfig<DC, DO, false>;
+    if constexpr (!Cfg::kSupported) {
+        return hipErrorNotSupported;
+    } else {
+        const int n_tiles = (b.p[0].N + Cfg::BM - 1) / Cfg::BM;
+        const int single = (int64_t)b.p[0].BH * ((n_tiles + 1) / 2) < 256 ? 1 : 0;
+        for (int i = 0; i < count; ++i) b.p[i].n_tiles = n_tiles, b.p[i].single = single, b.p[i].state = nullptr;
+        const int64_t grid = (int64_t)8 * ((b.p[0].BH + 7) / 8) * (single ? n_tiles : (n_tiles + 1) / 2);
+        if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+        auto kern = tri_xyt_z_fast_batch_kernel<T, DC, DO>;
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM_BYTES);
+        if (e != hipSuccess) return e;
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid, (unsigned)count), dim3(256), Cfg::SMEM_BYTES, stream, b);
         return hipGetLastError();
     }
 }

@@ -59,6 +59,13 @@ struct TriParams {
 #endif
 };
 
+// Up to three products of identical shape in one launch (grid y selects the product): the
+// backward's dQ, dV and dK.  Workgroups of the next product fill the CUs the previous one's
+// tail leaves idle.
+struct TriBatch {
+    TriParams p[3];
+};
+
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
