@@ -145,7 +145,14 @@ def main() -> int:
     if args.algo == "chunked":
         from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
 
-        fwd, bwd = linear_attention_chunked_fwd, linear_attention_chunked_bwd
+        # as under autograd: forward hands its running state to backward
+        _, chunk_state = linear_attention_chunked_fwd(q, k, v, want_state=True)
+
+        def fwd(q_, k_, v_):
+            return linear_attention_chunked_fwd(q_, k_, v_, want_state=True)
+
+        def bwd(do_, q_, k_, v_):
+            return linear_attention_chunked_bwd(do_, q_, k_, v_, chunk_state)
     plain_fwd, plain_bwd = fwd, bwd
     if args.algo == "normalised":
         from flashy_linear_attention_amd.normalised import (
@@ -284,7 +291,7 @@ def main() -> int:
         gbs = bytes_step / (ms_step * 1e-3) / 1e9
         result["roofline"] = {
             "bound": "hbm",
-            "kernel": "chunk_state + chunk_scan + tri_xyt_z_fast (chunked) per product",
+            "kernel": "chunk_state + chunk_scan (two running states per step when shared, else one per product) + tri_xyt_z_fast (chunked) per product",
             "achieved": round(gbs, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",

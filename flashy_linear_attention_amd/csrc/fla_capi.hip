@@ -90,6 +90,7 @@ TriParams make_params(const View &x, const View &y, const View &z, const View &o
     p.n_tiles = 0;
     p.single = 0;
     p.state = nullptr;
+    p.state_transposed = 0;
     p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout), p.vec_out = vec_ok(out, dout);
 #ifdef FLA_DBG_TIMING
     {
@@ -141,6 +142,41 @@ int64_t chunked_bytes(int64_t B, int64_t H, int64_t N, int64_t dc, int64_t dout)
     return B * H * chunks * padded(dc) * padded(dout) * 6;
 }
 
+// ---- chunk-wise evaluation, in three steps per product:
+//   chunk_states: per-chunk Y_c^T Z_c in fp32, then the exclusive running sum over the chunks
+//                 before (lower) / after (upper) each chunk, rounded to the storage dtype;
+//   chunk_main:   diagonal blocks plus X_c . S_c, S_c taken as stored or transposed.
+
+// true when (x, y, z, out) of these widths can be evaluated chunk-wise: a fast kernel exists,
+// the operands qualify for it, and there is more than one chunk
+bool chunkable(const TriParams &p, int64_t dc, int64_t dout, int64_t N) {
+    const int rows = chunk_rows(dc, dout);
+    return rows != 0 && N > rows && fla::fast_path_ok(p);
+}
+
+int chunk_states(const View &y, const View &z, int64_t B, int64_t H, int64_t N, int64_t dc, int64_t dout, int upper,
+                 int dtype, float *w, void *state, void *stream) {
+    const int64_t rows = chunk_rows(dc, dout), chunks = (N + rows - 1) / rows, E = padded(dc) * padded(dout);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    fla::ChunkStateParams cp;
+    cp.y = y.ptr, cp.z = z.ptr, cp.w = w;
+    cp.ys_b = y.strides[0], cp.ys_h = y.strides[1], cp.ys_n = y.strides[2];
+    cp.zs_b = z.strides[0], cp.zs_h = z.strides[1], cp.zs_n = z.strides[2];
+    cp.H = (int32_t)H, cp.N = (int32_t)N, cp.BH = (int32_t)(B * H), cp.dc = (int32_t)dc, cp.dout = (int32_t)dout;
+    cp.n_chunks = (int32_t)chunks;
+    if (lookup_state(dtype, dc, dout)(cp, s) != hipSuccess) return FLA_ERR_LAUNCH;
+    const hipError_t e = dtype == FLA_DTYPE_BF16
+                             ? fla::launch_chunk_scan<__bf16>(w, state, B * H, (int)chunks, E, upper ? 1 : 0, s)
+                             : fla::launch_chunk_scan<_Float16>(w, state, B * H, (int)chunks, E, upper ? 1 : 0, s);
+    return e == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+}
+
+int chunk_main(TriParams p, int64_t dc, int64_t dout, int dtype, const void *state, int transposed, void *stream) {
+    p.state = state;
+    p.state_transposed = transposed;
+    return lookup(dtype, dc, dout)(p, static_cast<hipStream_t>(stream)) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+}
+
 // Out = mask(X Y^T) Z evaluated chunk-wise; same arguments as run_tri plus the workspace.
 // Falls back to the quadratic kernels when the operands do not qualify for the fast path
 // or the sequence is a single chunk.
@@ -156,49 +192,102 @@ int run_tri_chunked(const View &x, const View &y, const View &z, const View &out
         return run_tri_chunked(x, y, z_hi, out_hi, B, H, N, dc, dout - 128, upper, dtype, workspace, workspace_bytes,
                                stream);
     }
-    const int rows = chunk_rows(dc, dout);
-    TriParams p;
-    p.x = x.ptr, p.y = y.ptr, p.z = z.ptr, p.out = const_cast<void *>(out.ptr);
-    p.xs_b = x.strides[0], p.xs_h = x.strides[1], p.xs_n = x.strides[2];
-    p.ys_b = y.strides[0], p.ys_h = y.strides[1], p.ys_n = y.strides[2];
-    p.zs_b = z.strides[0], p.zs_h = z.strides[1], p.zs_n = z.strides[2];
-    p.os_b = out.strides[0], p.os_h = out.strides[1], p.os_n = out.strides[2];
-    p.H = (int32_t)H, p.N = (int32_t)N, p.BH = (int32_t)(B * H);
-    p.dc = (int32_t)dc, p.dout = (int32_t)dout;
-    p.upper = upper ? 1 : 0;
-    p.n_tiles = 0;
-    p.single = 0;
-    p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout), p.vec_out = vec_ok(out, dout);
-    p.state = nullptr;
-#ifdef FLA_DBG_TIMING
-    {
-        const char *e = getenv("FLA_DBG_TIMING_PTR");
-        p.dbg = e ? reinterpret_cast<unsigned long long *>(strtoull(e, nullptr, 16)) : nullptr;
-    }
-#endif
-    if (rows == 0 || N <= rows || !fla::fast_path_ok(p))
-        return run_tri(x, y, z, out, B, H, N, dc, dout, upper, dtype, stream);
-
-    const int64_t chunks = (N + rows - 1) / rows, E = padded(dc) * padded(dout), BH = B * H;
+    const TriParams p = make_params(x, y, z, out, B, H, N, dc, dout, upper);
+    if (!chunkable(p, dc, dout, N)) return run_tri(x, y, z, out, B, H, N, dc, dout, upper, dtype, stream);
+    const int64_t rows = chunk_rows(dc, dout), chunks = (N + rows - 1) / rows, E = padded(dc) * padded(dout);
+    const int64_t BH = B * H;
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < BH * chunks * E * 6)
         return FLA_ERR_WORKSPACE;
     float *w = static_cast<float *>(workspace);
     void *state = static_cast<char *>(workspace) + BH * chunks * E * 4;
-    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (int rc = chunk_states(y, z, B, H, N, dc, dout, upper, dtype, w, state, stream)) return rc;
+    return chunk_main(p, dc, dout, dtype, state, 0, stream);
+}
 
-    fla::ChunkStateParams cp;
-    cp.y = y.ptr, cp.z = z.ptr, cp.w = w;
-    cp.ys_b = p.ys_b, cp.ys_h = p.ys_h, cp.ys_n = p.ys_n;
-    cp.zs_b = p.zs_b, cp.zs_h = p.zs_h, cp.zs_n = p.zs_n;
-    cp.H = p.H, cp.N = p.N, cp.BH = p.BH, cp.dc = p.dc, cp.dout = p.dout;
-    cp.n_chunks = (int32_t)chunks;
-    if (lookup_state(dtype, dc, dout)(cp, s) != hipSuccess) return FLA_ERR_LAUNCH;
-    const hipError_t e = dtype == FLA_DTYPE_BF16
-                             ? fla::launch_chunk_scan<__bf16>(w, state, BH, (int)chunks, E, upper ? 1 : 0, s)
-                             : fla::launch_chunk_scan<_Float16>(w, state, BH, (int)chunks, E, upper ? 1 : 0, s);
-    if (e != hipSuccess) return FLA_ERR_LAUNCH;
-    p.state = state;
-    return lookup(dtype, dc, dout)(p, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+// ---- the whole operator chunk-wise, with running states shared between products.  With equal
+// padded head dims up to 128 all four products run the same square kernel, and
+//     state(dQ) = state(O)^T   (sum of K_c^T V_c over the chunks before)
+//     state(dK) = state(dV)^T  (sum of Q_c^T dO_c over the chunks after)
+// so forward can hand its state to backward, and backward computes one new state instead of
+// three.  Any other shape evaluates each product on its own.
+
+bool states_shareable(int64_t dqk, int64_t dv, int64_t N) {
+    if (pad_index(dqk) != pad_index(dv) || padded(dqk) > 128) return false;
+    const int rows = chunk_rows(dqk, dv);
+    return rows != 0 && N > rows;
+}
+
+// bytes of one rounded running state / of the scratch one state computation needs (fp32 chunk states)
+int64_t shared_state_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
+    if (!states_shareable(dqk, dv, N)) return 0;
+    const int64_t rows = chunk_rows(dqk, dv);
+    return B * H * ((N + rows - 1) / rows) * padded(dqk) * padded(dv) * 2;
+}
+
+int64_t chunked_op_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
+    const int64_t shared = shared_state_bytes(B, H, N, dqk, dv);
+    if (shared) return shared * 4;  // fp32 chunk states (2x) + two rounded states (backward without a saved one)
+    int64_t m = chunked_bytes(B, H, N, dqk, dv);
+    const int64_t t = chunked_bytes(B, H, N, dv, dqk);
+    return m > t ? m : t;
+}
+
+int chunked_forward(const View &q, const View &k, const View &v, const View &o, int64_t B, int64_t H, int64_t N,
+                    int64_t dqk, int64_t dv, int dtype, void *state_out, int32_t *state_valid, void *workspace,
+                    int64_t workspace_bytes, void *stream) {
+    if (state_valid) *state_valid = 0;
+    const View all[] = {q, k, v, o};
+    for (const View &t : all)
+        if (int rc = check_view(t)) return rc;
+    if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    const TriParams p = make_params(q, k, v, o, B, H, N, dqk, dv, 0);
+    if (!states_shareable(dqk, dv, N) || !fla::fast_path_ok(p))
+        return run_tri_chunked(q, k, v, o, B, H, N, dqk, dv, 0, dtype, workspace, workspace_bytes, stream);
+    const int64_t sb = shared_state_bytes(B, H, N, dqk, dv);
+    if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < sb * (state_out ? 2 : 3))
+        return FLA_ERR_WORKSPACE;
+    if (state_out && reinterpret_cast<uintptr_t>(state_out) % 16 != 0) return FLA_ERR_WORKSPACE;
+    float *w = static_cast<float *>(workspace);
+    void *state = state_out ? state_out : static_cast<char *>(workspace) + 2 * sb;
+    if (int rc = chunk_states(k, v, B, H, N, dqk, dv, 0, dtype, w, state, stream)) return rc;
+    if (int rc = chunk_main(p, dqk, dv, dtype, state, 0, stream)) return rc;
+    if (state_out && state_valid) *state_valid = 1;
+    return FLA_OK;
+}
+
+int chunked_backward(const View &go, const View &q, const View &k, const View &v, const View &dq, const View &dk,
+                     const View &dvv, int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv, int dtype,
+                     const void *state_in, void *workspace, int64_t workspace_bytes, void *stream) {
+    const View all[] = {go, q, k, v, dq, dk, dvv};
+    for (const View &t : all)
+        if (int rc = check_view(t)) return rc;
+    if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    const TriParams pq = make_params(go, v, k, dq, B, H, N, dv, dqk, 0);   // dQ = lower(dO V^T) K
+    const TriParams pv = make_params(k, q, go, dvv, B, H, N, dqk, dv, 1);  // dV = upper(K Q^T) dO
+    const TriParams pk = make_params(v, go, q, dk, B, H, N, dv, dqk, 1);   // dK = upper(V dO^T) Q
+    if (!states_shareable(dqk, dv, N) || !fla::fast_path_ok(pq) || !fla::fast_path_ok(pv) || !fla::fast_path_ok(pk)) {
+        if (int rc = run_tri_chunked(go, v, k, dq, B, H, N, dv, dqk, 0, dtype, workspace, workspace_bytes, stream))
+            return rc;
+        if (int rc = run_tri_chunked(k, q, go, dvv, B, H, N, dqk, dv, 1, dtype, workspace, workspace_bytes, stream))
+            return rc;
+        return run_tri_chunked(v, go, q, dk, B, H, N, dv, dqk, 1, dtype, workspace, workspace_bytes, stream);
+    }
+    const int64_t sb = shared_state_bytes(B, H, N, dqk, dv);
+    if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < sb * (state_in ? 3 : 4))
+        return FLA_ERR_WORKSPACE;
+    float *w = static_cast<float *>(workspace);
+    void *state_v = static_cast<char *>(workspace) + 2 * sb;
+    const void *state_f = state_in;
+    if (!state_f) {
+        void *mine = static_cast<char *>(workspace) + 3 * sb;
+        if (int rc = chunk_states(k, v, B, H, N, dqk, dv, 0, dtype, w, mine, stream)) return rc;
+        state_f = mine;
+    }
+    // dQ reads the forward state [D_v][D_qk] as its own [D_c = D_v][D_o = D_qk] transposed state
+    if (int rc = chunk_main(pq, dv, dqk, dtype, state_f, 1, stream)) return rc;
+    if (int rc = chunk_states(q, go, B, H, N, dqk, dv, 1, dtype, w, state_v, stream)) return rc;
+    if (int rc = chunk_main(pv, dqk, dv, dtype, state_v, 0, stream)) return rc;
+    return chunk_main(pk, dv, dqk, dtype, state_v, 1, stream);
 }
 
 int forward(const View &q, const View &k, const View &v, const View &o, int64_t B, int64_t H, int64_t N,
@@ -443,6 +532,42 @@ int fla_tri_xyt_z_chunked(const void *x, const void *y, const void *z, void *out
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
     return run_tri_chunked(vx, vy, vz, vo, B, H, N, D_c, D_o, upper, dtype, workspace, workspace_bytes, stream);
+}
+
+int64_t fla_linear_attn_chunked_state_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v) {
+    if (B < 0 || H < 0 || N < 0 || D_qk < 1 || D_qk > 256 || D_v < 1 || D_v > 256) return 0;
+    return shared_state_bytes(B, H, N, D_qk, D_v);
+}
+
+int64_t fla_linear_attn_chunked_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v) {
+    if (B < 0 || H < 0 || N < 0 || D_qk < 1 || D_qk > 256 || D_v < 1 || D_v > 256) return 0;
+    return chunked_op_workspace_bytes(B, H, N, D_qk, D_v);
+}
+
+int fla_linear_attn_chunked_fwd(const void *q, const void *k, const void *v, void *o, int64_t B, int64_t H, int64_t N,
+                                int64_t D_qk, int64_t D_v, const int64_t *q_strides, const int64_t *k_strides,
+                                const int64_t *v_strides, const int64_t *o_strides, int dtype, void *state_out,
+                                int32_t *state_valid, void *workspace, int64_t workspace_bytes, void *stream) {
+    if (state_valid) *state_valid = 0;
+    if (int rc = check_common(B, H, N, dtype)) return rc;
+    if (D_qk < 1 || D_qk > 256) return FLA_ERR_HEAD_DIM;
+    if (D_v < 1 || D_v > 256) return FLA_ERR_V_HEAD_DIM;
+    return chunked_forward({q, q_strides}, {k, k_strides}, {v, v_strides}, {o, o_strides}, B, H, N, D_qk, D_v, dtype,
+                           state_out, state_valid, workspace, workspace_bytes, stream);
+}
+
+int fla_linear_attn_chunked_bwd(const void *grad_out, const void *q, const void *k, const void *v, void *dq, void *dk,
+                                void *dv, int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                                const int64_t *go_strides, const int64_t *q_strides, const int64_t *k_strides,
+                                const int64_t *v_strides, const int64_t *dq_strides, const int64_t *dk_strides,
+                                const int64_t *dv_strides, int dtype, const void *state_in, void *workspace,
+                                int64_t workspace_bytes, void *stream) {
+    if (int rc = check_common(B, H, N, dtype)) return rc;
+    if (D_qk < 1 || D_qk > 256) return FLA_ERR_HEAD_DIM;
+    if (D_v < 1 || D_v > 256) return FLA_ERR_V_HEAD_DIM;
+    return chunked_backward({grad_out, go_strides}, {q, q_strides}, {k, k_strides}, {v, v_strides}, {dq, dq_strides},
+                            {dk, dk_strides}, {dv, dv_strides}, B, H, N, D_qk, D_v, dtype, state_in, workspace,
+                            workspace_bytes, stream);
 }
 
 int64_t fla_normalised_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v) {

@@ -119,6 +119,8 @@ struct FastConfig {
     // whole 64-row units of the Y tile layout when the 160 KiB allow it
     static constexpr int STATE_BYTES = ((DO + 63) / 64) * Y_BYTES;
     static constexpr bool kStateInLds = CHUNKED && SMEM_BYTES + STATE_BYTES <= 160 * 1024;
+    // the transposed state ([DC rows][DO], Z tile layout) is read only by square instantiations
+    static constexpr bool kStateTransposable = kStateInLds && DC == DO;
     // Narrow shapes need half the LDS and about half the registers: holding the kernel to 256
     // registers lets two workgroups share a CU, which hides each other's prologue and epilogue.
     static constexpr int kMinWavesPerSimd = (DC <= 64 && DO <= 64) ? 2 : 1;
@@ -366,16 +368,31 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         if constexpr (Cfg::kStateInLds) {
             if (has_state) {
                 const u32x4 rs = make_rsrc(st, DO * DC * 2);
-                const int row = wave * (1024 / RY) + lane / CY;
-                const uint32_t sdma = (uint32_t)(row * RY + (((lane % CY) ^ swizzle_y<CY>(row)) << 4));
-                static_for<0, Cfg::STATE_BYTES / Y_BYTES>([&](auto uu) {
-                    constexpr int UNIT = decltype(uu)::value;
-                    static_for<0, NIY>([&](auto u) {
-                        constexpr int U = decltype(u)::value;
-                        dma_16B_per_lane<Cfg::SMEM_BYTES + UNIT * Y_BYTES + U * 4096>(
-                            rs, lds_wave, sdma, (uint32_t)((UNIT * 64 + U * YSTEP) * RY));
+                if (Cfg::kStateTransposable && p.state_transposed) {
+                    // [DC rows][DO] in the Z tile layout
+                    const int row = wave * (1024 / RZ) + lane / CZ;
+                    const uint32_t tdma = (uint32_t)(row * RZ + (((lane % CZ) ^ swizzle_z<CZ>(row)) << 4));
+                    static_for<0, (DC + 63) / 64>([&](auto uu) {
+                        constexpr int UNIT = decltype(uu)::value;
+                        static_for<0, NIZ>([&](auto u) {
+                            constexpr int U = decltype(u)::value;
+                            dma_16B_per_lane<Cfg::SMEM_BYTES + UNIT * Cfg::Z_BYTES + U * 4096>(
+                                rs, lds_wave, tdma, (uint32_t)((UNIT * 64 + U * ZSTEP) * RZ));
+                        });
                     });
-                });
+                } else {
+                    // [DO rows][DC] in the Y tile layout
+                    const int row = wave * (1024 / RY) + lane / CY;
+                    const uint32_t sdma = (uint32_t)(row * RY + (((lane % CY) ^ swizzle_y<CY>(row)) << 4));
+                    static_for<0, Cfg::STATE_BYTES / Y_BYTES>([&](auto uu) {
+                        constexpr int UNIT = decltype(uu)::value;
+                        static_for<0, NIY>([&](auto u) {
+                            constexpr int U = decltype(u)::value;
+                            dma_16B_per_lane<Cfg::SMEM_BYTES + UNIT * Y_BYTES + U * 4096>(
+                                rs, lds_wave, sdma, (uint32_t)((UNIT * 64 + U * YSTEP) * RY));
+                        });
+                    });
+                }
             }
         }
         wait_vm<0>();
@@ -522,7 +539,41 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         const int e_lane = 16 * ((l32 >> 2) & 1) + 4 * (l32 >> 3) + (l32 & 3);
         // two column blocks of fragments in flight: the loads of block db+1 overlap the MFMAs of db
         V8 sf[2][KC];
-        if constexpr (Cfg::kStateInLds) {
+        if (Cfg::kStateTransposable && p.state_transposed) {
+            // From LDS, stored as S[d][e]: the fragment is a column read, eight consecutive rows d of
+            // one column e per lane, i.e. the transposing read of the Z fragments with rows
+            // 8g .. 8g+7 of each 16-row k chunk (the k order of the X fragments) and the same
+            // lane -> column assignment as the accumulators.
+            int tl[ZQ];
+            {
+                const int srow = 8 * g + (lam >> 2);
+                const int sz = swizzle_z<CZ>(srow);
+                const int zc = lam & 3, beta = (lane >> 4) & 1;
+#pragma unroll
+                for (int j = 0; j < ZQ; ++j) {
+                    tl[j] = Cfg::SMEM_BYTES + srow * RZ + (((4 * j + 2 * (zc & 1) + beta) ^ sz) << 4) + 8 * (zc >> 1);
+                    asm volatile("" : "+v"(tl[j]));  // computed here, not once per kernel
+                }
+            }
+            auto load_block = [&](int db, V8 (&dst)[KC]) {
+#pragma unroll
+                for (int kc = 0; kc < KC; ++kc) {
+                    const unsigned char *zp = smem + tl[db % ZQ] + (16 * kc * RZ + (db / ZQ) * (ZQ * 64));
+                    const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(zp));
+                    const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(zp + 4 * RZ));
+                    dst[kc] = __builtin_bit_cast(V8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+                }
+            };
+            load_block(0, sf[0]);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                if (db + 1 < DB) load_block(db + 1, sf[(db + 1) & 1]);
+#pragma unroll
+                for (int kc = 0; kc < KC; ++kc)
+#pragma unroll
+                    for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(sf[db & 1][kc], xf[ib][kc], acc[ib][db]);
+            }
+        } else if constexpr (Cfg::kStateInLds) {
             // from LDS, in the Y tile layout (row e, chunk index XOR swizzle(e))
             int sl[YQ];
             const int sw = swizzle_y<CY>(e_lane);
@@ -748,6 +799,7 @@ hipError_t launch_tri_fast_variant(TriParams p, hipStream_t stream) {
     if constexpr (!Cfg::kSupported) {
         return hipErrorNotSupported;
     } else {
+        if (CHUNKED && p.state_transposed && !Cfg::kStateTransposable) return hipErrorNotSupported;
         p.n_tiles = (p.N + Cfg::BM - 1) / Cfg::BM;
         // Pairs of row tiles make all workgroups equal; a problem with fewer pairs than the chip has
         // CUs (256) would leave CUs idle and runs as single tiles instead (measured 10-20 % faster

@@ -54,6 +54,9 @@ struct TriParams {
     // Y_c^T Z_c over the chunks before (lower) / after (upper) the tile, stored transposed as
     // state[(bh * n_tiles + tile)][DO][DC] with the padded DO, DC of the instantiation.
     const void *state;
+    // 1: `state` holds the transpose instead, [DC][DO] per (bh, tile) -- the running state of the
+    // product with Y and Z exchanged, shared rather than recomputed (square instantiations only)
+    int32_t state_transposed;
 #ifdef FLA_DBG_TIMING
     unsigned long long *dbg;      // 16 clock stamps per workgroup (experimental builds only)
 #endif

@@ -139,6 +139,37 @@ int fla_tri_xyt_z_chunked(const void *x, const void *y, const void *z, void *out
                           const int64_t *z_strides, const int64_t *out_strides,
                           int upper, int dtype, void *workspace, int64_t workspace_bytes, void *stream);
 
+/* The whole operator evaluated chunk-wise, forward and backward, with the running states
+ * shared between products: O and dQ use the same state (sum of K_c^T V_c over earlier chunks),
+ * dV and dK the same one (sum of Q_c^T dO_c over later chunks), so a forward + backward pair
+ * computes two states instead of four.  Sharing needs equal padded head dims (next of 32 / 64 /
+ * 128) up to 128, operands that meet the speed-path alignment rules and more than one chunk;
+ * every other case evaluates each product with fla_tri_xyt_z_chunked's method, same results.
+ *
+ * forward:  `state_out` (optional, fla_linear_attn_chunked_state_bytes() bytes, 16-byte aligned)
+ *           receives the rounded running state for a later backward call; *state_valid (host
+ *           memory, optional) is set to 1 when it was written, else 0.
+ * backward: `state_in` is that buffer or NULL (the state is then recomputed).
+ * `workspace`: fla_linear_attn_chunked_workspace_bytes() bytes of scratch, 16-byte aligned.
+ * No counterpart in the reference (quadratic kernels only, linear_attn_kernels.py:63, 166-171). */
+int64_t fla_linear_attn_chunked_state_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v);
+int64_t fla_linear_attn_chunked_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v);
+int fla_linear_attn_chunked_fwd(const void *q, const void *k, const void *v, void *o,
+                                int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                                const int64_t *q_strides, const int64_t *k_strides,
+                                const int64_t *v_strides, const int64_t *o_strides,
+                                int dtype, void *state_out, int32_t *state_valid,
+                                void *workspace, int64_t workspace_bytes, void *stream);
+int fla_linear_attn_chunked_bwd(const void *grad_out, const void *q, const void *k, const void *v,
+                                void *dq, void *dk, void *dv,
+                                int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                                const int64_t *go_strides, const int64_t *q_strides,
+                                const int64_t *k_strides, const int64_t *v_strides,
+                                const int64_t *dq_strides, const int64_t *dk_strides,
+                                const int64_t *dv_strides,
+                                int dtype, const void *state_in,
+                                void *workspace, int64_t workspace_bytes, void *stream);
+
 /* Normalised causal linear attention, the full operator a caller of the reference assembles
  * in PyTorch around LinearAttention.apply (README.md:27-30 of the reference):
  *

@@ -101,3 +101,52 @@ def test_chunked_workspace_errors(gpu_device):
     rc = lib.fla_tri_xyt_z_chunked(x.data_ptr(), x.data_ptr(), x.data_ptr(), out.data_ptr(), 1, 1, 1024, 64, 64,
                                    st, st, st, st, 0, 0, None, 0, None)
     assert rc == -9
+
+
+def test_chunked_backward_with_and_without_the_forward_state(gpu_device):
+    """Backward given the forward's running state, and backward that recomputes it, return the
+    same gradients bit for bit; shapes that cannot share a state report none."""
+    from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
+
+    q, k, v, dy = (t.to(gpu_device) for t in reference_style_inputs(2, 3, 1280, 128, 128, torch.bfloat16, seed=31))
+    out, state = linear_attention_chunked_fwd(q, k, v, want_state=True)
+    assert state is not None
+    plain = linear_attention_chunked_fwd(q, k, v)
+    assert torch.equal(out, plain)
+    with_state = linear_attention_chunked_bwd(dy, q, k, v, state)
+    without = linear_attention_chunked_bwd(dy, q, k, v, None)
+    for a, b in zip(with_state, without):
+        assert torch.equal(a, b)
+    want = naive.causal_dot_product_grads(q.float().cpu(), k.float().cpu(), v.float().cpu(), dy.float().cpu())
+    for name, got, w in zip(("dQ", "dK", "dV"), with_state, want):
+        assert_close(name, got, w)
+    # widths that differ after padding (small V), and a single chunk: no shared state
+    q2, k2, v2, _ = (t.to(gpu_device) for t in reference_style_inputs(1, 2, 1024, 256, 64, torch.bfloat16, seed=32))
+    assert linear_attention_chunked_fwd(q2, k2, v2, want_state=True)[1] is None
+    assert linear_attention_chunked_fwd(q[:, :, :256], k[:, :, :256], v[:, :, :256], want_state=True)[1] is None
+
+
+def test_chunked_operator_workspace_is_checked(gpu_device):
+    import ctypes
+
+    from flashy_linear_attention_amd import _lib
+
+    lib = _lib.load()
+    q, k, v, dy = (t.to(gpu_device) for t in reference_style_inputs(1, 2, 1024, 64, 64, torch.bfloat16, seed=2))
+    out = torch.empty_like(v)
+    st = _lib.strides_arg
+    stream = torch.cuda.current_stream().cuda_stream
+    need = lib.fla_linear_attn_chunked_workspace_bytes(1, 2, 1024, 64, 64)
+    sbytes = lib.fla_linear_attn_chunked_state_bytes(1, 2, 1024, 64, 64)
+    assert need > 0 and sbytes == 2 * 4 * 64 * 64 * 2
+    valid = ctypes.c_int32(7)
+    rc = lib.fla_linear_attn_chunked_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), 1, 2, 1024, 64, 64,
+                                         st(q), st(k), st(v), st(out), 0, None, ctypes.byref(valid), None, 0, stream)
+    assert rc == -9 and valid.value == 0
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    work = torch.empty(need, dtype=torch.uint8, device=gpu_device)
+    rc = lib.fla_linear_attn_chunked_bwd(dy.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), dq.data_ptr(),
+                                         dk.data_ptr(), dv.data_ptr(), 1, 2, 1024, 64, 64, st(dy), st(q), st(k), st(v),
+                                         st(dq), st(dk), st(dv), 0, None, work.data_ptr(), 3 * sbytes, stream)
+    assert rc == -9  # without a saved state the call needs room for four
+    torch.cuda.synchronize()
