@@ -57,11 +57,12 @@ def _parse():
     ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU oracle timing")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target seconds of CPU work for the baseline")
-    ap.add_argument("--algo", default="quadratic", choices=["quadratic", "chunked", "normalised"],
+    ap.add_argument("--algo", default="quadratic", choices=["quadratic", "chunked", "normalised", "normalised-chunked"],
                     help="quadratic: the tiled O(N^2 D) kernels the headline metric is defined on (default); "
                          "chunked: the O(N) chunk-state path, reported with its own FLOP count and an HBM roofline; "
                          "normalised: the quadratic kernels plus the fused normaliser (out / (q . cumsum(k) + eps)), "
-                         "with the normaliser's own time, bytes and the PyTorch recipe's time beside it")
+                         "with the normaliser's own time, bytes and the PyTorch recipe's time beside it; "
+                         "normalised-chunked: the same with the chunk-wise product")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain device copy of 256 MiB (a known-size reference for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -142,7 +143,9 @@ def main() -> int:
     q, k, v, do = (t.to(dev) for t in make_inputs(w, seed=0))
     fwd = linear_flash_wrapper_fwd_smallv_hd if w.small_v else linear_flash_wrapper_fwd
     bwd = linear_flash_wrapper_bwd_smallv_hd if w.small_v else linear_flash_wrapper_bwd
-    if args.algo == "chunked":
+    normalised = args.algo.startswith("normalised")
+    chunked = args.algo in ("chunked", "normalised-chunked")
+    if chunked:
         from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
 
         # as under autograd: forward hands its running state to backward
@@ -154,19 +157,19 @@ def main() -> int:
         def bwd(do_, q_, k_, v_):
             return linear_attention_chunked_bwd(do_, q_, k_, v_, chunk_state)
     plain_fwd, plain_bwd = fwd, bwd
-    if args.algo == "normalised":
+    if normalised:
         from flashy_linear_attention_amd.normalised import (
             linear_attention_normalised_bwd,
             linear_attention_normalised_fwd,
         )
 
-        norm_out, norm_denom = linear_attention_normalised_fwd(q, k, v, 1e-5)
+        norm_out, norm_denom = linear_attention_normalised_fwd(q, k, v, 1e-5, chunked)
 
         def fwd(q_, k_, v_):
-            return linear_attention_normalised_fwd(q_, k_, v_, 1e-5)
+            return linear_attention_normalised_fwd(q_, k_, v_, 1e-5, chunked)
 
         def bwd(do_, q_, k_, v_):
-            return linear_attention_normalised_bwd(do_, q_, k_, v_, norm_out, norm_denom)
+            return linear_attention_normalised_bwd(do_, q_, k_, v_, norm_out, norm_denom, chunked)
 
     def step():
         fwd(q, k, v)
@@ -271,7 +274,7 @@ def main() -> int:
             "avg_launch_ms": round(ms_launch, 4),
         },
     }
-    if args.algo == "chunked":
+    if chunked:
         # The chunked path does different (far less) arithmetic, so it is never priced in the
         # quadratic algorithm's FLOPs: its own count, and the HBM roofline that bounds it.
         chunk = 256 if (w.d_qk // 2 + w.d_v <= 192 and w.d_v // 2 + w.d_qk <= 192) else 128
@@ -299,7 +302,7 @@ def main() -> int:
             "traffic": None,
             "algorithmic_bytes_per_step": bytes_step,
         }
-    if args.algo == "normalised":
+    if normalised:
         # The product kernels are unchanged; what is new are the memory-bound passes around them.
         # Their time is the difference to the plain step in this same run, their algorithmic bytes:
         # forward reads q, k, O and writes out (+ n); backward reads g, out (pre-pass, writes dO) and
@@ -331,12 +334,14 @@ def main() -> int:
             recipe_step()
         ms_recipe = _time_region(torch, recipe_step, max(10, args.steps // 5)) / max(10, args.steps // 5)
         # the dominant kernel is still the product kernel: its per-launch figures come from the plain step
-        plain_flops = flops_product * (4 if w.backward else 1)
-        result["roofline"]["kernel"] = "fla::tri_xyt_z_fast_kernel / _batch_kernel (all product launches of the plain step)"
-        result["roofline"]["avg_launch_ms"] = round(ms_plain / launches, 4)
-        result["roofline"]["flops_per_launch"] = plain_flops / launches
-        result["roofline"]["achieved"] = round(plain_flops / (ms_plain * 1e-3) / 1e12, 2)
-        result["roofline"]["frac"] = round(result["roofline"]["achieved"] / peak, 4)
+        if not chunked:
+            plain_flops = flops_product * (4 if w.backward else 1)
+            result["roofline"]["kernel"] = ("fla::tri_xyt_z_fast_kernel / _batch_kernel "
+                                            "(all product launches of the plain step)")
+            result["roofline"]["avg_launch_ms"] = round(ms_plain / launches, 4)
+            result["roofline"]["flops_per_launch"] = plain_flops / launches
+            result["roofline"]["achieved"] = round(plain_flops / (ms_plain * 1e-3) / 1e12, 2)
+            result["roofline"]["frac"] = round(result["roofline"]["achieved"] / peak, 4)
         result["metric"] = result["metric"].replace("causal linear attention", "normalised causal linear attention")
         result["config"]["workload"] += "; fused normaliser out / (q . cumsum(k) + 1e-5)"
         result["config"]["normaliser"] = {

@@ -335,9 +335,11 @@ int backward(const View &go, const View &q, const View &k, const View &v, const 
 struct NormLayout {
     int lpr;
     int64_t chunks, sums_bytes, do_bytes, dn_bytes;
+    int64_t norm_bytes;   // the normaliser's own scratch: dO, dn, two sets of chunk sums
+    int64_t chunk_bytes;  // behind it: scratch of the chunk-wise product evaluation (0 when quadratic)
 };
 
-NormLayout norm_layout(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
+NormLayout norm_layout(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv, int chunked) {
     NormLayout l;
     l.lpr = fla::norm_lanes_per_row((int)(dqk > dv ? dqk : dv));
     const int64_t rows = fla::norm_chunk_rows(l.lpr);
@@ -345,6 +347,9 @@ NormLayout norm_layout(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv)
     l.sums_bytes = B * H * l.chunks * (l.lpr * 8) * 4;
     l.do_bytes = (B * H * N * dv * 2 + 15) / 16 * 16;
     l.dn_bytes = (B * H * N * 4 + 15) / 16 * 16;
+    l.sums_bytes = (l.sums_bytes + 15) / 16 * 16;
+    l.norm_bytes = l.do_bytes + l.dn_bytes + 2 * l.sums_bytes;
+    l.chunk_bytes = chunked ? chunked_op_workspace_bytes(B, H, N, dqk, dv) : 0;
     return l;
 }
 
@@ -379,17 +384,24 @@ int check_norm_args(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv, in
 }
 
 int normalised_forward(const View &q, const View &k, const View &v, const View &o, float *denom, int64_t B, int64_t H,
-                       int64_t N, int64_t dqk, int64_t dv, float eps, int dtype, void *workspace,
+                       int64_t N, int64_t dqk, int64_t dv, float eps, int dtype, int chunked, void *workspace,
                        int64_t workspace_bytes, void *stream) {
     const View all[] = {q, k, v, o};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
     if (!denom) return FLA_ERR_NULL_POINTER;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
-    const NormLayout l = norm_layout(B, H, N, dqk, dv);
-    if (l.chunks > 1 && (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < l.sums_bytes))
+    const NormLayout l = norm_layout(B, H, N, dqk, dv, chunked);
+    if ((l.chunks > 1 || l.chunk_bytes > 0) &&
+        (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < l.norm_bytes + l.chunk_bytes))
         return FLA_ERR_WORKSPACE;
-    if (int rc = run_tri(q, k, v, o, B, H, N, dqk, dv, 0, dtype, stream)) return rc;
+    if (chunked) {
+        if (int rc = chunked_forward(q, k, v, o, B, H, N, dqk, dv, dtype, nullptr, nullptr,
+                                     static_cast<char *>(workspace) + l.norm_bytes, l.chunk_bytes, stream))
+            return rc;
+    } else if (int rc = run_tri(q, k, v, o, B, H, N, dqk, dv, 0, dtype, stream)) {
+        return rc;
+    }
     fla::NormParams p;
     norm_common(p, q, k, B, H, N, dqk, dv, l);
     p.a = o.ptr, p.out = const_cast<void *>(o.ptr);  // normalised in place
@@ -403,16 +415,15 @@ int normalised_forward(const View &q, const View &k, const View &v, const View &
 
 int normalised_backward(const View &go, const View &q, const View &k, const View &v, const View &o,
                         const float *denom, const View &dq, const View &dk, const View &dvv, int64_t B, int64_t H,
-                        int64_t N, int64_t dqk, int64_t dv, int dtype, void *workspace, int64_t workspace_bytes,
-                        void *stream) {
+                        int64_t N, int64_t dqk, int64_t dv, int dtype, int chunked, void *workspace,
+                        int64_t workspace_bytes, void *stream) {
     const View all[] = {go, q, k, v, o, dq, dk, dvv};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
     if (!denom) return FLA_ERR_NULL_POINTER;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
-    const NormLayout l = norm_layout(B, H, N, dqk, dv);
-    if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 ||
-        workspace_bytes < l.do_bytes + l.dn_bytes + 2 * l.sums_bytes)
+    const NormLayout l = norm_layout(B, H, N, dqk, dv, chunked);
+    if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < l.norm_bytes + l.chunk_bytes)
         return FLA_ERR_WORKSPACE;
     char *ws = static_cast<char *>(workspace);
     void *dO = ws;
@@ -431,7 +442,13 @@ int normalised_backward(const View &go, const View &q, const View &k, const View
     p.out = dO, p.os_b = do_strides[0], p.os_h = do_strides[1], p.os_n = do_strides[2], p.vec_out = vec_ok(dOv, dv);
     if (norm_launch(1, dtype, l.lpr, p, stream) != hipSuccess) return FLA_ERR_LAUNCH;
     // gradients of the unnormalised product
-    if (int rc = backward_products(dOv, q, k, v, dq, dk, dvv, B, H, N, dqk, dv, dtype, stream)) return rc;
+    if (chunked) {
+        if (int rc = chunked_backward(dOv, q, k, v, dq, dk, dvv, B, H, N, dqk, dv, dtype, nullptr, ws + l.norm_bytes,
+                                      l.chunk_bytes, stream))
+            return rc;
+    } else if (int rc = backward_products(dOv, q, k, v, dq, dk, dvv, B, H, N, dqk, dv, dtype, stream)) {
+        return rc;
+    }
     // the normaliser's own terms
     p.dq = const_cast<void *>(dq.ptr), p.dqs_b = dq.strides[0], p.dqs_h = dq.strides[1], p.dqs_n = dq.strides[2];
     p.dk = const_cast<void *>(dk.ptr), p.dks_b = dk.strides[0], p.dks_h = dk.strides[1], p.dks_n = dk.strides[2];
@@ -570,19 +587,20 @@ int fla_linear_attn_chunked_bwd(const void *grad_out, const void *q, const void 
                             workspace_bytes, stream);
 }
 
-int64_t fla_normalised_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v) {
+int64_t fla_normalised_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v, int chunked) {
     if (B < 0 || H < 0 || N < 0 || D_qk < 1 || D_qk > 256 || D_v < 1 || D_v > 256) return 0;
-    const NormLayout l = norm_layout(B, H, N, D_qk, D_v);
-    return l.do_bytes + l.dn_bytes + 2 * l.sums_bytes;
+    const NormLayout l = norm_layout(B, H, N, D_qk, D_v, chunked);
+    return l.norm_bytes + l.chunk_bytes;
 }
 
 int fla_linear_attn_normalised_fwd(const void *q, const void *k, const void *v, void *o, float *denom, int64_t B,
                                    int64_t H, int64_t N, int64_t D_qk, int64_t D_v, const int64_t *q_strides,
                                    const int64_t *k_strides, const int64_t *v_strides, const int64_t *o_strides,
-                                   float eps, int dtype, void *workspace, int64_t workspace_bytes, void *stream) {
+                                   float eps, int dtype, int chunked, void *workspace, int64_t workspace_bytes,
+                                   void *stream) {
     if (int rc = check_norm_args(B, H, N, D_qk, D_v, dtype)) return rc;
     return normalised_forward({q, q_strides}, {k, k_strides}, {v, v_strides}, {o, o_strides}, denom, B, H, N, D_qk,
-                              D_v, eps, dtype, workspace, workspace_bytes, stream);
+                              D_v, eps, dtype, chunked, workspace, workspace_bytes, stream);
 }
 
 int fla_linear_attn_normalised_bwd(const void *grad_out, const void *q, const void *k, const void *v, const void *o,
@@ -590,12 +608,12 @@ int fla_linear_attn_normalised_bwd(const void *grad_out, const void *q, const vo
                                    int64_t N, int64_t D_qk, int64_t D_v, const int64_t *go_strides,
                                    const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
                                    const int64_t *o_strides, const int64_t *dq_strides, const int64_t *dk_strides,
-                                   const int64_t *dv_strides, int dtype, void *workspace, int64_t workspace_bytes,
-                                   void *stream) {
+                                   const int64_t *dv_strides, int dtype, int chunked, void *workspace,
+                                   int64_t workspace_bytes, void *stream) {
     if (int rc = check_norm_args(B, H, N, D_qk, D_v, dtype)) return rc;
     return normalised_backward({grad_out, go_strides}, {q, q_strides}, {k, k_strides}, {v, v_strides},
                                {o, o_strides}, denom, {dq, dq_strides}, {dk, dk_strides}, {dv, dv_strides}, B, H, N,
-                               D_qk, D_v, dtype, workspace, workspace_bytes, stream);
+                               D_qk, D_v, dtype, chunked, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"

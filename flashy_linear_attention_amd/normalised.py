@@ -3,7 +3,8 @@ normaliser to the caller, README.md:27-30 of the reference):
 
     out = LinearAttention.apply(q, k, v) / ((q * k.cumsum(-2)).sum(-1, keepdim=True) + eps)
 
-``LinearAttentionNormalised.apply(q, k, v, eps)`` returns the same tensor.  The product runs on
+``LinearAttentionNormalised.apply(q, k, v, eps, chunked=False)`` returns the same tensor
+(``chunked=True``: the product is evaluated chunk-wise, O(N), for long sequences).  The product runs on
 the kernels of ``LinearAttention``; the cumulative sum, the dot with q, eps and the division
 are one fused pass in fp32 (``fla_linear_attn_normalised_fwd``), and backward adds the
 normaliser's own gradient terms with two more fused passes instead of an autograd graph of
@@ -21,15 +22,17 @@ from . import _lib
 from .kernels._common import dtype_code, prepare, stream_handle
 
 
-def _workspace(lib, b: int, h: int, n: int, dqk: int, dv: int, device: torch.device) -> Tuple[torch.Tensor, int]:
-    nbytes = lib.fla_normalised_workspace_bytes(b, h, n, dqk, dv)
+def _workspace(lib, b: int, h: int, n: int, dqk: int, dv: int, chunked: bool,
+               device: torch.device) -> Tuple[torch.Tensor, int]:
+    nbytes = lib.fla_normalised_workspace_bytes(b, h, n, dqk, dv, int(chunked))
     return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device), nbytes
 
 
 def linear_attention_normalised_fwd(
-    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, eps: float = 1e-5
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, eps: float = 1e-5, chunked: bool = False
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    """(out, denom): the normalised output in the dtype of q and the fp32 normaliser (B, H, N)."""
+    """(out, denom): the normalised output in the dtype of q and the fp32 normaliser (B, H, N).
+    ``chunked`` evaluates the product chunk-wise (O(N)) instead of with the quadratic kernels."""
     assert q.shape == k.shape and v.shape[:3] == q.shape[:3], "q, k: (B,H,N,D_qk); v: (B,H,N,D_v)"
     assert q.shape[-1] <= 256 and v.shape[-1] <= 256, "Only head_dims <= 256 are supported."
     q, k, v = prepare(q, k, v)
@@ -39,13 +42,13 @@ def linear_attention_normalised_fwd(
     denom = torch.empty(b, h, n, dtype=torch.float32, device=q.device)
     lib = _lib.load()
     with torch.cuda.device(q.device):
-        work, nbytes = _workspace(lib, b, h, n, dqk, dv, q.device)
+        work, nbytes = _workspace(lib, b, h, n, dqk, dv, chunked, q.device)
         _lib.check(
             "fla_linear_attn_normalised_fwd",
             lib.fla_linear_attn_normalised_fwd(
                 q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), denom.data_ptr(), b, h, n, dqk, dv,
                 _lib.strides_arg(q), _lib.strides_arg(k), _lib.strides_arg(v), _lib.strides_arg(out),
-                float(eps), dtype_code(q), work.data_ptr(), nbytes, stream_handle(q.device),
+                float(eps), dtype_code(q), int(chunked), work.data_ptr(), nbytes, stream_handle(q.device),
             ),
         )
     return out, denom
@@ -53,7 +56,7 @@ def linear_attention_normalised_fwd(
 
 def linear_attention_normalised_bwd(
     grad_output: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor,
-    denom: torch.Tensor,
+    denom: torch.Tensor, chunked: bool = False,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """(dq, dk, dv) for d(out) = grad_output, given forward's ``out`` and ``denom``."""
     grad_output, q, k, v, out = prepare(grad_output, q, k, v, out)
@@ -65,7 +68,7 @@ def linear_attention_normalised_bwd(
     dvv = torch.empty_like(v, memory_format=torch.contiguous_format)
     lib = _lib.load()
     with torch.cuda.device(q.device):
-        work, nbytes = _workspace(lib, b, h, n, dqk, dv, q.device)
+        work, nbytes = _workspace(lib, b, h, n, dqk, dv, chunked, q.device)
         _lib.check(
             "fla_linear_attn_normalised_bwd",
             lib.fla_linear_attn_normalised_bwd(
@@ -73,7 +76,7 @@ def linear_attention_normalised_bwd(
                 dq.data_ptr(), dk.data_ptr(), dvv.data_ptr(), b, h, n, dqk, dv,
                 _lib.strides_arg(grad_output), _lib.strides_arg(q), _lib.strides_arg(k), _lib.strides_arg(v),
                 _lib.strides_arg(out), _lib.strides_arg(dq), _lib.strides_arg(dk), _lib.strides_arg(dvv),
-                dtype_code(q), work.data_ptr(), nbytes, stream_handle(q.device),
+                dtype_code(q), int(chunked), work.data_ptr(), nbytes, stream_handle(q.device),
             ),
         )
     return dq, dk, dvv
@@ -82,14 +85,16 @@ def linear_attention_normalised_bwd(
 class LinearAttentionNormalised(Function):
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.bfloat16)
-    def forward(ctx: Any, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, eps: float = 1e-5) -> torch.Tensor:
-        out, denom = linear_attention_normalised_fwd(q, k, v, eps)
+    def forward(ctx: Any, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, eps: float = 1e-5,
+                chunked: bool = False) -> torch.Tensor:
+        out, denom = linear_attention_normalised_fwd(q, k, v, eps, chunked)
         ctx.save_for_backward(q, k, v, out, denom)
+        ctx.chunked = chunked
         return out
 
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx: Any, grad_output: torch.Tensor):
         q, k, v, out, denom = ctx.saved_tensors
-        dq, dk, dv = linear_attention_normalised_bwd(grad_output, q, k, v, out, denom)
-        return dq, dk, dv, None
+        dq, dk, dv = linear_attention_normalised_bwd(grad_output, q, k, v, out, denom, ctx.chunked)
+        return dq, dk, dv, None, None

@@ -179,17 +179,19 @@ int fla_linear_attn_chunked_bwd(const void *grad_out, const void *q, const void 
  * dot with q, eps) and divides in place; `denom` receives n as fp32, contiguous (B, H, N), for
  * the backward call.  Backward takes d(out), the forward's `o` and `denom`, and returns the
  * gradients of q, k, v including the normaliser's own terms.  D_qk and D_v are independent
- * (1..256).  `workspace`: at least fla_normalised_workspace_bytes() bytes of 16-byte aligned
- * device memory, scratch, not needed by forward when N fits one chunk.  B*H must not exceed
- * 65535.  No counterpart in the reference's kernels; replaces the caller-side recipe and its
+ * (1..256).  `chunked` != 0 evaluates the products chunk-wise (fla_linear_attn_chunked_fwd/bwd's
+ * method) instead of with the quadratic kernels.  `workspace`: at least
+ * fla_normalised_workspace_bytes() bytes (same `chunked`) of 16-byte aligned device memory,
+ * scratch.  B*H must not exceed 65535.  No counterpart in the reference's kernels; replaces the caller-side recipe and its
  * autograd graph (a cumsum, two elementwise products, a row sum and a division, each a full
  * pass over memory, forward and backward). */
-int64_t fla_normalised_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v);
+int64_t fla_normalised_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v, int chunked);
 int fla_linear_attn_normalised_fwd(const void *q, const void *k, const void *v, void *o, float *denom,
                                    int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
                                    const int64_t *q_strides, const int64_t *k_strides,
                                    const int64_t *v_strides, const int64_t *o_strides,
-                                   float eps, int dtype, void *workspace, int64_t workspace_bytes, void *stream);
+                                   float eps, int dtype, int chunked,
+                                   void *workspace, int64_t workspace_bytes, void *stream);
 int fla_linear_attn_normalised_bwd(const void *grad_out, const void *q, const void *k, const void *v,
                                    const void *o, const float *denom, void *dq, void *dk, void *dv,
                                    int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
@@ -197,7 +199,8 @@ int fla_linear_attn_normalised_bwd(const void *grad_out, const void *q, const vo
                                    const int64_t *k_strides, const int64_t *v_strides,
                                    const int64_t *o_strides, const int64_t *dq_strides,
                                    const int64_t *dk_strides, const int64_t *dv_strides,
-                                   int dtype, void *workspace, int64_t workspace_bytes, void *stream);
+                                   int dtype, int chunked,
+                                   void *workspace, int64_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus
 }

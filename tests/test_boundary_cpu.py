@@ -85,19 +85,21 @@ def test_c_abi_validation_codes():
     assert t(P, P, P, P, 1, 2, 64, 32, 32, S, S, S, S, 1, 5, None) == -2
     nf = lib.fla_linear_attn_normalised_fwd
     eps = ctypes.c_float(1e-5)
-    assert nf(P, P, P, P, P, 1, 2, 64, 32, 32, S, S, S, S, eps, 9, None, 0, None) == -2
-    assert nf(P, P, P, P, P, 1, 2, 64, 257, 32, S, S, S, S, eps, 0, None, 0, None) == -3
-    assert nf(P, P, P, P, P, 1, 2, 64, 32, 0, S, S, S, S, eps, 0, None, 0, None) == -4
-    assert nf(P, P, P, P, P, 300, 300, 64, 32, 32, S, S, S, S, eps, 0, None, 0, None) == -5   # B H > 65535
-    assert nf(P, P, P, P, None, 1, 2, 64, 32, 32, S, S, S, S, eps, 0, None, 0, None) == -1    # denom
-    assert nf(P, P, P, P, P, 1, 2, 64, 32, 32, S, S, BAD_S, S, eps, 0, None, 0, None) == -6
-    assert nf(P, P, P, P, P, 1, 2, 4096, 32, 32, S, S, S, S, eps, 0, None, 0, None) == -9     # chunk sums need workspace
-    assert nf(P, P, P, P, P, 1, 0, 64, 32, 32, S, S, S, S, eps, 0, None, 0, None) == 0
+    assert nf(P, P, P, P, P, 1, 2, 64, 32, 32, S, S, S, S, eps, 9, 0, None, 0, None) == -2
+    assert nf(P, P, P, P, P, 1, 2, 64, 257, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -3
+    assert nf(P, P, P, P, P, 1, 2, 64, 32, 0, S, S, S, S, eps, 0, 0, None, 0, None) == -4
+    assert nf(P, P, P, P, P, 300, 300, 64, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -5   # B H > 65535
+    assert nf(P, P, P, P, None, 1, 2, 64, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -1    # denom
+    assert nf(P, P, P, P, P, 1, 2, 64, 32, 32, S, S, BAD_S, S, eps, 0, 0, None, 0, None) == -6
+    assert nf(P, P, P, P, P, 1, 2, 4096, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -9     # chunk sums need workspace
+    assert nf(P, P, P, P, P, 1, 0, 64, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == 0
     nb = lib.fla_linear_attn_normalised_bwd
-    assert nb(P, P, P, P, P, P, P, P, P, 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, None, 0, None) == -9
-    assert nb(P, P, P, P, P, None, P, P, P, 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, P, 1 << 30, None) == -1
-    assert lib.fla_normalised_workspace_bytes(1, 2, 64, 32, 32) >= 2 * 64 * 32 * 2 + 2 * 64 * 4
-    assert lib.fla_normalised_workspace_bytes(1, 2, 64, 300, 32) == 0
+    assert nb(P, P, P, P, P, P, P, P, P, 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, 0, None, 0, None) == -9
+    assert nb(P, P, P, P, P, None, P, P, P, 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, 1, P, 1 << 30, None) == -1
+    assert lib.fla_normalised_workspace_bytes(1, 2, 64, 32, 32, 0) >= 2 * 64 * 32 * 2 + 2 * 64 * 4
+    assert lib.fla_normalised_workspace_bytes(1, 2, 64, 300, 32, 0) == 0
+    assert (lib.fla_normalised_workspace_bytes(1, 2, 4096, 64, 64, 1)
+            > lib.fla_normalised_workspace_bytes(1, 2, 4096, 64, 64, 0))
     for code in range(0, -10, -1):
         assert lib.fla_strerror(code)
     assert lib.fla_strerror(-3) == b"Only head_dims <= 256 are supported."

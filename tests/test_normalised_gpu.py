@@ -154,17 +154,33 @@ def test_normalised_workspace_is_checked(gpu_device):
     denom = torch.empty(1, 2, 1024, dtype=torch.float32, device=gpu_device)
     st = _lib.strides_arg
     stream = torch.cuda.current_stream().cuda_stream
-    need = lib.fla_normalised_workspace_bytes(1, 2, 1024, 64, 64)
+    need = lib.fla_normalised_workspace_bytes(1, 2, 1024, 64, 64, 0)
     assert need > 0
     rc = lib.fla_linear_attn_normalised_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                             denom.data_ptr(), 1, 2, 1024, 64, 64, st(q), st(k), st(v), st(out),
-                                            ctypes.c_float(1e-5), 0, None, 0, stream)
+                                            ctypes.c_float(1e-5), 0, 0, None, 0, stream)
     assert rc == -9  # FLA_ERR_WORKSPACE: several chunks need the chunk sums
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     work = torch.empty(need, dtype=torch.uint8, device=gpu_device)
     rc = lib.fla_linear_attn_normalised_bwd(dy.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                             denom.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
                                             1, 2, 1024, 64, 64, st(dy), st(q), st(k), st(v), st(out), st(dq), st(dk),
-                                            st(dv), 0, work.data_ptr(), need - 1, stream)
+                                            st(dv), 0, 0, work.data_ptr(), need - 1, stream)
     assert rc == -9
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dims", [(2, 2, 1536, 128, 128), (1, 2, 2304, 64, 64), (1, 2, 1024, 256, 64), (1, 1, 256, 64, 64)],
+                         ids=lambda d: "x".join(map(str, d)))
+def test_normalised_with_chunkwise_product(dims, gpu_device):
+    """chunked=True: the product goes through the chunk states, the normaliser passes are the
+    same; parity against the oracle as for the quadratic product."""
+    bs, nh, sq, dqk, dv = dims
+    q, k, v, dy = reference_style_inputs(bs, nh, sq, dqk, dv, torch.bfloat16, seed=sum(dims) + 1)
+    want_o, _, want_dq, want_dk, want_dv = _oracle(q, k, v, dy, 1e-5)
+    qg, kg, vg = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v))
+    out = LinearAttentionNormalised.apply(qg, kg, vg, 1e-5, True)
+    out.backward(dy.to(gpu_device))
+    assert_close("out", out, want_o)
+    for name, got, want in (("dQ", qg.grad, want_dq), ("dK", kg.grad, want_dk), ("dV", vg.grad, want_dv)):
+        assert_close(name, got, want, tol_fro=1e-2, tol_max=5e-2)
