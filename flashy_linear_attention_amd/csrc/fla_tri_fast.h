@@ -6,8 +6,8 @@
 // pipelined:
 //
 //   * Y/Z tiles (BN = 64 rows) go HBM -> LDS with buffer_load_dwordx4 ... lds
-//     (no staging registers, no ds_write), into a ring of three LDS buffers.
-//     One wave instruction fills 1 KiB of LDS in lane order, so the bank
+//     (no staging registers, no ds_write), into a ring of three to five LDS
+//     slots.  One wave instruction fills 1 KiB of LDS in lane order, so the bank
 //     spreading that padding would give is done by an XOR swizzle of the
 //     16-byte chunk index instead: a lane fetches the global chunk that belongs
 //     at its LDS slot.  Rows beyond N and chunks beyond the real width are
@@ -20,9 +20,13 @@
 //     its MFMA and the two MFMA chains of a phase are independent.
 //     One barrier per tile, placed between the phases of the tile's second
 //     sub-tile: it publishes the next tile and retires the previous one.
-//   * The BM x BM block on the diagonal is handled afterwards by a plain
-//     S -> mask -> P -> PV sequence per sub-tile that skips the (block, sub-tile)
-//     pairs the mask removes entirely.
+//   * The BM x BM block on the diagonal is handled afterwards, with all of its
+//     tiles resident, by a barrier-free S -> mask -> P -> PV sequence per sub-tile
+//     that skips the (block, sub-tile) pairs the mask removes entirely.
+//   * Variants of the same body: the plain kernel (one product), the batched
+//     kernel (grid y selects one of up to three products: the backward's dQ, dV,
+//     dK in one launch) and the chunked kernel (CHUNKED: diagonal block plus
+//     the running state of the chunk-wise evaluation, no tile ring).
 #pragma once
 
 #include <hip/hip_runtime.h>
