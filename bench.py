@@ -303,9 +303,9 @@ def main() -> int:
             "algorithmic_bytes_per_step": bytes_step,
         }
     if normalised:
-        # The product kernels are unchanged; what is new are the memory-bound passes around them.
-        # Their time is the difference to the plain step in this same run, their algorithmic bytes:
-        # forward reads q, k, O and writes out (+ n); backward reads g, out (pre-pass, writes dO) and
+        # What is new are the memory-bound passes around the product kernels.  Their time is the
+        # difference to the plain step in this same run, their algorithmic bytes: forward (separate pass)
+        # reads q, k, O and writes out (+ n); backward reads g, out (pre-pass, writes dO) and
         # q, k, dq, dk (post-pass, writes dq, dk); 2 bytes per element, fp32 vectors of length N aside.
         def plain_step():
             plain_fwd(q, k, v)
@@ -313,8 +313,10 @@ def main() -> int:
                 plain_bwd(do, q, k, v)
 
         ms_plain = _time_region(torch, plain_step, args.steps) / args.steps
+        # (with the quadratic product the forward normaliser lives inside the product kernel -- row sums
+        # of the scores -- and moves no extra bytes; only the chunk-wise product needs the forward pass)
         e = float(w.batch * w.heads * w.seq)
-        nbytes = 2.0 * e * (2 * w.d_qk + 2 * w.d_v)
+        nbytes = 2.0 * e * (2 * w.d_qk + 2 * w.d_v) if chunked else 4.0 * e
         if w.backward:
             nbytes += 2.0 * e * (3 * w.d_v + 6 * w.d_qk)
         extra_ms = ms_step - ms_plain

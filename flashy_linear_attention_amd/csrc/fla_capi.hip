@@ -91,6 +91,8 @@ TriParams make_params(const View &x, const View &y, const View &z, const View &o
     p.single = 0;
     p.state = nullptr;
     p.state_transposed = 0;
+    p.denom = nullptr;
+    p.eps = 0.f;
     p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout), p.vec_out = vec_ok(out, dout);
 #ifdef FLA_DBG_TIMING
     {
@@ -383,6 +385,27 @@ int check_norm_args(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv, in
     return FLA_OK;
 }
 
+// Forward with the normaliser inside the product kernel: the row sums of the masked scores are
+// the normaliser (q_i . sum_{j<=i} k_j = sum_j q_i . k_j), so the fast kernel divides before it
+// stores and no extra pass runs.  Returns 1 when this shape / layout has no such kernel (the
+// caller then normalises with the separate passes), 0 on success, a negative code on failure.
+int fused_normalised_forward(const View &q, const View &k, const View &v, const View &o, float *denom, int64_t B,
+                             int64_t H, int64_t N, int64_t dqk, int64_t dv, float eps, int dtype, void *stream) {
+    const bool split = dv > 128 && (dqk <= 64 || dqk > 128);
+    const int64_t w0 = split ? 128 : dv;
+    TriParams p0 = make_params(q, k, v, o, B, H, N, dqk, w0, 0);
+    if (chunk_rows(dqk, w0) == 0 || !fla::fast_path_ok(p0)) return 1;
+    p0.denom = denom, p0.eps = eps;
+    if (!split) return lookup(dtype, dqk, w0)(p0, static_cast<hipStream_t>(stream)) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+    const View v_hi{static_cast<const char *>(v.ptr) + 128 * 2, v.strides};
+    const View o_hi{static_cast<const char *>(o.ptr) + 128 * 2, o.strides};
+    TriParams p1 = make_params(q, k, v_hi, o_hi, B, H, N, dqk, dv - 128, 0);
+    if (chunk_rows(dqk, dv - 128) == 0 || !fla::fast_path_ok(p1)) return 1;
+    p1.denom = denom, p1.eps = eps;  // both halves see the same scores and write the same n
+    if (lookup(dtype, dqk, w0)(p0, static_cast<hipStream_t>(stream)) != hipSuccess) return FLA_ERR_LAUNCH;
+    return lookup(dtype, dqk, dv - 128)(p1, static_cast<hipStream_t>(stream)) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+}
+
 int normalised_forward(const View &q, const View &k, const View &v, const View &o, float *denom, int64_t B, int64_t H,
                        int64_t N, int64_t dqk, int64_t dv, float eps, int dtype, int chunked, void *workspace,
                        int64_t workspace_bytes, void *stream) {
@@ -395,6 +418,10 @@ int normalised_forward(const View &q, const View &k, const View &v, const View &
     if ((l.chunks > 1 || l.chunk_bytes > 0) &&
         (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < l.norm_bytes + l.chunk_bytes))
         return FLA_ERR_WORKSPACE;
+    if (!chunked) {
+        const int rc = fused_normalised_forward(q, k, v, o, denom, B, H, N, dqk, dv, eps, dtype, stream);
+        if (rc <= 0) return rc;
+    }
     if (chunked) {
         if (int rc = chunked_forward(q, k, v, o, B, H, N, dqk, dv, dtype, nullptr, nullptr,
                                      static_cast<char *>(workspace) + l.norm_bytes, l.chunk_bytes, stream))

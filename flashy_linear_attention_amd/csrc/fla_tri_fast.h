@@ -150,8 +150,9 @@ __device__ __forceinline__ int swizzle_z(int row) {
 }
 
 // The work of one workgroup; `wg_index` is its index within one product's grid.
-template <typename T, int DC, int DO, bool CHUNKED>
+template <typename T, int DC, int DO, bool CHUNKED, bool NORM = false>
 __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_index) {
+    static_assert(!(CHUNKED && NORM), "the in-kernel normaliser belongs to the quadratic walk");
     // The body is compiled in the device pass only: hipcc's host pass silently
     // drops the launch stub of a kernel template whose body calls the LDS-DMA
     // builtin from inside a lambda, and the host needs nothing but the stub.
@@ -312,6 +313,16 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         for (int db = 0; db < DB; ++db)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[ib][db][v] = 0.f;
+    // NORM: running sum of this lane's masked scores per row block (row l32, the 16 key rows of
+    // every sub-tile that fall to this half-wave); the two halves are added in the epilogue
+    float rsum[NIB];
+#pragma unroll
+    for (int ib = 0; ib < NIB; ++ib) rsum[ib] = 0.f;
+    auto add_scores = [&](const f32x16 &sc, float &dst) {
+        float t0 = (sc[0] + sc[1]) + (sc[2] + sc[3]), t1 = (sc[4] + sc[5]) + (sc[6] + sc[7]);
+        float t2 = (sc[8] + sc[9]) + (sc[10] + sc[11]), t3 = (sc[12] + sc[13]) + (sc[14] + sc[15]);
+        dst += (t0 + t1) + (t2 + t3);
+    };
 
     // ---- LDS read offsets inside a stage.  Only the chunk bits the swizzle touches need a
     // register; the rest of (sub-tile, kc / t, db) is an immediate offset of the DS instruction.
@@ -475,6 +486,12 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
                 for (int kc = 0; kc < KC; ++kc)
                     if (kc * NZF / KC == f) asm volatile("" : "+v"(yf[kc]));
 #endif
+                if constexpr (NORM) {
+                    if (f == NZF / 2) {
+#pragma unroll
+                        for (int ib = 0; ib < NIB; ++ib) add_scores(s[ib], rsum[ib]);
+                    }
+                }
                 // S of this sub-tile is complete once a couple of the independent MFMAs above have
                 // issued; its rounding is spread over the second half of the phase
 #pragma unroll
@@ -688,6 +705,7 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
                         sd[ib][v] = keep ? sd[ib][v] : 0.f;
                     }
                 }
+                if constexpr (NORM) add_scores(sd[ib], rsum[ib]);
                 V8 pf[2];
 #pragma unroll
                 for (int t = 0; t < 2; ++t)
@@ -726,6 +744,19 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     // Out[row l32 of block ib][column 32 db + 16 g + v]: 16 consecutive columns per lane.
     // They go to LDS as two 16-byte writes (the ring is idle: every wave has passed the last
     // barrier of the walk), and the tile leaves as whole rows, 16 bytes per lane.
+    if constexpr (NORM) {
+#pragma unroll
+        for (int ib = 0; ib < NIB; ++ib) {
+            const float n = rsum[ib] + __shfl_xor(rsum[ib], 32, 64) + p.eps;
+            const float inv = 1.0f / n;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[ib][db][v] *= inv;
+            const int row = i0 + blk[ib] * 32 + l32;
+            if (g == 0 && row < N) p.denom[(int64_t)bh * N + row] = n;
+        }
+    }
     {
         constexpr int RO = Cfg::RO;
 #pragma unroll
@@ -766,10 +797,10 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
 #endif
 }
 
-template <typename T, int DC, int DO, bool CHUNKED>
+template <typename T, int DC, int DO, bool CHUNKED, bool NORM>
 __global__ __launch_bounds__(256, (FastConfig<DC, DO, CHUNKED>::kMinWavesPerSimd)) void tri_xyt_z_fast_kernel(
     const TriParams p) {
-    tri_fast_body<T, DC, DO, CHUNKED>(p, blockIdx.x);
+    tri_fast_body<T, DC, DO, CHUNKED, NORM>(p, blockIdx.x);
 }
 
 // grid y = product index
@@ -788,16 +819,17 @@ inline bool fast_path_ok(const TriParams &p) {
     return n * p.xs_n * 2 <= kMaxFastExtent && n * p.ys_n * 2 <= kMaxFastExtent && n * p.zs_n * 2 <= kMaxFastExtent;
 }
 
-template <typename T, int DC, int DO, bool CHUNKED>
+template <typename T, int DC, int DO, bool CHUNKED, bool NORM>
 hipError_t launch_tri_fast_variant(TriParams p, hipStream_t stream);
 
 template <typename T, int DC, int DO>
 hipError_t launch_tri_fast(const TriParams &p, hipStream_t stream) {
-    return p.state ? launch_tri_fast_variant<T, DC, DO, true>(p, stream)
-                   : launch_tri_fast_variant<T, DC, DO, false>(p, stream);
+    if (p.state) return p.denom ? hipErrorNotSupported : launch_tri_fast_variant<T, DC, DO, true, false>(p, stream);
+    return p.denom ? launch_tri_fast_variant<T, DC, DO, false, true>(p, stream)
+                   : launch_tri_fast_variant<T, DC, DO, false, false>(p, stream);
 }
 
-template <typename T, int DC, int DO, bool CHUNKED>
+template <typename T, int DC, int DO, bool CHUNKED, bool NORM>
 hipError_t launch_tri_fast_variant(TriParams p, hipStream_t stream) {
     using Cfg = FastConfig<DC, DO, CHUNKED>;
     if constexpr (!Cfg::kSupported) {
@@ -811,7 +843,7 @@ hipError_t launch_tri_fast_variant(TriParams p, hipStream_t stream) {
         p.single = (!CHUNKED && (int64_t)p.BH * ((p.n_tiles + 1) / 2) < 256) ? 1 : 0;
         const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * ((CHUNKED || p.single) ? p.n_tiles : (p.n_tiles + 1) / 2);
         if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-        auto kern = tri_xyt_z_fast_kernel<T, DC, DO, CHUNKED>;
+        auto kern = tri_xyt_z_fast_kernel<T, DC, DO, CHUNKED, NORM>;
         const int smem = Cfg::SMEM_BYTES + (Cfg::kStateInLds ? Cfg::STATE_BYTES : 0);
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, smem);

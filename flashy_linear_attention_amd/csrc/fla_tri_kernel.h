@@ -57,6 +57,11 @@ struct TriParams {
     // 1: `state` holds the transpose instead, [DC][DO] per (bh, tile) -- the running state of the
     // product with Y and Z exchanged, shared rather than recomputed (square instantiations only)
     int32_t state_transposed;
+    // Normalised output (quadratic fast path only): when non-null, each row of Out is divided by
+    // n = (sum of its masked scores, in fp32 before rounding) + eps, and n is written here as
+    // fp32, contiguous (B H, N).
+    float *denom;
+    float eps;
 #ifdef FLA_DBG_TIMING
     unsigned long long *dbg;      // 16 clock stamps per workgroup (experimental builds only)
 #endif
