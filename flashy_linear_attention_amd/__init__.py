@@ -5,5 +5,7 @@ from .chunked import LinearAttentionChunked
 from .linear_attn import LinearAttention
 from .linear_attn_smallv_hd import LinearAttentionSmallVHD
 from .normalised import LinearAttentionNormalised
+from .poly import PolynomialLinearAttention
 
-__all__ = ["LinearAttention", "LinearAttentionSmallVHD", "LinearAttentionChunked", "LinearAttentionNormalised"]
+__all__ = ["LinearAttention", "LinearAttentionSmallVHD", "LinearAttentionChunked", "LinearAttentionNormalised",
+           "PolynomialLinearAttention"]

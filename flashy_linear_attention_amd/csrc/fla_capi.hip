@@ -93,6 +93,8 @@ TriParams make_params(const View &x, const View &y, const View &z, const View &o
     p.state_transposed = 0;
     p.denom = nullptr;
     p.eps = 0.f;
+    p.poly[0] = p.poly[1] = p.poly[2] = 0.f;
+    p.poly_on = 0;
     p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout), p.vec_out = vec_ok(out, dout);
 #ifdef FLA_DBG_TIMING
     {
@@ -483,6 +485,113 @@ int normalised_backward(const View &go, const View &q, const View &k, const View
     return norm_launch(2, dtype, l.lpr, p, stream) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
 }
 
+// ---- polynomial score map: out = lower(f(Xq Xk^T)) V, f(u) = c0 + c1 u + c2 u^2
+
+// [a | x] side by side, 8 elements per thread: columns [0, split) hold a (zero beyond its width),
+// columns [split, split + rp) hold x (zero beyond its width); out is contiguous (B, H, N, split + rp)
+__global__ __launch_bounds__(256) void pack_pair_kernel(const uint16_t *a, int64_t as_b, int64_t as_h, int64_t as_n, int wa,
+                                                        const uint16_t *x, int64_t xs_b, int64_t xs_h, int64_t xs_n, int wx,
+                                                        uint16_t *out, int H, int64_t N, int split, int rp, int64_t total) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    const int cpr = (split + rp) / 8;  // 8-element chunks per row
+    const int64_t row = t / cpr;
+    const int c8 = (int)(t - row * cpr) * 8;
+    const int64_t bh = row / N, n = row - bh * N;
+    const int64_t b = bh / H, h = bh - b * H;
+    fla::u32x4 w = {0u, 0u, 0u, 0u};
+    if (c8 < split) {
+        if (c8 < wa) w = *reinterpret_cast<const fla::u32x4 *>(a + b * as_b + h * as_h + n * as_n + c8);
+    } else if (c8 - split < wx) {
+        w = *reinterpret_cast<const fla::u32x4 *>(x + b * xs_b + h * xs_h + n * xs_n + (c8 - split));
+    }
+    *reinterpret_cast<fla::u32x4 *>(out + row * (split + rp) + c8) = w;
+}
+
+struct PolyLayout {
+    int64_t split, rp, width, packed_bytes;
+};
+
+// split: where the second operand starts = half of the padded contraction the dual-score kernel is
+// built for; rp: r rounded up to whole 16-byte chunks
+PolyLayout poly_layout(int64_t B, int64_t H, int64_t N, int64_t r, int64_t dv) {
+    PolyLayout l;
+    l.split = dv <= 32 ? 32 : dv <= 64 ? 64 : 128;
+    l.rp = (r + 7) / 8 * 8;
+    l.width = l.split + l.rp;
+    l.packed_bytes = (B * H * N * l.width * 2 + 15) / 16 * 16;
+    return l;
+}
+
+int check_poly_args(int64_t B, int64_t H, int64_t N, int64_t r, int64_t dv, int dtype, const float *coef) {
+    if (int rc = check_common(B, H, N, dtype)) return rc;
+    if (!coef) return FLA_ERR_NULL_POINTER;
+    if (r < 1 || r > 32) return FLA_ERR_HEAD_DIM;
+    if (dv < 1 || dv > 128) return FLA_ERR_V_HEAD_DIM;
+    return FLA_OK;
+}
+
+// every product of this operator exists only as a fast-path kernel
+bool poly_ok(const TriParams &p, int64_t dc, int64_t dout) { return chunk_rows(dc, dout) != 0 && fla::fast_path_ok(p); }
+
+int launch_poly(TriParams p, int64_t dc, int64_t dout, int dtype, int mode, float c0, float c1, float c2, void *stream) {
+    p.poly[0] = c0, p.poly[1] = c1, p.poly[2] = c2, p.poly_on = mode;
+    const hipError_t e = lookup(dtype, dc, dout)(p, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? FLA_OK : e == hipErrorNotSupported ? FLA_ERR_UNSUPPORTED : FLA_ERR_LAUNCH;
+}
+
+int poly_forward(const View &xq, const View &xk, const View &v, const View &o, float *denom, int64_t B, int64_t H,
+                 int64_t N, int64_t r, int64_t dv, const float *coef, float eps, int dtype, void *stream) {
+    const View all[] = {xq, xk, v, o};
+    for (const View &t : all)
+        if (int rc = check_view(t)) return rc;
+    if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    if (denom && B * H > 65535) return FLA_ERR_SHAPE;
+    TriParams p = make_params(xq, xk, v, o, B, H, N, r, dv, 0);
+    if (!poly_ok(p, r, dv)) return FLA_ERR_UNSUPPORTED;
+    p.denom = denom, p.eps = eps;
+    return launch_poly(p, r, dv, dtype, 1, coef[0], coef[1], coef[2], stream);
+}
+
+int poly_backward(const View &go, const View &xq, const View &xk, const View &v, const View &dxq, const View &dxk,
+                  const View &dvv, int64_t B, int64_t H, int64_t N, int64_t r, int64_t dv, const float *coef,
+                  int dtype, void *workspace, int64_t workspace_bytes, void *stream) {
+    const View all[] = {go, xq, xk, v, dxq, dxk, dvv};
+    for (const View &t : all)
+        if (int rc = check_view(t)) return rc;
+    if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    const PolyLayout l = poly_layout(B, H, N, r, dv);
+    if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < 2 * l.packed_bytes)
+        return FLA_ERR_WORKSPACE;
+    // the packing kernel and the products below use 16-byte accesses throughout
+    if (!(vec_ok(go, dv) && vec_ok(v, dv) && vec_ok(xq, r) && vec_ok(xk, r) && vec_ok(dxq, r) && vec_ok(dxk, r) &&
+          vec_ok(dvv, dv)))
+        return FLA_ERR_UNSUPPORTED;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    uint16_t *p1 = static_cast<uint16_t *>(workspace);                                               // [dO | xq]
+    uint16_t *p2 = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + l.packed_bytes);    // [V | xk]
+    const int64_t total = B * H * N * (l.width / 8);
+    const dim3 grid((unsigned)((total + 255) / 256));
+    hipLaunchKernelGGL(pack_pair_kernel, grid, dim3(256), 0, s, static_cast<const uint16_t *>(go.ptr), go.strides[0],
+                       go.strides[1], go.strides[2], (int)dv, static_cast<const uint16_t *>(xq.ptr), xq.strides[0],
+                       xq.strides[1], xq.strides[2], (int)r, p1, (int)H, N, (int)l.split, (int)l.rp, total);
+    hipLaunchKernelGGL(pack_pair_kernel, grid, dim3(256), 0, s, static_cast<const uint16_t *>(v.ptr), v.strides[0],
+                       v.strides[1], v.strides[2], (int)dv, static_cast<const uint16_t *>(xk.ptr), xk.strides[0],
+                       xk.strides[1], xk.strides[2], (int)r, p2, (int)H, N, (int)l.split, (int)l.rp, total);
+    if (hipGetLastError() != hipSuccess) return FLA_ERR_LAUNCH;
+    const int64_t ps[4] = {H * N * l.width, N * l.width, l.width, 1};
+    const View P1{p1, ps}, P2{p2, ps};
+    // dV = upper(f(Xk Xq^T)) dO
+    const TriParams pv = make_params(xk, xq, go, dvv, B, H, N, r, dv, 1);
+    // dXq = lower((dO V^T) f'(Xq Xk^T)) Xk, dXk = upper((V dO^T) f'(Xk Xq^T)) Xq; f'(u) = c1 + 2 c2 u
+    const TriParams pq = make_params(P1, P2, xk, dxq, B, H, N, l.width, r, 0);
+    const TriParams pk = make_params(P2, P1, xq, dxk, B, H, N, l.width, r, 1);
+    if (!poly_ok(pv, r, dv) || !poly_ok(pq, l.width, r) || !poly_ok(pk, l.width, r)) return FLA_ERR_UNSUPPORTED;
+    if (int rc = launch_poly(pv, r, dv, dtype, 1, coef[0], coef[1], coef[2], stream)) return rc;
+    if (int rc = launch_poly(pq, l.width, r, dtype, 2, coef[1], 2.0f * coef[2], 0.f, stream)) return rc;
+    return launch_poly(pk, l.width, r, dtype, 2, coef[1], 2.0f * coef[2], 0.f, stream);
+}
+
 }  // namespace
 
 extern "C" {
@@ -612,6 +721,31 @@ int fla_linear_attn_chunked_bwd(const void *grad_out, const void *q, const void 
     return chunked_backward({grad_out, go_strides}, {q, q_strides}, {k, k_strides}, {v, v_strides}, {dq, dq_strides},
                             {dk, dk_strides}, {dv, dv_strides}, B, H, N, D_qk, D_v, dtype, state_in, workspace,
                             workspace_bytes, stream);
+}
+
+int64_t fla_poly_attn_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t R, int64_t D_v) {
+    if (B < 0 || H < 0 || N < 0 || R < 1 || R > 32 || D_v < 1 || D_v > 128) return 0;
+    return 2 * poly_layout(B, H, N, R, D_v).packed_bytes;
+}
+
+int fla_poly_attn_fwd(const void *xq, const void *xk, const void *v, void *o, float *denom, int64_t B, int64_t H,
+                      int64_t N, int64_t R, int64_t D_v, const int64_t *xq_strides, const int64_t *xk_strides,
+                      const int64_t *v_strides, const int64_t *o_strides, const float *coef, float eps, int dtype,
+                      void *stream) {
+    if (int rc = check_poly_args(B, H, N, R, D_v, dtype, coef)) return rc;
+    return poly_forward({xq, xq_strides}, {xk, xk_strides}, {v, v_strides}, {o, o_strides}, denom, B, H, N, R, D_v,
+                        coef, eps, dtype, stream);
+}
+
+int fla_poly_attn_bwd(const void *grad_out, const void *xq, const void *xk, const void *v, void *dxq, void *dxk,
+                      void *dv, int64_t B, int64_t H, int64_t N, int64_t R, int64_t D_v, const int64_t *go_strides,
+                      const int64_t *xq_strides, const int64_t *xk_strides, const int64_t *v_strides,
+                      const int64_t *dxq_strides, const int64_t *dxk_strides, const int64_t *dv_strides,
+                      const float *coef, int dtype, void *workspace, int64_t workspace_bytes, void *stream) {
+    if (int rc = check_poly_args(B, H, N, R, D_v, dtype, coef)) return rc;
+    return poly_backward({grad_out, go_strides}, {xq, xq_strides}, {xk, xk_strides}, {v, v_strides},
+                         {dxq, dxq_strides}, {dxk, dxk_strides}, {dv, dv_strides}, B, H, N, R, D_v, coef, dtype,
+                         workspace, workspace_bytes, stream);
 }
 
 int64_t fla_normalised_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v, int chunked) {

@@ -150,9 +150,22 @@ __device__ __forceinline__ int swizzle_z(int row) {
 }
 
 // The work of one workgroup; `wg_index` is its index within one product's grid.
-template <typename T, int DC, int DO, bool CHUNKED, bool NORM = false>
+// FLAGS of the quadratic walk: kNormFlag divides each output row by the sum of its masked scores
+// (the normaliser of linear attention); kPolyFlag maps every score through a quadratic polynomial
+// (second-order Taylor feature map without the features).
+// kDualFlag: two scores from one pass over the contraction -- columns [0, D_c/2) of X and Y give
+// u1, columns [D_c/2, D_c/2 + 32) give u2, and the score is u1 (poly[0] + poly[1] u2 + poly[2] u2^2):
+// the gradient of the polynomial score map with respect to its argument, e.g.
+// lower((dO V^T) . f'(Xq Xk^T)) Xk with X = [dO | xq] and Y = [V | xk] packed side by side.
+constexpr int kNormFlag = 1, kPolyFlag = 2, kDualFlag = 4;
+constexpr int kPolyMaxContraction = 64;  // polynomial variants are built for D_c <= 64 only
+
+template <typename T, int DC, int DO, bool CHUNKED, int FLAGS = 0>
 __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_index) {
-    static_assert(!(CHUNKED && NORM), "the in-kernel normaliser belongs to the quadratic walk");
+    constexpr bool NORM = (FLAGS & kNormFlag) != 0, POLY = (FLAGS & kPolyFlag) != 0, DUAL = (FLAGS & kDualFlag) != 0;
+    static_assert(!(DUAL && (POLY || NORM)), "the dual-score walk has its own score map and no normaliser");
+    static_assert(!DUAL || DC >= 64, "the dual-score walk needs room for two contractions");
+    static_assert(!(CHUNKED && FLAGS != 0), "score maps and the in-kernel normaliser belong to the quadratic walk");
     // The body is compiled in the device pass only: hipcc's host pass silently
     // drops the launch stub of a kernel template whose body calls the LDS-DMA
     // builtin from inside a lambda, and the host needs nothing but the stub.
@@ -166,6 +179,9 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     constexpr int RY = Cfg::RY, RZ = Cfg::RZ, CY = Cfg::CY, CZ = Cfg::CZ;
     constexpr int NIY = Cfg::NIY, NIZ = Cfg::NIZ;
     constexpr int STAGE = Cfg::STAGE_BYTES, Y_BYTES = Cfg::Y_BYTES;
+    // chunks of the contraction that feed the first score / that are used at all (DUAL: the
+    // second score takes two chunks, 32 columns, right after the first half)
+    constexpr int KC1 = DUAL ? KC / 2 : KC, KCU = DUAL ? KC / 2 + 2 : KC;
     constexpr int YQ = KC < 4 ? KC : 4;  // Y read addresses that differ by more than an immediate
     constexpr int ZQ = DB < 2 ? DB : 2;  // same for Z
 
@@ -299,7 +315,7 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     for (int ib = 0; ib < NIB; ++ib) {
         const int row = i0 + blk[ib] * 32 + l32;
 #pragma unroll
-        for (int kc = 0; kc < KC; ++kc) {
+        for (int kc = 0; kc < KCU; ++kc) {
             const int col = kc * 16 + 8 * g;
             const uint32_t off = (uint32_t)(row * xs2 + col * 2) + (col < p.dc ? 0u : kOobOffset);
             xf[ib][kc] = __builtin_bit_cast(V8, __builtin_amdgcn_raw_buffer_load_b128(rx, off, 0, 0));
@@ -318,6 +334,15 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     float rsum[NIB];
 #pragma unroll
     for (int ib = 0; ib < NIB; ++ib) rsum[ib] = 0.f;
+    const float pc0 = p.poly[0], pc1 = p.poly[1], pc2 = p.poly[2];
+    auto map_scores = [&](f32x16 &sc) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sc[v] = __builtin_fmaf(__builtin_fmaf(pc2, sc[v], pc1), sc[v], pc0);
+    };
+    auto combine_scores = [&](f32x16 &sc, const f32x16 &sc2) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sc[v] *= __builtin_fmaf(__builtin_fmaf(pc2, sc2[v], pc1), sc2[v], pc0);
+    };
     auto add_scores = [&](const f32x16 &sc, float &dst) {
         float t0 = (sc[0] + sc[1]) + (sc[2] + sc[3]), t1 = (sc[4] + sc[5]) + (sc[6] + sc[7]);
         float t2 = (sc[8] + sc[9]) + (sc[10] + sc[11]), t3 = (sc[12] + sc[13]) + (sc[14] + sc[15]);
@@ -435,30 +460,35 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     // ================= tiles fully inside the mask: pipelined, no masking =================
     if (n_full > 0) {
         V8 yf[KC], zf[NZF], pfa[NIB][2], pfb[NIB][2];
-        f32x16 s[NIB];
+        f32x16 s[NIB], s2[NIB];
         const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         {
             int ya0[YQ], za0[ZQ];
             slot_addrs(0, ya0, za0);
 #pragma unroll
-            for (int kc = 0; kc < KC; ++kc) yf[kc] = y_read(ya0, 0, kc);
+            for (int kc = 0; kc < KCU; ++kc) yf[kc] = y_read(ya0, 0, kc);
         }
 
         // phase 1 of sub-tile s: S = Y_s X^T, interleaved with the Z fragment reads of the previous sub-tile
         auto phase1 = [&](auto with_z, const int (&za)[ZQ], int zsub) {
 #pragma unroll
-            for (int kc = 0; kc < KC; ++kc) {
+            for (int kc = 0; kc < KCU; ++kc) {
 #pragma unroll
-                for (int ib = 0; ib < NIB; ++ib) s[ib] = M::mma(yf[kc], xf[ib][kc], kc == 0 ? zero : s[ib]);
+                for (int ib = 0; ib < NIB; ++ib) {
+                    if (kc < KC1)
+                        s[ib] = M::mma(yf[kc], xf[ib][kc], kc == 0 ? zero : s[ib]);
+                    else
+                        s2[ib] = M::mma(yf[kc], xf[ib][kc], kc == KC1 ? zero : s2[ib]);
+                }
                 if constexpr (decltype(with_z)::value) {
 #ifndef FLA_DBG_NO_ZREAD
 #pragma unroll
                     for (int f = 0; f < NZF; ++f)
-                        if (f * KC / NZF == kc) zf[f] = z_read(za, zsub, f);
+                        if (f * KCU / NZF == kc) zf[f] = z_read(za, zsub, f);
 #else
 #pragma unroll
                     for (int f = 0; f < NZF; ++f)
-                        if (f * KC / NZF == kc) asm volatile("" : "+v"(zf[f]));
+                        if (f * KCU / NZF == kc) asm volatile("" : "+v"(zf[f]));
 #endif
                 }
                 __builtin_amdgcn_sched_barrier(0);
@@ -479,13 +509,25 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
                 }
 #ifndef FLA_DBG_NO_YREAD
 #pragma unroll
-                for (int kc = 0; kc < KC; ++kc)
-                    if (kc * NZF / KC == f) yf[kc] = y_read(ya, ysub, kc);
+                for (int kc = 0; kc < KCU; ++kc)
+                    if (kc * NZF / KCU == f) yf[kc] = y_read(ya, ysub, kc);
 #else
 #pragma unroll
-                for (int kc = 0; kc < KC; ++kc)
-                    if (kc * NZF / KC == f) asm volatile("" : "+v"(yf[kc]));
+                for (int kc = 0; kc < KCU; ++kc)
+                    if (kc * NZF / KCU == f) asm volatile("" : "+v"(yf[kc]));
 #endif
+                if constexpr (POLY) {
+                    if (f == NZF / 2) {
+#pragma unroll
+                        for (int ib = 0; ib < NIB; ++ib) map_scores(s[ib]);
+                    }
+                }
+                if constexpr (DUAL) {
+                    if (f == NZF / 2) {
+#pragma unroll
+                        for (int ib = 0; ib < NIB; ++ib) combine_scores(s[ib], s2[ib]);
+                    }
+                }
                 if constexpr (NORM) {
                     if (f == NZF / 2) {
 #pragma unroll
@@ -677,26 +719,30 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
 #pragma unroll
             for (int j = 0; j < ZQ; ++j) za[j] = zlane[j] + so + (s8 & 1) * (32 * RZ);
 #pragma unroll
-            for (int kc = 0; kc < KC; ++kc) yf[kc] = y_read(ya, 0, kc);
+            for (int kc = 0; kc < KCU; ++kc) yf[kc] = y_read(ya, 0, kc);
 #pragma unroll
             for (int f = 0; f < NZF; ++f) zf[f] = z_read(za, 0, f);
         };
         auto compute_sub = [&](int s8, const V8 (&yf)[KC], const V8 (&zf)[NZF]) {
             bool act[NIB];
-            f32x16 sd[NIB];
+            f32x16 sd[NIB], sd2[NIB];
 #pragma unroll
             for (int ib = 0; ib < NIB; ++ib) {
                 act[ib] = upper ? s8 >= blk[ib] : s8 <= blk[ib];
                 if (act[ib]) {
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) sd[ib][v] = 0.f;
+                    for (int v = 0; v < 16; ++v) sd[ib][v] = 0.f, sd2[ib][v] = 0.f;
 #pragma unroll
-                    for (int kc = 0; kc < KC; ++kc) sd[ib] = M::mma(yf[kc], xf[ib][kc], sd[ib]);
+                    for (int kc = 0; kc < KC1; ++kc) sd[ib] = M::mma(yf[kc], xf[ib][kc], sd[ib]);
+#pragma unroll
+                    for (int kc = KC1; kc < KCU; ++kc) sd2[ib] = M::mma(yf[kc], xf[ib][kc], sd2[ib]);
+                    if constexpr (DUAL) combine_scores(sd[ib], sd2[ib]);
                 }
             }
 #pragma unroll
             for (int ib = 0; ib < NIB; ++ib) {
                 if (!act[ib]) continue;
+                if constexpr (POLY) map_scores(sd[ib]);  // before the mask: masked scores stay zero
                 if (s8 == blk[ib]) {  // the 32 x 32 block on the diagonal itself
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
@@ -797,10 +843,10 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
 #endif
 }
 
-template <typename T, int DC, int DO, bool CHUNKED, bool NORM>
+template <typename T, int DC, int DO, bool CHUNKED, int FLAGS>
 __global__ __launch_bounds__(256, (FastConfig<DC, DO, CHUNKED>::kMinWavesPerSimd)) void tri_xyt_z_fast_kernel(
     const TriParams p) {
-    tri_fast_body<T, DC, DO, CHUNKED, NORM>(p, blockIdx.x);
+    tri_fast_body<T, DC, DO, CHUNKED, FLAGS>(p, blockIdx.x);
 }
 
 // grid y = product index
@@ -819,17 +865,33 @@ inline bool fast_path_ok(const TriParams &p) {
     return n * p.xs_n * 2 <= kMaxFastExtent && n * p.ys_n * 2 <= kMaxFastExtent && n * p.zs_n * 2 <= kMaxFastExtent;
 }
 
-template <typename T, int DC, int DO, bool CHUNKED, bool NORM>
+template <typename T, int DC, int DO, bool CHUNKED, int FLAGS>
 hipError_t launch_tri_fast_variant(TriParams p, hipStream_t stream);
 
 template <typename T, int DC, int DO>
 hipError_t launch_tri_fast(const TriParams &p, hipStream_t stream) {
-    if (p.state) return p.denom ? hipErrorNotSupported : launch_tri_fast_variant<T, DC, DO, true, false>(p, stream);
-    return p.denom ? launch_tri_fast_variant<T, DC, DO, false, true>(p, stream)
-                   : launch_tri_fast_variant<T, DC, DO, false, false>(p, stream);
+    if (p.state)
+        return (p.denom || p.poly_on) ? hipErrorNotSupported : launch_tri_fast_variant<T, DC, DO, true, 0>(p, stream);
+    if (p.poly_on == 2) {  // dual-score walk: built for 32-wide outputs (the argument of the score map)
+        if constexpr (DC >= 64 && DO == 32) {
+            return p.denom ? hipErrorNotSupported : launch_tri_fast_variant<T, DC, DO, false, kDualFlag>(p, stream);
+        } else {
+            return hipErrorNotSupported;
+        }
+    }
+    if (p.poly_on) {
+        if constexpr (DC <= kPolyMaxContraction) {
+            return p.denom ? launch_tri_fast_variant<T, DC, DO, false, kPolyFlag | kNormFlag>(p, stream)
+                           : launch_tri_fast_variant<T, DC, DO, false, kPolyFlag>(p, stream);
+        } else {
+            return hipErrorNotSupported;
+        }
+    }
+    return p.denom ? launch_tri_fast_variant<T, DC, DO, false, kNormFlag>(p, stream)
+                   : launch_tri_fast_variant<T, DC, DO, false, 0>(p, stream);
 }
 
-template <typename T, int DC, int DO, bool CHUNKED, bool NORM>
+template <typename T, int DC, int DO, bool CHUNKED, int FLAGS>
 hipError_t launch_tri_fast_variant(TriParams p, hipStream_t stream) {
     using Cfg = FastConfig<DC, DO, CHUNKED>;
     if constexpr (!Cfg::kSupported) {
@@ -843,7 +905,7 @@ hipError_t launch_tri_fast_variant(TriParams p, hipStream_t stream) {
         p.single = (!CHUNKED && (int64_t)p.BH * ((p.n_tiles + 1) / 2) < 256) ? 1 : 0;
         const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * ((CHUNKED || p.single) ? p.n_tiles : (p.n_tiles + 1) / 2);
         if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-        auto kern = tri_xyt_z_fast_kernel<T, DC, DO, CHUNKED, NORM>;
+        auto kern = tri_xyt_z_fast_kernel<T, DC, DO, CHUNKED, FLAGS>;
         const int smem = Cfg::SMEM_BYTES + (Cfg::kStateInLds ? Cfg::STATE_BYTES : 0);
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, smem);

@@ -62,6 +62,14 @@ struct TriParams {
     // fp32, contiguous (B H, N).
     float *denom;
     float eps;
+    // Polynomial score map (quadratic fast path, contraction width <= 64): when poly_on != 0 every
+    // score u = x . y is replaced by poly[0] + poly[1] u + poly[2] u^2 before masking and rounding --
+    // causal linear attention with a second-order Taylor feature map, the features never built.
+    // poly_on == 2: dual-score walk (32-wide outputs only).  X and Y carry two operands side by side,
+    // columns [0, DC/2) and [DC/2, DC/2 + 32) of the instantiation's padded width DC; the score is
+    // u1 (poly[0] + poly[1] u2 + poly[2] u2^2).
+    float poly[3];
+    int32_t poly_on;
 #ifdef FLA_DBG_TIMING
     unsigned long long *dbg;      // 16 clock stamps per workgroup (experimental builds only)
 #endif

@@ -170,6 +170,38 @@ int fla_linear_attn_chunked_bwd(const void *grad_out, const void *q, const void 
                                 int dtype, const void *state_in,
                                 void *workspace, int64_t workspace_bytes, void *stream);
 
+/* Causal linear attention with a polynomial score map,
+ *
+ *     out = lower(f(Xq Xk^T)) V,    f(u) = coef[0] + coef[1] u + coef[2] u^2,
+ *
+ * i.e. LinearAttentionSmallVHD on second-order Taylor features phi(x) with
+ * phi(x) . phi(y) = f(x . y) (the reference's README.md:3 use case: 256 features from a 16-wide
+ * x, coef = {0, 0, 1/2}; the full Taylor map is {1, 1, 1/2}) -- with the features never built:
+ * scores cost an R-wide contraction instead of an R^2-wide one.  xq, xk: (B, H, N, R), R <= 32;
+ * v, o: (B, H, N, D_v), D_v <= 128.  When `denom` is non-NULL the output rows are divided by
+ * n = (row sum of the masked scores) + eps and n is stored there (fp32, contiguous (B, H, N));
+ * backward is for the un-normalised product (denom == NULL).  Backward forms
+ *     dV  = upper(f(Xk Xq^T)) dO
+ *     dXq = lower((dO V^T) . f'(Xq Xk^T)) Xk,   dXk = upper((V dO^T) . f'(Xk Xq^T)) Xq
+ * and needs fla_poly_attn_workspace_bytes() bytes of 16-byte aligned scratch.  Fast-path kernels
+ * only: every operand 16-byte aligned with widths and outer strides multiples of 8 elements,
+ * else FLA_ERR_UNSUPPORTED.  No counterpart in the reference (it multiplies materialised
+ * features, linear_attn_kernels_smallv_hd.py:78-86). */
+int64_t fla_poly_attn_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t R, int64_t D_v);
+int fla_poly_attn_fwd(const void *xq, const void *xk, const void *v, void *o, float *denom,
+                      int64_t B, int64_t H, int64_t N, int64_t R, int64_t D_v,
+                      const int64_t *xq_strides, const int64_t *xk_strides,
+                      const int64_t *v_strides, const int64_t *o_strides,
+                      const float *coef, float eps, int dtype, void *stream);
+int fla_poly_attn_bwd(const void *grad_out, const void *xq, const void *xk, const void *v,
+                      void *dxq, void *dxk, void *dv,
+                      int64_t B, int64_t H, int64_t N, int64_t R, int64_t D_v,
+                      const int64_t *go_strides, const int64_t *xq_strides,
+                      const int64_t *xk_strides, const int64_t *v_strides,
+                      const int64_t *dxq_strides, const int64_t *dxk_strides,
+                      const int64_t *dv_strides,
+                      const float *coef, int dtype, void *workspace, int64_t workspace_bytes, void *stream);
+
 /* Normalised causal linear attention, the full operator a caller of the reference assembles
  * in PyTorch around LinearAttention.apply (README.md:27-30 of the reference):
  *

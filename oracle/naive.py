@@ -120,3 +120,46 @@ def causal_dot_product_grads_blocked(
         dk[..., :r1, :] += torch.matmul(m.transpose(-2, -1), q[..., r0:r1, :])
         dq[..., r0:r1, :] = torch.matmul(m, k[..., :r1, :])
     return dq, dk, dv
+
+
+def taylor2_features(x: torch.Tensor, coef: Tuple[float, float, float]) -> torch.Tensor:
+    """Feature vector phi(x) with phi(x) . phi(y) = c0 + c1 (x . y) + c2 (x . y)^2 for
+    non-negative (c0, c1, c2): [sqrt(c0), sqrt(c1) x, sqrt(c2) vec(x x^T)].  With (0, 0, 1/2) this
+    is the map ``flatten(x (x) x) / sqrt 2`` of the reference's small-V use case (README.md:3 of
+    the reference: Based / Taylor features in front of ``LinearAttentionSmallVHD``)."""
+    c0, c1, c2 = coef
+    parts = []
+    if c0:
+        parts.append(torch.full((*x.shape[:-1], 1), c0 ** 0.5, dtype=x.dtype, device=x.device))
+    if c1:
+        parts.append(c1 ** 0.5 * x)
+    if c2:
+        parts.append(c2 ** 0.5 * (x[..., :, None] * x[..., None, :]).flatten(-2))
+    return torch.cat(parts, dim=-1)
+
+
+def poly_causal_dot_product(
+    xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, coef: Tuple[float, float, float]
+) -> torch.Tensor:
+    """O = tril(f(Xq Xk^T)) V with f(u) = c0 + c1 u + c2 u^2 applied to every score: what
+    :func:`causal_dot_product` gives on ``taylor2_features`` of xq and xk, with the features
+    never built (the two must agree to rounding; tests/test_oracle.py checks it)."""
+    c0, c1, c2 = coef
+    n = xq.shape[-2]
+    u = torch.matmul(xq, xk.transpose(-2, -1))
+    scores = (c0 + c1 * u + c2 * u * u) * _tril_mask(n, xq.device).to(u.dtype)
+    return torch.matmul(scores, v)
+
+
+def poly_causal_dot_product_grads(
+    xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, do: torch.Tensor, coef: Tuple[float, float, float]
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dXq, dXk, dV) of :func:`poly_causal_dot_product` in closed form:
+    dV = S^T dO,  dU = tril(dO V^T) * f'(U),  dXq = dU Xk,  dXk = dU^T Xq."""
+    c0, c1, c2 = coef
+    n = xq.shape[-2]
+    mask = _tril_mask(n, xq.device).to(xq.dtype)
+    u = torch.matmul(xq, xk.transpose(-2, -1))
+    s = (c0 + c1 * u + c2 * u * u) * mask
+    du = torch.matmul(do, v.transpose(-2, -1)) * mask * (c1 + 2.0 * c2 * u)
+    return torch.matmul(du, xk), torch.matmul(du.transpose(-2, -1), xq), torch.matmul(s.transpose(-2, -1), do)

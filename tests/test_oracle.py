@@ -158,3 +158,26 @@ def test_normalised_recipe_is_a_weighted_average():
 def test_c_oracle_rejects_bad_arguments():
     lib = c_oracle._load()
     assert lib.oracle_causal_dot_product_fwd(None, None, None, None, 1, 1, 1, 1) == -1
+
+
+@pytest.mark.parametrize("coef", [(0.0, 0.0, 0.5), (1.0, 1.0, 0.5), (0.25, 2.0, 0.0)], ids=["square", "taylor", "affine"])
+def test_polynomial_score_map_equals_explicit_features(coef):
+    """f(x . y) = phi(x) . phi(y): the polynomial form against the plain oracle on the explicit
+    feature vectors, forward and all three gradients (the latter by autograd through the
+    explicit features, an independent route), in fp64."""
+    g = torch.Generator().manual_seed(3)
+    xq = torch.randn(2, 2, 40, 6, generator=g, dtype=torch.float64)
+    xk = torch.randn(2, 2, 40, 6, generator=g, dtype=torch.float64)
+    v = torch.randn(2, 2, 40, 5, generator=g, dtype=torch.float64)
+    do = torch.randn(2, 2, 40, 5, generator=g, dtype=torch.float64)
+    a, b, c = (t.clone().requires_grad_(True) for t in (xq, xk, v))
+    ref = naive.causal_dot_product(naive.taylor2_features(a, coef), naive.taylor2_features(b, coef), c)
+    ref.backward(do)
+    got = naive.poly_causal_dot_product(xq, xk, v, coef)
+    assert torch.allclose(got, ref.detach(), rtol=1e-12, atol=1e-12)
+    dxq, dxk, dv = naive.poly_causal_dot_product_grads(xq, xk, v, do, coef)
+    for x, y in ((dxq, a.grad), (dxk, b.grad), (dv, c.grad)):
+        assert torch.allclose(x, y, rtol=1e-11, atol=1e-11)
+    # the reference's feature recipe for the small-V operator is the pure square with c2 = 1/2
+    phi = (xq[..., :, None] * xq[..., None, :]).flatten(-2) / 2 ** 0.5
+    assert torch.allclose(naive.taylor2_features(xq, (0.0, 0.0, 0.5)), phi)
