@@ -57,12 +57,14 @@ def _parse():
     ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU oracle timing")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target seconds of CPU work for the baseline")
-    ap.add_argument("--algo", default="quadratic", choices=["quadratic", "chunked", "normalised", "normalised-chunked"],
+    ap.add_argument("--algo", default="quadratic", choices=["quadratic", "chunked", "normalised", "normalised-chunked", "poly"],
                     help="quadratic: the tiled O(N^2 D) kernels the headline metric is defined on (default); "
                          "chunked: the O(N) chunk-state path, reported with its own FLOP count and an HBM roofline; "
                          "normalised: the quadratic kernels plus the fused normaliser (out / (q . cumsum(k) + eps)), "
                          "with the normaliser's own time, bytes and the PyTorch recipe's time beside it; "
-                         "normalised-chunked: the same with the chunk-wise product")
+                         "normalised-chunked: the same with the chunk-wise product; "
+                         "poly (workload C4 only): the same function as C4 computed from the 16-wide x behind its "
+                         "Taylor features with the polynomial score map, priced in its own FLOPs")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain device copy of 256 MiB (a known-size reference for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -115,6 +117,79 @@ def _cpu_baseline(torch, w, target_seconds):
     }
 
 
+def _bench_poly(torch, args, w, dev, time_region) -> int:
+    """C4's function, O = tril(phi(xq) phi(xk)^T) V with phi(x) = flatten(x (x) x) / sqrt 2, evaluated
+    from the 16-wide x with the polynomial score map f(u) = u^2 / 2, next to the same step on the
+    materialised 256-wide features (LinearAttentionSmallVHD's kernels) in the same run."""
+    import math
+
+    from flashy_linear_attention_amd.kernels import linear_flash_wrapper_bwd_smallv_hd, linear_flash_wrapper_fwd_smallv_hd
+    from flashy_linear_attention_amd.poly import poly_attention_bwd, poly_attention_fwd
+
+    if w.features != "taylor2":
+        print("bench.py: --algo poly needs a workload whose q, k are Taylor features (C4)", file=sys.stderr)
+        return 2
+    r = math.isqrt(w.d_qk)
+    gen = torch.Generator().manual_seed(0)
+    xq = (0.5 * torch.randn(w.batch, w.heads, w.seq, r, generator=gen)).to(w.dtype)
+    xk = (0.5 * torch.randn(w.batch, w.heads, w.seq, r, generator=gen)).to(w.dtype)
+    v = torch.randn(w.batch, w.heads, w.seq, w.d_v, generator=gen).to(w.dtype)
+    do = torch.randn(w.batch, w.heads, w.seq, w.d_v, generator=gen).to(w.dtype)
+
+    def phi(x):
+        return ((x.float()[..., :, None] * x.float()[..., None, :]).flatten(-2) / math.sqrt(2.0)).to(w.dtype)
+
+    q, k = phi(xq).to(dev), phi(xk).to(dev)
+    xq, xk, v, do = (t.to(dev) for t in (xq, xk, v, do))
+    coef = (0.0, 0.0, 0.5)
+
+    def step():
+        poly_attention_fwd(xq, xk, v, coef)
+        poly_attention_bwd(do, xq, xk, v, coef)
+
+    def plain_step():
+        linear_flash_wrapper_fwd_smallv_hd(q, k, v)
+        linear_flash_wrapper_bwd_smallv_hd(do, q, k, v)
+
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < args.settle_seconds:
+        for _ in range(8):
+            step()
+        torch.cuda.synchronize()
+    for _ in range(args.warmup):
+        step()
+    ms_step = time_region(torch, step, args.steps) / args.steps
+    ms_fwd = time_region(torch, lambda: poly_attention_fwd(xq, xk, v, coef), args.steps) / args.steps
+    ms_bwd = time_region(torch, lambda: poly_attention_bwd(do, xq, xk, v, coef), args.steps) / args.steps
+    for _ in range(20):
+        plain_step()
+    ms_plain = time_region(torch, plain_step, args.steps) / args.steps
+    bh, n = float(w.batch * w.heads), float(w.seq)
+    # causal-counted FLOPs of what is evaluated: scores over r columns, second products as they are
+    f_fwd = bh * n * n * (r + w.d_v)
+    f_bwd = bh * n * n * ((r + w.d_v) + 2 * (w.d_v + r + r))
+    value = (f_fwd + f_bwd) / (ms_step * 1e-3) / 1e12
+    result = {
+        "metric": f"causal linear attention with polynomial score map fwd+bwd TFLOP/s (its own causal-counted FLOPs), "
+                  f"B={w.batch} H={w.heads} N={w.seq} R={r} D_v={w.d_v}, 1 MI355X",
+        "value": round(value, 2), "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "workload": f"{w.name} evaluated from x: q, k = flatten(x (x) x) / sqrt 2 of a {r}-wide x = 0.5 randn, "
+                        f"f(u) = u^2 / 2; v and dO randn, seed 0",
+            "flops_per_step": f_fwd + f_bwd, "fwd_ms": round(ms_fwd, 4), "bwd_ms": round(ms_bwd, 4),
+            "materialised_features_step_ms": round(ms_plain, 4),
+            "speedup_vs_materialised_features": round(ms_plain / ms_step, 2),
+        },
+        "roofline": {"bound": "mfma", "kernel": "fla::tri_xyt_z_fast_kernel, polynomial and dual-score variants",
+                     "achieved": round(value, 2), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
+                     "frac": round(value / PEAK_TFLOPS["bf16"], 4), "traffic": None},
+    }
+    print(json.dumps(result))
+    return 0
+
+
 def main() -> int:
     args = _parse()
     if args.gpus != 1:
@@ -143,6 +218,8 @@ def main() -> int:
     q, k, v, do = (t.to(dev) for t in make_inputs(w, seed=0))
     fwd = linear_flash_wrapper_fwd_smallv_hd if w.small_v else linear_flash_wrapper_fwd
     bwd = linear_flash_wrapper_bwd_smallv_hd if w.small_v else linear_flash_wrapper_bwd
+    if args.algo == "poly":
+        return _bench_poly(torch, args, w, dev, _time_region)
     normalised = args.algo.startswith("normalised")
     chunked = args.algo in ("chunked", "normalised-chunked")
     if chunked:
