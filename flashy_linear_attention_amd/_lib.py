@@ -43,7 +43,7 @@ SIGNATURES = {
     "fla_poly_attn_workspace_bytes": ([_i64] * 5, ctypes.c_int64),
     "fla_poly_attn_fwd": ([_ptr] * 5 + [_i64] * 5 + [_strides] * 4
                           + [ctypes.POINTER(ctypes.c_float), ctypes.c_float, ctypes.c_int, _ptr], ctypes.c_int),
-    "fla_poly_attn_bwd": ([_ptr] * 7 + [_i64] * 5 + [_strides] * 7
+    "fla_poly_attn_bwd": ([_ptr] * 9 + [_i64] * 5 + [_strides] * 8
                           + [ctypes.POINTER(ctypes.c_float), ctypes.c_int, _ptr, _i64, _ptr], ctypes.c_int),
     "fla_normalised_workspace_bytes": ([_i64] * 5 + [ctypes.c_int], ctypes.c_int64),
     "fla_linear_attn_normalised_fwd": ([_ptr] * 5 + [_i64] * 5 + [_strides] * 4

@@ -488,10 +488,13 @@ int normalised_backward(const View &go, const View &q, const View &k, const View
 // ---- polynomial score map: out = lower(f(Xq Xk^T)) V, f(u) = c0 + c1 u + c2 u^2
 
 // [a | x] side by side, 8 elements per thread: columns [0, split) hold a (zero beyond its width),
-// columns [split, split + rp) hold x (zero beyond its width); out is contiguous (B, H, N, split + rp)
-__global__ __launch_bounds__(256) void pack_pair_kernel(const uint16_t *a, int64_t as_b, int64_t as_h, int64_t as_n, int wa,
-                                                        const uint16_t *x, int64_t xs_b, int64_t xs_h, int64_t xs_n, int wx,
-                                                        uint16_t *out, int H, int64_t N, int split, int rp, int64_t total) {
+// columns [split, split + rp) hold x (zero beyond its width); out is contiguous (B, H, N, split + rp).
+// bias_mode 1 / 2 puts one more value right after a, in column wa: bias[row] / the constant 1.
+template <typename T>
+__global__ __launch_bounds__(256) void pack_pair_kernel(const T *a, int64_t as_b, int64_t as_h, int64_t as_n, int wa,
+                                                        const T *x, int64_t xs_b, int64_t xs_h, int64_t xs_n, int wx,
+                                                        T *out, int H, int64_t N, int split, int rp, int64_t total,
+                                                        int bias_mode, const float *bias) {
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (t >= total) return;
     const int cpr = (split + rp) / 8;  // 8-element chunks per row
@@ -501,25 +504,54 @@ __global__ __launch_bounds__(256) void pack_pair_kernel(const uint16_t *a, int64
     const int64_t b = bh / H, h = bh - b * H;
     fla::u32x4 w = {0u, 0u, 0u, 0u};
     if (c8 < split) {
-        if (c8 < wa) w = *reinterpret_cast<const fla::u32x4 *>(a + b * as_b + h * as_h + n * as_n + c8);
+        if (c8 < wa) {
+            w = *reinterpret_cast<const fla::u32x4 *>(a + b * as_b + h * as_h + n * as_n + c8);
+        } else if (c8 == wa && bias_mode) {
+            const T one = static_cast<T>(bias_mode == 1 ? bias[row] : 1.0f);
+            w[0] = (uint32_t)__builtin_bit_cast(unsigned short, one);
+        }
     } else if (c8 - split < wx) {
         w = *reinterpret_cast<const fla::u32x4 *>(x + b * xs_b + h * xs_h + n * xs_n + (c8 - split));
     }
     *reinterpret_cast<fla::u32x4 *>(out + row * (split + rp) + c8) = w;
 }
 
+template <typename T>
+void launch_pack(const View &a, int wa, const View &x, int wx, void *out, int64_t B, int64_t H, int64_t N, int split,
+                 int rp, int bias_mode, const float *bias, hipStream_t s) {
+    const int64_t total = B * H * N * ((split + rp) / 8);
+    hipLaunchKernelGGL((pack_pair_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+                       static_cast<const T *>(a.ptr), a.strides[0], a.strides[1], a.strides[2], wa,
+                       static_cast<const T *>(x.ptr), x.strides[0], x.strides[1], x.strides[2], wx,
+                       static_cast<T *>(out), (int)H, N, split, rp, total, bias_mode, bias);
+}
+
 struct PolyLayout {
     int64_t split, rp, width, packed_bytes;
+    int mode;  // TriParams::poly_on of the dual-score products: 2 (half layout) or 3 (tail layout)
+    // normalised backward: dO = g / n and dn, then the packed operands
+    int64_t do_bytes, dn_bytes;
 };
 
-// split: where the second operand starts = half of the padded contraction the dual-score kernel is
-// built for; rp: r rounded up to whole 16-byte chunks
-PolyLayout poly_layout(int64_t B, int64_t H, int64_t N, int64_t r, int64_t dv) {
+// split: where the second operand starts; rp: r rounded up to whole 16-byte chunks.  Without the
+// bias column the first operand is padded to half of the contraction the dual-score kernel is built
+// for (the kernel skips the empty chunks); with it (normalised backward) D_v + 1 columns are needed,
+// and when those do not fit the half the second operand goes to the last 32 columns instead.
+PolyLayout poly_layout(int64_t B, int64_t H, int64_t N, int64_t r, int64_t dv, int with_bias) {
     PolyLayout l;
-    l.split = dv <= 32 ? 32 : dv <= 64 ? 64 : 128;
-    l.rp = (r + 7) / 8 * 8;
+    const int64_t need = dv + (with_bias ? 8 : 0);  // the bias takes a 16-byte chunk of its own
+    const int64_t half = need <= 32 ? 32 : need <= 64 ? 64 : need <= 128 ? 128 : 0;
+    const int64_t dc_tail = need + 32 <= 64 ? 64 : need + 32 <= 128 ? 128 : 256;
+    if (half != 0 && 2 * half <= dc_tail) {
+        l.split = half, l.mode = 2;
+    } else {
+        l.split = dc_tail - 32, l.mode = 3;
+    }
+    l.rp = l.mode == 3 ? 32 : (r + 7) / 8 * 8;
     l.width = l.split + l.rp;
     l.packed_bytes = (B * H * N * l.width * 2 + 15) / 16 * 16;
+    l.do_bytes = with_bias ? (B * H * N * dv * 2 + 15) / 16 * 16 : 0;
+    l.dn_bytes = with_bias ? (B * H * N * 4 + 15) / 16 * 16 : 0;
     return l;
 }
 
@@ -553,43 +585,68 @@ int poly_forward(const View &xq, const View &xk, const View &v, const View &o, f
     return launch_poly(p, r, dv, dtype, 1, coef[0], coef[1], coef[2], stream);
 }
 
-int poly_backward(const View &go, const View &xq, const View &xk, const View &v, const View &dxq, const View &dxk,
-                  const View &dvv, int64_t B, int64_t H, int64_t N, int64_t r, int64_t dv, const float *coef,
-                  int dtype, void *workspace, int64_t workspace_bytes, void *stream) {
+int poly_backward(const View &go, const View &xq, const View &xk, const View &v, const View *o, const float *denom,
+                  const View &dxq, const View &dxk, const View &dvv, int64_t B, int64_t H, int64_t N, int64_t r,
+                  int64_t dv, const float *coef, int dtype, void *workspace, int64_t workspace_bytes, void *stream) {
     const View all[] = {go, xq, xk, v, dxq, dxk, dvv};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
+    const bool normalised = o != nullptr;
+    if (normalised) {
+        if (int rc = check_view(*o)) return rc;
+        if (!denom) return FLA_ERR_NULL_POINTER;
+        if (B * H > 65535) return FLA_ERR_SHAPE;
+    }
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
-    const PolyLayout l = poly_layout(B, H, N, r, dv);
-    if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < 2 * l.packed_bytes)
+    const PolyLayout l = poly_layout(B, H, N, r, dv, normalised);
+    if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 ||
+        workspace_bytes < 2 * l.packed_bytes + l.do_bytes + l.dn_bytes)
         return FLA_ERR_WORKSPACE;
     // the packing kernel and the products below use 16-byte accesses throughout
     if (!(vec_ok(go, dv) && vec_ok(v, dv) && vec_ok(xq, r) && vec_ok(xk, r) && vec_ok(dxq, r) && vec_ok(dxk, r) &&
           vec_ok(dvv, dv)))
         return FLA_ERR_UNSUPPORTED;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    uint16_t *p1 = static_cast<uint16_t *>(workspace);                                               // [dO | xq]
-    uint16_t *p2 = reinterpret_cast<uint16_t *>(static_cast<char *>(workspace) + l.packed_bytes);    // [V | xk]
-    const int64_t total = B * H * N * (l.width / 8);
-    const dim3 grid((unsigned)((total + 255) / 256));
-    hipLaunchKernelGGL(pack_pair_kernel, grid, dim3(256), 0, s, static_cast<const uint16_t *>(go.ptr), go.strides[0],
-                       go.strides[1], go.strides[2], (int)dv, static_cast<const uint16_t *>(xq.ptr), xq.strides[0],
-                       xq.strides[1], xq.strides[2], (int)r, p1, (int)H, N, (int)l.split, (int)l.rp, total);
-    hipLaunchKernelGGL(pack_pair_kernel, grid, dim3(256), 0, s, static_cast<const uint16_t *>(v.ptr), v.strides[0],
-                       v.strides[1], v.strides[2], (int)dv, static_cast<const uint16_t *>(xk.ptr), xk.strides[0],
-                       xk.strides[1], xk.strides[2], (int)r, p2, (int)H, N, (int)l.split, (int)l.rp, total);
+    char *ws = static_cast<char *>(workspace);
+    void *p1 = ws, *p2 = ws + l.packed_bytes;  // [dO (| dn) | xq], [V (| 1) | xk]
+    void *dO = ws + 2 * l.packed_bytes;
+    float *dn = reinterpret_cast<float *>(ws + 2 * l.packed_bytes + l.do_bytes);
+    const int64_t do_strides[4] = {H * N * dv, N * dv, dv, 1};
+    View g = go;
+    if (normalised) {
+        // out = O / n: dO = g / n, dn = -(g . out) / n; the dn term enters u1 as a bias column
+        const int lpr = fla::norm_lanes_per_row((int)dv);
+        fla::NormParams np{};
+        np.H = (int32_t)H, np.N = (int32_t)N, np.BH = (int32_t)(B * H), np.dqk = (int32_t)dv, np.dv = (int32_t)dv;
+        const int64_t rows = fla::norm_chunk_rows(lpr);
+        np.n_chunks = (int32_t)((N + rows - 1) / rows);
+        np.denom = const_cast<float *>(denom), np.dn = dn;
+        np.a = go.ptr, np.as_b = go.strides[0], np.as_h = go.strides[1], np.as_n = go.strides[2], np.vec_a = vec_ok(go, dv);
+        np.b = o->ptr, np.bs_b = o->strides[0], np.bs_h = o->strides[1], np.bs_n = o->strides[2], np.vec_b = vec_ok(*o, dv);
+        np.out = dO, np.os_b = do_strides[0], np.os_h = do_strides[1], np.os_n = do_strides[2], np.vec_out = 1;
+        if (norm_launch(1, dtype, lpr, np, stream) != hipSuccess) return FLA_ERR_LAUNCH;
+        g = View{dO, do_strides};
+    }
+    const int bias1 = normalised ? 1 : 0, bias2 = normalised ? 2 : 0;
+    if (dtype == FLA_DTYPE_BF16) {
+        launch_pack<__bf16>(g, (int)dv, xq, (int)r, p1, B, H, N, (int)l.split, (int)l.rp, bias1, dn, s);
+        launch_pack<__bf16>(v, (int)dv, xk, (int)r, p2, B, H, N, (int)l.split, (int)l.rp, bias2, nullptr, s);
+    } else {
+        launch_pack<_Float16>(g, (int)dv, xq, (int)r, p1, B, H, N, (int)l.split, (int)l.rp, bias1, dn, s);
+        launch_pack<_Float16>(v, (int)dv, xk, (int)r, p2, B, H, N, (int)l.split, (int)l.rp, bias2, nullptr, s);
+    }
     if (hipGetLastError() != hipSuccess) return FLA_ERR_LAUNCH;
     const int64_t ps[4] = {H * N * l.width, N * l.width, l.width, 1};
     const View P1{p1, ps}, P2{p2, ps};
     // dV = upper(f(Xk Xq^T)) dO
-    const TriParams pv = make_params(xk, xq, go, dvv, B, H, N, r, dv, 1);
-    // dXq = lower((dO V^T) f'(Xq Xk^T)) Xk, dXk = upper((V dO^T) f'(Xk Xq^T)) Xq; f'(u) = c1 + 2 c2 u
+    const TriParams pv = make_params(xk, xq, g, dvv, B, H, N, r, dv, 1);
+    // dXq = lower((dO V^T + dn 1^T) f'(Xq Xk^T)) Xk, dXk = upper((V dO^T + 1 dn^T) f'(Xk Xq^T)) Xq; f'(u) = c1 + 2 c2 u
     const TriParams pq = make_params(P1, P2, xk, dxq, B, H, N, l.width, r, 0);
     const TriParams pk = make_params(P2, P1, xq, dxk, B, H, N, l.width, r, 1);
     if (!poly_ok(pv, r, dv) || !poly_ok(pq, l.width, r) || !poly_ok(pk, l.width, r)) return FLA_ERR_UNSUPPORTED;
     if (int rc = launch_poly(pv, r, dv, dtype, 1, coef[0], coef[1], coef[2], stream)) return rc;
-    if (int rc = launch_poly(pq, l.width, r, dtype, 2, coef[1], 2.0f * coef[2], 0.f, stream)) return rc;
-    return launch_poly(pk, l.width, r, dtype, 2, coef[1], 2.0f * coef[2], 0.f, stream);
+    if (int rc = launch_poly(pq, l.width, r, dtype, l.mode, coef[1], 2.0f * coef[2], 0.f, stream)) return rc;
+    return launch_poly(pk, l.width, r, dtype, l.mode, coef[1], 2.0f * coef[2], 0.f, stream);
 }
 
 }  // namespace
@@ -725,7 +782,8 @@ int fla_linear_attn_chunked_bwd(const void *grad_out, const void *q, const void 
 
 int64_t fla_poly_attn_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t R, int64_t D_v) {
     if (B < 0 || H < 0 || N < 0 || R < 1 || R > 32 || D_v < 1 || D_v > 128) return 0;
-    return 2 * poly_layout(B, H, N, R, D_v).packed_bytes;
+    const PolyLayout l = poly_layout(B, H, N, R, D_v, 1);  // the normalised backward needs the most
+    return 2 * l.packed_bytes + l.do_bytes + l.dn_bytes;
 }
 
 int fla_poly_attn_fwd(const void *xq, const void *xk, const void *v, void *o, float *denom, int64_t B, int64_t H,
@@ -737,15 +795,17 @@ int fla_poly_attn_fwd(const void *xq, const void *xk, const void *v, void *o, fl
                         coef, eps, dtype, stream);
 }
 
-int fla_poly_attn_bwd(const void *grad_out, const void *xq, const void *xk, const void *v, void *dxq, void *dxk,
-                      void *dv, int64_t B, int64_t H, int64_t N, int64_t R, int64_t D_v, const int64_t *go_strides,
-                      const int64_t *xq_strides, const int64_t *xk_strides, const int64_t *v_strides,
-                      const int64_t *dxq_strides, const int64_t *dxk_strides, const int64_t *dv_strides,
-                      const float *coef, int dtype, void *workspace, int64_t workspace_bytes, void *stream) {
+int fla_poly_attn_bwd(const void *grad_out, const void *xq, const void *xk, const void *v, const void *o,
+                      const float *denom, void *dxq, void *dxk, void *dv, int64_t B, int64_t H, int64_t N, int64_t R,
+                      int64_t D_v, const int64_t *go_strides, const int64_t *xq_strides, const int64_t *xk_strides,
+                      const int64_t *v_strides, const int64_t *o_strides, const int64_t *dxq_strides,
+                      const int64_t *dxk_strides, const int64_t *dv_strides, const float *coef, int dtype,
+                      void *workspace, int64_t workspace_bytes, void *stream) {
     if (int rc = check_poly_args(B, H, N, R, D_v, dtype, coef)) return rc;
+    const View ov{o, o_strides};
     return poly_backward({grad_out, go_strides}, {xq, xq_strides}, {xk, xk_strides}, {v, v_strides},
-                         {dxq, dxq_strides}, {dxk, dxk_strides}, {dv, dv_strides}, B, H, N, R, D_v, coef, dtype,
-                         workspace, workspace_bytes, stream);
+                         o ? &ov : nullptr, denom, {dxq, dxq_strides}, {dxk, dxk_strides}, {dv, dv_strides}, B, H, N,
+                         R, D_v, coef, dtype, workspace, workspace_bytes, stream);
 }
 
 int64_t fla_normalised_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v, int chunked) {

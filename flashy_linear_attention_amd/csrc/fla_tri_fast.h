@@ -157,7 +157,10 @@ __device__ __forceinline__ int swizzle_z(int row) {
 // u1, columns [D_c/2, D_c/2 + 32) give u2, and the score is u1 (poly[0] + poly[1] u2 + poly[2] u2^2):
 // the gradient of the polynomial score map with respect to its argument, e.g.
 // lower((dO V^T) . f'(Xq Xk^T)) Xk with X = [dO | xq] and Y = [V | xk] packed side by side.
-constexpr int kNormFlag = 1, kPolyFlag = 2, kDualFlag = 4;
+// kTailFlag (with kDualFlag): the second operand sits in the last 32 columns of the padded
+// contraction instead, [D_c - 32, D_c), which leaves the first one D_c - 32 columns -- room for an
+// extra column that adds a per-row bias to u1 ([.. | b_i] . [.. | 1]).
+constexpr int kNormFlag = 1, kPolyFlag = 2, kDualFlag = 4, kTailFlag = 8;
 constexpr int kPolyMaxContraction = 64;  // polynomial variants are built for D_c <= 64 only
 
 template <typename T, int DC, int DO, bool CHUNKED, int FLAGS = 0>
@@ -181,7 +184,9 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     constexpr int STAGE = Cfg::STAGE_BYTES, Y_BYTES = Cfg::Y_BYTES;
     // chunks of the contraction that feed the first score / that are used at all (DUAL: the
     // second score takes two chunks, 32 columns, right after the first half)
-    constexpr int KC1 = DUAL ? KC / 2 : KC, KCU = DUAL ? KC / 2 + 2 : KC;
+    constexpr bool TAIL = (FLAGS & kTailFlag) != 0;
+    static_assert(!TAIL || DUAL, "the tail layout is a layout of the dual-score walk");
+    constexpr int KC1 = !DUAL ? KC : TAIL ? KC - 2 : KC / 2, KCU = (DUAL && !TAIL) ? KC / 2 + 2 : KC;
     constexpr int YQ = KC < 4 ? KC : 4;  // Y read addresses that differ by more than an immediate
     constexpr int ZQ = DB < 2 ? DB : 2;  // same for Z
 
@@ -875,6 +880,14 @@ hipError_t launch_tri_fast(const TriParams &p, hipStream_t stream) {
     if (p.poly_on == 2) {  // dual-score walk: built for 32-wide outputs (the argument of the score map)
         if constexpr (DC >= 64 && DO == 32) {
             return p.denom ? hipErrorNotSupported : launch_tri_fast_variant<T, DC, DO, false, kDualFlag>(p, stream);
+        } else {
+            return hipErrorNotSupported;
+        }
+    }
+    if (p.poly_on == 3) {  // dual-score walk, second operand in the last 32 columns
+        if constexpr (DC >= 64 && DO == 32) {
+            return p.denom ? hipErrorNotSupported
+                           : launch_tri_fast_variant<T, DC, DO, false, kDualFlag | kTailFlag>(p, stream);
         } else {
             return hipErrorNotSupported;
         }

@@ -67,7 +67,8 @@ struct TriParams {
     // causal linear attention with a second-order Taylor feature map, the features never built.
     // poly_on == 2: dual-score walk (32-wide outputs only).  X and Y carry two operands side by side,
     // columns [0, DC/2) and [DC/2, DC/2 + 32) of the instantiation's padded width DC; the score is
-    // u1 (poly[0] + poly[1] u2 + poly[2] u2^2).
+    // u1 (poly[0] + poly[1] u2 + poly[2] u2^2).  poly_on == 3: the same with the second operand in the
+    // last 32 columns, [DC - 32, DC).
     float poly[3];
     int32_t poly_on;
 #ifdef FLA_DBG_TIMING

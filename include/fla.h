@@ -179,11 +179,14 @@ int fla_linear_attn_chunked_bwd(const void *grad_out, const void *q, const void 
  * x, coef = {0, 0, 1/2}; the full Taylor map is {1, 1, 1/2}) -- with the features never built:
  * scores cost an R-wide contraction instead of an R^2-wide one.  xq, xk: (B, H, N, R), R <= 32;
  * v, o: (B, H, N, D_v), D_v <= 128.  When `denom` is non-NULL the output rows are divided by
- * n = (row sum of the masked scores) + eps and n is stored there (fp32, contiguous (B, H, N));
- * backward is for the un-normalised product (denom == NULL).  Backward forms
+ * n = (row sum of the masked scores) + eps and n is stored there (fp32, contiguous (B, H, N)).
+ * Backward forms
  *     dV  = upper(f(Xk Xq^T)) dO
  *     dXq = lower((dO V^T) . f'(Xq Xk^T)) Xk,   dXk = upper((V dO^T) . f'(Xk Xq^T)) Xq
- * and needs fla_poly_attn_workspace_bytes() bytes of 16-byte aligned scratch.  Fast-path kernels
+ * and needs fla_poly_attn_workspace_bytes() bytes of 16-byte aligned scratch.  For the
+ * normalised forward pass the forward's `o` and `denom` to backward (both NULL otherwise): dO
+ * becomes g / n, and the normaliser's own gradient dn = -(g . o) / n enters the first score of
+ * dXq and dXk as a bias (dO V^T + dn 1^T); B*H must then not exceed 65535.  Fast-path kernels
  * only: every operand 16-byte aligned with widths and outer strides multiples of 8 elements,
  * else FLA_ERR_UNSUPPORTED.  No counterpart in the reference (it multiplies materialised
  * features, linear_attn_kernels_smallv_hd.py:78-86). */
@@ -194,10 +197,11 @@ int fla_poly_attn_fwd(const void *xq, const void *xk, const void *v, void *o, fl
                       const int64_t *v_strides, const int64_t *o_strides,
                       const float *coef, float eps, int dtype, void *stream);
 int fla_poly_attn_bwd(const void *grad_out, const void *xq, const void *xk, const void *v,
+                      const void *o, const float *denom,
                       void *dxq, void *dxk, void *dv,
                       int64_t B, int64_t H, int64_t N, int64_t R, int64_t D_v,
                       const int64_t *go_strides, const int64_t *xq_strides,
-                      const int64_t *xk_strides, const int64_t *v_strides,
+                      const int64_t *xk_strides, const int64_t *v_strides, const int64_t *o_strides,
                       const int64_t *dxq_strides, const int64_t *dxk_strides,
                       const int64_t *dv_strides,
                       const float *coef, int dtype, void *workspace, int64_t workspace_bytes, void *stream);

@@ -151,6 +151,19 @@ def poly_causal_dot_product(
     return torch.matmul(scores, v)
 
 
+def poly_linear_attention_normalised(
+    xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, coef: Tuple[float, float, float], eps: float = 1e-5
+) -> torch.Tensor:
+    """:func:`linear_attention_normalised` on ``taylor2_features`` of xq and xk without the
+    features: every row of :func:`poly_causal_dot_product` divided by the sum of its masked
+    scores plus eps (differentiable; tests/test_oracle.py checks it against the explicit form)."""
+    c0, c1, c2 = coef
+    n = xq.shape[-2]
+    u = torch.matmul(xq, xk.transpose(-2, -1))
+    scores = (c0 + c1 * u + c2 * u * u) * _tril_mask(n, xq.device).to(u.dtype)
+    return torch.matmul(scores, v) / (scores.sum(dim=-1, keepdim=True) + eps)
+
+
 def poly_causal_dot_product_grads(
     xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, do: torch.Tensor, coef: Tuple[float, float, float]
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:

@@ -181,3 +181,24 @@ def test_polynomial_score_map_equals_explicit_features(coef):
     # the reference's feature recipe for the small-V operator is the pure square with c2 = 1/2
     phi = (xq[..., :, None] * xq[..., None, :]).flatten(-2) / 2 ** 0.5
     assert torch.allclose(naive.taylor2_features(xq, (0.0, 0.0, 0.5)), phi)
+
+
+def test_normalised_polynomial_equals_normalised_recipe_on_explicit_features():
+    """The normalised polynomial form against the reference's README recipe (cumsum-based
+    normaliser) applied to the explicit features: two routes to the row sums (masked scores
+    summed / q . cumsum(k)), output and gradients by autograd on both, in fp64."""
+    coef = (1.0, 1.0, 0.5)  # positive scores
+    g = torch.Generator().manual_seed(8)
+    xq = torch.randn(1, 3, 33, 5, generator=g, dtype=torch.float64)
+    xk = torch.randn(1, 3, 33, 5, generator=g, dtype=torch.float64)
+    v = torch.randn(1, 3, 33, 7, generator=g, dtype=torch.float64)
+    do = torch.randn(1, 3, 33, 7, generator=g, dtype=torch.float64)
+    a, b, c = (t.clone().requires_grad_(True) for t in (xq, xk, v))
+    ref = naive.linear_attention_normalised(naive.taylor2_features(a, coef), naive.taylor2_features(b, coef), c, 1e-6)
+    ref.backward(do)
+    a2, b2, c2 = (t.clone().requires_grad_(True) for t in (xq, xk, v))
+    got = naive.poly_linear_attention_normalised(a2, b2, c2, coef, 1e-6)
+    got.backward(do)
+    assert torch.allclose(got.detach(), ref.detach(), rtol=1e-11, atol=1e-11)
+    for x, y in ((a2.grad, a.grad), (b2.grad, b.grad), (c2.grad, c.grad)):
+        assert torch.allclose(x, y, rtol=1e-10, atol=1e-10)
