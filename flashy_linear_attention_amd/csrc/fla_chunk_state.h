@@ -71,11 +71,13 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(const ChunkStateParams
     // whole chunk -> LDS (rows beyond N and columns beyond the true widths arrive as zeros);
     // same lane -> chunk assignment as the main kernel's tile loads
     constexpr int YSTEP = 4 * (1024 / RY), ZSTEP = 4 * (1024 / RZ);
-    uint32_t ydma, zdma;
-    {
-        const int row = wave * (1024 / RY) + lane / CY;
+    constexpr int NYD = Cfg::NYD;
+    uint32_t ydma[NYD], zdma;
+#pragma unroll
+    for (int v = 0; v < NYD; ++v) {
+        const int row = v * YSTEP + wave * (1024 / RY) + lane / CY;
         const int c = (lane % CY) ^ swizzle_y<CY>(row);
-        ydma = (uint32_t)(row * ys2 + c * 16) + (c * 8 < p.dc ? 0u : kOobOffset);
+        ydma[v] = (uint32_t)(row * ys2 + c * 16) + (c * 8 < p.dc ? 0u : kOobOffset);
     }
     {
         const int row = wave * (1024 / RZ) + lane / CZ;
@@ -88,7 +90,8 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(const ChunkStateParams
         const int row0 = r0 + t * BN;
         static_for<0, NIY>([&](auto u) {
             constexpr int U = decltype(u)::value;
-            dma_16B_per_lane<t * STAGE + U * 4096>(ry, lds_wave, ydma, (uint32_t)((row0 + U * YSTEP) * ys2));
+            dma_16B_per_lane<t * STAGE + U * 4096>(ry, lds_wave, ydma[U % NYD],
+                                                   (uint32_t)((row0 + (U - U % NYD) * YSTEP) * ys2));
         });
         static_for<0, NIZ>([&](auto u) {
             constexpr int U = decltype(u)::value;

@@ -50,6 +50,9 @@ typedef short s16x8 __attribute__((ext_vector_type(8)));
 // written: the loads of one tile then need a single scalar base between them.
 template <int LDS_IMM>
 __device__ __forceinline__ void dma_16B_per_lane(u32x4 rsrc, uint32_t lds_base, uint32_t voffset, uint32_t soffset) {
+#ifdef FLA_DBG_NO_DMA
+    return;
+#endif
     asm volatile("s_add_u32 m0, %0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset), "n"(LDS_IMM)
@@ -92,12 +95,17 @@ __device__ __forceinline__ uint32_t round_pack_pinned(float lo, float hi) {
     pr[0] = static_cast<T>(lo);
     pr[1] = static_cast<T>(hi);
     uint32_t r = __builtin_bit_cast(uint32_t, pr);
+#ifdef FLA_DBG_NO_CVT
+    r = __builtin_bit_cast(uint32_t, lo);
+#endif
     asm volatile("" : "+v"(r));
     return r;
 }
 
 constexpr uint32_t kOobOffset = 0x40000000u;  // added to a buffer offset to force an out-of-range (zero) access
 constexpr int64_t kMaxFastExtent = 0x3fffffff;  // per-(b,h) byte extent the 32-bit buffer offsets can address
+
+constexpr int kSwizzlePeriodY = 16;  // rows after which swizzle_y (below) repeats
 
 // CHUNKED = false: the quadratic walk over all tiles under the mask; true: chunk-wise evaluation
 // (diagonal block plus running state), compiled as a kernel of its own.
@@ -131,6 +139,9 @@ struct FastConfig {
     // wave-level 1 KiB DMA instructions per tile and wave
     static constexpr int NIY = Y_BYTES / 4096, NIZ = Z_BYTES / 4096;
     static constexpr int NT = NIY + NIZ;  // buffer loads per wave and tile
+    // distinct per-lane source offsets among the Y loads of a tile (see swizzle_y)
+    static constexpr int NYD = (4 * (1024 / RY)) % kSwizzlePeriodY == 0 ? 1 : 2;
+    static_assert((NYD * 4 * (1024 / RY)) % kSwizzlePeriodY == 0 && (NIY % NYD) == 0, "Y swizzle period");
     // output staging in LDS: BM rows of DO 16-bit values, 16 bytes of padding per row
     static constexpr int RO = DO * 2 + 16;
     static_assert(BM * RO <= SMEM_BYTES, "output staging must fit in the ring");
@@ -138,10 +149,17 @@ struct FastConfig {
 };
 
 // XOR applied to the chunk index of LDS row `row` (row counted inside the tile).
+// Y: a 16-byte-per-lane read is served 16 lanes at a time out of 64 banks of 4 bytes, and the 16
+// lanes read one chunk index of 16 consecutive rows: the 16 rows must land in the 16 different
+// 16-byte slots of a 256-byte window (measured: 4-5 clocks per instruction then, 8 with only 8
+// slots covered).  Rows of 256 bytes and more all start at bank 0, so the row's low 4 bits go
+// into the chunk index; with 128- / 64-byte rows the low 1 / 2 row bits already pick a different
+// part of the window and the next 3 / 2 bits are folded in.
 template <int CY>
 __device__ __forceinline__ int swizzle_y(int row) {
-    if constexpr (CY == 4) return (row >> 1) & 3;  // 64-byte rows: two rows share 128 bytes
-    else return row & 7;  // 8 consecutive rows hit 8 different 16-byte slots of a 128-byte window
+    if constexpr (CY == 4) return (row >> 2) & 3;
+    else if constexpr (CY == 8) return (row >> 1) & 7;
+    else return row & 15;
 }
 template <int CZ>
 __device__ __forceinline__ int swizzle_z(int row) {
@@ -187,7 +205,7 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     constexpr bool TAIL = (FLAGS & kTailFlag) != 0;
     static_assert(!TAIL || DUAL, "the tail layout is a layout of the dual-score walk");
     constexpr int KC1 = !DUAL ? KC : TAIL ? KC - 2 : KC / 2, KCU = (DUAL && !TAIL) ? KC / 2 + 2 : KC;
-    constexpr int YQ = KC < 4 ? KC : 4;  // Y read addresses that differ by more than an immediate
+    constexpr int YQ = KC < 8 ? KC : 8;  // Y read addresses that differ by more than an immediate
     constexpr int ZQ = DB < 2 ? DB : 2;  // same for Z
 
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -267,17 +285,19 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     const int n_seq = n_full + n_diag;
 
     // ---- HBM -> LDS: per-lane source offsets (constant over tiles).  Load u of a wave covers
-    // rows u * YSTEP + wave * (1024 / RY) + lane / CY of the tile; YSTEP is a multiple of the
-    // swizzle period, so the lane's chunk is the same for every u and the row advance goes into
-    // the scalar offset: one address register per operand, no vector work per load.
+    // rows u * YSTEP + wave * (1024 / RY) + lane / CY of the tile.  Where YSTEP is a multiple of
+    // the swizzle period the lane's chunk is the same for every u and the row advance goes into
+    // the scalar offset: one address register per operand, no vector work per load (512-byte Y
+    // rows: the period is two steps, so two registers, for even and odd u).
     constexpr int YSTEP = 4 * (1024 / RY), ZSTEP = 4 * (1024 / RZ);
-    static_assert(NIY == 1 || YSTEP % 8 == 0, "Y swizzle must not depend on the load index");
+    constexpr int NYD = Cfg::NYD;
     static_assert(NIZ == 1 || ZSTEP % 4 == 0, "Z swizzle must not depend on the load index");
-    uint32_t ydma, zdma;
-    {
-        const int row = wave * (1024 / RY) + lane / CY;
+    uint32_t ydma[NYD], zdma;
+#pragma unroll
+    for (int v = 0; v < NYD; ++v) {
+        const int row = v * YSTEP + wave * (1024 / RY) + lane / CY;
         const int c = (lane % CY) ^ swizzle_y<CY>(row);
-        ydma = (uint32_t)(row * ys2 + c * 16) + (c * 8 < p.dc ? 0u : kOobOffset);
+        ydma[v] = (uint32_t)(row * ys2 + c * 16) + (c * 8 < p.dc ? 0u : kOobOffset);
     }
     {
         const int row = wave * (1024 / RZ) + lane / CZ;
@@ -286,18 +306,30 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     }
     const uint32_t lds_wave = lds0 + wave * 1024;
     // tile q of the sequence -> ring slot q % NBUF, tracked incrementally by the caller
+    auto tile_row0 = [&](int q) { return q < n_full ? full_row0 + q * BN : i0 + (q - n_full) * BN; };
+    // load I of the NT wave-level loads of the tile whose first row is row0, into the slot at yb
+    auto issue_part = [&](auto ii, int row0, uint32_t yb) {
+        constexpr int I = decltype(ii)::value;
+        if constexpr (I < NIY) {
+            dma_16B_per_lane<I * 4096>(ry, yb, ydma[I % NYD], (uint32_t)((row0 + (I - I % NYD) * YSTEP) * ys2));
+        } else {
+            constexpr int U = I - NIY;
+            dma_16B_per_lane<Y_BYTES + U * 4096>(rz, yb, zdma, (uint32_t)((row0 + U * ZSTEP) * zs2));
+        }
+    };
+    // the same with the scalar offset given (kOobOffset: a tile that does not exist, zeros arrive)
+    auto issue_part_at = [&](auto ii, uint32_t soffset, uint32_t yb) {
+        constexpr int I = decltype(ii)::value;
+        if constexpr (I < NIY)
+            dma_16B_per_lane<I * 4096>(ry, yb, ydma[I % NYD], soffset);
+        else
+            dma_16B_per_lane<Y_BYTES + (I - NIY) * 4096>(rz, yb, zdma, soffset);
+    };
     auto issue_tile = [&](int q, int slot_off) {
         if (q < n_seq) {
-            const int row0 = q < n_full ? full_row0 + q * BN : i0 + (q - n_full) * BN;
+            const int row0 = tile_row0(q);
             const uint32_t yb = lds_wave + slot_off;
-            static_for<0, NIY>([&](auto u) {
-                constexpr int U = decltype(u)::value;
-                dma_16B_per_lane<U * 4096>(ry, yb, ydma, (uint32_t)((row0 + U * YSTEP) * ys2));
-            });
-            static_for<0, NIZ>([&](auto u) {
-                constexpr int U = decltype(u)::value;
-                dma_16B_per_lane<Y_BYTES + U * 4096>(rz, yb, zdma, (uint32_t)((row0 + U * ZSTEP) * zs2));
-            });
+            static_for<0, Cfg::NT>([&](auto ii) { issue_part(ii, row0, yb); });
         }
     };
     auto next_slot = [](int off) { return off + STAGE == Cfg::NBUF * STAGE ? 0 : off + STAGE; };
@@ -427,14 +459,18 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
                     });
                 } else {
                     // [DO rows][DC] in the Y tile layout
-                    const int row = wave * (1024 / RY) + lane / CY;
-                    const uint32_t sdma = (uint32_t)(row * RY + (((lane % CY) ^ swizzle_y<CY>(row)) << 4));
+                    uint32_t sdma[NYD];
+#pragma unroll
+                    for (int v = 0; v < NYD; ++v) {
+                        const int row = v * YSTEP + wave * (1024 / RY) + lane / CY;
+                        sdma[v] = (uint32_t)(row * RY + (((lane % CY) ^ swizzle_y<CY>(row)) << 4));
+                    }
                     static_for<0, Cfg::STATE_BYTES / Y_BYTES>([&](auto uu) {
                         constexpr int UNIT = decltype(uu)::value;
                         static_for<0, NIY>([&](auto u) {
                             constexpr int U = decltype(u)::value;
                             dma_16B_per_lane<Cfg::SMEM_BYTES + UNIT * Y_BYTES + U * 4096>(
-                                rs, lds_wave, sdma, (uint32_t)((UNIT * 64 + U * YSTEP) * RY));
+                                rs, lds_wave, sdma[U % NYD], (uint32_t)((UNIT * 64 + (U - U % NYD) * YSTEP) * RY));
                         });
                     });
                 }
@@ -502,11 +538,11 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         // phase 2: Out += P_prev Z_prev, interleaved with the Y fragment reads of the next sub-tile
         // and the rounding of S into `pcur`
         auto phase2 = [&](auto with_pv, V8 (&pprev)[NIB][2], V8 (&pcur)[NIB][2], const int (&ya)[YQ], int ysub,
-                          auto &&after_first_group) {
+                          auto &&after_group) {
             constexpr int NPK = NIB * 8;  // packed pairs that make up P of one sub-tile
             u32x4 pk[NIB][2];
-#pragma unroll
-            for (int f = 0; f < NZF; ++f) {
+            static_for<0, NZF>([&](auto ff) {
+                constexpr int f = decltype(ff)::value;
                 if constexpr (decltype(with_pv)::value) {
                     const int t = f / DB, db = f % DB;
 #pragma unroll
@@ -548,9 +584,9 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
                         pk[ib][t][w] = round_pack_pinned<T>(s[ib][8 * t + 2 * w], s[ib][8 * t + 2 * w + 1]);
                     }
                 }
-                if (f == 0) after_first_group();
+                after_group(ff);
                 __builtin_amdgcn_sched_barrier(0);
-            }
+            });
 #pragma unroll
             for (int ib = 0; ib < NIB; ++ib)
 #pragma unroll
@@ -564,7 +600,7 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
             slot_addrs(next_off, ya_next, unused_z);
             // first sub-tile: Z of the previous tile's second sub-tile, then Y of this tile's second
             phase1(std::integral_constant<bool, !kFirst>{}, za_prev, 1);
-            phase2(std::integral_constant<bool, !kFirst>{}, pfb, pfa, ya_cur, 1, [] {});
+            phase2(std::integral_constant<bool, !kFirst>{}, pfb, pfa, ya_cur, 1, [](auto) {});
             // second sub-tile
             phase1(std::true_type{}, za_cur, 0);
 #ifndef FLA_DBG_NO_WAIT
@@ -573,12 +609,41 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
 #ifndef FLA_DBG_NO_BARRIER
             __builtin_amdgcn_s_barrier();  // tile q+1 has landed; nobody reads tile q-1 any more
 #endif
-#ifdef FLA_DMA_LATE
-            phase2(std::true_type{}, pfa, pfb, ya_next, 0, [&] { issue_tile(q + Cfg::NBUF - 1, issue_off); });
+#ifdef FLA_DMA_BURST
+            constexpr bool kSpread = false;
 #else
-            issue_tile(q + Cfg::NBUF - 1, issue_off);
-            phase2(std::true_type{}, pfa, pfb, ya_next, 0, [] {});
+            constexpr bool kSpread = FLAGS == 0;  // the variants with score maps have no registers to spare
 #endif
+            if constexpr (!kSpread) {
+                issue_tile(q + Cfg::NBUF - 1, issue_off);
+                phase2(std::true_type{}, pfa, pfb, ya_next, 0, [](auto) {});
+            } else
+            // The loads of tile q + NBUF - 1 go into the slot the barrier has just retired.  A wave
+            // issues one instruction every few clocks and a load to LDS holds it for longer than
+            // that, so all of them in a row would leave the matrix pipe idle: one (or a few) after
+            // each group of MFMAs instead.
+            {
+                // scalar offsets of all loads up front; past the end of the sequence the loads
+                // are issued all the same, out of range: zeros land in a slot nobody reads any
+                // more (the slot retired just now), and the instruction stream has no branch
+                const bool more = q + Cfg::NBUF - 1 < n_seq;
+                const int row0 = tile_row0(q + Cfg::NBUF - 1);
+                const uint32_t ybase = more ? (uint32_t)(row0 * ys2) : kOobOffset;
+                const uint32_t zbase = more ? (uint32_t)(row0 * zs2) : kOobOffset;
+                uint32_t so[Cfg::NT];
+                static_for<0, Cfg::NT>([&](auto ii) {
+                    constexpr int I = decltype(ii)::value;
+                    so[I] = I < NIY ? ybase + (uint32_t)((I - I % NYD) * YSTEP * ys2)
+                                    : zbase + (uint32_t)((I - NIY) * ZSTEP * zs2);
+                });
+                const uint32_t yb = lds_wave + issue_off;
+                phase2(std::true_type{}, pfa, pfb, ya_next, 0, [&](auto ff) {
+                    static_for<0, Cfg::NT>([&](auto ii) {
+                        if constexpr (decltype(ii)::value * NZF / Cfg::NT == decltype(ff)::value)
+                            issue_part_at(ii, so[decltype(ii)::value], yb);
+                    });
+                });
+            }
             advance();
             ++q;
         };
