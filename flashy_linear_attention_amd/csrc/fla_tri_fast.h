@@ -307,17 +307,7 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     const uint32_t lds_wave = lds0 + wave * 1024;
     // tile q of the sequence -> ring slot q % NBUF, tracked incrementally by the caller
     auto tile_row0 = [&](int q) { return q < n_full ? full_row0 + q * BN : i0 + (q - n_full) * BN; };
-    // load I of the NT wave-level loads of the tile whose first row is row0, into the slot at yb
-    auto issue_part = [&](auto ii, int row0, uint32_t yb) {
-        constexpr int I = decltype(ii)::value;
-        if constexpr (I < NIY) {
-            dma_16B_per_lane<I * 4096>(ry, yb, ydma[I % NYD], (uint32_t)((row0 + (I - I % NYD) * YSTEP) * ys2));
-        } else {
-            constexpr int U = I - NIY;
-            dma_16B_per_lane<Y_BYTES + U * 4096>(rz, yb, zdma, (uint32_t)((row0 + U * ZSTEP) * zs2));
-        }
-    };
-    // the same with the scalar offset given (kOobOffset: a tile that does not exist, zeros arrive)
+    // load I of the NT wave-level loads of a tile, into the slot at yb
     auto issue_part_at = [&](auto ii, uint32_t soffset, uint32_t yb) {
         constexpr int I = decltype(ii)::value;
         if constexpr (I < NIY)
@@ -325,23 +315,33 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         else
             dma_16B_per_lane<Y_BYTES + (I - NIY) * 4096>(rz, yb, zdma, soffset);
     };
+    // Scalar offsets of the NT loads of tile q.  A tile past the end of the sequence is loaded
+    // all the same, from out of range: zeros arrive in a slot nobody reads (callers only name
+    // slots that are free), and the count of loads in flight is the same at every step, which
+    // keeps branches out of the instruction stream and makes wait_tile a constant.
+    auto tile_offsets = [&](int q, uint32_t (&so)[Cfg::NT]) {
+        const bool exists = q < n_seq;
+        const int row0 = tile_row0(q);
+        const uint32_t ybase = exists ? (uint32_t)(row0 * ys2) : kOobOffset;
+        const uint32_t zbase = exists ? (uint32_t)(row0 * zs2) : kOobOffset;
+        static_for<0, Cfg::NT>([&](auto ii) {
+            constexpr int I = decltype(ii)::value;
+            so[I] = I < NIY ? ybase + (uint32_t)((I - I % NYD) * YSTEP * ys2) : zbase + (uint32_t)((I - NIY) * ZSTEP * zs2);
+        });
+    };
     auto issue_tile = [&](int q, int slot_off) {
-        if (q < n_seq) {
-            const int row0 = tile_row0(q);
-            const uint32_t yb = lds_wave + slot_off;
-            static_for<0, Cfg::NT>([&](auto ii) { issue_part(ii, row0, yb); });
-        }
+        uint32_t so[Cfg::NT];
+        tile_offsets(q, so);
+        const uint32_t yb = lds_wave + slot_off;
+        static_for<0, Cfg::NT>([&](auto ii) { issue_part_at(ii, so[decltype(ii)::value], yb); });
     };
     auto next_slot = [](int off) { return off + STAGE == Cfg::NBUF * STAGE ? 0 : off + STAGE; };
-    // Wait until tile `q` has landed, given that every tile up to q + NBUF - 3 has been issued:
-    // the loads of the NBUF - 3 tiles after it may stay in flight (when all of them exist).
-    auto wait_tile = [&](int q) {
+    // Wait until a tile has landed, given that exactly the NBUF - 3 tiles after it have been
+    // issued since: their loads may stay in flight.
+    auto wait_tile = [&]() {
         constexpr int AHEAD = Cfg::NBUF > 3 ? Cfg::NBUF - 3 : 0;
         static_assert(AHEAD * Cfg::NT < 64, "vmcnt is a 6-bit field");
-        if (AHEAD > 0 && q + AHEAD < n_seq)
-            wait_vm<AHEAD * Cfg::NT>();
-        else
-            wait_vm<0>();
+        wait_vm<AHEAD * Cfg::NT>();
     };
 
     issue_tile(0, 0);
@@ -435,7 +435,7 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     };
 
     // ring state: byte offsets of the slots of tile q-1, q, q+1 and of the next tile to issue
-    int prev_off = (Cfg::NBUF - 1) * STAGE, cur_off = 0, next_off = STAGE, issue_off = STAGE;
+    int prev_off = (Cfg::NBUF - 1) * STAGE, cur_off = 0, next_off = STAGE;
     const bool has_state = chunked && (upper ? tile + 1 < p.n_tiles : tile > 0);
     const T *st = has_state ? static_cast<const T *>(p.state) + ((int64_t)bh * p.n_tiles + tile) * (DO * DC) : nullptr;
     if constexpr (chunked) {
@@ -482,19 +482,17 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     } else {
         // tiles 1 .. NBUF-3 before the first wait, tile NBUF-2 right after it
         static_for<1, Cfg::NBUF - 2>([&](auto qq) { issue_tile(decltype(qq)::value, decltype(qq)::value * STAGE); });
-        issue_off = (Cfg::NBUF - 2) * STAGE;
-        wait_tile(0);
+        wait_tile();
         __builtin_amdgcn_s_barrier();  // tile 0 (and the X fragments) have landed
         FLA_STAMP(1);
-        issue_tile(Cfg::NBUF - 2, issue_off);
-        issue_off = next_slot(issue_off);
+        issue_tile(Cfg::NBUF - 2, (Cfg::NBUF - 2) * STAGE);
     }
-    // from here on: tiles up to q + NBUF - 2 are issued while tile q is consumed
+    // from here on: tiles up to q + NBUF - 2 are issued while tile q is consumed, and tile
+    // q + NBUF - 1 goes into the slot of tile q - 1 (prev_off) once that one is retired
     auto advance = [&]() {
         prev_off = cur_off;
         cur_off = next_off;
         next_off = next_slot(next_off);
-        issue_off = next_slot(issue_off);
     };
     int q = 0;
 
@@ -604,7 +602,7 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
             // second sub-tile
             phase1(std::true_type{}, za_cur, 0);
 #ifndef FLA_DBG_NO_WAIT
-            wait_tile(q + 1);
+            wait_tile();
 #endif
 #ifndef FLA_DBG_NO_BARRIER
             __builtin_amdgcn_s_barrier();  // tile q+1 has landed; nobody reads tile q-1 any more
@@ -615,7 +613,7 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
             constexpr bool kSpread = FLAGS == 0;  // the variants with score maps have no registers to spare
 #endif
             if constexpr (!kSpread) {
-                issue_tile(q + Cfg::NBUF - 1, issue_off);
+                issue_tile(q + Cfg::NBUF - 1, prev_off);
                 phase2(std::true_type{}, pfa, pfb, ya_next, 0, [](auto) {});
             } else
             // The loads of tile q + NBUF - 1 go into the slot the barrier has just retired.  A wave
@@ -623,20 +621,9 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
             // that, so all of them in a row would leave the matrix pipe idle: one (or a few) after
             // each group of MFMAs instead.
             {
-                // scalar offsets of all loads up front; past the end of the sequence the loads
-                // are issued all the same, out of range: zeros land in a slot nobody reads any
-                // more (the slot retired just now), and the instruction stream has no branch
-                const bool more = q + Cfg::NBUF - 1 < n_seq;
-                const int row0 = tile_row0(q + Cfg::NBUF - 1);
-                const uint32_t ybase = more ? (uint32_t)(row0 * ys2) : kOobOffset;
-                const uint32_t zbase = more ? (uint32_t)(row0 * zs2) : kOobOffset;
                 uint32_t so[Cfg::NT];
-                static_for<0, Cfg::NT>([&](auto ii) {
-                    constexpr int I = decltype(ii)::value;
-                    so[I] = I < NIY ? ybase + (uint32_t)((I - I % NYD) * YSTEP * ys2)
-                                    : zbase + (uint32_t)((I - NIY) * ZSTEP * zs2);
-                });
-                const uint32_t yb = lds_wave + issue_off;
+                tile_offsets(q + Cfg::NBUF - 1, so);
+                const uint32_t yb = lds_wave + prev_off;
                 phase2(std::true_type{}, pfa, pfb, ya_next, 0, [&](auto ff) {
                     static_for<0, Cfg::NT>([&](auto ii) {
                         if constexpr (decltype(ii)::value * NZF / Cfg::NT == decltype(ff)::value)
@@ -764,7 +751,7 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         static_assert(BM / BN <= Cfg::NBUF, "the diagonal block must fit in the LDS ring");
         if (n_full > 0) __builtin_amdgcn_s_barrier();  // every wave is done with the last full tile
         if constexpr (!chunked) {
-            issue_tile(q + Cfg::NBUF - 1, issue_off);  // the one tile not yet requested (if any)
+            issue_tile(q + Cfg::NBUF - 1, prev_off);  // the one tile not yet requested (if any)
             wait_vm<0>();
             __builtin_amdgcn_s_barrier();
         }
