@@ -358,6 +358,15 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
             xf[ib][kc] = __builtin_bit_cast(V8, __builtin_amdgcn_raw_buffer_load_b128(rx, off, 0, 0));
         }
     }
+    // The last row block's fragments are held in accumulation registers (MFMA reads its A / B
+    // operands from there as well).  Left to itself the register allocator parks them there
+    // anyway, the architectural file being full, but then copies each one to a second
+    // accumulation register before every use: four moves per MFMA in the main loop.
+    // (Only where a wave has the whole register file: with two waves per SIMD nothing is parked.)
+    if constexpr (Cfg::kMinWavesPerSimd == 1) {
+#pragma unroll
+        for (int kc = 0; kc < KCU; ++kc) asm volatile("" : "+a"(xf[NIB - 1][kc]));
+    }
 
     f32x16 acc[NIB][DB];
 #pragma unroll
