@@ -261,28 +261,32 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         p.dbg[(size_t)wg_index * 16 + 7] = (__builtin_amdgcn_s_memrealtime() & 0xffffffffffull) |
                                              ((unsigned long long)__builtin_amdgcn_s_getreg(63492) << 40);
 #endif
-    for (int pass = 0; pass < 2; ++pass) {
-    FLA_STAMP(0);
-    // unpaired tiles go heaviest first (last row tile under a lower mask, first under an upper one)
-    const int tile = chunked ? rank : single ? (upper ? rank : p.n_tiles - 1 - rank) : (pass == 0 ? p.n_tiles - 1 - rank : rank);
-    // odd tile count: the middle tile has no partner; chunked: a single tile per workgroup
-    if (pass == 1 && (single || tile == p.n_tiles - 1 - rank)) break;
-    const int i0 = tile * BM;
-
-    // ---- tile sequence: tiles fully inside the mask first, then the diagonal block
-    const int diag_rows = (N - i0 < BM) ? (N - i0) : BM;
-    const int n_diag = (diag_rows + BN - 1) / BN;
-    int n_full, full_row0;
-    if (upper) {
-        const int rest = N - (i0 + BM);
-        n_full = rest > 0 ? (rest + BN - 1) / BN : 0;
-        full_row0 = i0 + BM;
-    } else {
-        n_full = i0 / BN;
-        full_row0 = 0;
-    }
-    if (chunked) n_full = 0;  // everything off the diagonal block arrives through the state
-    const int n_seq = n_full + n_diag;
+    // ---- the row tiles of this workgroup, in the order they are done: unpaired tiles go heaviest
+    // first (last row tile under a lower mask, first under an upper one); with an odd tile
+    // count the middle tile has no partner; chunked: a single tile per workgroup
+    auto stream_tile = [&](int pass) {
+        return chunked ? rank : single ? (upper ? rank : p.n_tiles - 1 - rank) : (pass == 0 ? p.n_tiles - 1 - rank : rank);
+    };
+    const int n_pass = (single || rank == p.n_tiles - 1 - rank) ? 1 : 2;
+    // geometry of the tile being set up; the tile sequence is the tiles fully inside the mask
+    // first, then the diagonal block
+    int tile = 0, i0 = 0, diag_rows = 0, n_diag = 0, n_full = 0, full_row0 = 0, n_seq = 0;
+    auto set_tile = [&](int t) {
+        tile = t;
+        i0 = t * BM;
+        diag_rows = (N - i0 < BM) ? (N - i0) : BM;
+        n_diag = (diag_rows + BN - 1) / BN;
+        if (upper) {
+            const int rest = N - (i0 + BM);
+            n_full = rest > 0 ? (rest + BN - 1) / BN : 0;
+            full_row0 = i0 + BM;
+        } else {
+            n_full = i0 / BN;
+            full_row0 = 0;
+        }
+        if (chunked) n_full = 0;  // everything off the diagonal block arrives through the state
+        n_seq = n_full + n_diag;
+    };
 
     // ---- HBM -> LDS: per-lane source offsets (constant over tiles).  Load u of a wave covers
     // rows u * YSTEP + wave * (1024 / RY) + lane / CY of the tile.  Where YSTEP is a multiple of
@@ -344,29 +348,45 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         wait_vm<AHEAD * Cfg::NT>();
     };
 
-    issue_tile(0, 0);
+    constexpr int RING = Cfg::NBUF * STAGE;
+    auto wrap_slot = [](int off) { return off >= RING ? off - RING : off; };
 
     // ---- resident X fragments
     V8 xf[NIB][KC];
+    auto load_x = [&]() {
 #pragma unroll
-    for (int ib = 0; ib < NIB; ++ib) {
-        const int row = i0 + blk[ib] * 32 + l32;
+        for (int ib = 0; ib < NIB; ++ib) {
+            const int row = i0 + blk[ib] * 32 + l32;
 #pragma unroll
-        for (int kc = 0; kc < KCU; ++kc) {
-            const int col = kc * 16 + 8 * g;
-            const uint32_t off = (uint32_t)(row * xs2 + col * 2) + (col < p.dc ? 0u : kOobOffset);
-            xf[ib][kc] = __builtin_bit_cast(V8, __builtin_amdgcn_raw_buffer_load_b128(rx, off, 0, 0));
+            for (int kc = 0; kc < KCU; ++kc) {
+                const int col = kc * 16 + 8 * g;
+                const uint32_t off = (uint32_t)(row * xs2 + col * 2) + (col < p.dc ? 0u : kOobOffset);
+                xf[ib][kc] = __builtin_bit_cast(V8, __builtin_amdgcn_raw_buffer_load_b128(rx, off, 0, 0));
+            }
         }
-    }
-    // The last row block's fragments are held in accumulation registers (MFMA reads its A / B
-    // operands from there as well).  Left to itself the register allocator parks them there
-    // anyway, the architectural file being full, but then copies each one to a second
-    // accumulation register before every use: four moves per MFMA in the main loop.
-    // (Only where a wave has the whole register file: with two waves per SIMD nothing is parked.)
-    if constexpr (Cfg::kMinWavesPerSimd == 1) {
-#pragma unroll
-        for (int kc = 0; kc < KCU; ++kc) asm volatile("" : "+a"(xf[NIB - 1][kc]));
-    }
+    };
+    // First requests of a row tile: tile 0 of its sequence, the X fragments, then tiles up to
+    // kPre - 1, into ring slots starting at byte offset ring0.  For the second row tile of a
+    // workgroup this runs before the first one's epilogue (kOverlap): the epilogue stages the
+    // output in the first kStageSlots slots, the requests go to the slots behind them, and the
+    // latency of the first loads is hidden behind the epilogue.
+    constexpr int kStageSlots = (BM * Cfg::RO + STAGE - 1) / STAGE;
+    constexpr int kFreeSlots = Cfg::NBUF - kStageSlots;
+    constexpr bool kOverlap = !CHUNKED && kFreeSlots >= 1 && Cfg::NBUF >= 3;
+    constexpr int kPreMax = Cfg::NBUF - 2 < 2 ? Cfg::NBUF - 2 : 2;
+    constexpr int kPre = !kOverlap ? 1 : (kFreeSlots < kPreMax ? kFreeSlots : kPreMax);
+    static_assert(kPre >= 1, "tile 0 is always requested up front");
+    int ring0 = 0;
+    auto start_tile = [&]() {
+        issue_tile(0, ring0);
+        load_x();
+        static_for<1, kPre>([&](auto qq) { issue_tile(decltype(qq)::value, wrap_slot(ring0 + decltype(qq)::value * STAGE)); });
+    };
+    set_tile(stream_tile(0));
+    start_tile();
+
+    for (int pass = 0;; ++pass) {
+    FLA_STAMP(0);
 
     f32x16 acc[NIB][DB];
 #pragma unroll
@@ -444,13 +464,25 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     };
 
     // ring state: byte offsets of the slots of tile q-1, q, q+1 and of the next tile to issue
-    int prev_off = (Cfg::NBUF - 1) * STAGE, cur_off = 0, next_off = STAGE;
+    int prev_off = wrap_slot(ring0 + (Cfg::NBUF - 1) * STAGE), cur_off = ring0, next_off = wrap_slot(ring0 + STAGE);
+    // The last row block's X fragments are held in accumulation registers (MFMA reads its A / B
+    // operands from there as well).  Left to itself the register allocator parks them there
+    // anyway, the architectural file being full, but then copies each one to a second
+    // accumulation register before every use: four moves per MFMA in the main loop.
+    // (Only where a wave has the whole register file: with two waves per SIMD nothing is parked.
+    // Placed after the first wait for loaded data: the statement needs the values.)
+    auto pin_x = [&]() {
+        if constexpr (Cfg::kMinWavesPerSimd == 1) {
+#pragma unroll
+            for (int kc = 0; kc < KCU; ++kc) asm volatile("" : "+a"(xf[NIB - 1][kc]));
+        }
+    };
     const bool has_state = chunked && (upper ? tile + 1 < p.n_tiles : tile > 0);
     const T *st = has_state ? static_cast<const T *>(p.state) + ((int64_t)bh * p.n_tiles + tile) * (DO * DC) : nullptr;
     if constexpr (chunked) {
         // everything this workgroup will ever read is requested at once: the rest of the diagonal
         // block's tiles and the running state (the kernel is latency-bound in this mode)
-        static_for<1, BM / BN>([&](auto qq) { issue_tile(decltype(qq)::value, decltype(qq)::value * STAGE); });
+        static_for<kPre, BM / BN>([&](auto qq) { issue_tile(decltype(qq)::value, decltype(qq)::value * STAGE); });
         if constexpr (Cfg::kStateInLds) {
             if (has_state) {
                 const u32x4 rs = make_rsrc(st, DO * DC * 2);
@@ -487,14 +519,17 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         }
         wait_vm<0>();
         __builtin_amdgcn_s_barrier();
+        pin_x();
         FLA_STAMP(1);
     } else {
-        // tiles 1 .. NBUF-3 before the first wait, tile NBUF-2 right after it
-        static_for<1, Cfg::NBUF - 2>([&](auto qq) { issue_tile(decltype(qq)::value, decltype(qq)::value * STAGE); });
+        // tiles up to NBUF-3 before the first wait, tile NBUF-2 right after it
+        static_for<kPre, Cfg::NBUF - 2>(
+            [&](auto qq) { issue_tile(decltype(qq)::value, wrap_slot(ring0 + decltype(qq)::value * STAGE)); });
         wait_tile();
         __builtin_amdgcn_s_barrier();  // tile 0 (and the X fragments) have landed
+        pin_x();
         FLA_STAMP(1);
-        issue_tile(Cfg::NBUF - 2, (Cfg::NBUF - 2) * STAGE);
+        issue_tile(Cfg::NBUF - 2, wrap_slot(ring0 + (Cfg::NBUF - 2) * STAGE));
     }
     // from here on: tiles up to q + NBUF - 2 are issued while tile q is consumed, and tile
     // q + NBUF - 1 goes into the slot of tile q - 1 (prev_off) once that one is retired
@@ -512,7 +547,7 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         {
             int ya0[YQ], za0[ZQ];
-            slot_addrs(0, ya0, za0);
+            slot_addrs(cur_off, ya0, za0);
 #pragma unroll
             for (int kc = 0; kc < KCU; ++kc) yf[kc] = y_read(ya0, 0, kc);
         }
@@ -766,7 +801,6 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         }
         FLA_STAMP(5);
 
-        constexpr int RING = Cfg::NBUF * STAGE;
         const int nsub = (diag_rows + 31) >> 5;  // sub-tiles with at least one valid row
         int blk_min = blk[0], blk_max = blk[0];
         if constexpr (NIB == 2) {
@@ -851,6 +885,16 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     }
 
     FLA_STAMP(3);
+    // ---- the next row tile's first requests go out before this one's epilogue
+    const int out_i0 = i0;
+    const bool more = pass + 1 < n_pass;
+    if constexpr (kOverlap) {
+        if (more) {
+            set_tile(stream_tile(pass + 1));
+            ring0 = kStageSlots * STAGE;
+            start_tile();
+        }
+    }
     // ---- epilogue.  The second product is issued as Out^T += Z^T P^T (the two register
     // operands swapped), and with the column permutation of the Z fragments acc[ib][db][v] is
     // Out[row l32 of block ib][column 32 db + 16 g + v]: 16 consecutive columns per lane.
@@ -865,7 +909,7 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
             for (int db = 0; db < DB; ++db)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[ib][db][v] *= inv;
-            const int row = i0 + blk[ib] * 32 + l32;
+            const int row = out_i0 + blk[ib] * 32 + l32;
             if (g == 0 && row < N) p.denom[(int64_t)bh * N + row] = n;
         }
     }
@@ -885,20 +929,35 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
                 }
             }
         }
-        __syncthreads();
+        // LDS writes done, then a bare barrier: __syncthreads() would also wait for every load in
+        // flight, and the next row tile's first loads are in flight here
+        asm volatile("" ::: "memory");  // the compiler keeps the staging writes above, the reads below
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
         constexpr int CO = DO / 8;  // 16-byte chunks per output row
 #pragma unroll
         for (int u = 0; u < BM * CO / 256; ++u) {
             const int c = tid + 256 * u, r = c / CO, cc = c - r * CO;
-            const int row = i0 + r;
+            const int row = out_i0 + r;
             if (row < N && cc * 8 < p.dout) {
                 const u32x4 val = *reinterpret_cast<const u32x4 *>(smem + r * RO + cc * 16);
                 *reinterpret_cast<u32x4 *>(O + (int64_t)row * p.os_n + cc * 8) = val;
             }
         }
-        __syncthreads();  // the staging area is ring space again
+        // Every wave has read its part of the staging area (the stores above hold the values):
+        // it is ring space again.  The stores themselves need not have completed.
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
     }
     FLA_STAMP(4);
+    if (!more) break;
+    if constexpr (!kOverlap) {
+        set_tile(stream_tile(pass + 1));
+        ring0 = 0;
+        start_tile();
+    }
     }  // pass
 #ifdef FLA_DBG_TIMING
     if (p.dbg && tid == 0) p.dbg[(size_t)wg_index * 16 + 15] = __builtin_amdgcn_s_memrealtime() & 0xffffffffffull;
