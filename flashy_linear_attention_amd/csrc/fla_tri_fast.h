@@ -373,8 +373,7 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     constexpr int kStageSlots = (BM * Cfg::RO + STAGE - 1) / STAGE;
     constexpr int kFreeSlots = Cfg::NBUF - kStageSlots;
     constexpr bool kOverlap = !CHUNKED && kFreeSlots >= 1 && Cfg::NBUF >= 3;
-    constexpr int kPreMax = Cfg::NBUF - 2 < 2 ? Cfg::NBUF - 2 : 2;
-    constexpr int kPre = !kOverlap ? 1 : (kFreeSlots < kPreMax ? kFreeSlots : kPreMax);
+    constexpr int kPre = 1;  // (two tiles up front measured no better than one)
     static_assert(kPre >= 1, "tile 0 is always requested up front");
     int ring0 = 0;
     auto start_tile = [&]() {
@@ -936,14 +935,20 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         constexpr int CO = DO / 8;  // 16-byte chunks per output row
+        // all LDS reads first (the accumulators are dead, registers are free), then the stores:
+        // read, wait, store per row would pay the LDS latency once per row
+        constexpr int NOUT = BM * CO / 256;
+        u32x4 val[NOUT];
 #pragma unroll
-        for (int u = 0; u < BM * CO / 256; ++u) {
+        for (int u = 0; u < NOUT; ++u) {
+            const int c = tid + 256 * u, r = c / CO, cc = c - r * CO;
+            val[u] = *reinterpret_cast<const u32x4 *>(smem + r * RO + cc * 16);
+        }
+#pragma unroll
+        for (int u = 0; u < NOUT; ++u) {
             const int c = tid + 256 * u, r = c / CO, cc = c - r * CO;
             const int row = out_i0 + r;
-            if (row < N && cc * 8 < p.dout) {
-                const u32x4 val = *reinterpret_cast<const u32x4 *>(smem + r * RO + cc * 16);
-                *reinterpret_cast<u32x4 *>(O + (int64_t)row * p.os_n + cc * 8) = val;
-            }
+            if (row < N && cc * 8 < p.dout) *reinterpret_cast<u32x4 *>(O + (int64_t)row * p.os_n + cc * 8) = val[u];
         }
         // Every wave has read its part of the staging area (the stores above hold the values):
         // it is ring space again.  The stores themselves need not have completed.
