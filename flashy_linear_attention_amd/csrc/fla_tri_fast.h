@@ -653,7 +653,7 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
 #ifdef FLA_DMA_BURST
             constexpr bool kSpread = false;
 #else
-            constexpr bool kSpread = FLAGS == 0;  // the variants with score maps have no registers to spare
+            constexpr bool kSpread = true;
 #endif
             if constexpr (!kSpread) {
                 issue_tile(q + Cfg::NBUF - 1, prev_off);
