@@ -166,7 +166,7 @@ def _gpu_fp32_reference(q, k, v, do, backward, heads_per_chunk=8):
 
 @pytest.mark.parametrize("name", ["C2", "C3", "C4", "C5"])
 def test_benchmark_workload(name, gpu_device):
-    """Each BASELINE workload at full size: every head against the oracle's
+    """Each benchmark workload at full size: every head against the oracle's
     formula in fp32 on the GPU, and a sample of heads against the oracle run in
     fp32 on the CPU (one head of C5 alone is 2x137 GFLOP there)."""
     w = WORKLOADS[name]
