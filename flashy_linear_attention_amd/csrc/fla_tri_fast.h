@@ -20,9 +20,19 @@
 //     its MFMA and the two MFMA chains of a phase are independent.
 //     One barrier per tile, placed between the phases of the tile's second
 //     sub-tile: it publishes the next tile and retires the previous one.
+//     With one wave per SIMD a wave issues one instruction every four clocks and
+//     an MFMA holds the pipe for 32, so at most seven other instructions fit
+//     between two MFMAs: the loads of the tile that goes into the retired slot
+//     are issued one per MFMA group of the following phase, with their scalar
+//     offsets computed beforehand, unconditionally (a tile past the end of the
+//     sequence is fetched from out of range) so that no branch or variable wait
+//     count sits in the loop.
 //   * The BM x BM block on the diagonal is handled afterwards, with all of its
 //     tiles resident, by a barrier-free S -> mask -> P -> PV sequence per sub-tile
 //     that skips the (block, sub-tile) pairs the mask removes entirely.
+//   * A workgroup does two row tiles (r and n_tiles-1-r).  The second one's first
+//     tile and X fragments are requested before the first one's epilogue, into
+//     ring slots behind the epilogue's staging area.
 //   * Variants of the same body: the plain kernel (one product), the batched
 //     kernel (grid y selects one of up to three products: the backward's dQ, dV,
 //     dK in one launch) and the chunked kernel (CHUNKED: diagonal block plus
