@@ -123,3 +123,23 @@ def test_backward_entry_point_on_ragged_lengths(dims, gpu_device):
     assert rc == 0
     for name, got, w in zip(("dQ", "dK", "dV"), (dq, dk, dv), want):
         assert_close(name + " (chunked)", got, w)
+
+
+@pytest.mark.parametrize("dims", [(1, 64, 2300, 64, 64), (2, 26, 2300, 128, 128), (1, 64, 1990, 32, 64)],
+                         ids=lambda d: "x".join(map(str, d)))
+@pytest.mark.parametrize("upper", [0, 1], ids=["lower", "upper"])
+def test_paired_row_tiles_on_ragged_lengths(dims, upper, gpu_device):
+    """Enough (head, tile-pair) work for one workgroup to take two row tiles (the second tile's
+    first loads overlap the first tile's epilogue), with an odd tile count (the middle tile has
+    no partner) and a last tile that is cut short.  Every head against the formula in fp32 on
+    the GPU, four heads against the CPU oracle."""
+    b, h, n, dc, do = dims
+    x, y, z = _inputs(b, h, n, dc, do, torch.bfloat16, seed=sum(dims) + upper)
+    xg, yg, zg = (t.to(gpu_device) for t in (x, y, z))
+    got = _call("tri", xg, yg, zg, upper, chunked=False)
+    s = torch.matmul(xg.float(), yg.float().transpose(-2, -1))
+    s = s.triu() if upper else s.tril()
+    assert_close("all heads (fp32 GPU)", got, torch.matmul(s, zg.float()).cpu())
+    heads = [0, h // 3, h // 2, h - 1]
+    want = _oracle(x[-1:, heads], y[-1:, heads], z[-1:, heads], upper)
+    assert_close("sampled heads (CPU oracle)", got[-1:, heads], want)
