@@ -232,7 +232,12 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     constexpr bool chunked = CHUNKED;
     const bool single = chunked || p.single != 0;
     const int n_pairs = single ? p.n_tiles : (p.n_tiles + 1) >> 1;
-    const int hl = slot / n_pairs, rank = slot - hl * n_pairs;
+    // Pairs: the workgroups of one head are neighbours (they stream the same Y / Z rows at the
+    // same time).  Single tiles differ in work, so they are ordered heaviest first across all
+    // heads: whatever CU frees up next takes the heaviest tile left.
+    const int n_hl = (p.BH + 7) >> 3;
+    const int hl = (single && !chunked) ? slot % n_hl : slot / n_pairs;
+    const int rank = (single && !chunked) ? slot / n_hl : slot - hl * n_pairs;
     const int bh = hl * 8 + xcd;
     if (bh >= p.BH) return;
     const bool upper = p.upper != 0;
@@ -1005,6 +1010,15 @@ inline bool fast_path_ok(const TriParams &p) {
     return n * p.xs_n * 2 <= kMaxFastExtent && n * p.ys_n * 2 <= kMaxFastExtent && n * p.zs_n * 2 <= kMaxFastExtent;
 }
 
+// A problem with fewer tile pairs than workgroups fit on the chip at once (256 CUs, one or two
+// workgroups each) runs as single tiles, heaviest first: pairs would leave slots idle (measured
+// 7-20 % faster there).  Exactly one pair per CU stays paired: every CU then has the same work
+// (1-4 % faster than single tiles).
+constexpr int kCuCount = 256;
+inline int run_single_tiles(int64_t pairs, int workgroups_per_cu) {
+    return pairs < (int64_t)kCuCount * workgroups_per_cu && pairs % kCuCount != 0;
+}
+
 template <typename T, int DC, int DO, bool CHUNKED, int FLAGS>
 hipError_t launch_tri_fast_variant(TriParams p, hipStream_t stream);
 
@@ -1047,10 +1061,7 @@ hipError_t launch_tri_fast_variant(TriParams p, hipStream_t stream) {
     } else {
         if (CHUNKED && p.state_transposed && !Cfg::kStateTransposable) return hipErrorNotSupported;
         p.n_tiles = (p.N + Cfg::BM - 1) / Cfg::BM;
-        // Pairs of row tiles make all workgroups equal; a problem with fewer pairs than the chip has
-        // CUs (256) would leave CUs idle and runs as single tiles instead (measured 10-20 % faster
-        // there, while at exactly one pair per CU the equal pairs still win).
-        p.single = (!CHUNKED && (int64_t)p.BH * ((p.n_tiles + 1) / 2) < 256) ? 1 : 0;
+        p.single = (!CHUNKED && run_single_tiles((int64_t)p.BH * ((p.n_tiles + 1) / 2), Cfg::kMinWavesPerSimd)) ? 1 : 0;
         const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * ((CHUNKED || p.single) ? p.n_tiles : (p.n_tiles + 1) / 2);
         if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
         auto kern = tri_xyt_z_fast_kernel<T, DC, DO, CHUNKED, FLAGS>;
@@ -1071,7 +1082,7 @@ hipError_t launch_tri_fast_batch(TriBatch b, int count, hipStream_t stream) {
         return hipErrorNotSupported;
     } else {
         const int n_tiles = (b.p[0].N + Cfg::BM - 1) / Cfg::BM;
-        const int single = (int64_t)b.p[0].BH * ((n_tiles + 1) / 2) < 256 ? 1 : 0;
+        const int single = run_single_tiles((int64_t)b.p[0].BH * ((n_tiles + 1) / 2), Cfg::kMinWavesPerSimd);
         for (int i = 0; i < count; ++i) b.p[i].n_tiles = n_tiles, b.p[i].single = single, b.p[i].state = nullptr;
         const int64_t grid = (int64_t)8 * ((b.p[0].BH + 7) / 8) * (single ? n_tiles : (n_tiles + 1) / 2);
         if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
