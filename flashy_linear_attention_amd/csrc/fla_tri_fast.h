@@ -224,6 +224,15 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, g = lane >> 5, lam = lane & 15;
+#ifdef FLA_DBG_FILL_LDS
+    // ablation builds without the loads: LDS holds pseudo-random 16-bit values of magnitude ~1
+    for (int i = threadIdx.x; i < Cfg::SMEM_BYTES / 4; i += 256) {
+        uint32_t h = (uint32_t)i * 2654435761u + blockIdx.x * 40503u;
+        h ^= h >> 15;
+        reinterpret_cast<uint32_t *>(smem)[i] = 0x3f003f00u | (h & 0x80ff80ffu);
+    }
+    __syncthreads();
+#endif
 
     const int wg = wg_index, xcd = wg & 7, slot = wg >> 3;
     // Each workgroup takes two row tiles of one head, r and n_tiles-1-r: under a triangular
