@@ -37,6 +37,14 @@
 //     kernel (grid y selects one of up to three products: the backward's dQ, dV,
 //     dK in one launch) and the chunked kernel (CHUNKED: diagonal block plus
 //     the running state of the chunk-wise evaluation, no tile ring).
+//
+// Measurement switches (never defined in a product build; results of such builds are wrong):
+//   FLA_DBG_TIMING     every workgroup writes shader-clock stamps of its phases to TriParams::dbg
+//   FLA_DBG_NO_DMA / NO_ZREAD / NO_YREAD / NO_WAIT / NO_BARRIER / NO_CVT / NO_DIAG
+//                      drop the tile loads / the Z or Y fragment reads / the waits for tiles /
+//                      the per-tile barrier / the rounding / the diagonal walk
+//   FLA_DBG_FILL_LDS   fill LDS with random 16-bit values at workgroup start (with NO_DMA)
+//   FLA_DMA_BURST      issue a tile's loads in one burst after the barrier instead of spread out
 #pragma once
 
 #include <hip/hip_runtime.h>
