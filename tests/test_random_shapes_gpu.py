@@ -143,3 +143,17 @@ def test_paired_row_tiles_on_ragged_lengths(dims, upper, gpu_device):
     heads = [0, h // 3, h // 2, h - 1]
     want = _oracle(x[-1:, heads], y[-1:, heads], z[-1:, heads], upper)
     assert_close("sampled heads (CPU oracle)", got[-1:, heads], want)
+
+
+@pytest.mark.parametrize("dims", [(8, 40, 300, 64, 64), (5, 13, 520, 128, 128), (4, 80, 257, 32, 32)],
+                         ids=lambda d: "x".join(map(str, d)))
+@pytest.mark.parametrize("upper", [0, 1], ids=["lower", "upper"])
+def test_many_heads_short_sequences(dims, upper, gpu_device):
+    """Many heads, few row tiles each: single-tile workgroups ordered heaviest first across heads,
+    head counts that are no multiple of 8 (idle slots in the last group of eight)."""
+    b, h, n, dc, do = dims
+    x, y, z = _inputs(b, h, n, dc, do, torch.float16, seed=sum(dims) + upper)
+    want = _oracle(x, y, z, upper)
+    xg, yg, zg = (t.to(gpu_device) for t in (x, y, z))
+    assert_close("quadratic", _call("tri", xg, yg, zg, upper, chunked=False), want)
+    assert_close("chunked", _call("tri_chunked", xg, yg, zg, upper, chunked=True), want)
