@@ -34,6 +34,15 @@ struct ChunkStateParams {
     int32_t n_chunks;
 };
 
+// LDS footprint of the state kernel: at most half of the CU's 160 KiB, so that two workgroups fit
+template <int DC, int DO>
+struct ChunkStateLds {
+    using Cfg = FastConfig<DC, DO>;
+    static constexpr int kTiles = Cfg::BM / Cfg::BN;
+    static constexpr int kRoundTiles = (kTiles * Cfg::STAGE_BYTES > 80 * 1024 && kTiles % 2 == 0) ? kTiles / 2 : kTiles;
+    static constexpr int kBytes = kRoundTiles * Cfg::STAGE_BYTES;
+};
+
 template <typename T, int DC, int DO>
 __global__ __launch_bounds__(256) void chunk_state_kernel(const ChunkStateParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -44,8 +53,11 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(const ChunkStateParams
     constexpr int RY = Cfg::RY, RZ = Cfg::RZ, CY = Cfg::CY, CZ = Cfg::CZ;
     constexpr int NIY = Cfg::NIY, NIZ = Cfg::NIZ;
     constexpr int STAGE = Cfg::STAGE_BYTES, Y_BYTES = Cfg::Y_BYTES;
-    constexpr int NTILE = BM / BN;  // 64-row tiles per chunk, all resident in LDS at once
-    static_assert(NTILE <= Cfg::NBUF, "a chunk must fit in the LDS ring");
+    constexpr int NTILE = BM / BN;  // 64-row tiles per chunk
+    // tiles resident in LDS at once: the whole chunk when that leaves room for two workgroups
+    // per CU (one loads while the other computes), else half of it, in two rounds
+    constexpr int RT = ChunkStateLds<DC, DO>::kRoundTiles;
+    static_assert(RT <= Cfg::NBUF && NTILE % RT == 0, "a round must fit in LDS and divide the chunk");
     constexpr int EB = DO / 32, DBK = DC / 32;     // 32 x 32 output blocks
     constexpr int NBW = (EB * DBK + 3) / 4;        // blocks per wave (block b goes to wave b % 4)
 
@@ -85,21 +97,34 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(const ChunkStateParams
         zdma = (uint32_t)(row * zs2 + c * 16) + (c * 8 < p.dout ? 0u : kOobOffset);
     }
     const uint32_t lds_wave = lds0 + wave * 1024;
-    static_for<0, NTILE>([&](auto tt) {
-        constexpr int t = decltype(tt)::value;
-        const int row0 = r0 + t * BN;
-        static_for<0, NIY>([&](auto u) {
-            constexpr int U = decltype(u)::value;
-            dma_16B_per_lane<t * STAGE + U * 4096>(ry, lds_wave, ydma[U % NYD],
-                                                   (uint32_t)((row0 + (U - U % NYD) * YSTEP) * ys2));
+    // (the load instruction takes its descriptor, LDS base and row offset in scalar registers;
+    // the values are uniform, and said to be so where the compiler loses track of it)
+    auto uniform = [](uint32_t x) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)x); };
+    auto uniform4 = [&](const u32x4 &r) {
+        u32x4 o = {uniform(r[0]), uniform(r[1]), uniform(r[2]), uniform(r[3])};
+        return o;
+    };
+    auto load_round = [&](auto rr) {
+        constexpr int R = decltype(rr)::value;
+        const u32x4 ryu = uniform4(ry), rzu = uniform4(rz);
+        const uint32_t ldsu = uniform(lds_wave);
+        static_for<0, RT>([&](auto tt) {
+            constexpr int t = decltype(tt)::value;
+            const int row0 = r0 + (R * RT + t) * BN;
+            static_for<0, NIY>([&](auto u) {
+                constexpr int U = decltype(u)::value;
+                dma_16B_per_lane<t * STAGE + U * 4096>(ryu, ldsu, ydma[U % NYD],
+                                                       uniform((uint32_t)((row0 + (U - U % NYD) * YSTEP) * ys2)));
+            });
+            static_for<0, NIZ>([&](auto u) {
+                constexpr int U = decltype(u)::value;
+                dma_16B_per_lane<t * STAGE + Y_BYTES + U * 4096>(rzu, ldsu, zdma,
+                                                                 uniform((uint32_t)((row0 + U * ZSTEP) * zs2)));
+            });
         });
-        static_for<0, NIZ>([&](auto u) {
-            constexpr int U = decltype(u)::value;
-            dma_16B_per_lane<t * STAGE + Y_BYTES + U * 4096>(rz, lds_wave, zdma, (uint32_t)((row0 + U * ZSTEP) * zs2));
-        });
-    });
-    wait_vm<0>();
-    __builtin_amdgcn_s_barrier();
+        wait_vm<0>();
+        __builtin_amdgcn_s_barrier();
+    };
 
     // Column fragment of a row-major tile: rows R0 + {4g..4g+3, 8+4g..8+4g+3}, column 32 cb + l32.
     // Source lane `lam` of a 16-lane group addresses row lam/4, chunk lam%4 of the 16 columns
@@ -120,23 +145,27 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(const ChunkStateParams
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
 
+    static_for<0, NTILE / RT>([&](auto rr) {
+        if constexpr (decltype(rr)::value > 0) __builtin_amdgcn_s_barrier();  // the previous round's tiles are read
+        load_round(rr);
 #pragma unroll 1
-    for (int t = 0; t < NTILE; ++t) {
-        const unsigned char *ytile = smem + t * STAGE, *ztile = ytile + Y_BYTES;
+        for (int t = 0; t < RT; ++t) {
+            const unsigned char *ytile = smem + t * STAGE, *ztile = ytile + Y_BYTES;
 #pragma unroll
-        for (int ks = 0; ks < BN / 16; ++ks) {
+            for (int ks = 0; ks < BN / 16; ++ks) {
 #pragma unroll
-            for (int i = 0; i < NBW; ++i) {
-                const int blk = wave + 4 * i;  // = eb * DBK + dbk
-                if (blk < EB * DBK) {
-                    const int eb = blk / DBK, dbk = blk % DBK;
-                    const V8 a = col_frag(ztile, RZ, eb, 16 * ks, [](int r) { return swizzle_z<CZ>(r); });
-                    const V8 bfr = col_frag(ytile, RY, dbk, 16 * ks, [](int r) { return swizzle_y<CY>(r); });
-                    acc[i] = M::mma(a, bfr, acc[i]);
+                for (int i = 0; i < NBW; ++i) {
+                    const int blk = wave + 4 * i;  // = eb * DBK + dbk
+                    if (blk < EB * DBK) {
+                        const int eb = blk / DBK, dbk = blk % DBK;
+                        const V8 a = col_frag(ztile, RZ, eb, 16 * ks, [](int r) { return swizzle_z<CZ>(r); });
+                        const V8 bfr = col_frag(ytile, RY, dbk, 16 * ks, [](int r) { return swizzle_y<CY>(r); });
+                        acc[i] = M::mma(a, bfr, acc[i]);
+                    }
                 }
             }
         }
-    }
+    });
 
     // acc[i][v] = W^T[e = 32 eb + 8(v/4) + 4g + v%4][d = 32 dbk + l32]
     float *W = p.w + ((int64_t)bh * p.n_chunks + chunk) * (DO * DC);
@@ -211,10 +240,11 @@ hipError_t launch_chunk_state(ChunkStateParams p, hipStream_t stream) {
         const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_chunks;
         if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
         auto kern = chunk_state_kernel<T, DC, DO>;
+        constexpr int smem = ChunkStateLds<DC, DO>::kBytes;
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM_BYTES);
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), Cfg::SMEM_BYTES, stream, p);
+        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
         return hipGetLastError();
     }
 }
