@@ -186,8 +186,8 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(const ChunkStateParams
 // Exclusive running sum over the chunk axis of w[bh][chunk][E] (fp32), rounded to T.
 // reverse == 0: state[c] = sum_{c' < c} w[c'];  reverse != 0: state[c] = sum_{c' > c} w[c'].
 // One thread per pair of elements (many sequences have few (b, h) pairs, so parallelism has to
-// come from the state elements); the chunk loop is unrolled by 8 so that eight independent
-// loads are in flight per thread.
+// come from the state elements); the chunk loop runs in batches of 16 (then 4) independent loads
+// per thread.
 template <typename T>
 __global__ __launch_bounds__(256) void chunk_scan_kernel(const float *w, T *state, int n_chunks, int64_t E,
                                                         int64_t total2, int reverse) {
@@ -205,21 +205,26 @@ __global__ __launch_bounds__(256) void chunk_scan_kernel(const float *w, T *stat
     }
     f32x2 run = {0.f, 0.f};
     int k = 0;
-    for (; k + 8 <= n_chunks; k += 8) {
-        f32x2 v[8];
+    auto batch = [&](auto nn) {
+        constexpr int NB = decltype(nn)::value;
+        for (; k + NB <= n_chunks; k += NB) {
+            f32x2 v[NB];
 #pragma unroll
-        for (int u = 0; u < 8; ++u) v[u] = *reinterpret_cast<const f32x2 *>(wp + u * step);
+            for (int u = 0; u < NB; ++u) v[u] = *reinterpret_cast<const f32x2 *>(wp + u * step);
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            t2 o;
-            o[0] = static_cast<T>(run[0]);
-            o[1] = static_cast<T>(run[1]);
-            *reinterpret_cast<t2 *>(sp + u * step) = o;
-            run += v[u];
+            for (int u = 0; u < NB; ++u) {
+                t2 o;
+                o[0] = static_cast<T>(run[0]);
+                o[1] = static_cast<T>(run[1]);
+                *reinterpret_cast<t2 *>(sp + u * step) = o;
+                run += v[u];
+            }
+            wp += NB * step;
+            sp += NB * step;
         }
-        wp += 8 * step;
-        sp += 8 * step;
-    }
+    };
+    batch(std::integral_constant<int, 16>{});
+    batch(std::integral_constant<int, 4>{});
     for (; k < n_chunks; ++k) {
         t2 o;
         o[0] = static_cast<T>(run[0]);
