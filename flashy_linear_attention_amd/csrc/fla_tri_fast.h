@@ -511,9 +511,14 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     const bool has_state = chunked && (upper ? tile + 1 < p.n_tiles : tile > 0);
     const T *st = has_state ? static_cast<const T *>(p.state) + ((int64_t)bh * p.n_tiles + tile) * (DO * DC) : nullptr;
     if constexpr (chunked) {
-        // everything this workgroup will ever read is requested at once: the rest of the diagonal
-        // block's tiles and the running state (the kernel is latency-bound in this mode)
-        static_for<kPre, BM / BN>([&](auto qq) { issue_tile(decltype(qq)::value, decltype(qq)::value * STAGE); });
+        // The kernel is bound by its loads.  With two workgroups on a CU everything is requested at
+        // once (the other workgroup computes meanwhile).  A workgroup that has the CU to itself
+        // requests what the state product below needs first -- the X fragments and the running
+        // state, with tile 0 -- and the other tiles once that has landed, so that the product runs
+        // while they arrive: asked for together, all of it would arrive at the end.
+        constexpr bool kLateTiles = Cfg::kMinWavesPerSimd == 1;
+        if constexpr (!kLateTiles)
+            static_for<kPre, BM / BN>([&](auto qq) { issue_tile(decltype(qq)::value, decltype(qq)::value * STAGE); });
         if constexpr (Cfg::kStateInLds) {
             if (has_state) {
                 const u32x4 rs = make_rsrc(st, DO * DC * 2);
@@ -551,6 +556,8 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         wait_vm<0>();
         __builtin_amdgcn_s_barrier();
         pin_x();
+        if constexpr (kLateTiles)
+            static_for<kPre, BM / BN>([&](auto qq) { issue_tile(decltype(qq)::value, decltype(qq)::value * STAGE); });
         FLA_STAMP(1);
     } else {
         // tiles up to NBUF-3 before the first wait, tile NBUF-2 right after it
@@ -825,11 +832,9 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     {
         static_assert(BM / BN <= Cfg::NBUF, "the diagonal block must fit in the LDS ring");
         if (n_full > 0) __builtin_amdgcn_s_barrier();  // every wave is done with the last full tile
-        if constexpr (!chunked) {
-            issue_tile(q + Cfg::NBUF - 1, prev_off);  // the one tile not yet requested (if any)
-            wait_vm<0>();
-            __builtin_amdgcn_s_barrier();
-        }
+        if constexpr (!chunked) issue_tile(q + Cfg::NBUF - 1, prev_off);  // the one tile not yet requested (if any)
+        wait_vm<0>();
+        __builtin_amdgcn_s_barrier();
         FLA_STAMP(5);
 
         const int nsub = (diag_rows + 31) >> 5;  // sub-tiles with at least one valid row
