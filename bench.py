@@ -42,7 +42,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per kernel launch (mean over the launches of one step), measured with
 # `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`, each scaled by what the same counter
 # reads for a 256 MiB device copy (fetch x2.0, write x1.0); see profiles/*_pmc.md.
-MEASURED_TRAFFIC_BYTES = {"C3": 2.416e9}
+MEASURED_TRAFFIC_BYTES = {"C3": 2.420e9}
 
 
 def _parse():
