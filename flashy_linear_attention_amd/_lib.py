@@ -11,8 +11,7 @@ import os
 import threading
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
-# FLA_LIB_PATH points at another build of the same library (e.g. an experimental one)
-LIB_PATH = os.environ.get("FLA_LIB_PATH") or os.path.join(_PKG_DIR, "libfla_gfx950.so")
+LIB_PATH = os.path.join(_PKG_DIR, "libfla_gfx950.so")
 ABI_VERSION = 1
 
 FLA_DTYPE_BF16 = 0

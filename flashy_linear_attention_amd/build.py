@@ -60,16 +60,8 @@ def _compile_inst(args) -> str:
     return obj
 
 
-def build(jobs: int | None = None, verbose: bool = True, extra_flags: List[str] | None = None,
-          lib_path: str | None = None) -> str:
-    """Compile every kernel instantiation and link the shared library.  Always recompiles.
-    ``extra_flags`` / ``lib_path`` build an experimental variant somewhere else."""
-    global HIPCC_FLAGS, LIB_PATH, OBJ_DIR
-    if extra_flags:
-        HIPCC_FLAGS = HIPCC_FLAGS + list(extra_flags)
-    if lib_path:
-        LIB_PATH = lib_path
-        OBJ_DIR = os.path.join(os.path.dirname(lib_path), "_obj")
+def build(jobs: int | None = None, verbose: bool = True) -> str:
+    """Compile every kernel instantiation and link the shared library.  Always recompiles."""
     os.makedirs(OBJ_DIR, exist_ok=True)
     jobs = jobs or min(8, os.cpu_count() or 1)
     work = [(t, dc, do) for t in (0, 1) for dc in DIMS for do in DIMS]
@@ -86,10 +78,5 @@ def build(jobs: int | None = None, verbose: bool = True, extra_flags: List[str] 
 
 
 if __name__ == "__main__":
-    # usage: python -m flashy_linear_attention_amd.build [--out LIB.so] [extra hipcc flags...]
-    argv = sys.argv[1:]
-    out = None
-    if argv[:1] == ["--out"]:
-        out, argv = argv[1], argv[2:]
-    build(extra_flags=argv, lib_path=out)
+    build()
     sys.exit(0)

@@ -4,7 +4,6 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
-#include <stdlib.h>
 
 #include "fla_dispatch.h"
 #include "fla_norm.h"
@@ -68,12 +67,56 @@ int vec_ok(const View &t, int64_t width) {
            t.strides[1] % 8 == 0 && t.strides[2] % 8 == 0;
 }
 
+// The kernels read tiles of the inputs while other workgroups already write results: an output
+// that shares memory with an input (or with another output) would be read half-updated.  The
+// test is on the byte ranges [first element, one past the last addressed element).
+struct Span {
+    uintptr_t lo, hi;
+};
+
+Span span_of(const View &t, int64_t B, int64_t H, int64_t N, int64_t width) {
+    if (B <= 0 || H <= 0 || N <= 0 || !t.ptr || !t.strides) return {0, 0};
+    const int64_t last = (B - 1) * t.strides[0] + (H - 1) * t.strides[1] + (N - 1) * t.strides[2] + width;
+    const uintptr_t lo = reinterpret_cast<uintptr_t>(t.ptr);
+    return {lo, lo + (uintptr_t)last * 2};
+}
+
+bool overlap(const Span &a, const Span &b) { return a.lo < b.hi && b.lo < a.hi; }
+
+int check_alias(const Span *ins, int n_in, const Span *outs, int n_out) {
+    for (int o = 0; o < n_out; ++o) {
+        for (int i = 0; i < n_in; ++i)
+            if (overlap(outs[o], ins[i])) return FLA_ERR_ALIAS;
+        for (int o2 = o + 1; o2 < n_out; ++o2)
+            if (overlap(outs[o], outs[o2])) return FLA_ERR_ALIAS;
+    }
+    return FLA_OK;
+}
+
 int check_common(int64_t B, int64_t H, int64_t N, int dtype) {
     if (dtype != FLA_DTYPE_BF16 && dtype != FLA_DTYPE_F16) return FLA_ERR_DTYPE;
     if (B < 0 || H < 0 || N < 0) return FLA_ERR_SHAPE;
     if (N > (int64_t)1 << 30) return FLA_ERR_SHAPE;
     if (H > 0 && B > ((int64_t)1 << 30) / H) return FLA_ERR_SHAPE;
     return FLA_OK;
+}
+
+// forward-shaped call: two operands of width dc and one of width dout in, one of width dout out
+int check_alias_fwd(const View &x, const View &y, const View &z, const View &out, int64_t B, int64_t H, int64_t N,
+                    int64_t dc, int64_t dout) {
+    const Span ins[] = {span_of(x, B, H, N, dc), span_of(y, B, H, N, dc), span_of(z, B, H, N, dout)};
+    const Span outs[] = {span_of(out, B, H, N, dout)};
+    return check_alias(ins, 3, outs, 1);
+}
+
+// backward-shaped call: go, v (and the forward's output `o`, when given) of width dv, q, k of width
+// dqk in; dq, dk of width dqk and dv of width dv out
+int check_alias_bwd(const View &go, const View &q, const View &k, const View &v, const View *o, const View &dq,
+                    const View &dk, const View &dvv, int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
+    const Span ins[] = {span_of(go, B, H, N, dv), span_of(q, B, H, N, dqk), span_of(k, B, H, N, dqk),
+                        span_of(v, B, H, N, dv), o ? span_of(*o, B, H, N, dv) : Span{0, 0}};
+    const Span outs[] = {span_of(dq, B, H, N, dqk), span_of(dk, B, H, N, dqk), span_of(dvv, B, H, N, dv)};
+    return check_alias(ins, 5, outs, 3);
 }
 
 TriParams make_params(const View &x, const View &y, const View &z, const View &out, int64_t B, int64_t H, int64_t N,
@@ -96,12 +139,6 @@ TriParams make_params(const View &x, const View &y, const View &z, const View &o
     p.poly[0] = p.poly[1] = p.poly[2] = 0.f;
     p.poly_on = 0;
     p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout), p.vec_out = vec_ok(out, dout);
-#ifdef FLA_DBG_TIMING
-    {
-        const char *e = getenv("FLA_DBG_TIMING_PTR");
-        p.dbg = e ? reinterpret_cast<unsigned long long *>(strtoull(e, nullptr, 16)) : nullptr;
-    }
-#endif
     return p;
 }
 
@@ -243,6 +280,7 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
     const View all[] = {q, k, v, o};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
+    if (int rc = check_alias_fwd(q, k, v, o, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
     const TriParams p = make_params(q, k, v, o, B, H, N, dqk, dv, 0);
     if (!states_shareable(dqk, dv, N) || !fla::fast_path_ok(p))
@@ -265,6 +303,7 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
     const View all[] = {go, q, k, v, dq, dk, dvv};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
+    if (int rc = check_alias_bwd(go, q, k, v, nullptr, dq, dk, dvv, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
     const TriParams pq = make_params(go, v, k, dq, B, H, N, dv, dqk, 0);   // dQ = lower(dO V^T) K
     const TriParams pv = make_params(k, q, go, dvv, B, H, N, dqk, dv, 1);  // dV = upper(K Q^T) dO
@@ -299,6 +338,7 @@ int forward(const View &q, const View &k, const View &v, const View &o, int64_t 
     const View all[] = {q, k, v, o};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
+    if (int rc = check_alias_fwd(q, k, v, o, B, H, N, dqk, dv)) return rc;
     return run_tri(q, k, v, o, B, H, N, dqk, dv, 0, dtype, stream);
 }
 
@@ -331,6 +371,7 @@ int backward(const View &go, const View &q, const View &k, const View &v, const 
     const View all[] = {go, q, k, v, dq, dk, dv};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
+    if (int rc = check_alias_bwd(go, q, k, v, nullptr, dq, dk, dv, B, H, N, dqk, dvw)) return rc;
     return backward_products(go, q, k, v, dq, dk, dv, B, H, N, dqk, dvw, dtype, stream);
 }
 
@@ -415,6 +456,7 @@ int normalised_forward(const View &q, const View &k, const View &v, const View &
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
     if (!denom) return FLA_ERR_NULL_POINTER;
+    if (int rc = check_alias_fwd(q, k, v, o, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
     const NormLayout l = norm_layout(B, H, N, dqk, dv, chunked);
     if ((l.chunks > 1 || l.chunk_bytes > 0) &&
@@ -450,6 +492,7 @@ int normalised_backward(const View &go, const View &q, const View &k, const View
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
     if (!denom) return FLA_ERR_NULL_POINTER;
+    if (int rc = check_alias_bwd(go, q, k, v, &o, dq, dk, dvv, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
     const NormLayout l = norm_layout(B, H, N, dqk, dv, chunked);
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < l.norm_bytes + l.chunk_bytes)
@@ -517,13 +560,13 @@ __global__ __launch_bounds__(256) void pack_pair_kernel(const T *a, int64_t as_b
 }
 
 template <typename T>
-void launch_pack(const View &a, int wa, const View &x, int wx, void *out, int64_t B, int64_t H, int64_t N, int split,
+hipError_t launch_pack(const View &a, int wa, const View &x, int wx, void *out, int64_t B, int64_t H, int64_t N, int split,
                  int rp, int bias_mode, const float *bias, hipStream_t s) {
     const int64_t total = B * H * N * ((split + rp) / 8);
-    hipLaunchKernelGGL((pack_pair_kernel<T>), dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
-                       static_cast<const T *>(a.ptr), a.strides[0], a.strides[1], a.strides[2], wa,
-                       static_cast<const T *>(x.ptr), x.strides[0], x.strides[1], x.strides[2], wx,
-                       static_cast<T *>(out), (int)H, N, split, rp, total, bias_mode, bias);
+    return fla::launch_kernel(pack_pair_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+                              static_cast<const T *>(a.ptr), a.strides[0], a.strides[1], a.strides[2], wa,
+                              static_cast<const T *>(x.ptr), x.strides[0], x.strides[1], x.strides[2], wx,
+                              static_cast<T *>(out), (int)H, N, split, rp, total, bias_mode, bias);
 }
 
 struct PolyLayout {
@@ -577,6 +620,7 @@ int poly_forward(const View &xq, const View &xk, const View &v, const View &o, f
     const View all[] = {xq, xk, v, o};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
+    if (int rc = check_alias_fwd(xq, xk, v, o, B, H, N, r, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
     if (denom && B * H > 65535) return FLA_ERR_SHAPE;
     TriParams p = make_params(xq, xk, v, o, B, H, N, r, dv, 0);
@@ -597,6 +641,7 @@ int poly_backward(const View &go, const View &xq, const View &xk, const View &v,
         if (!denom) return FLA_ERR_NULL_POINTER;
         if (B * H > 65535) return FLA_ERR_SHAPE;
     }
+    if (int rc = check_alias_bwd(go, xq, xk, v, o, dxq, dxk, dvv, B, H, N, r, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
     const PolyLayout l = poly_layout(B, H, N, r, dv, normalised);
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 ||
@@ -628,14 +673,10 @@ int poly_backward(const View &go, const View &xq, const View &xk, const View &v,
         g = View{dO, do_strides};
     }
     const int bias1 = normalised ? 1 : 0, bias2 = normalised ? 2 : 0;
-    if (dtype == FLA_DTYPE_BF16) {
-        launch_pack<__bf16>(g, (int)dv, xq, (int)r, p1, B, H, N, (int)l.split, (int)l.rp, bias1, dn, s);
-        launch_pack<__bf16>(v, (int)dv, xk, (int)r, p2, B, H, N, (int)l.split, (int)l.rp, bias2, nullptr, s);
-    } else {
-        launch_pack<_Float16>(g, (int)dv, xq, (int)r, p1, B, H, N, (int)l.split, (int)l.rp, bias1, dn, s);
-        launch_pack<_Float16>(v, (int)dv, xk, (int)r, p2, B, H, N, (int)l.split, (int)l.rp, bias2, nullptr, s);
-    }
-    if (hipGetLastError() != hipSuccess) return FLA_ERR_LAUNCH;
+    const auto pack = dtype == FLA_DTYPE_BF16 ? launch_pack<__bf16> : launch_pack<_Float16>;
+    if (pack(g, (int)dv, xq, (int)r, p1, B, H, N, (int)l.split, (int)l.rp, bias1, dn, s) != hipSuccess) return FLA_ERR_LAUNCH;
+    if (pack(v, (int)dv, xk, (int)r, p2, B, H, N, (int)l.split, (int)l.rp, bias2, nullptr, s) != hipSuccess)
+        return FLA_ERR_LAUNCH;
     const int64_t ps[4] = {H * N * l.width, N * l.width, l.width, 1};
     const View P1{p1, ps}, P2{p2, ps};
     // dV = upper(f(Xk Xq^T)) dO
@@ -668,6 +709,7 @@ const char *fla_strerror(int status) {
         case FLA_ERR_LAUNCH: return "the HIP runtime rejected the kernel launch";
         case FLA_ERR_UNSUPPORTED: return "no kernel was built for this combination";
         case FLA_ERR_WORKSPACE: return "workspace is NULL, not 16-byte aligned, or smaller than fla_chunked_workspace_bytes()";
+        case FLA_ERR_ALIAS: return "an output tensor overlaps an input or another output in memory";
         default: return "unknown fla status";
     }
 }
@@ -723,6 +765,7 @@ int fla_tri_xyt_z(const void *x, const void *y, const void *z, void *out, int64_
     const View all[] = {vx, vy, vz, vo};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
+    if (int rc = check_alias_fwd(vx, vy, vz, vo, B, H, N, D_c, D_o)) return rc;
     return run_tri(vx, vy, vz, vo, B, H, N, D_c, D_o, upper, dtype, stream);
 }
 
@@ -741,6 +784,7 @@ int fla_tri_xyt_z_chunked(const void *x, const void *y, const void *z, void *out
     const View all[] = {vx, vy, vz, vo};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
+    if (int rc = check_alias_fwd(vx, vy, vz, vo, B, H, N, D_c, D_o)) return rc;
     return run_tri_chunked(vx, vy, vz, vo, B, H, N, D_c, D_o, upper, dtype, workspace, workspace_bytes, stream);
 }
 

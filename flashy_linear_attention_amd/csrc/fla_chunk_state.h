@@ -244,13 +244,10 @@ hipError_t launch_chunk_state(ChunkStateParams p, hipStream_t stream) {
     } else {
         const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_chunks;
         if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-        auto kern = chunk_state_kernel<T, DC, DO>;
+        constexpr auto kern = chunk_state_kernel<T, DC, DO>;
         constexpr int smem = ChunkStateLds<DC, DO>::kBytes;
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
-        return hipGetLastError();
+        if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
+        return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
     }
 }
 
@@ -260,9 +257,8 @@ hipError_t launch_chunk_scan(const float *w, void *state, int64_t BH, int n_chun
     const int64_t total2 = BH * E / 2;
     const int64_t grid = (total2 + 255) / 256;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-    hipLaunchKernelGGL(chunk_scan_kernel<T>, dim3((unsigned)grid), dim3(256), 0, stream, w, static_cast<T *>(state),
-                       n_chunks, E, total2, reverse);
-    return hipGetLastError();
+    return launch_kernel(chunk_scan_kernel<T>, dim3((unsigned)grid), dim3(256), 0, stream, w, static_cast<T *>(state),
+                         n_chunks, E, total2, reverse);
 }
 
 }  // namespace fla

@@ -380,31 +380,28 @@ inline int norm_chunk_rows(int lpr) { return 4 * (64 / lpr) * kNormSegRows; }
 
 inline hipError_t launch_norm_scan(const NormParams &p, int dp, bool with_w, hipStream_t s) {
     const int64_t threads = (int64_t)p.BH * dp;
-    hipLaunchKernelGGL(norm_scan_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, p.ksum,
-                       with_w ? p.wsum : nullptr, p.BH, p.n_chunks, dp);
-    return hipGetLastError();
+    return launch_kernel(norm_scan_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, p.ksum,
+                         with_w ? p.wsum : nullptr, p.BH, p.n_chunks, dp);
 }
 
 // which: 0 forward, 1 backward-pre, 2 backward-post
 template <typename T, int LPR, bool VEC>
 hipError_t launch_norm_lpr(int which, const NormParams &p, hipStream_t s) {
     const dim3 grid((unsigned)p.n_chunks, (unsigned)p.BH);
+    // every launch is checked on its own: nothing further is enqueued after a failed one
     if (which == 0) {
         if (p.n_chunks > 1) {
-            hipLaunchKernelGGL((norm_chunk_sums_kernel<T, LPR, VEC, false>), grid, dim3(256), 0, s, p);
-            launch_norm_scan(p, LPR * 8, false, s);
+            if (hipError_t e = launch_kernel(norm_chunk_sums_kernel<T, LPR, VEC, false>, grid, dim3(256), 0, s, p)) return e;
+            if (hipError_t e = launch_norm_scan(p, LPR * 8, false, s)) return e;
         }
-        hipLaunchKernelGGL((norm_fwd_kernel<T, LPR, VEC>), grid, dim3(256), 0, s, p);
-    } else if (which == 1) {
-        hipLaunchKernelGGL((norm_bwd_pre_kernel<T, LPR, VEC>), grid, dim3(256), 0, s, p);
-    } else {
-        if (p.n_chunks > 1) {
-            hipLaunchKernelGGL((norm_chunk_sums_kernel<T, LPR, VEC, true>), grid, dim3(256), 0, s, p);
-            launch_norm_scan(p, LPR * 8, true, s);
-        }
-        hipLaunchKernelGGL((norm_bwd_post_kernel<T, LPR, VEC>), dim3(grid.x, grid.y, 2), dim3(256), 0, s, p);
+        return launch_kernel(norm_fwd_kernel<T, LPR, VEC>, grid, dim3(256), 0, s, p);
     }
-    return hipGetLastError();
+    if (which == 1) return launch_kernel(norm_bwd_pre_kernel<T, LPR, VEC>, grid, dim3(256), 0, s, p);
+    if (p.n_chunks > 1) {
+        if (hipError_t e = launch_kernel(norm_chunk_sums_kernel<T, LPR, VEC, true>, grid, dim3(256), 0, s, p)) return e;
+        if (hipError_t e = launch_norm_scan(p, LPR * 8, true, s)) return e;
+    }
+    return launch_kernel(norm_bwd_post_kernel<T, LPR, VEC>, dim3(grid.x, grid.y, 2), dim3(256), 0, s, p);
 }
 
 // lpr from norm_lanes_per_row; vec: every operand of this call qualifies for 16-byte accesses

@@ -37,14 +37,6 @@
 //     kernel (grid y selects one of up to three products: the backward's dQ, dV,
 //     dK in one launch) and the chunked kernel (CHUNKED: diagonal block plus
 //     the running state of the chunk-wise evaluation, no tile ring).
-//
-// Measurement switches (never defined in a product build; results of such builds are wrong):
-//   FLA_DBG_TIMING     every workgroup writes shader-clock stamps of its phases to TriParams::dbg
-//   FLA_DBG_NO_DMA / NO_ZREAD / NO_YREAD / NO_WAIT / NO_BARRIER / NO_CVT / NO_DIAG
-//                      drop the tile loads / the Z or Y fragment reads / the waits for tiles /
-//                      the per-tile barrier / the rounding / the diagonal walk
-//   FLA_DBG_FILL_LDS   fill LDS with random 16-bit values at workgroup start (with NO_DMA)
-//   FLA_DMA_BURST      issue a tile's loads in one burst after the barrier instead of spread out
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -68,9 +60,6 @@ typedef short s16x8 __attribute__((ext_vector_type(8)));
 // written: the loads of one tile then need a single scalar base between them.
 template <int LDS_IMM>
 __device__ __forceinline__ void dma_16B_per_lane(u32x4 rsrc, uint32_t lds_base, uint32_t voffset, uint32_t soffset) {
-#ifdef FLA_DBG_NO_DMA
-    return;
-#endif
     asm volatile("s_add_u32 m0, %0, %4\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :
                  : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset), "n"(LDS_IMM)
@@ -113,9 +102,6 @@ __device__ __forceinline__ uint32_t round_pack_pinned(float lo, float hi) {
     pr[0] = static_cast<T>(lo);
     pr[1] = static_cast<T>(hi);
     uint32_t r = __builtin_bit_cast(uint32_t, pr);
-#ifdef FLA_DBG_NO_CVT
-    r = __builtin_bit_cast(uint32_t, lo);
-#endif
     asm volatile("" : "+v"(r));
     return r;
 }
@@ -232,15 +218,6 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, g = lane >> 5, lam = lane & 15;
-#ifdef FLA_DBG_FILL_LDS
-    // ablation builds without the loads: LDS holds pseudo-random 16-bit values of magnitude ~1
-    for (int i = threadIdx.x; i < Cfg::SMEM_BYTES / 4; i += 256) {
-        uint32_t h = (uint32_t)i * 2654435761u + blockIdx.x * 40503u;
-        h ^= h >> 15;
-        reinterpret_cast<uint32_t *>(smem)[i] = 0x3f003f00u | (h & 0x80ff80ffu);
-    }
-    __syncthreads();
-#endif
 
     const int wg = wg_index, xcd = wg & 7, slot = wg >> 3;
     // Each workgroup takes two row tiles of one head, r and n_tiles-1-r: under a triangular
@@ -276,23 +253,6 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     blk[0] = wave;
     if constexpr (NIB == 2) blk[1] = NBLK - 1 - wave;
 
-    // FLA_DBG_TIMING builds record the shader clock at the phase boundaries of every workgroup
-#ifdef FLA_DBG_TIMING
-#define FLA_STAMP(k)                                                                                           \
-    do {                                                                                                       \
-        if (p.dbg && tid == 0) p.dbg[(size_t)wg_index * 16 + pass * 8 + (k)] = __builtin_readcyclecounter(); \
-    } while (0)
-#else
-#define FLA_STAMP(k) \
-    do {             \
-    } while (0)
-#endif
-#ifdef FLA_DBG_TIMING
-    // slot 7: constant-rate (100 MHz) clock at workgroup start, hardware id in the top bits; slot 15: at the end
-    if (p.dbg && tid == 0)
-        p.dbg[(size_t)wg_index * 16 + 7] = (__builtin_amdgcn_s_memrealtime() & 0xffffffffffull) |
-                                             ((unsigned long long)__builtin_amdgcn_s_getreg(63492) << 40);
-#endif
     // ---- the row tiles of this workgroup, in the order they are done: unpaired tiles go heaviest
     // first (last row tile under a lower mask, first under an upper one); with an odd tile
     // count the middle tile has no partner; chunked: a single tile per workgroup
@@ -417,7 +377,6 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     start_tile();
 
     for (int pass = 0;; ++pass) {
-    FLA_STAMP(0);
 
     f32x16 acc[NIB][DB];
 #pragma unroll
@@ -558,7 +517,6 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         pin_x();
         if constexpr (kLateTiles)
             static_for<kPre, BM / BN>([&](auto qq) { issue_tile(decltype(qq)::value, decltype(qq)::value * STAGE); });
-        FLA_STAMP(1);
     } else {
         // tiles up to NBUF-3 before the first wait, tile NBUF-2 right after it
         static_for<kPre, Cfg::NBUF - 2>(
@@ -566,7 +524,6 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         wait_tile();
         __builtin_amdgcn_s_barrier();  // tile 0 (and the X fragments) have landed
         pin_x();
-        FLA_STAMP(1);
         issue_tile(Cfg::NBUF - 2, wrap_slot(ring0 + (Cfg::NBUF - 2) * STAGE));
     }
     // from here on: tiles up to q + NBUF - 2 are issued while tile q is consumed, and tile
@@ -602,15 +559,9 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
                         s2[ib] = M::mma(yf[kc], xf[ib][kc], kc == KC1 ? zero : s2[ib]);
                 }
                 if constexpr (decltype(with_z)::value) {
-#ifndef FLA_DBG_NO_ZREAD
 #pragma unroll
                     for (int f = 0; f < NZF; ++f)
                         if (f * KCU / NZF == kc) zf[f] = z_read(za, zsub, f);
-#else
-#pragma unroll
-                    for (int f = 0; f < NZF; ++f)
-                        if (f * KCU / NZF == kc) asm volatile("" : "+v"(zf[f]));
-#endif
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
@@ -628,15 +579,9 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
 #pragma unroll
                     for (int ib = 0; ib < NIB; ++ib) acc[ib][db] = M::mma(zf[f], pprev[ib][t], acc[ib][db]);
                 }
-#ifndef FLA_DBG_NO_YREAD
 #pragma unroll
                 for (int kc = 0; kc < KCU; ++kc)
                     if (kc * NZF / KCU == f) yf[kc] = y_read(ya, ysub, kc);
-#else
-#pragma unroll
-                for (int kc = 0; kc < KCU; ++kc)
-                    if (kc * NZF / KCU == f) asm volatile("" : "+v"(yf[kc]));
-#endif
                 if constexpr (POLY) {
                     if (f == NZF / 2) {
 #pragma unroll
@@ -683,21 +628,8 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
             phase2(std::integral_constant<bool, !kFirst>{}, pfb, pfa, ya_cur, 1, [](auto) {});
             // second sub-tile
             phase1(std::true_type{}, za_cur, 0);
-#ifndef FLA_DBG_NO_WAIT
             wait_tile();
-#endif
-#ifndef FLA_DBG_NO_BARRIER
             __builtin_amdgcn_s_barrier();  // tile q+1 has landed; nobody reads tile q-1 any more
-#endif
-#ifdef FLA_DMA_BURST
-            constexpr bool kSpread = false;
-#else
-            constexpr bool kSpread = true;
-#endif
-            if constexpr (!kSpread) {
-                issue_tile(q + Cfg::NBUF - 1, prev_off);
-                phase2(std::true_type{}, pfa, pfb, ya_next, 0, [](auto) {});
-            } else
             // The loads of tile q + NBUF - 1 go into the slot the barrier has just retired.  A wave
             // issues one instruction every few clocks and a load to LDS holds it for longer than
             // that, so all of them in a row would leave the matrix pipe idle: one (or a few) after
@@ -824,7 +756,6 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         }
     }
 
-    FLA_STAMP(2);
     // ================= the diagonal block =================
     // Its tiles (BM / BN of them, never more than the ring holds) are all made resident first;
     // then every wave walks the 32-row sub-tiles its two row blocks touch, without barriers,
@@ -835,7 +766,6 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         if constexpr (!chunked) issue_tile(q + Cfg::NBUF - 1, prev_off);  // the one tile not yet requested (if any)
         wait_vm<0>();
         __builtin_amdgcn_s_barrier();
-        FLA_STAMP(5);
 
         const int nsub = (diag_rows + 31) >> 5;  // sub-tiles with at least one valid row
         int blk_min = blk[0], blk_max = blk[0];
@@ -897,7 +827,6 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
                 for (int f = 0; f < NZF; ++f) acc[ib][f % DB] = M::mma(zf[f], pf[f / DB], acc[ib][f % DB]);
             }
         };
-#ifndef FLA_DBG_NO_DIAG
         if (s_lo <= s_hi) {
             V8 yfa[KC], zfa[NZF], yfb[KC], zfb[NZF];
             load_sub(s_lo, yfa, zfa);
@@ -915,12 +844,9 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
                 }
             }
         }
-#endif
-        FLA_STAMP(6);
         __builtin_amdgcn_s_barrier();  // all LDS reads of the walk are done: the ring can be reused
     }
 
-    FLA_STAMP(3);
     // ---- the next row tile's first requests go out before this one's epilogue
     const int out_i0 = i0;
     const bool more = pass + 1 < n_pass;
@@ -993,7 +919,6 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     }
-    FLA_STAMP(4);
     if (!more) break;
     if constexpr (!kOverlap) {
         set_tile(stream_tile(pass + 1));
@@ -1001,9 +926,6 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         start_tile();
     }
     }  // pass
-#ifdef FLA_DBG_TIMING
-    if (p.dbg && tid == 0) p.dbg[(size_t)wg_index * 16 + 15] = __builtin_amdgcn_s_memrealtime() & 0xffffffffffull;
-#endif
 #else
     (void)p;
     (void)wg_index;
@@ -1086,13 +1008,10 @@ hipError_t launch_tri_fast_variant(TriParams p, hipStream_t stream) {
         p.single = (!CHUNKED && run_single_tiles((int64_t)p.BH * ((p.n_tiles + 1) / 2), Cfg::kMinWavesPerSimd)) ? 1 : 0;
         const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * ((CHUNKED || p.single) ? p.n_tiles : (p.n_tiles + 1) / 2);
         if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-        auto kern = tri_xyt_z_fast_kernel<T, DC, DO, CHUNKED, FLAGS>;
-        const int smem = Cfg::SMEM_BYTES + (Cfg::kStateInLds ? Cfg::STATE_BYTES : 0);
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
-        return hipGetLastError();
+        constexpr auto kern = tri_xyt_z_fast_kernel<T, DC, DO, CHUNKED, FLAGS>;
+        constexpr int smem = Cfg::SMEM_BYTES + (Cfg::kStateInLds ? Cfg::STATE_BYTES : 0);
+        if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
+        return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
     }
 }
 
@@ -1108,12 +1027,9 @@ hipError_t launch_tri_fast_batch(TriBatch b, int count, hipStream_t stream) {
         for (int i = 0; i < count; ++i) b.p[i].n_tiles = n_tiles, b.p[i].single = single, b.p[i].state = nullptr;
         const int64_t grid = (int64_t)8 * ((b.p[0].BH + 7) / 8) * (single ? n_tiles : (n_tiles + 1) / 2);
         if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-        auto kern = tri_xyt_z_fast_batch_kernel<T, DC, DO>;
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM_BYTES);
-        if (e != hipSuccess) return e;
-        hipLaunchKernelGGL(kern, dim3((unsigned)grid, (unsigned)count), dim3(256), Cfg::SMEM_BYTES, stream, b);
-        return hipGetLastError();
+        constexpr auto kern = tri_xyt_z_fast_batch_kernel<T, DC, DO>;
+        if (hipError_t e = ensure_dynamic_lds<kern>(Cfg::SMEM_BYTES)) return e;
+        return launch_kernel(kern, dim3((unsigned)grid, (unsigned)count), dim3(256), Cfg::SMEM_BYTES, stream, b);
     }
 }
 

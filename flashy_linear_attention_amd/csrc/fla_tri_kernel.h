@@ -33,6 +33,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "fla_launch.h"
+
 namespace fla {
 
 struct TriParams {
@@ -71,9 +73,6 @@ struct TriParams {
     // last 32 columns, [DC - 32, DC).
     float poly[3];
     int32_t poly_on;
-#ifdef FLA_DBG_TIMING
-    unsigned long long *dbg;      // 16 clock stamps per workgroup (experimental builds only)
-#endif
 };
 
 // Up to three products of identical shape in one launch (grid y selects the product): the
@@ -359,12 +358,9 @@ hipError_t launch_tri(TriParams p, hipStream_t stream) {
     p.n_tiles = (p.N + Cfg::BM - 1) / Cfg::BM;
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_tiles;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-    auto kern = tri_xyt_z_kernel<T, DC, DO>;
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, Cfg::SMEM_BYTES);
-    if (e != hipSuccess) return e;
-    hipLaunchKernelGGL(kern, dim3((unsigned)grid), dim3(256), Cfg::SMEM_BYTES, stream, p);
-    return hipGetLastError();
+    constexpr auto kern = tri_xyt_z_kernel<T, DC, DO>;
+    if (hipError_t e = ensure_dynamic_lds<kern>(Cfg::SMEM_BYTES)) return e;
+    return launch_kernel(kern, dim3((unsigned)grid), dim3(256), Cfg::SMEM_BYTES, stream, p);
 }
 
 }  // namespace fla

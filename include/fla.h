@@ -14,7 +14,10 @@
  *     run on bf16 / fp16 MFMA with fp32 accumulation; outputs are rounded once.
  *   - `stream` is a hipStream_t (NULL = the null stream).  Calls only enqueue
  *     work; they never synchronise, allocate or free.  Outputs must not alias
- *     inputs.
+ *     inputs or each other: the byte range each tensor spans (first to last
+ *     addressed element) is compared on the host and an overlap is rejected with
+ *     FLA_ERR_ALIAS (the reference's wrappers always allocate fresh outputs,
+ *     linear_attn_kernels.py:327, 366-368).
  *   - Re-entrant, no global mutable state (except the no-allocation variant
  *     documented at its declaration, if present).
  *   - Return value: FLA_OK or a negative FLA_ERR_* code; fla_strerror() names it.
@@ -47,7 +50,8 @@ enum fla_status {
     FLA_ERR_STRIDE = -6,       /* strides[3] != 1, a NULL strides array, or a negative stride */
     FLA_ERR_LAUNCH = -7,       /* the HIP runtime rejected the launch */
     FLA_ERR_UNSUPPORTED = -8,  /* no kernel was built for this combination */
-    FLA_ERR_WORKSPACE = -9     /* chunked call: workspace missing, misaligned or too small */
+    FLA_ERR_WORKSPACE = -9,    /* chunked call: workspace missing, misaligned or too small */
+    FLA_ERR_ALIAS = -10        /* an output tensor's byte range overlaps an input's or another output's */
 };
 
 /* ABI revision of the loaded library (== FLA_ABI_VERSION it was built with). */

@@ -55,54 +55,95 @@ def _null_call(name, *tail):
 
 S = (ctypes.c_int64 * 4)(4096, 2048, 32, 1)
 BAD_S = (ctypes.c_int64 * 4)(4096, 2048, 64, 2)
-P = ctypes.c_void_p(0x1000)  # never dereferenced: every call below fails validation first
+# fake device pointers 4 GiB apart (distinct tensors must not overlap); never dereferenced:
+# every call below fails validation first
+A = [ctypes.c_void_p((i + 1) << 32) for i in range(10)]
+P = A[0]
 
 
 def test_c_abi_validation_codes():
     lib = _lib.load()
     f = lib.fla_linear_attn_fwd
-    assert f(P, P, P, P, 1, 2, 64, 32, S, S, S, S, 7, None) == -2          # dtype
-    assert f(P, P, P, P, 1, 2, 64, 257, S, S, S, S, 0, None) == -3         # head dim
-    assert f(P, P, P, P, 1, 2, 64, 0, S, S, S, S, 0, None) == -3
-    assert f(P, P, P, P, -1, 2, 64, 32, S, S, S, S, 0, None) == -5         # shape
-    assert f(None, P, P, P, 1, 2, 64, 32, S, S, S, S, 0, None) == -1       # null pointer
-    assert f(P, P, P, P, 1, 2, 64, 32, S, BAD_S, S, S, 0, None) == -6      # innermost stride
-    assert f(P, P, P, P, 1, 2, 64, 32, S, S, None, S, 0, None) == -6       # missing strides
-    assert f(P, P, P, P, 0, 2, 64, 32, S, S, S, S, 0, None) == 0           # empty problem: no-op
-    assert f(P, P, P, P, 1, 2, 0, 32, S, S, S, S, 1, None) == 0
+    assert f(A[0], A[1], A[2], A[3], 1, 2, 64, 32, S, S, S, S, 7, None) == -2          # dtype
+    assert f(A[0], A[1], A[2], A[3], 1, 2, 64, 257, S, S, S, S, 0, None) == -3         # head dim
+    assert f(A[0], A[1], A[2], A[3], 1, 2, 64, 0, S, S, S, S, 0, None) == -3
+    assert f(A[0], A[1], A[2], A[3], -1, 2, 64, 32, S, S, S, S, 0, None) == -5         # shape
+    assert f(None, A[1], A[2], A[3], 1, 2, 64, 32, S, S, S, S, 0, None) == -1       # null pointer
+    assert f(A[0], A[1], A[2], A[3], 1, 2, 64, 32, S, BAD_S, S, S, 0, None) == -6      # innermost stride
+    assert f(A[0], A[1], A[2], A[3], 1, 2, 64, 32, S, S, None, S, 0, None) == -6       # missing strides
+    assert f(A[0], A[1], A[2], A[3], 0, 2, 64, 32, S, S, S, S, 0, None) == 0           # empty problem: no-op
+    assert f(A[0], A[1], A[2], A[3], 1, 2, 0, 32, S, S, S, S, 1, None) == 0
     b = lib.fla_linear_attn_bwd
-    assert b(P, P, P, P, P, P, P, 1, 2, 64, 300, S, S, S, S, S, S, S, 0, None) == -3
-    assert b(P, P, P, P, P, None, P, 1, 2, 64, 32, S, S, S, S, S, S, S, 0, None) == -1
+    assert b(A[0], A[1], A[2], A[3], A[4], A[5], A[6], 1, 2, 64, 300, S, S, S, S, S, S, S, 0, None) == -3
+    assert b(A[0], A[1], A[2], A[3], A[4], None, A[6], 1, 2, 64, 32, S, S, S, S, S, S, S, 0, None) == -1
     sf = lib.fla_linear_attn_smallv_fwd
-    assert sf(P, P, P, P, 1, 2, 64, 64, 24, S, S, S, S, 0, None) == -4     # D_v not a power of two
-    assert sf(P, P, P, P, 1, 2, 64, 32, 64, S, S, S, S, 0, None) == -4     # D_v above padded D_qk
-    assert sf(P, P, P, P, 1, 2, 64, 300, 64, S, S, S, S, 0, None) == -3
-    assert sf(P, P, P, P, 1, 0, 64, 37, 64, S, S, S, S, 0, None) == 0      # 64 <= next_pow2(37): accepted
+    assert sf(A[0], A[1], A[2], A[3], 1, 2, 64, 64, 24, S, S, S, S, 0, None) == -4     # D_v not a power of two
+    assert sf(A[0], A[1], A[2], A[3], 1, 2, 64, 32, 64, S, S, S, S, 0, None) == -4     # D_v above padded D_qk
+    assert sf(A[0], A[1], A[2], A[3], 1, 2, 64, 300, 64, S, S, S, S, 0, None) == -3
+    assert sf(A[0], A[1], A[2], A[3], 1, 0, 64, 37, 64, S, S, S, S, 0, None) == 0      # 64 <= next_pow2(37): accepted
     sb = lib.fla_linear_attn_smallv_bwd
-    assert sb(P, P, P, P, P, P, P, 1, 2, 64, 257, 16, S, S, S, S, S, S, S, 0, None) == -3
+    assert sb(A[0], A[1], A[2], A[3], A[4], A[5], A[6], 1, 2, 64, 257, 16, S, S, S, S, S, S, S, 0, None) == -3
     t = lib.fla_tri_xyt_z
-    assert t(P, P, P, P, 1, 2, 64, 32, 300, S, S, S, S, 0, 0, None) == -3
-    assert t(P, P, P, P, 1, 2, 64, 32, 32, S, S, S, S, 1, 5, None) == -2
+    assert t(A[0], A[1], A[2], A[3], 1, 2, 64, 32, 300, S, S, S, S, 0, 0, None) == -3
+    assert t(A[0], A[1], A[2], A[3], 1, 2, 64, 32, 32, S, S, S, S, 1, 5, None) == -2
     nf = lib.fla_linear_attn_normalised_fwd
     eps = ctypes.c_float(1e-5)
-    assert nf(P, P, P, P, P, 1, 2, 64, 32, 32, S, S, S, S, eps, 9, 0, None, 0, None) == -2
-    assert nf(P, P, P, P, P, 1, 2, 64, 257, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -3
-    assert nf(P, P, P, P, P, 1, 2, 64, 32, 0, S, S, S, S, eps, 0, 0, None, 0, None) == -4
-    assert nf(P, P, P, P, P, 300, 300, 64, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -5   # B H > 65535
-    assert nf(P, P, P, P, None, 1, 2, 64, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -1    # denom
-    assert nf(P, P, P, P, P, 1, 2, 64, 32, 32, S, S, BAD_S, S, eps, 0, 0, None, 0, None) == -6
-    assert nf(P, P, P, P, P, 1, 2, 4096, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -9     # chunk sums need workspace
-    assert nf(P, P, P, P, P, 1, 0, 64, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == 0
+    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 64, 32, 32, S, S, S, S, eps, 9, 0, None, 0, None) == -2
+    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 64, 257, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -3
+    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 64, 32, 0, S, S, S, S, eps, 0, 0, None, 0, None) == -4
+    assert nf(A[0], A[1], A[2], A[3], A[4], 300, 300, 64, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -5   # B H > 65535
+    assert nf(A[0], A[1], A[2], A[3], None, 1, 2, 64, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -1    # denom
+    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 64, 32, 32, S, S, BAD_S, S, eps, 0, 0, None, 0, None) == -6
+    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 4096, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -9     # chunk sums need workspace
+    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 0, 64, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == 0
     nb = lib.fla_linear_attn_normalised_bwd
-    assert nb(P, P, P, P, P, P, P, P, P, 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, 0, None, 0, None) == -9
-    assert nb(P, P, P, P, P, None, P, P, P, 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, 1, P, 1 << 30, None) == -1
+    assert nb(A[0], A[1], A[2], A[3], A[4], A[5], A[6], A[7], A[8], 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, 0, None, 0, None) == -9
+    assert nb(A[0], A[1], A[2], A[3], A[4], None, A[6], A[7], A[8], 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, 1, A[9], 1 << 30, None) == -1
     assert lib.fla_normalised_workspace_bytes(1, 2, 64, 32, 32, 0) >= 2 * 64 * 32 * 2 + 2 * 64 * 4
     assert lib.fla_normalised_workspace_bytes(1, 2, 64, 300, 32, 0) == 0
     assert (lib.fla_normalised_workspace_bytes(1, 2, 4096, 64, 64, 1)
             > lib.fla_normalised_workspace_bytes(1, 2, 4096, 64, 64, 0))
-    for code in range(0, -10, -1):
+    for code in range(0, -11, -1):
         assert lib.fla_strerror(code)
     assert lib.fla_strerror(-3) == b"Only head_dims <= 256 are supported."
+
+
+def test_c_abi_rejects_outputs_that_overlap_inputs():
+    """The reference's wrappers allocate fresh outputs (linear_attn_kernels.py:327,366-368); the C
+    ABI takes caller-owned outputs, so an overlap with an input or another output is an error."""
+    lib = _lib.load()
+    q, k, v, o, g, dq, dk, dv = A[:8]
+    inside_q = ctypes.c_void_p(q.value + 2 * 64 * 32)  # second head of q
+    just_past_q = ctypes.c_void_p(q.value + 2 * (4096 + 2048 + 63 * 32 + 32))
+    f = lib.fla_linear_attn_fwd
+    assert f(q, k, v, q, 2, 2, 64, 32, S, S, S, S, 0, None) == -10
+    assert f(q, k, v, inside_q, 2, 2, 64, 32, S, S, S, S, 0, None) == -10
+    assert f(q, k, v, just_past_q, 2, 0, 64, 32, S, S, S, S, 0, None) == 0     # empty problem: nothing to overlap
+    assert f(q, k, q, q, 2, 2, 64, 32, S, S, S, S, 7, None) == -2              # argument errors come first
+    b = lib.fla_linear_attn_bwd
+    assert b(g, q, k, v, dq, dk, q, 1, 2, 64, 32, S, S, S, S, S, S, S, 0, None) == -10     # dV on q
+    assert b(g, q, k, v, dq, dq, dv, 1, 2, 64, 32, S, S, S, S, S, S, S, 0, None) == -10    # dQ and dK shared
+    assert b(g, q, k, v, g, dk, dv, 1, 2, 64, 32, S, S, S, S, S, S, S, 0, None) == -10     # in-place on dO
+    sb = lib.fla_linear_attn_smallv_bwd
+    assert sb(g, q, k, v, dq, k, dv, 1, 2, 64, 64, 16, S, S, S, S, S, S, S, 0, None) == -10
+    t = lib.fla_tri_xyt_z
+    assert t(q, k, v, v, 1, 2, 64, 32, 32, S, S, S, S, 0, 0, None) == -10
+    tc = lib.fla_tri_xyt_z_chunked
+    assert tc(q, k, v, k, 1, 2, 64, 32, 32, S, S, S, S, 0, 0, None, 0, None) == -10
+    cf = lib.fla_linear_attn_chunked_fwd
+    assert cf(q, k, v, q, 1, 2, 64, 32, 32, S, S, S, S, 0, None, None, None, 0, None) == -10
+    cb = lib.fla_linear_attn_chunked_bwd
+    assert cb(g, q, k, v, dq, dk, v, 1, 2, 64, 32, 32, S, S, S, S, S, S, S, 0, None, None, 0, None) == -10
+    eps = ctypes.c_float(1e-5)
+    nf = lib.fla_linear_attn_normalised_fwd
+    assert nf(q, k, v, k, A[8], 1, 2, 64, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -10
+    nb = lib.fla_linear_attn_normalised_bwd
+    # the forward's output is an input of backward: a gradient must not land on it
+    assert nb(g, q, k, v, o, A[8], dq, o, dv, 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, 0, A[9], 1 << 30, None) == -10
+    coef = (ctypes.c_float * 3)(0.0, 0.0, 0.5)
+    pf = lib.fla_poly_attn_fwd
+    assert pf(q, k, v, v, None, 1, 2, 64, 16, 32, S, S, S, S, coef, eps, 0, None) == -10
+    assert lib.fla_strerror(-10)
 
 
 def test_wrapper_assertions_match_reference():
