@@ -10,19 +10,23 @@ the one the headline metric is quoted on: bf16, B=4 H=32 N=4096 D_qk=D_v=128.
 
 Before the W warm-up steps the same step runs untimed for ``--settle-seconds``
 (default 0.3 s) so that the shader clock has left its idle state; the timed
-region is exactly K steps between two synchronisations.
+region is exactly K steps between two synchronisations (``ms_per_step``,
+``value``).  After it, forward, backward, the step and the step through autograd
+(``LinearAttention.apply`` + ``torch.autograd.grad``) are each timed once more
+with one HIP event pair per iteration; ``config.median_ms`` holds the medians.
 
 Prints ONE JSON line.  ``value`` is causal-counted algorithmic TFLOP/s of the
-whole step, N^2 (4 D_qk + 3 D_v) per (b, h) (five products: S, dS, dV, dK, dQ
-in backward, two in forward).  ``roofline`` describes the dominant kernel.  All
-launches evaluate products Out = mask(X Y^T) Z of N^2 (D_c + D_o) B H algorithmic
-FLOPs each; forward is one such launch, and with equal head dims up to 128 the
-three backward products are ONE launch of the batched kernel, which is then the
-dominant one: its FLOPs (three products) over the duration of the backward-only
-region timed here with HIP events on the launch stream, against the dense bf16
-MFMA peak.  ``cpu_baseline`` times the oracle's naive PyTorch formula on the
-host cores over a bounded sample (whole (b, h) slices at full N and D), in the
-same unit.
+whole step, N^2 (4 D_qk + 3 D_v) per (b, h): five products in backward (S, dS,
+dV, dK, dQ), two in forward.  ``roofline`` describes the dominant kernel.  With
+equal head dims up to 128 that is the batched backward kernel (dQ, dV and dK in
+one launch): ``achieved`` = the backward's algorithmic FLOPs, N^2 (3 D_qk + 2
+D_v) B H, over the average duration of the backward-only region timed here with
+HIP events on the launch stream; ``frac`` = that over the dense bf16 MFMA peak.
+The kernel executes six product-units for those five (dO V^T is formed for dQ
+and again for dK): ``executed_tflops`` / ``executed_frac`` price what it issues.
+``cpu_baseline`` times the oracle's naive PyTorch formula on the host cores
+over a bounded sample, in the same unit.  ``config.other_workloads`` holds
+short runs of the other benchmark workloads (default run only).
 """
 
 from __future__ import annotations
@@ -30,6 +34,7 @@ from __future__ import annotations
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -39,10 +44,18 @@ if ROOT not in sys.path:
 
 PEAK_TFLOPS = {"bf16": 2500.0, "f16": 2500.0}  # MI355X dense MFMA, published
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per kernel launch (mean over the launches of one step), measured with
-# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE`, each scaled by what the same counter
-# reads for a 256 MiB device copy (fetch x2.0, write x1.0); see profiles/*_pmc.md.
-MEASURED_TRAFFIC_BYTES = {"C3": 2.420e9}
+# HBM bytes per launch of a workload's dominant kernel, from rocprofv3 --pmc FETCH_SIZE and
+# --pmc WRITE_SIZE runs (each scaled by what the same counter reads for a device copy of known
+# size): (workload, algo) -> (bytes, the summary under profiles/ that holds the readings).
+# Workloads without an entry report `traffic: null`.
+PROFILED_TRAFFIC = {
+    ("C3", "quadratic"): (2.420e9, "profiles/tri_xyt_z_fast_kernels_C3_pmc.md"),
+}
+# MFMA operations the dominant kernel issues over those of its product-units (rocprofv3
+# SQ_INSTS_VALU_MFMA_MOPS_BF16 x 512 FLOPs; the excess is the 32 x 32 blocks on the diagonal)
+PROFILED_MFMA_RATIO = {("C3", "quadratic"): (1.008, "profiles/tri_xyt_z_fast_kernels_C3_pmc.md")}
+
+ALGOS = ["quadratic", "chunked", "normalised", "normalised-chunked", "poly"]
 
 
 def _parse():
@@ -57,7 +70,10 @@ def _parse():
     ap.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true", help="skip the host-CPU oracle timing")
     ap.add_argument("--cpu-seconds", type=float, default=12.0, help="target seconds of CPU work for the baseline")
-    ap.add_argument("--algo", default="quadratic", choices=["quadratic", "chunked", "normalised", "normalised-chunked", "poly"],
+    ap.add_argument("--no-other-workloads", action="store_true",
+                    help="skip the short runs of the other workloads that the default run appends")
+    ap.add_argument("--other-steps", type=int, default=50, help="timed iterations per entry of other_workloads")
+    ap.add_argument("--algo", default="quadratic", choices=ALGOS,
                     help="quadratic: the tiled O(N^2 D) kernels the headline metric is defined on (default); "
                          "chunked: the O(N) chunk-state path, reported with its own FLOP count and an HBM roofline; "
                          "normalised: the quadratic kernels plus the fused normaliser (out / (q . cumsum(k) + eps)), "
@@ -72,7 +88,8 @@ def _parse():
 
 
 def _time_region(torch, fn, steps):
-    """Milliseconds for `steps` calls of fn, HIP events on the current stream."""
+    """Milliseconds for `steps` back-to-back calls of fn: one HIP event pair on the current stream
+    around the whole region, a synchronisation on either side."""
     torch.cuda.synchronize()
     e0 = torch.cuda.Event(enable_timing=True)
     e1 = torch.cuda.Event(enable_timing=True)
@@ -84,14 +101,139 @@ def _time_region(torch, fn, steps):
     return e0.elapsed_time(e1)
 
 
-def _cpu_baseline(torch, w, target_seconds):
-    """The oracle's naive formula, fp32, on the host: whole (b, h) slices of the
-    workload at full N and D, forward (+ backward), until ~target_seconds."""
+def _time_each(torch, fn, steps):
+    """Milliseconds of each of `steps` back-to-back calls of fn: an event between every two calls
+    (the GPU stays busy throughout, so the clock does not drop between iterations)."""
+    torch.cuda.synchronize()
+    ev = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    ev[0].record()
+    for i in range(steps):
+        fn()
+        ev[i + 1].record()
+    torch.cuda.synchronize()
+    return [ev[i].elapsed_time(ev[i + 1]) for i in range(steps)]
+
+
+def _median_ms(torch, fn, steps):
+    return statistics.median(_time_each(torch, fn, steps))
+
+
+def _settle(torch, step, seconds):
+    n, t0 = 0, time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(8):
+            step()
+        n += 8
+        torch.cuda.synchronize()
+    return n
+
+
+def _pad(d):
+    return 32 if d <= 32 else 64 if d <= 64 else 128 if d <= 128 else 256
+
+
+def _chunk_rows(w):
+    return 256 if (w.d_qk // 2 + w.d_v <= 192 and w.d_v // 2 + w.d_qk <= 192) else 128
+
+
+def _chunked_flops(w):
+    """(forward, backward) FLOPs of the chunk-wise algorithm itself: causal-counted diagonal blocks
+    plus Y^T Z per chunk and X . S, per product; backward is three products of the same shape."""
+    bh, n, chunk = w.batch * w.heads, w.seq, _chunk_rows(w)
+    fwd = float(bh) * n * chunk * (w.d_qk + w.d_v) + 4.0 * bh * n * w.d_qk * w.d_v
+    return fwd, (3.0 * fwd if w.backward else 0.0)
+
+
+def _ops(torch, w, algo, dev):
+    """Device inputs and the forward / backward / autograd callables of one (workload, algo)."""
+    from flashy_linear_attention_amd import LinearAttention, LinearAttentionChunked, LinearAttentionSmallVHD
+    from flashy_linear_attention_amd.kernels import (
+        linear_flash_wrapper_bwd,
+        linear_flash_wrapper_bwd_smallv_hd,
+        linear_flash_wrapper_fwd,
+        linear_flash_wrapper_fwd_smallv_hd,
+    )
     from flashy_linear_attention_amd.synthetic import make_inputs
+
+    q, k, v, do = (t.to(dev) for t in make_inputs(w, seed=0))
+    fwd = linear_flash_wrapper_fwd_smallv_hd if w.small_v else linear_flash_wrapper_fwd
+    bwd = linear_flash_wrapper_bwd_smallv_hd if w.small_v else linear_flash_wrapper_bwd
+    op = LinearAttentionSmallVHD if w.small_v else LinearAttention
+    if algo in ("chunked", "normalised-chunked"):
+        from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
+
+        # as under autograd: forward hands its running state to backward
+        _, chunk_state = linear_attention_chunked_fwd(q, k, v, want_state=True)
+
+        def fwd(q_, k_, v_):
+            return linear_attention_chunked_fwd(q_, k_, v_, want_state=True)
+
+        def bwd(do_, q_, k_, v_):
+            return linear_attention_chunked_bwd(do_, q_, k_, v_, chunk_state)
+
+        op = LinearAttentionChunked
+    qa, ka, va = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+
+    def autograd_step():
+        out = op.apply(qa, ka, va)
+        if w.backward:
+            torch.autograd.grad(out, (qa, ka, va), do)
+
+    return {"q": q, "k": k, "v": v, "do": do, "fwd": lambda: fwd(q, k, v), "bwd": lambda: bwd(do, q, k, v),
+            "fwd_fn": fwd, "bwd_fn": bwd, "autograd_step": autograd_step, "op": op}
+
+
+def _other_workload(torch, name, algo, dev, steps):
+    """A short run of another workload: medians of per-iteration HIP event pairs."""
+    from flashy_linear_attention_amd.synthetic import WORKLOADS
+
+    w = WORKLOADS[name]
+    o = _ops(torch, w, algo, dev)
+
+    def step():
+        o["fwd"]()
+        if w.backward:
+            o["bwd"]()
+
+    _settle(torch, step, 0.15)
+    for _ in range(10):
+        step()
+    ms_step = _median_ms(torch, step, steps)
+    ms_fwd = _median_ms(torch, o["fwd"], steps)
+    ms_bwd = _median_ms(torch, o["bwd"], steps) if w.backward else None
+    dt_name = {torch.bfloat16: "bf16", torch.float16: "f16"}[w.dtype]
+    rec = {"workload": name, "algo": algo, "dtype": dt_name, "steps": steps,
+           "shape": f"B={w.batch} H={w.heads} N={w.seq} D_qk={w.d_qk} D_v={w.d_v}",
+           "median_step_ms": round(ms_step, 4), "median_fwd_ms": round(ms_fwd, 4),
+           "median_bwd_ms": None if ms_bwd is None else round(ms_bwd, 4)}
+    if algo == "quadratic":
+        flops = w.flops_fwd + (w.flops_bwd if w.backward else 0.0)
+        tf = flops / (ms_step * 1e-3) / 1e12
+        rec.update({"tflops": round(tf, 1), "bound": "mfma", "frac_of_peak": round(tf / PEAK_TFLOPS[dt_name], 4),
+                    "flops": "quadratic algorithm, causal-counted"})
+    else:
+        nbytes = w.bytes_fwd + (w.bytes_bwd if w.backward else 0.0)
+        gbs = nbytes / (ms_step * 1e-3) / 1e9
+        ff, fb = _chunked_flops(w)
+        rec.update({"gbps_algorithmic": round(gbs, 1), "bound": "hbm", "frac_of_peak": round(gbs / HBM_PEAK_GBS, 4),
+                    "own_tflops": round((ff + fb) / (ms_step * 1e-3) / 1e12, 1),
+                    "bytes": "each operand read once, each result written once"})
+    del o
+    torch.cuda.empty_cache()
+    return rec
+
+
+def _cpu_baseline(torch, w, target_seconds):
+    """The oracle's naive formula, fp32, on the host cores: (i) one (b, h) slice of the workload
+    at full N and D, forward (+ backward), repeated until ~target_seconds, extrapolated to all
+    slices; (ii) the small normalised workload C1 in full (forward + backward through autograd,
+    with the denominator), median of 21 runs."""
+    from flashy_linear_attention_amd.synthetic import WORKLOADS, make_inputs
     from oracle import naive
 
     q, k, v, do = (t.float() for t in make_inputs(w, seed=1, batch=1, heads=1))
-    flops_slice = (w.flops_fwd + (w.flops_bwd if w.backward else 0.0)) / (w.batch * w.heads)
+    slices = w.batch * w.heads
+    flops_slice = (w.flops_fwd + (w.flops_bwd if w.backward else 0.0)) / slices
 
     def one():
         naive.causal_dot_product_blocked(q, k, v, block=2048)
@@ -104,20 +246,44 @@ def _cpu_baseline(torch, w, target_seconds):
         one()
         n += 1
         dt = time.perf_counter() - t0
-        if dt >= target_seconds or n >= 4 * w.batch * w.heads:
+        if dt >= target_seconds or n >= 1000:
             break
+
+    c1 = WORKLOADS["C1"]
+    q1, k1, v1, g1 = make_inputs(c1, seed=0)
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q1, k1, v1))
+
+    def c1_step():
+        out = naive.linear_attention_normalised(qa, ka, va, eps=1e-5)
+        torch.autograd.grad(out, (qa, ka, va), g1)
+
+    for _ in range(3):
+        c1_step()
+    c1_ms = []
+    for _ in range(21):
+        t1 = time.perf_counter()
+        c1_step()
+        c1_ms.append((time.perf_counter() - t1) * 1e3)
+    c1_flops = c1.flops_fwd + c1.flops_bwd
     return {
         "value": round(flops_slice * n / dt / 1e12, 4),
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"{n} of {w.batch * w.heads} (b,h) slices at full N={w.seq}, D_qk={w.d_qk}, D_v={w.d_v}, "
-                  f"fp32 naive PyTorch fwd{'+bwd' if w.backward else ''}, {dt:.1f} s; os.cpu_count()={os.cpu_count()}",
-        "ms_per_step_extrapolated": round(dt / n * w.batch * w.heads * 1e3, 1),
+        "sample": f"{n} repeats of one (b,h) slice (of the workload's {slices}) at full N={w.seq}, D_qk={w.d_qk}, "
+                  f"D_v={w.d_v}, fp32 naive PyTorch fwd{'+bwd' if w.backward else ''}, {dt:.1f} s; "
+                  f"os.cpu_count()={os.cpu_count()}, torch threads={torch.get_num_threads()}",
+        "ms_per_step_extrapolated": round(dt / n * slices * 1e3, 1),
+        "c1": {
+            "what": f"C1 in full: fp32 B={c1.batch} H={c1.heads} N={c1.seq} D={c1.d_qk}, naive tril(QK^T)V / "
+                    f"((Q*cumsum(K)).sum(-1)+1e-5), forward + backward by autograd, median of {len(c1_ms)} runs",
+            "median_ms": round(statistics.median(c1_ms), 3),
+            "tflops_causal_counted": round(c1_flops / (statistics.median(c1_ms) * 1e-3) / 1e12, 4),
+        },
     }
 
 
-def _bench_poly(torch, args, w, dev, time_region) -> int:
+def _bench_poly(torch, args, w, dev) -> int:
     """C4's function, O = tril(phi(xq) phi(xk)^T) V with phi(x) = flatten(x (x) x) / sqrt 2, evaluated
     from the 16-wide x with the polynomial score map f(u) = u^2 / 2, next to the same step on the
     materialised 256-wide features (LinearAttentionSmallVHD's kernels) in the same run."""
@@ -151,19 +317,15 @@ def _bench_poly(torch, args, w, dev, time_region) -> int:
         linear_flash_wrapper_fwd_smallv_hd(q, k, v)
         linear_flash_wrapper_bwd_smallv_hd(do, q, k, v)
 
-    t0 = time.perf_counter()
-    while time.perf_counter() - t0 < args.settle_seconds:
-        for _ in range(8):
-            step()
-        torch.cuda.synchronize()
+    _settle(torch, step, args.settle_seconds)
     for _ in range(args.warmup):
         step()
-    ms_step = time_region(torch, step, args.steps) / args.steps
-    ms_fwd = time_region(torch, lambda: poly_attention_fwd(xq, xk, v, coef), args.steps) / args.steps
-    ms_bwd = time_region(torch, lambda: poly_attention_bwd(do, xq, xk, v, coef), args.steps) / args.steps
+    ms_step = _time_region(torch, step, args.steps) / args.steps
+    ms_fwd = _median_ms(torch, lambda: poly_attention_fwd(xq, xk, v, coef), args.steps)
+    ms_bwd = _median_ms(torch, lambda: poly_attention_bwd(do, xq, xk, v, coef), args.steps)
     for _ in range(20):
         plain_step()
-    ms_plain = time_region(torch, plain_step, args.steps) / args.steps
+    ms_plain = _median_ms(torch, plain_step, args.steps)
     bh, n = float(w.batch * w.heads), float(w.seq)
     # causal-counted FLOPs of what is evaluated: scores over r columns, second products as they are
     f_fwd = bh * n * n * (r + w.d_v)
@@ -200,13 +362,7 @@ def main() -> int:
     import torch
 
     from flashy_linear_attention_amd import _lib
-    from flashy_linear_attention_amd.kernels import (
-        linear_flash_wrapper_bwd,
-        linear_flash_wrapper_bwd_smallv_hd,
-        linear_flash_wrapper_fwd,
-        linear_flash_wrapper_fwd_smallv_hd,
-    )
-    from flashy_linear_attention_amd.synthetic import WORKLOADS, make_inputs
+    from flashy_linear_attention_amd.synthetic import WORKLOADS
 
     if not torch.cuda.is_available():
         print("bench.py: no ROCm GPU visible", file=sys.stderr)
@@ -215,26 +371,17 @@ def main() -> int:
 
     w = WORKLOADS[args.workload]
     dev = torch.device("cuda:0")
-    q, k, v, do = (t.to(dev) for t in make_inputs(w, seed=0))
-    fwd = linear_flash_wrapper_fwd_smallv_hd if w.small_v else linear_flash_wrapper_fwd
-    bwd = linear_flash_wrapper_bwd_smallv_hd if w.small_v else linear_flash_wrapper_bwd
     if args.algo == "poly":
-        return _bench_poly(torch, args, w, dev, _time_region)
+        return _bench_poly(torch, args, w, dev)
     normalised = args.algo.startswith("normalised")
     chunked = args.algo in ("chunked", "normalised-chunked")
-    if chunked:
-        from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
-
-        # as under autograd: forward hands its running state to backward
-        _, chunk_state = linear_attention_chunked_fwd(q, k, v, want_state=True)
-
-        def fwd(q_, k_, v_):
-            return linear_attention_chunked_fwd(q_, k_, v_, want_state=True)
-
-        def bwd(do_, q_, k_, v_):
-            return linear_attention_chunked_bwd(do_, q_, k_, v_, chunk_state)
+    o = _ops(torch, w, "chunked" if chunked else "quadratic", dev)
+    q, k, v, do = o["q"], o["k"], o["v"], o["do"]
+    fwd, bwd = o["fwd_fn"], o["bwd_fn"]
     plain_fwd, plain_bwd = fwd, bwd
+    autograd_step = o["autograd_step"]
     if normalised:
+        from flashy_linear_attention_amd import LinearAttentionNormalised
         from flashy_linear_attention_amd.normalised import (
             linear_attention_normalised_bwd,
             linear_attention_normalised_fwd,
@@ -248,6 +395,13 @@ def main() -> int:
         def bwd(do_, q_, k_, v_):
             return linear_attention_normalised_bwd(do_, q_, k_, v_, norm_out, norm_denom, chunked)
 
+        qa, ka, va = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+
+        def autograd_step():
+            out = LinearAttentionNormalised.apply(qa, ka, va, 1e-5, chunked)
+            if w.backward:
+                torch.autograd.grad(out, (qa, ka, va), do)
+
     def step():
         fwd(q, k, v)
         if w.backward:
@@ -260,56 +414,62 @@ def main() -> int:
         torch.cuda.synchronize()
         del src, dst
 
-    settle_steps = 0
-    t_settle = time.perf_counter()
-    while time.perf_counter() - t_settle < args.settle_seconds:
-        for _ in range(8):
-            step()
-        settle_steps += 8
-        torch.cuda.synchronize()
+    settle_steps = _settle(torch, step, args.settle_seconds)
     for _ in range(args.warmup):
         step()
+    # the timed region: exactly K steps between two synchronisations
     ms_total = _time_region(torch, step, args.steps)
     ms_step = ms_total / args.steps
 
-    # secondary figures: each half alone (same event method)
+    # each half alone over a region of K launches (the dominant kernel's average launch duration
+    # comes from here), then per-iteration event pairs for the medians
     ms_fwd = _time_region(torch, lambda: fwd(q, k, v), args.steps) / args.steps
     ms_bwd = _time_region(torch, lambda: bwd(do, q, k, v), args.steps) / args.steps if w.backward else None
+    med_step = _median_ms(torch, step, args.steps)
+    med_fwd = _median_ms(torch, lambda: fwd(q, k, v), args.steps)
+    med_bwd = _median_ms(torch, lambda: bwd(do, q, k, v), args.steps) if w.backward else None
+    for _ in range(5):
+        autograd_step()
+    med_autograd = _median_ms(torch, autograd_step, args.steps)
 
     flops_step = w.flops_fwd + (w.flops_bwd if w.backward else 0.0)
     dt_name = {torch.bfloat16: "bf16", torch.float16: "f16"}[w.dtype]
     peak = PEAK_TFLOPS[dt_name]
     tflops = flops_step / (ms_step * 1e-3) / 1e12
 
-    # The dominant kernel and its launches.  Every launch evaluates products Out = mask(X Y^T) Z of
-    # N^2 (D_c + D_o) B H algorithmic FLOPs each.  With equal padded widths up to 128 the three
-    # backward products go out as ONE launch of fla::tri_xyt_z_fast_batch_kernel (the dominant
-    # kernel: three quarters of the step); its duration is the backward-only region timed above.
-    # Otherwise every product is a launch of its own (two when an output wider than 128 columns
-    # meets a <=64- or 256-wide contraction: one per 128-column half) and the figures are means
-    # over the launches of a step.
+    # The dominant kernel.  Every launch evaluates products Out = mask(X Y^T) Z; one product
+    # executes N^2 (D_c + D_o) B H FLOPs (causal-counted).  With equal padded widths up to 128 the
+    # three backward products go out as ONE launch of fla::tri_xyt_z_fast_batch_kernel, three
+    # quarters of the step: its duration is the backward-only region timed above, its algorithmic
+    # FLOPs are the backward's five products (it executes six: dO V^T twice).  Otherwise every
+    # product is a launch of its own (two when an output wider than 128 columns meets a <= 64- or
+    # 256-wide contraction: one per 128-column half) and the figures are means over the launches
+    # of a step.
     def n_launches(dc, dout):
         return 2 if dout > 128 and (dc <= 64 or dc > 128) else 1
 
-    def pad(d):
-        return 32 if d <= 32 else 64 if d <= 64 else 128 if d <= 128 else 256
-
     flops_product = float(w.batch * w.heads) * w.seq * w.seq * (w.d_qk + w.d_v)
-    batched_bwd = w.backward and pad(w.d_qk) == pad(w.d_v) and pad(w.d_qk) <= 128
+    batched_bwd = w.backward and _pad(w.d_qk) == _pad(w.d_v) and _pad(w.d_qk) <= 128
     if batched_bwd:
         launches = 2
         kernel_name = "fla::tri_xyt_z_fast_batch_kernel (dQ, dV, dK: three products Out = mask(X Y^T) Z in one launch)"
-        flops_launch = 3.0 * flops_product
+        flops_launch = w.flops_bwd
+        executed_launch = 3.0 * flops_product
         ms_launch = ms_bwd
     else:
         launches = n_launches(w.d_qk, w.d_v)
         if w.backward:
             launches += n_launches(w.d_v, w.d_qk) * 2 + n_launches(w.d_qk, w.d_v)
         products = 1 + (3 if w.backward else 0)
-        kernel_name = "fla::tri_xyt_z_fast_kernel (Out = mask(X Y^T) Z)"
-        flops_launch = flops_product * products / launches
+        kernel_name = "fla::tri_xyt_z_fast_kernel (Out = mask(X Y^T) Z), mean over the launches of a step"
+        flops_launch = flops_step / launches
+        executed_launch = flops_product * products / launches
         ms_launch = ms_step / launches
     achieved = flops_launch / (ms_launch * 1e-3) / 1e12
+    executed = executed_launch / (ms_launch * 1e-3) / 1e12
+    traffic, traffic_src = PROFILED_TRAFFIC.get((w.name, "quadratic"), (None, None))
+    mfma_ratio, mfma_src = PROFILED_MFMA_RATIO.get((w.name, "quadratic"), (None, None))
+    alg_bytes_launch = (w.bytes_bwd if batched_bwd else (w.bytes_fwd + (w.bytes_bwd if w.backward else 0.0)) / launches)
 
     result = {
         "metric": f"causal linear attention {'fwd+bwd' if w.backward else 'fwd'} TFLOP/s "
@@ -336,6 +496,14 @@ def main() -> int:
             "fwd_tflops": round(w.flops_fwd / (ms_fwd * 1e-3) / 1e12, 2),
             "bwd_tflops": None if ms_bwd is None else round(w.flops_bwd / (ms_bwd * 1e-3) / 1e12, 2),
             "pct_of_mfma_peak": round(100.0 * tflops / peak, 2),
+            "median_ms": {
+                "note": f"medians of {args.steps} iterations, one HIP event pair each; autograd_step = "
+                        f"{o['op'].__name__ if not normalised else 'LinearAttentionNormalised'}.apply + torch.autograd.grad",
+                "step": round(med_step, 4),
+                "fwd": round(med_fwd, 4),
+                "bwd": None if med_bwd is None else round(med_bwd, 4),
+                "autograd_step": round(med_autograd, 4),
+            },
         },
         "roofline": {
             "bound": "mfma",
@@ -344,26 +512,30 @@ def main() -> int:
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": round(achieved / peak, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES.get(w.name),
-            "traffic_note": "HBM bytes per launch of the dominant kernel, rocprofv3 FETCH_SIZE/WRITE_SIZE (profiles/)",
+            "traffic": traffic,
+            "traffic_source": traffic_src,
+            "algorithmic_bytes_per_launch": alg_bytes_launch,
+            "traffic_over_algorithmic_bytes": None if traffic is None else round(traffic / alg_bytes_launch, 2),
             "launches_per_step": launches,
             "flops_per_launch": flops_launch,
             "avg_launch_ms": round(ms_launch, 4),
+            "executed_tflops": round(executed, 2),
+            "executed_frac": round(executed / peak, 4),
+            "executed_note": "FLOPs of the product-units the kernel executes (backward: six for the five counted, "
+                             "dO V^T is formed for dQ and again for dK)"
+                             + ("" if mfma_ratio is None else
+                                f"; MFMA operations issued / those FLOPs = {mfma_ratio} ({mfma_src})"),
         },
     }
     if chunked:
         # The chunked path does different (far less) arithmetic, so it is never priced in the
         # quadratic algorithm's FLOPs: its own count, and the HBM roofline that bounds it.
-        chunk = 256 if (w.d_qk // 2 + w.d_v <= 192 and w.d_v // 2 + w.d_qk <= 192) else 128
-        bh, n = w.batch * w.heads, w.seq
-        f_intra = float(bh) * n * chunk * (w.d_qk + w.d_v)          # causal-counted diagonal blocks
-        f_state = 4.0 * bh * n * w.d_qk * w.d_v                     # Y^T Z per chunk + X . S
-        flops_fwd = f_intra + f_state
-        flops_bwd = 3.0 * flops_fwd if w.backward else 0.0          # three products of the same shape
+        flops_fwd, flops_bwd = _chunked_flops(w)
         bytes_step = w.bytes_fwd + (w.bytes_bwd if w.backward else 0.0)
+        traffic, traffic_src = PROFILED_TRAFFIC.get((w.name, "chunked"), (None, None))
         result["metric"] = result["metric"].replace("TFLOP/s (causal-counted)", "TFLOP/s (chunked algorithm's own FLOPs)")
         result["value"] = round((flops_fwd + flops_bwd) / (ms_step * 1e-3) / 1e12, 2)
-        result["config"]["workload"] += f"; chunk-wise evaluation, {chunk}-row chunks"
+        result["config"]["workload"] += f"; chunk-wise evaluation, {_chunk_rows(w)}-row chunks"
         result["config"]["flops_per_step"] = flops_fwd + flops_bwd
         result["config"]["fwd_tflops"] = round(flops_fwd / (ms_fwd * 1e-3) / 1e12, 2)
         result["config"]["bwd_tflops"] = None if ms_bwd is None else round(flops_bwd / (ms_bwd * 1e-3) / 1e12, 2)
@@ -371,19 +543,23 @@ def main() -> int:
         gbs = bytes_step / (ms_step * 1e-3) / 1e9
         result["roofline"] = {
             "bound": "hbm",
-            "kernel": "chunk_state + chunk_scan (two running states per step when shared, else one per product) + tri_xyt_z_fast (chunked) per product",
+            "kernel": "all kernels of a chunk-wise step (chunk states and their running sums, diagonal blocks + state product)",
             "achieved": round(gbs, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(gbs / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": traffic,
+            "traffic_source": traffic_src,
             "algorithmic_bytes_per_step": bytes_step,
+            "traffic_over_algorithmic_bytes": None if traffic is None else round(traffic / bytes_step, 2),
         }
     if normalised:
         # What is new are the memory-bound passes around the product kernels.  Their time is the
         # difference to the plain step in this same run, their algorithmic bytes: forward (separate pass)
         # reads q, k, O and writes out (+ n); backward reads g, out (pre-pass, writes dO) and
         # q, k, dq, dk (post-pass, writes dq, dk); 2 bytes per element, fp32 vectors of length N aside.
+        from flashy_linear_attention_amd import LinearAttention, LinearAttentionSmallVHD
+
         def plain_step():
             plain_fwd(q, k, v)
             if w.backward:
@@ -399,28 +575,29 @@ def main() -> int:
         extra_ms = ms_step - ms_plain
 
         def recipe_step():
-            qa, ka, va = (t.detach().requires_grad_(w.backward) for t in (q, k, v))
+            qr, kr, vr = (t.detach().requires_grad_(w.backward) for t in (q, k, v))
             op = LinearAttentionSmallVHD if w.small_v else LinearAttention
-            num = op.apply(qa, ka, va)
-            den = (qa * ka.cumsum(-2)).sum(dim=-1, keepdim=True) + 1e-5
+            num = op.apply(qr, kr, vr)
+            den = (qr * kr.cumsum(-2)).sum(dim=-1, keepdim=True) + 1e-5
             out = num / den
             if w.backward:
                 out.backward(do)
-
-        from flashy_linear_attention_amd import LinearAttention, LinearAttentionSmallVHD
 
         for _ in range(10):
             recipe_step()
         ms_recipe = _time_region(torch, recipe_step, max(10, args.steps // 5)) / max(10, args.steps // 5)
         # the dominant kernel is still the product kernel: its per-launch figures come from the plain step
         if not chunked:
-            plain_flops = flops_product * (4 if w.backward else 1)
             result["roofline"]["kernel"] = ("fla::tri_xyt_z_fast_kernel / _batch_kernel "
                                             "(all product launches of the plain step)")
             result["roofline"]["avg_launch_ms"] = round(ms_plain / launches, 4)
-            result["roofline"]["flops_per_launch"] = plain_flops / launches
-            result["roofline"]["achieved"] = round(plain_flops / (ms_plain * 1e-3) / 1e12, 2)
+            result["roofline"]["flops_per_launch"] = flops_step / launches
+            result["roofline"]["achieved"] = round(flops_step / (ms_plain * 1e-3) / 1e12, 2)
             result["roofline"]["frac"] = round(result["roofline"]["achieved"] / peak, 4)
+            for key in ("executed_tflops", "executed_frac", "executed_note", "traffic", "traffic_source",
+                        "algorithmic_bytes_per_launch", "traffic_over_algorithmic_bytes"):
+                result["roofline"].pop(key, None)
+            result["roofline"]["traffic"] = None
         result["metric"] = result["metric"].replace("causal linear attention", "normalised causal linear attention")
         result["config"]["workload"] += "; fused normaliser out / (q . cumsum(k) + 1e-5)"
         result["config"]["normaliser"] = {
@@ -432,6 +609,15 @@ def main() -> int:
             "pytorch_recipe_step_ms": round(ms_recipe, 4),
             "speedup_vs_pytorch_recipe": round(ms_recipe / ms_step, 2),
         }
+    if args.workload == "C3" and args.algo == "quadratic" and not args.no_other_workloads:
+        # the other benchmark workloads, briefly, so that one run of this script times them all
+        del o, q, k, v, do
+        torch.cuda.empty_cache()
+        result["config"]["other_workloads"] = [
+            _other_workload(torch, name, algo, dev, args.other_steps)
+            for name, algo in (("C2", "quadratic"), ("C4", "quadratic"), ("C5", "quadratic"),
+                               ("C3", "chunked"), ("C4", "chunked"), ("C5", "chunked"))
+        ]
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = _cpu_baseline(torch, w, args.cpu_seconds)
     print(json.dumps(result))
