@@ -5,10 +5,36 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "fla_dispatch.h"
 #include "fla_norm.h"
 
+// Scratch of fla_linear_attn_chunked_fwd_static: one copy per GPU, at its own address on each.
+// Host code never uses the array's name as an address; it asks the runtime for the device
+// address once per device (static_scratch below) and passes that pointer on.  (No `used`
+// attribute: it would pin the device symbol to local binding, where the runtime's lookup by
+// name cannot find it; the reference from host code below is what keeps the array and makes
+// the compiler give it global binding.)
+static __device__ __align__(256) unsigned char scratch[FLA_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device (looked up on the first call per device).
+int static_scratch(void **out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return FLA_ERR_LAUNCH;
+    void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)) != hipSuccess || !ptr) return FLA_ERR_LAUNCH;
+        g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return FLA_OK;
+}
 
 using fla::TriParams;
 typedef hipError_t (*launch_fn)(const TriParams &, hipStream_t);
@@ -808,6 +834,21 @@ int fla_linear_attn_chunked_fwd(const void *q, const void *k, const void *v, voi
     if (D_v < 1 || D_v > 256) return FLA_ERR_V_HEAD_DIM;
     return chunked_forward({q, q_strides}, {k, k_strides}, {v, v_strides}, {o, o_strides}, B, H, N, D_qk, D_v, dtype,
                            state_out, state_valid, workspace, workspace_bytes, stream);
+}
+
+int fla_linear_attn_chunked_fwd_static(const void *q, const void *k, const void *v, void *o, int64_t B, int64_t H,
+                                       int64_t N, int64_t D_qk, int64_t D_v, const int64_t *q_strides,
+                                       const int64_t *k_strides, const int64_t *v_strides, const int64_t *o_strides,
+                                       int dtype, void *stream) {
+    if (int rc = check_common(B, H, N, dtype)) return rc;
+    if (D_qk < 1 || D_qk > 256) return FLA_ERR_HEAD_DIM;
+    if (D_v < 1 || D_v > 256) return FLA_ERR_V_HEAD_DIM;
+    const int64_t need = chunked_op_workspace_bytes(B, H, N, D_qk, D_v);
+    if (need > (int64_t)FLA_STATIC_SCRATCH_BYTES) return FLA_ERR_WORKSPACE;
+    void *ws = nullptr;
+    if (int rc = static_scratch(&ws)) return rc;
+    return chunked_forward({q, q_strides}, {k, k_strides}, {v, v_strides}, {o, o_strides}, B, H, N, D_qk, D_v, dtype,
+                           nullptr, nullptr, ws, FLA_STATIC_SCRATCH_BYTES, stream);
 }
 
 int fla_linear_attn_chunked_bwd(const void *grad_out, const void *q, const void *k, const void *v, void *dq, void *dk,

@@ -174,6 +174,23 @@ int fla_linear_attn_chunked_bwd(const void *grad_out, const void *q, const void 
                                 int dtype, const void *state_in,
                                 void *workspace, int64_t workspace_bytes, void *stream);
 
+/* fla_linear_attn_chunked_fwd for callers that cannot allocate device memory or pass a workspace
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
+ * counterpart in the reference.  Same arguments and results as fla_linear_attn_chunked_fwd with
+ * state_out = NULL; the scratch its kernels need (per-chunk states and their running sums) lives
+ * in a static device array of FLA_STATIC_SCRATCH_BYTES that every GPU the library runs on holds
+ * until the process ends.  The call allocates and frees nothing.  Problems whose
+ * fla_linear_attn_chunked_workspace_bytes() exceeds FLA_STATIC_SCRATCH_BYTES are rejected with
+ * FLA_ERR_WORKSPACE before anything is enqueued.  All calls on one GPU share that array (it keeps
+ * the previous call's contents; the kernels overwrite what they read): calls that overlap in
+ * time on one GPU -- different streams, different host threads -- race; calls on one stream do not. */
+#define FLA_STATIC_SCRATCH_BYTES (64 * 1024 * 1024)
+int fla_linear_attn_chunked_fwd_static(const void *q, const void *k, const void *v, void *o,
+                                       int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                                       const int64_t *q_strides, const int64_t *k_strides,
+                                       const int64_t *v_strides, const int64_t *o_strides,
+                                       int dtype, void *stream);
+
 /* Causal linear attention with a polynomial score map,
  *
  *     out = lower(f(Xq Xk^T)) V,    f(u) = coef[0] + coef[1] u + coef[2] u^2,
