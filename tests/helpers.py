@@ -60,3 +60,26 @@ def load_golden(name: str):
 
 
 GOLDEN_CASES = ("equal_d_b1_h1_n128_d32", "small_v_b1_h1_n128_dqk64_dv16")
+
+
+def _naive():
+    from oracle import naive
+
+    return naive
+
+
+def gpu_fp32_reference(q, k, v, do, backward, heads_per_chunk=8):
+    """The oracle's blocked formula evaluated in fp32 on the GPU, a few heads at
+    a time (the full score tensor of C3 would be 8.6 GB)."""
+    b, h = q.shape[:2]
+    o = torch.empty(*q.shape[:3], v.shape[-1], dtype=torch.float32, device=q.device)
+    grads = [torch.empty(t.shape, dtype=torch.float32, device=q.device) for t in (q, k, v)] if backward else None
+    for bi in range(b):
+        for h0 in range(0, h, heads_per_chunk):
+            sl = (slice(bi, bi + 1), slice(h0, h0 + heads_per_chunk))
+            qs, ks, vs = q[sl].float(), k[sl].float(), v[sl].float()
+            o[sl] = _naive().causal_dot_product_blocked(qs, ks, vs, block=2048)
+            if backward:
+                for gbuf, gval in zip(grads, _naive().causal_dot_product_grads_blocked(qs, ks, vs, do[sl].float(), block=2048)):
+                    gbuf[sl] = gval
+    return o, grads

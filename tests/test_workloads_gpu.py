@@ -17,7 +17,7 @@ from flashy_linear_attention_amd.kernels import (
 from flashy_linear_attention_amd.synthetic import WORKLOADS, make_inputs
 from oracle import c_oracle, naive
 
-from helpers import GOLDEN_CASES, assert_close, load_golden, reference_style_inputs
+from helpers import GOLDEN_CASES, assert_close, gpu_fp32_reference, load_golden, reference_style_inputs
 
 pytestmark = pytest.mark.gpu
 
@@ -147,23 +147,6 @@ def test_small_v_equals_equal_d_on_padded_v(gpu_device):
 
 
 # ------------------------------------------------------- benchmark workloads
-def _gpu_fp32_reference(q, k, v, do, backward, heads_per_chunk=8):
-    """The oracle's blocked formula evaluated in fp32 on the GPU, a few heads at
-    a time (the full score tensor of C3 would be 8.6 GB)."""
-    b, h = q.shape[:2]
-    o = torch.empty(*q.shape[:3], v.shape[-1], dtype=torch.float32, device=q.device)
-    grads = [torch.empty(t.shape, dtype=torch.float32, device=q.device) for t in (q, k, v)] if backward else None
-    for bi in range(b):
-        for h0 in range(0, h, heads_per_chunk):
-            sl = (slice(bi, bi + 1), slice(h0, h0 + heads_per_chunk))
-            qs, ks, vs = q[sl].float(), k[sl].float(), v[sl].float()
-            o[sl] = naive.causal_dot_product_blocked(qs, ks, vs, block=2048)
-            if backward:
-                for gbuf, gval in zip(grads, naive.causal_dot_product_grads_blocked(qs, ks, vs, do[sl].float(), block=2048)):
-                    gbuf[sl] = gval
-    return o, grads
-
-
 @pytest.mark.parametrize("name", ["C2", "C3", "C4", "C5"])
 def test_benchmark_workload(name, gpu_device):
     """Each benchmark workload at full size: every head against the oracle's
@@ -180,7 +163,7 @@ def test_benchmark_workload(name, gpu_device):
     got = [out.detach()] + ([qg.grad, kg.grad, vg.grad] if w.backward else [])
     names = ["O", "dQ", "dK", "dV"][: len(got)]
 
-    o_ref, g_ref = _gpu_fp32_reference(q, k, v, do, w.backward, heads_per_chunk=8 if w.seq <= 4096 else 1)
+    o_ref, g_ref = gpu_fp32_reference(q, k, v, do, w.backward, heads_per_chunk=8 if w.seq <= 4096 else 1)
     for n, x, y in zip(names, got, [o_ref] + (g_ref or [])):
         assert_close(f"{name} {n} (all heads, fp32 GPU)", x, y)
 
