@@ -118,6 +118,30 @@ def _median_ms(torch, fn, steps):
     return statistics.median(_time_each(torch, fn, steps))
 
 
+def _host_side(torch, fn, calls=200):
+    """What a caller sees per call of fn (a launch wrapper): host time to enqueue one call
+    (perf_counter over `calls` back-to-back calls, no synchronisation inside the loop; when the
+    GPU is the slower side this is the GPU's time per call instead) and the wall time of an
+    isolated call, synchronised before and after (launch latency + kernel + completion)."""
+    for _ in range(20):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(calls):
+        fn()
+    t1 = time.perf_counter()
+    torch.cuda.synchronize()
+    iso = []
+    for _ in range(50):
+        torch.cuda.synchronize()
+        a = time.perf_counter()
+        fn()
+        torch.cuda.synchronize()
+        iso.append((time.perf_counter() - a) * 1e6)
+    return {"enqueue_loop_us_per_call": round((t1 - t0) / calls * 1e6, 2),
+            "isolated_call_us_median": round(statistics.median(iso), 2)}
+
+
 def _settle(torch, step, seconds):
     n, t0 = 0, time.perf_counter()
     while time.perf_counter() - t0 < seconds:
@@ -202,10 +226,14 @@ def _other_workload(torch, name, algo, dev, steps):
     ms_fwd = _median_ms(torch, o["fwd"], steps)
     ms_bwd = _median_ms(torch, o["bwd"], steps) if w.backward else None
     dt_name = {torch.bfloat16: "bf16", torch.float16: "f16"}[w.dtype]
+    host = _host_side(torch, o["fwd"]) if w.seq * w.batch * w.heads <= 1 << 18 else None
     rec = {"workload": name, "algo": algo, "dtype": dt_name, "steps": steps,
            "shape": f"B={w.batch} H={w.heads} N={w.seq} D_qk={w.d_qk} D_v={w.d_v}",
            "median_step_ms": round(ms_step, 4), "median_fwd_ms": round(ms_fwd, 4),
            "median_bwd_ms": None if ms_bwd is None else round(ms_bwd, 4)}
+    if host is not None:  # launch-bound sizes: the region mean (no events between launches) and the host's view
+        rec["back_to_back_fwd_ms"] = round(_time_region(torch, o["fwd"], 4 * steps) / (4 * steps), 4)
+        rec["host_forward_wrapper"] = host
     if algo == "quadratic":
         flops = w.flops_fwd + (w.flops_bwd if w.backward else 0.0)
         tf = flops / (ms_step * 1e-3) / 1e12
@@ -496,6 +524,7 @@ def main() -> int:
             "fwd_tflops": round(w.flops_fwd / (ms_fwd * 1e-3) / 1e12, 2),
             "bwd_tflops": None if ms_bwd is None else round(w.flops_bwd / (ms_bwd * 1e-3) / 1e12, 2),
             "pct_of_mfma_peak": round(100.0 * tflops / peak, 2),
+            "host_forward_wrapper": _host_side(torch, lambda: fwd(q, k, v)),
             "median_ms": {
                 "note": f"medians of {args.steps} iterations, one HIP event pair each; autograd_step = "
                         f"{o['op'].__name__ if not normalised else 'LinearAttentionNormalised'}.apply + torch.autograd.grad",
