@@ -178,6 +178,14 @@ batch_fn lookup_batch(int dtype, int64_t d) {
     return table[pad_index(d)][dtype];
 }
 
+batch_fn lookup_chunked_batch(int dtype, int64_t d) {
+    static const batch_fn table[4][2] = {{fla::FLA_CBATCH_NAME(0, 32), fla::FLA_CBATCH_NAME(1, 32)},
+                                         {fla::FLA_CBATCH_NAME(0, 64), fla::FLA_CBATCH_NAME(1, 64)},
+                                         {fla::FLA_CBATCH_NAME(0, 128), fla::FLA_CBATCH_NAME(1, 128)},
+                                         {fla::FLA_CBATCH_NAME(0, 256), fla::FLA_CBATCH_NAME(1, 256)}};
+    return table[pad_index(d)][dtype];
+}
+
 // Out = mask(X Y^T) Z; all arguments already validated.
 int run_tri(const View &x, const View &y, const View &z, const View &out, int64_t B, int64_t H, int64_t N,
             int64_t dc, int64_t dout, int upper, int dtype, void *stream) {
@@ -352,11 +360,16 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         if (int rc = chunk_states(k, v, B, H, N, dqk, dv, 0, dtype, w, mine, stream)) return rc;
         state_f = mine;
     }
-    // dQ reads the forward state [D_v][D_qk] as its own [D_c = D_v][D_o = D_qk] transposed state
-    if (int rc = chunk_main(pq, dv, dqk, dtype, state_f, 1, stream)) return rc;
     if (int rc = chunk_states(q, go, B, H, N, dqk, dv, 1, dtype, w, state_v, stream)) return rc;
-    if (int rc = chunk_main(pv, dqk, dv, dtype, state_v, 0, stream)) return rc;
-    return chunk_main(pk, dv, dqk, dtype, state_v, 1, stream);
+    // One launch for the three products: a workgroup evaluates dQ, dV and dK of its chunk in turn,
+    // so q, k, v and dO come from memory once.  dQ reads the forward state [D_v][D_qk] as its own
+    // [D_c = D_v][D_o = D_qk] transposed state; dK reads the state of dV transposed.
+    fla::TriBatch b;
+    b.p[0] = pq, b.p[0].state = state_f, b.p[0].state_transposed = 1;
+    b.p[1] = pv, b.p[1].state = state_v, b.p[1].state_transposed = 0;
+    b.p[2] = pk, b.p[2].state = state_v, b.p[2].state_transposed = 1;
+    return lookup_chunked_batch(dtype, dqk)(b, 3, static_cast<hipStream_t>(stream)) == hipSuccess ? FLA_OK
+                                                                                                   : FLA_ERR_LAUNCH;
 }
 
 int forward(const View &q, const View &k, const View &v, const View &o, int64_t B, int64_t H, int64_t N,

@@ -19,6 +19,8 @@
 #define FLA_STATE_NAME(t, dc, dout) FLA_STATE_NAME_(t, dc, dout)
 #define FLA_BATCH_NAME_(t, d) fla_launch_batch_t##t##_d##d
 #define FLA_BATCH_NAME(t, d) FLA_BATCH_NAME_(t, d)
+#define FLA_CBATCH_NAME_(t, d) fla_launch_chunked_batch_t##t##_d##d
+#define FLA_CBATCH_NAME(t, d) FLA_CBATCH_NAME_(t, d)
 
 namespace fla {
 #define FLA_DECLARE(dc, dout)                                                               \
@@ -32,7 +34,9 @@ FLA_FOR_EACH_DIM_PAIR(FLA_DECLARE)
 // several products of one square shape in a single launch (fast path only; hipErrorNotSupported otherwise)
 #define FLA_DECLARE_BATCH(d)                                                                  \
     hipError_t FLA_BATCH_NAME(0, d)(const TriBatch &b, int count, hipStream_t stream);        \
-    hipError_t FLA_BATCH_NAME(1, d)(const TriBatch &b, int count, hipStream_t stream);
+    hipError_t FLA_BATCH_NAME(1, d)(const TriBatch &b, int count, hipStream_t stream);        \
+    hipError_t FLA_CBATCH_NAME(0, d)(const TriBatch &b, int count, hipStream_t stream);       \
+    hipError_t FLA_CBATCH_NAME(1, d)(const TriBatch &b, int count, hipStream_t stream);
 FLA_DECLARE_BATCH(32) FLA_DECLARE_BATCH(64) FLA_DECLARE_BATCH(128) FLA_DECLARE_BATCH(256)
 #undef FLA_DECLARE_BATCH
 }  // namespace fla

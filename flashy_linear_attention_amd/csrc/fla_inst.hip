@@ -33,6 +33,10 @@ hipError_t FLA_BATCH_NAME(FLA_INST_DTYPE, FLA_INST_DC)(const TriBatch &b, int co
     if (!FastConfig<FLA_INST_DC, FLA_INST_DO>::kSupported) return hipErrorNotSupported;
     return launch_tri_fast_batch<InstT, FLA_INST_DC, FLA_INST_DO>(b, count, stream);
 }
+
+hipError_t FLA_CBATCH_NAME(FLA_INST_DTYPE, FLA_INST_DC)(const TriBatch &b, int count, hipStream_t stream) {
+    return launch_tri_fast_chunked_batch<InstT, FLA_INST_DC, FLA_INST_DO>(b, count, stream);
+}
 #endif
 
 #if FLA_INST_DTYPE == 0

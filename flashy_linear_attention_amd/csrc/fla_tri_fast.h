@@ -945,6 +945,17 @@ __global__ __launch_bounds__(256, (FastConfig<DC, DO, false>::kMinWavesPerSimd))
     tri_fast_body<T, DC, DO, false>(b.p[blockIdx.y], blockIdx.x);
 }
 
+// Chunk-wise evaluation of up to three products of one square shape by the same workgroup, one
+// after the other, for the same (head, chunk): the backward's dQ, dV and dK read the same rows
+// of q, k, v and dO in different roles, so after the first product the others find them in the
+// caches instead of fetching them from memory again.
+template <typename T, int DC, int DO>
+__global__ __launch_bounds__(256, (FastConfig<DC, DO, true>::kMinWavesPerSimd)) void tri_xyt_z_fast_chunked_batch_kernel(
+    const TriBatch b, const int count) {
+#pragma unroll 1
+    for (int i = 0; i < count; ++i) tri_fast_body<T, DC, DO, true>(b.p[i], blockIdx.x);
+}
+
 // True when the fast kernel can take this problem: every operand 16-byte
 // aligned with widths in whole chunks, and each (b, h) slice addressable with
 // 32-bit byte offsets.
@@ -1030,6 +1041,28 @@ hipError_t launch_tri_fast_batch(TriBatch b, int count, hipStream_t stream) {
         constexpr auto kern = tri_xyt_z_fast_batch_kernel<T, DC, DO>;
         if (hipError_t e = ensure_dynamic_lds<kern>(Cfg::SMEM_BYTES)) return e;
         return launch_kernel(kern, dim3((unsigned)grid, (unsigned)count), dim3(256), Cfg::SMEM_BYTES, stream, b);
+    }
+}
+
+// `count` chunk-wise products of one square shape, every TriParams with its state set, evaluated
+// by the same workgroups in sequence (see tri_xyt_z_fast_chunked_batch_kernel).
+template <typename T, int DC, int DO>
+hipError_t launch_tri_fast_chunked_batch(TriBatch b, int count, hipStream_t stream) {
+    using Cfg = FastConfig<DC, DO, true>;
+    if constexpr (!Cfg::kSupported || DC != DO) {
+        return hipErrorNotSupported;
+    } else {
+        const int n_tiles = (b.p[0].N + Cfg::BM - 1) / Cfg::BM;
+        for (int i = 0; i < count; ++i) {
+            if (!b.p[i].state || (b.p[i].state_transposed && !Cfg::kStateTransposable)) return hipErrorNotSupported;
+            b.p[i].n_tiles = n_tiles, b.p[i].single = 0;
+        }
+        const int64_t grid = (int64_t)8 * ((b.p[0].BH + 7) / 8) * n_tiles;
+        if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+        constexpr auto kern = tri_xyt_z_fast_chunked_batch_kernel<T, DC, DO>;
+        constexpr int smem = Cfg::SMEM_BYTES + (Cfg::kStateInLds ? Cfg::STATE_BYTES : 0);
+        if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
+        return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, b, count);
     }
 }
 
