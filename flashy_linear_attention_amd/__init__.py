@@ -2,10 +2,11 @@
 the Python surface of ``flashlinear`` (flashlinear/__init__.py:1-2)."""
 
 from .chunked import LinearAttentionChunked
+from .feature import FeatureMapLinearAttention
 from .linear_attn import LinearAttention
 from .linear_attn_smallv_hd import LinearAttentionSmallVHD
 from .normalised import LinearAttentionNormalised
 from .poly import PolynomialLinearAttention
 
 __all__ = ["LinearAttention", "LinearAttentionSmallVHD", "LinearAttentionChunked", "LinearAttentionNormalised",
-           "PolynomialLinearAttention"]
+           "PolynomialLinearAttention", "FeatureMapLinearAttention"]

@@ -164,6 +164,9 @@ TriParams make_params(const View &x, const View &y, const View &z, const View &o
     p.eps = 0.f;
     p.poly[0] = p.poly[1] = p.poly[2] = 0.f;
     p.poly_on = 0;
+    p.map_x = p.map_y = p.map_z = p.map_out = 0;
+    p.omap = nullptr;
+    p.ms_b = p.ms_h = p.ms_n = 0;
     p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout), p.vec_out = vec_ok(out, dout);
     return p;
 }
@@ -230,7 +233,7 @@ bool chunkable(const TriParams &p, int64_t dc, int64_t dout, int64_t N) {
 }
 
 int chunk_states(const View &y, const View &z, int64_t B, int64_t H, int64_t N, int64_t dc, int64_t dout, int upper,
-                 int dtype, float *w, void *state, void *stream) {
+                 int dtype, float *w, void *state, void *stream, int map_y = 0, int map_z = 0) {
     const int64_t rows = chunk_rows(dc, dout), chunks = (N + rows - 1) / rows, E = padded(dc) * padded(dout);
     hipStream_t s = static_cast<hipStream_t>(stream);
     fla::ChunkStateParams cp;
@@ -239,6 +242,7 @@ int chunk_states(const View &y, const View &z, int64_t B, int64_t H, int64_t N, 
     cp.zs_b = z.strides[0], cp.zs_h = z.strides[1], cp.zs_n = z.strides[2];
     cp.H = (int32_t)H, cp.N = (int32_t)N, cp.BH = (int32_t)(B * H), cp.dc = (int32_t)dc, cp.dout = (int32_t)dout;
     cp.n_chunks = (int32_t)chunks;
+    cp.map_y = map_y, cp.map_z = map_z;
     if (lookup_state(dtype, dc, dout)(cp, s) != hipSuccess) return FLA_ERR_LAUNCH;
     const hipError_t e = dtype == FLA_DTYPE_BF16
                              ? fla::launch_chunk_scan<__bf16>(w, state, B * H, (int)chunks, E, upper ? 1 : 0, s)
@@ -249,7 +253,24 @@ int chunk_states(const View &y, const View &z, int64_t B, int64_t H, int64_t N, 
 int chunk_main(TriParams p, int64_t dc, int64_t dout, int dtype, const void *state, int transposed, void *stream) {
     p.state = state;
     p.state_transposed = transposed;
-    return lookup(dtype, dc, dout)(p, static_cast<hipStream_t>(stream)) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+    const hipError_t e = lookup(dtype, dc, dout)(p, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? FLA_OK : e == hipErrorNotSupported ? FLA_ERR_UNSUPPORTED : FLA_ERR_LAUNCH;
+}
+
+// Feature maps of one product (fla_feature.h): phi on the operands as they are loaded, and the
+// output multiplied by phi'(omap).  Only the chunk-wise fast-path kernels implement them.
+struct Maps {
+    int x = 0, y = 0, z = 0, out = 0;
+    View omap{nullptr, nullptr};
+    bool any() const { return x || y || z || omap.ptr; }
+};
+
+void set_maps(TriParams &p, const Maps &m) {
+    p.map_x = m.x, p.map_y = m.y, p.map_z = m.z;
+    if (m.omap.ptr) {
+        p.map_out = m.out, p.omap = m.omap.ptr;
+        p.ms_b = m.omap.strides[0], p.ms_h = m.omap.strides[1], p.ms_n = m.omap.strides[2];
+    }
 }
 
 // Out = mask(X Y^T) Z evaluated chunk-wise; same arguments as run_tri plus the workspace.
@@ -257,25 +278,35 @@ int chunk_main(TriParams p, int64_t dc, int64_t dout, int dtype, const void *sta
 // or the sequence is a single chunk.
 int run_tri_chunked(const View &x, const View &y, const View &z, const View &out, int64_t B, int64_t H, int64_t N,
                     int64_t dc, int64_t dout, int upper, int dtype, void *workspace, int64_t workspace_bytes,
-                    void *stream) {
+                    void *stream, const Maps &maps = Maps{}) {
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
     if (dout > 128 && (dc <= 64 || dc > 128)) {
         const View z_hi{static_cast<const char *>(z.ptr) + 128 * 2, z.strides};
         const View out_hi{static_cast<const char *>(out.ptr) + 128 * 2, out.strides};
-        if (int rc = run_tri_chunked(x, y, z, out, B, H, N, dc, 128, upper, dtype, workspace, workspace_bytes, stream))
+        Maps maps_hi = maps;
+        if (maps.omap.ptr) maps_hi.omap.ptr = static_cast<const char *>(maps.omap.ptr) + 128 * 2;
+        if (int rc = run_tri_chunked(x, y, z, out, B, H, N, dc, 128, upper, dtype, workspace, workspace_bytes, stream,
+                                     maps))
             return rc;
         return run_tri_chunked(x, y, z_hi, out_hi, B, H, N, dc, dout - 128, upper, dtype, workspace, workspace_bytes,
-                               stream);
+                               stream, maps_hi);
     }
-    const TriParams p = make_params(x, y, z, out, B, H, N, dc, dout, upper);
-    if (!chunkable(p, dc, dout, N)) return run_tri(x, y, z, out, B, H, N, dc, dout, upper, dtype, stream);
+    TriParams p = make_params(x, y, z, out, B, H, N, dc, dout, upper);
+    set_maps(p, maps);
+    if (!chunkable(p, dc, dout, N)) {
+        if (!maps.any()) return run_tri(x, y, z, out, B, H, N, dc, dout, upper, dtype, stream);
+        // feature maps exist in the chunk-wise kernel only: a sequence of a single chunk runs it
+        // without a state (the pointer merely selects the kernel; a single chunk never reads it)
+        if (chunk_rows(dc, dout) == 0 || N > chunk_rows(dc, dout) || !fla::fast_path_ok(p)) return FLA_ERR_UNSUPPORTED;
+        return chunk_main(p, dc, dout, dtype, p.x, 0, stream);
+    }
     const int64_t rows = chunk_rows(dc, dout), chunks = (N + rows - 1) / rows, E = padded(dc) * padded(dout);
     const int64_t BH = B * H;
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < BH * chunks * E * 6)
         return FLA_ERR_WORKSPACE;
     float *w = static_cast<float *>(workspace);
     void *state = static_cast<char *>(workspace) + BH * chunks * E * 4;
-    if (int rc = chunk_states(y, z, B, H, N, dc, dout, upper, dtype, w, state, stream)) return rc;
+    if (int rc = chunk_states(y, z, B, H, N, dc, dout, upper, dtype, w, state, stream, maps.y, maps.z)) return rc;
     return chunk_main(p, dc, dout, dtype, state, 0, stream);
 }
 
@@ -307,25 +338,30 @@ int64_t chunked_op_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk,
     return m > t ? m : t;
 }
 
+// fmap != 0: q and k are the arguments of the feature map phi, applied as they are loaded
 int chunked_forward(const View &q, const View &k, const View &v, const View &o, int64_t B, int64_t H, int64_t N,
                     int64_t dqk, int64_t dv, int dtype, void *state_out, int32_t *state_valid, void *workspace,
-                    int64_t workspace_bytes, void *stream) {
+                    int64_t workspace_bytes, void *stream, int fmap = 0) {
     if (state_valid) *state_valid = 0;
     const View all[] = {q, k, v, o};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
     if (int rc = check_alias_fwd(q, k, v, o, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
-    const TriParams p = make_params(q, k, v, o, B, H, N, dqk, dv, 0);
-    if (!states_shareable(dqk, dv, N) || !fla::fast_path_ok(p))
-        return run_tri_chunked(q, k, v, o, B, H, N, dqk, dv, 0, dtype, workspace, workspace_bytes, stream);
+    TriParams p = make_params(q, k, v, o, B, H, N, dqk, dv, 0);
+    p.map_x = p.map_y = fmap;
+    if (!states_shareable(dqk, dv, N) || !fla::fast_path_ok(p)) {
+        Maps m;
+        m.x = m.y = fmap;
+        return run_tri_chunked(q, k, v, o, B, H, N, dqk, dv, 0, dtype, workspace, workspace_bytes, stream, m);
+    }
     const int64_t sb = shared_state_bytes(B, H, N, dqk, dv);
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < sb * (state_out ? 2 : 3))
         return FLA_ERR_WORKSPACE;
     if (state_out && reinterpret_cast<uintptr_t>(state_out) % 16 != 0) return FLA_ERR_WORKSPACE;
     float *w = static_cast<float *>(workspace);
     void *state = state_out ? state_out : static_cast<char *>(workspace) + 2 * sb;
-    if (int rc = chunk_states(k, v, B, H, N, dqk, dv, 0, dtype, w, state, stream)) return rc;
+    if (int rc = chunk_states(k, v, B, H, N, dqk, dv, 0, dtype, w, state, stream, fmap, 0)) return rc;
     if (int rc = chunk_main(p, dqk, dv, dtype, state, 0, stream)) return rc;
     if (state_out && state_valid) *state_valid = 1;
     return FLA_OK;
@@ -333,21 +369,30 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
 
 int chunked_backward(const View &go, const View &q, const View &k, const View &v, const View &dq, const View &dk,
                      const View &dvv, int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv, int dtype,
-                     const void *state_in, void *workspace, int64_t workspace_bytes, void *stream) {
+                     const void *state_in, void *workspace, int64_t workspace_bytes, void *stream, int fmap = 0) {
     const View all[] = {go, q, k, v, dq, dk, dvv};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
     if (int rc = check_alias_bwd(go, q, k, v, nullptr, dq, dk, dvv, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
-    const TriParams pq = make_params(go, v, k, dq, B, H, N, dv, dqk, 0);   // dQ = lower(dO V^T) K
-    const TriParams pv = make_params(k, q, go, dvv, B, H, N, dqk, dv, 1);  // dV = upper(K Q^T) dO
-    const TriParams pk = make_params(v, go, q, dk, B, H, N, dv, dqk, 1);   // dK = upper(V dO^T) Q
+    // With a feature map q and k are its arguments: K and Q are mapped wherever they are loaded, and
+    // the gradients with respect to phi(xq), phi(xk) leave multiplied by phi'(xq), phi'(xk).
+    Maps mq, mv, mk;
+    if (fmap) {
+        mq.z = fmap, mq.out = fmap, mq.omap = q;  // dXq = (lower(dO V^T) phi(Xk)) . phi'(Xq)
+        mv.x = mv.y = fmap;                       // dV  = upper(phi(Xk) phi(Xq)^T) dO
+        mk.z = fmap, mk.out = fmap, mk.omap = k;  // dXk = (upper(V dO^T) phi(Xq)) . phi'(Xk)
+    }
+    TriParams pq = make_params(go, v, k, dq, B, H, N, dv, dqk, 0);   // dQ = lower(dO V^T) K
+    TriParams pv = make_params(k, q, go, dvv, B, H, N, dqk, dv, 1);  // dV = upper(K Q^T) dO
+    TriParams pk = make_params(v, go, q, dk, B, H, N, dv, dqk, 1);   // dK = upper(V dO^T) Q
+    set_maps(pq, mq), set_maps(pv, mv), set_maps(pk, mk);
     if (!states_shareable(dqk, dv, N) || !fla::fast_path_ok(pq) || !fla::fast_path_ok(pv) || !fla::fast_path_ok(pk)) {
-        if (int rc = run_tri_chunked(go, v, k, dq, B, H, N, dv, dqk, 0, dtype, workspace, workspace_bytes, stream))
+        if (int rc = run_tri_chunked(go, v, k, dq, B, H, N, dv, dqk, 0, dtype, workspace, workspace_bytes, stream, mq))
             return rc;
-        if (int rc = run_tri_chunked(k, q, go, dvv, B, H, N, dqk, dv, 1, dtype, workspace, workspace_bytes, stream))
+        if (int rc = run_tri_chunked(k, q, go, dvv, B, H, N, dqk, dv, 1, dtype, workspace, workspace_bytes, stream, mv))
             return rc;
-        return run_tri_chunked(v, go, q, dk, B, H, N, dv, dqk, 1, dtype, workspace, workspace_bytes, stream);
+        return run_tri_chunked(v, go, q, dk, B, H, N, dv, dqk, 1, dtype, workspace, workspace_bytes, stream, mk);
     }
     const int64_t sb = shared_state_bytes(B, H, N, dqk, dv);
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < sb * (state_in ? 3 : 4))
@@ -357,10 +402,10 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
     const void *state_f = state_in;
     if (!state_f) {
         void *mine = static_cast<char *>(workspace) + 3 * sb;
-        if (int rc = chunk_states(k, v, B, H, N, dqk, dv, 0, dtype, w, mine, stream)) return rc;
+        if (int rc = chunk_states(k, v, B, H, N, dqk, dv, 0, dtype, w, mine, stream, fmap, 0)) return rc;
         state_f = mine;
     }
-    if (int rc = chunk_states(q, go, B, H, N, dqk, dv, 1, dtype, w, state_v, stream)) return rc;
+    if (int rc = chunk_states(q, go, B, H, N, dqk, dv, 1, dtype, w, state_v, stream, fmap, 0)) return rc;
     // One launch for the three products: a workgroup evaluates dQ, dV and dK of its chunk in turn,
     // so q, k, v and dO come from memory once.  dQ reads the forward state [D_v][D_qk] as its own
     // [D_c = D_v][D_o = D_qk] transposed state; dK reads the state of dV transposed.
@@ -862,6 +907,34 @@ int fla_linear_attn_chunked_fwd_static(const void *q, const void *k, const void 
     if (int rc = static_scratch(&ws)) return rc;
     return chunked_forward({q, q_strides}, {k, k_strides}, {v, v_strides}, {o, o_strides}, B, H, N, D_qk, D_v, dtype,
                            nullptr, nullptr, ws, FLA_STATIC_SCRATCH_BYTES, stream);
+}
+
+int fla_feature_attn_fwd(const void *xq, const void *xk, const void *v, void *o, int64_t B, int64_t H, int64_t N,
+                         int64_t D_qk, int64_t D_v, const int64_t *xq_strides, const int64_t *xk_strides,
+                         const int64_t *v_strides, const int64_t *o_strides, int feature_map, int dtype,
+                         void *state_out, int32_t *state_valid, void *workspace, int64_t workspace_bytes, void *stream) {
+    if (state_valid) *state_valid = 0;
+    if (int rc = check_common(B, H, N, dtype)) return rc;
+    if (D_qk < 1 || D_qk > 256) return FLA_ERR_HEAD_DIM;
+    if (D_v < 1 || D_v > 256) return FLA_ERR_V_HEAD_DIM;
+    if (feature_map != FLA_MAP_ELU1 && feature_map != FLA_MAP_SOFTPLUS) return FLA_ERR_UNSUPPORTED;
+    return chunked_forward({xq, xq_strides}, {xk, xk_strides}, {v, v_strides}, {o, o_strides}, B, H, N, D_qk, D_v,
+                           dtype, state_out, state_valid, workspace, workspace_bytes, stream, feature_map);
+}
+
+int fla_feature_attn_bwd(const void *grad_out, const void *xq, const void *xk, const void *v, void *dxq, void *dxk,
+                         void *dv, int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                         const int64_t *go_strides, const int64_t *xq_strides, const int64_t *xk_strides,
+                         const int64_t *v_strides, const int64_t *dxq_strides, const int64_t *dxk_strides,
+                         const int64_t *dv_strides, int feature_map, int dtype, const void *state_in, void *workspace,
+                         int64_t workspace_bytes, void *stream) {
+    if (int rc = check_common(B, H, N, dtype)) return rc;
+    if (D_qk < 1 || D_qk > 256) return FLA_ERR_HEAD_DIM;
+    if (D_v < 1 || D_v > 256) return FLA_ERR_V_HEAD_DIM;
+    if (feature_map != FLA_MAP_ELU1 && feature_map != FLA_MAP_SOFTPLUS) return FLA_ERR_UNSUPPORTED;
+    return chunked_backward({grad_out, go_strides}, {xq, xq_strides}, {xk, xk_strides}, {v, v_strides},
+                            {dxq, dxq_strides}, {dxk, dxk_strides}, {dv, dv_strides}, B, H, N, D_qk, D_v, dtype,
+                            state_in, workspace, workspace_bytes, stream, feature_map);
 }
 
 int fla_linear_attn_chunked_bwd(const void *grad_out, const void *q, const void *k, const void *v, void *dq, void *dk,

@@ -32,6 +32,7 @@ struct ChunkStateParams {
     int32_t H, N, BH;
     int32_t dc, dout;
     int32_t n_chunks;
+    int32_t map_y, map_z;  // feature map applied to Y / Z as the tiles arrive (fla_feature.h), 0: none
 };
 
 // LDS footprint of the state kernel: at most half of the CU's 160 KiB, so that two workgroups fit
@@ -124,6 +125,27 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(const ChunkStateParams
         });
         wait_vm<0>();
         __builtin_amdgcn_s_barrier();
+        if (p.map_y | p.map_z) {
+            // feature map on load: rewrite the landed tiles in place; zero padding stays zero
+            auto map_tiles = [&](int map, int region, int row_bytes, int cpr, int width, auto swz) {
+#pragma unroll 1
+                for (int t = 0; t < RT; ++t) {
+                    unsigned char *tile = smem + t * STAGE + region;
+                    const int row0 = r0 + (R * RT + t) * BN;
+#pragma unroll 1
+                    for (int u = tid; u < BN * cpr; u += 256) {
+                        const int r = u / cpr, c = (u - r * cpr) ^ swz(r);
+                        if (row0 + r < N && c * 8 < width) {
+                            u32x4 *ptr = reinterpret_cast<u32x4 *>(tile + r * row_bytes + ((u - r * cpr) << 4));
+                            *ptr = feature_map8<T>(map, *ptr);
+                        }
+                    }
+                }
+            };
+            if (p.map_y) map_tiles(p.map_y, 0, RY, CY, p.dc, [](int r) { return swizzle_y<CY>(r); });
+            if (p.map_z) map_tiles(p.map_z, Y_BYTES, RZ, CZ, p.dout, [](int r) { return swizzle_z<CZ>(r); });
+            __syncthreads();
+        }
     };
 
     // Column fragment of a row-major tile: rows R0 + {4g..4g+3, 8+4g..8+4g+3}, column 32 cb + l32.

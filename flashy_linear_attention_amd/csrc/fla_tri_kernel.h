@@ -73,6 +73,14 @@ struct TriParams {
     // last 32 columns, [DC - 32, DC).
     float poly[3];
     int32_t poly_on;
+    // Feature map on load (chunk-wise fast path only; fla_feature.h): a non-zero map_x / map_y /
+    // map_z replaces every element of that operand by phi(element) as it arrives (zero padding
+    // stays zero).  `omap`, when non-null, is a tensor of Out's shape (element strides ms_*): each
+    // output element is multiplied by phi'(omap element), map_out naming phi -- the chain rule of
+    // a gradient with respect to the argument of phi.
+    int32_t map_x, map_y, map_z, map_out;
+    const void *omap;
+    int64_t ms_b, ms_h, ms_n;
 };
 
 // Up to three products of identical shape in one launch (grid y selects the product): the

@@ -1,0 +1,121 @@
+"""Causal linear attention with the feature map inside the operator (an extension: callers of the
+reference apply the map in PyTorch before ``LinearAttention.apply``, README.md:27-30 and
+flashlinear/test_attn.py:36-40 of the reference):
+
+    FeatureMapLinearAttention.apply(xq, xk, v, "elu1")   ==   LinearAttention.apply(elu(xq) + 1, elu(xk) + 1, v)
+
+with ``"softplus"`` as the other map.  The product is evaluated chunk-wise
+(``LinearAttentionChunked``'s method) and the map is applied while the kernels load xq and xk,
+so phi(xq), phi(xk) are never written to memory and backward returns the gradients with respect
+to xq and xk themselves (``fla_feature_attn_fwd`` / ``fla_feature_attn_bwd``).
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Any, Optional, Tuple
+
+import torch
+from torch.autograd import Function
+
+from . import _lib
+from .kernels._common import dtype_code, prepare, stream_handle
+
+FEATURE_MAPS = {"elu1": 1, "softplus": 2}  # enum fla_feature_map
+
+
+def _map_code(feature: str) -> int:
+    try:
+        return FEATURE_MAPS[feature]
+    except KeyError:
+        raise ValueError(f"feature map must be one of {sorted(FEATURE_MAPS)}, got {feature!r}") from None
+
+
+def feature_attention_fwd(xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, feature: str = "elu1",
+                          want_state: bool = False):
+    """``O = tril(phi(xq) phi(xk)^T) v``.  With ``want_state`` returns ``(O, state)``, the running
+    state for :func:`feature_attention_bwd` (None when the shape does not allow sharing it)."""
+    assert xq.shape == xk.shape and v.shape[:3] == xq.shape[:3], "xq, xk: (B,H,N,D_qk); v: (B,H,N,D_v)"
+    assert xq.shape[-1] <= 256 and v.shape[-1] <= 256, "Only head_dims <= 256 are supported."
+    code = _map_code(feature)
+    xq, xk, v = prepare(xq, xk, v)
+    b, h, n, dqk = xq.shape
+    dv = v.shape[-1]
+    out = torch.empty_like(v, memory_format=torch.contiguous_format)
+    lib = _lib.load()
+    with torch.cuda.device(xq.device):
+        sbytes = lib.fla_linear_attn_chunked_state_bytes(b, h, n, dqk, dv) if want_state else 0
+        state = torch.empty(sbytes, dtype=torch.uint8, device=xq.device) if sbytes else None
+        wbytes = lib.fla_linear_attn_chunked_workspace_bytes(b, h, n, dqk, dv)
+        work = torch.empty(max(wbytes, 16), dtype=torch.uint8, device=xq.device)
+        valid = ctypes.c_int32(0)
+        _lib.check(
+            "fla_feature_attn_fwd",
+            lib.fla_feature_attn_fwd(
+                xq.data_ptr(), xk.data_ptr(), v.data_ptr(), out.data_ptr(), b, h, n, dqk, dv,
+                _lib.strides_arg(xq), _lib.strides_arg(xk), _lib.strides_arg(v), _lib.strides_arg(out),
+                code, dtype_code(xq), state.data_ptr() if state is not None else None, ctypes.byref(valid),
+                work.data_ptr(), wbytes, stream_handle(xq.device),
+            ),
+        )
+    if want_state:
+        return out, (state if valid.value else None)
+    return out
+
+
+def feature_attention_bwd(grad_output: torch.Tensor, xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor,
+                          feature: str = "elu1", state: Optional[torch.Tensor] = None,
+                          ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dxq, dxk, dv); ``state`` is what the forward call returned (or None)."""
+    code = _map_code(feature)
+    grad_output, xq, xk, v = prepare(grad_output, xq, xk, v)
+    b, h, n, dqk = xq.shape
+    dv = v.shape[-1]
+    dxq = torch.empty_like(xq, memory_format=torch.contiguous_format)
+    dxk = torch.empty_like(xk, memory_format=torch.contiguous_format)
+    dvv = torch.empty_like(v, memory_format=torch.contiguous_format)
+    lib = _lib.load()
+    with torch.cuda.device(xq.device):
+        if state is not None:
+            assert state.numel() == lib.fla_linear_attn_chunked_state_bytes(b, h, n, dqk, dv), "state of another shape"
+        wbytes = lib.fla_linear_attn_chunked_workspace_bytes(b, h, n, dqk, dv)
+        work = torch.empty(max(wbytes, 16), dtype=torch.uint8, device=xq.device)
+        _lib.check(
+            "fla_feature_attn_bwd",
+            lib.fla_feature_attn_bwd(
+                grad_output.data_ptr(), xq.data_ptr(), xk.data_ptr(), v.data_ptr(),
+                dxq.data_ptr(), dxk.data_ptr(), dvv.data_ptr(), b, h, n, dqk, dv,
+                _lib.strides_arg(grad_output), _lib.strides_arg(xq), _lib.strides_arg(xk), _lib.strides_arg(v),
+                _lib.strides_arg(dxq), _lib.strides_arg(dxk), _lib.strides_arg(dvv),
+                code, dtype_code(xq), state.data_ptr() if state is not None else None, work.data_ptr(), wbytes,
+                stream_handle(xq.device),
+            ),
+        )
+    return dxq, dxk, dvv
+
+
+class FeatureMapLinearAttention(Function):
+    @staticmethod
+    @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.bfloat16)
+    def forward(ctx: Any, xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, feature: str = "elu1") -> torch.Tensor:
+        if any(ctx.needs_input_grad[:3]):
+            out, state = feature_attention_fwd(xq, xk, v, feature, want_state=True)
+        else:
+            out, state = feature_attention_fwd(xq, xk, v, feature), None
+        ctx.feature = feature
+        ctx.has_state = state is not None
+        if state is not None:
+            ctx.save_for_backward(xq, xk, v, state)
+        else:
+            ctx.save_for_backward(xq, xk, v)
+        return out
+
+    @staticmethod
+    @torch.amp.custom_bwd(device_type="cuda")
+    def backward(ctx: Any, grad_output: torch.Tensor):
+        if ctx.has_state:
+            xq, xk, v, state = ctx.saved_tensors
+        else:
+            (xq, xk, v), state = ctx.saved_tensors, None
+        dxq, dxk, dv = feature_attention_bwd(grad_output, xq, xk, v, ctx.feature, state)
+        return dxq, dxk, dv, None

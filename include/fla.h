@@ -174,6 +174,40 @@ int fla_linear_attn_chunked_bwd(const void *grad_out, const void *q, const void 
                                 int dtype, const void *state_in,
                                 void *workspace, int64_t workspace_bytes, void *stream);
 
+/* Causal linear attention on q = phi(xq), k = phi(xk) for an element-wise feature map phi,
+ *
+ *     O = tril(phi(Xq) phi(Xk)^T) V,
+ *
+ * evaluated chunk-wise (fla_linear_attn_chunked_fwd/bwd's method) with phi applied as the
+ * operands are loaded: phi(xq) and phi(xk) never exist in memory, neither in forward nor in
+ * backward, and backward returns the gradients with respect to xq and xk directly,
+ *     dXq = (tril(dO V^T) phi(Xk)) . phi'(Xq),    dXk = (tril(dO V^T)^T phi(Xq)) . phi'(Xk)
+ * (the chain rule is applied to the accumulators before they are rounded and stored), plus dV.
+ * feature_map: FLA_MAP_ELU1 (elu(x) + 1) or FLA_MAP_SOFTPLUS (log(1 + e^x), the map the
+ * reference's tests put in front of its operators, flashlinear/test_attn.py:36-40); phi is
+ * evaluated in fp32 and rounded once to the storage dtype.  state_out / state_valid / state_in,
+ * workspace: exactly as for fla_linear_attn_chunked_fwd/bwd, same size queries.  Fast-path
+ * operands only (16-byte aligned, widths and outer strides multiples of 8 elements), else
+ * FLA_ERR_UNSUPPORTED.  No counterpart in the reference: its callers materialise phi(x) with a
+ * PyTorch pass before the operator and differentiate through it with another
+ * (README.md:27-30 of the reference). */
+enum fla_feature_map { FLA_MAP_NONE = 0, FLA_MAP_ELU1 = 1, FLA_MAP_SOFTPLUS = 2 };
+int fla_feature_attn_fwd(const void *xq, const void *xk, const void *v, void *o,
+                         int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                         const int64_t *xq_strides, const int64_t *xk_strides,
+                         const int64_t *v_strides, const int64_t *o_strides,
+                         int feature_map, int dtype, void *state_out, int32_t *state_valid,
+                         void *workspace, int64_t workspace_bytes, void *stream);
+int fla_feature_attn_bwd(const void *grad_out, const void *xq, const void *xk, const void *v,
+                         void *dxq, void *dxk, void *dv,
+                         int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                         const int64_t *go_strides, const int64_t *xq_strides,
+                         const int64_t *xk_strides, const int64_t *v_strides,
+                         const int64_t *dxq_strides, const int64_t *dxk_strides,
+                         const int64_t *dv_strides,
+                         int feature_map, int dtype, const void *state_in,
+                         void *workspace, int64_t workspace_bytes, void *stream);
+
 /* fla_linear_attn_chunked_fwd for callers that cannot allocate device memory or pass a workspace
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference.  Same arguments and results as fla_linear_attn_chunked_fwd with

@@ -176,3 +176,38 @@ def poly_causal_dot_product_grads(
     s = (c0 + c1 * u + c2 * u * u) * mask
     du = torch.matmul(do, v.transpose(-2, -1)) * mask * (c1 + 2.0 * c2 * u)
     return torch.matmul(du, xk), torch.matmul(du.transpose(-2, -1), xq), torch.matmul(s.transpose(-2, -1), do)
+
+
+def feature_map(x: torch.Tensor, kind: str) -> torch.Tensor:
+    """The element-wise positive maps callers put in front of the operators: ``"elu1"`` is
+    elu(x) + 1 (= x + 1 for x > 0, e^x otherwise), ``"softplus"`` is log(1 + e^x), the map of the
+    reference's tests (flashlinear/test_attn.py:36-40)."""
+    if kind == "elu1":
+        return torch.nn.functional.elu(x) + 1.0
+    if kind == "softplus":
+        return torch.nn.functional.softplus(x)
+    raise ValueError(kind)
+
+
+def feature_map_slope(x: torch.Tensor, kind: str) -> torch.Tensor:
+    """d phi / d x in closed form: elu1 -> 1 for x > 0, e^x otherwise; softplus -> sigmoid(x)."""
+    if kind == "elu1":
+        return torch.where(x > 0, torch.ones_like(x), torch.exp(x))
+    if kind == "softplus":
+        return torch.sigmoid(x)
+    raise ValueError(kind)
+
+
+def feature_causal_dot_product(xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, kind: str) -> torch.Tensor:
+    """O = tril(phi(Xq) phi(Xk)^T) V: the caller's recipe (feature map, then the operator;
+    README.md:27-30 of the reference) as one function of the raw xq, xk."""
+    return causal_dot_product(feature_map(xq, kind), feature_map(xk, kind), v)
+
+
+def feature_causal_dot_product_grads(
+    xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, do: torch.Tensor, kind: str
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dXq, dXk, dV) in closed form: the product's gradients with respect to phi(xq), phi(xk)
+    times the slope of phi."""
+    dq, dk, dv = causal_dot_product_grads(feature_map(xq, kind), feature_map(xk, kind), v, do)
+    return dq * feature_map_slope(xq, kind), dk * feature_map_slope(xk, kind), dv

@@ -202,3 +202,57 @@ def test_normalised_polynomial_equals_normalised_recipe_on_explicit_features():
     assert torch.allclose(got.detach(), ref.detach(), rtol=1e-11, atol=1e-11)
     for x, y in ((a2.grad, a.grad), (b2.grad, b.grad), (c2.grad, c.grad)):
         assert torch.allclose(x, y, rtol=1e-10, atol=1e-10)
+
+
+# ------------------------------------------------------------------ feature maps
+def test_feature_maps_closed_forms():
+    """elu1: x + 1 right of zero, e^x left of it, 1 at zero, continuous with slope 1 there;
+    softplus: log 2 at zero, softplus(x) - softplus(-x) = x, e^x far left, x far right.  A map
+    written without the '+ 1', or with the branches swapped, fails."""
+    import math
+
+    x = torch.tensor([-30.0, -3.0, -0.5, 0.0, 0.25, 2.0, 30.0], dtype=torch.float64)
+    e = naive.feature_map(x, "elu1")
+    for xi, ei in zip(x.tolist(), e.tolist()):
+        assert ei == pytest.approx(xi + 1.0 if xi > 0 else math.exp(xi), rel=1e-12)
+    s = naive.feature_map(x, "softplus")
+    assert s[3].item() == pytest.approx(math.log(2.0), rel=1e-12)
+    torch.testing.assert_close(s - naive.feature_map(-x, "softplus"), x, rtol=1e-12, atol=1e-12)
+    assert s[0].item() == pytest.approx(math.exp(-30.0), rel=1e-9) and s[-1].item() == pytest.approx(30.0, rel=1e-12)
+    assert (e > 0).all() and (s > 0).all()
+    with pytest.raises(ValueError):
+        naive.feature_map(x, "relu")
+
+
+@pytest.mark.parametrize("kind", ["elu1", "softplus"])
+def test_feature_map_slopes_against_central_differences(kind):
+    x = torch.linspace(-4.0, 4.0, 41, dtype=torch.float64) + 0.013  # keeps the elu kink off the grid
+    h = 1e-6
+    fd = (naive.feature_map(x + h, kind) - naive.feature_map(x - h, kind)) / (2 * h)
+    torch.testing.assert_close(naive.feature_map_slope(x, kind), fd, rtol=1e-7, atol=1e-8)
+
+
+@pytest.mark.parametrize("kind", ["elu1", "softplus"])
+def test_feature_operator_gradients(kind):
+    """Closed-form (dXq, dXk, dV) of O = tril(phi(Xq) phi(Xk)^T) V against autograd through the
+    composed function and against central differences of <dO, O> through the *recurrent* form of
+    the product: a missing slope factor, or the slope of the wrong operand, fails both."""
+    xq, xk, v, do = _rand((1, 2, 9, 4), 31), _rand((1, 2, 9, 4), 32), _rand((1, 2, 9, 3), 33), _rand((1, 2, 9, 3), 34)
+    got = naive.feature_causal_dot_product_grads(xq, xk, v, do, kind)
+    a, b, c = (t.clone().requires_grad_(True) for t in (xq, xk, v))
+    want = torch.autograd.grad(naive.feature_causal_dot_product(a, b, c, kind), (a, b, c), do)
+    for g, w in zip(got, want):
+        torch.testing.assert_close(g, w, rtol=1e-10, atol=1e-10)
+
+    def scalar(xq_, xk_, v_):
+        return (do * naive.causal_dot_product_recurrent(naive.feature_map(xq_, kind), naive.feature_map(xk_, kind), v_)).sum()
+
+    h = 1e-6
+    for which, g in enumerate(got):
+        base = [xq, xk, v]
+        for idx in [(0, 0, 0, 0), (0, 1, 4, 2), (0, 1, 8, 1)]:
+            plus, minus = [t.clone() for t in base], [t.clone() for t in base]
+            plus[which][idx] += h
+            minus[which][idx] -= h
+            fd = (scalar(*plus) - scalar(*minus)) / (2 * h)
+            assert g[idx].item() == pytest.approx(fd.item(), rel=1e-6, abs=1e-8)
