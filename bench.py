@@ -55,7 +55,7 @@ PROFILED_TRAFFIC = {
 # SQ_INSTS_VALU_MFMA_MOPS_BF16 x 512 FLOPs; the excess is the 32 x 32 blocks on the diagonal)
 PROFILED_MFMA_RATIO = {("C3", "quadratic"): (1.008, "profiles/tri_xyt_z_fast_kernels_C3_pmc.md")}
 
-ALGOS = ["quadratic", "chunked", "normalised", "normalised-chunked", "poly"]
+ALGOS = ["quadratic", "chunked", "normalised", "normalised-chunked", "poly", "feature"]
 
 
 def _parse():
@@ -80,7 +80,9 @@ def _parse():
                          "with the normaliser's own time, bytes and the PyTorch recipe's time beside it; "
                          "normalised-chunked: the same with the chunk-wise product; "
                          "poly (workload C4 only): the same function as C4 computed from the 16-wide x behind its "
-                         "Taylor features with the polynomial score map, priced in its own FLOPs")
+                         "Taylor features with the polynomial score map, priced in its own FLOPs; "
+                         "feature: the chunk-wise operator on raw xq, xk with elu(x) + 1 applied as the kernels load "
+                         "them, next to 'PyTorch elu pass + chunk-wise operator' through autograd in the same run")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain device copy of 256 MiB (a known-size reference for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -380,6 +382,82 @@ def _bench_poly(torch, args, w, dev) -> int:
     return 0
 
 
+def _bench_feature(torch, args, w, dev) -> int:
+    """The chunk-wise operator from the raw inputs xq, xk (q = elu(xq) + 1, k = elu(xk) + 1 formed while
+    the kernels load them, gradients with respect to xq, xk), against the same function built the
+    caller's way: elu passes in PyTorch around LinearAttentionChunked, differentiated by autograd."""
+    from flashy_linear_attention_amd import FeatureMapLinearAttention, LinearAttentionChunked
+    from flashy_linear_attention_amd.feature import feature_attention_bwd, feature_attention_fwd
+
+    if w.features != "elu1" or not w.backward:
+        print("bench.py: --algo feature needs a forward + backward workload with elu(x) + 1 features (C3, C5)", file=sys.stderr)
+        return 2
+    gen = torch.Generator().manual_seed(0)
+    xq, xk = (torch.randn(w.batch, w.heads, w.seq, w.d_qk, generator=gen).to(w.dtype).to(dev) for _ in range(2))
+    v, do = (torch.randn(w.batch, w.heads, w.seq, w.d_v, generator=gen).to(w.dtype).to(dev) for _ in range(2))
+    _, q_map, k_map, state = feature_attention_fwd(xq, xk, v, "elu1", want_state=True)
+
+    def fwd():
+        return feature_attention_fwd(xq, xk, v, "elu1", want_state=True)
+
+    def bwd():
+        return feature_attention_bwd(do, q_map, k_map, v, "elu1", state)
+
+    def step():
+        fwd()
+        bwd()
+
+    xa, xb, va = (t.detach().clone().requires_grad_(True) for t in (xq, xk, v))
+
+    def autograd_step():
+        torch.autograd.grad(FeatureMapLinearAttention.apply(xa, xb, va, "elu1"), (xa, xb, va), do)
+
+    def recipe_step():
+        q = torch.nn.functional.elu(xa) + 1
+        k = torch.nn.functional.elu(xb) + 1
+        torch.autograd.grad(LinearAttentionChunked.apply(q, k, va), (xa, xb, va), do)
+
+    _settle(torch, step, args.settle_seconds)
+    for _ in range(args.warmup):
+        step()
+    ms_step = _time_region(torch, step, args.steps) / args.steps
+    ms_fwd, ms_bwd = _median_ms(torch, fwd, args.steps), _median_ms(torch, bwd, args.steps)
+    for _ in range(5):
+        autograd_step()
+        recipe_step()
+    ms_auto, ms_recipe = _median_ms(torch, autograd_step, args.steps), _median_ms(torch, recipe_step, args.steps)
+    # the plain operator's tensors (xq, xk in place of q, k) plus the by-product q, k written in forward
+    bytes_step = w.bytes_fwd + w.bytes_bwd + 2.0 * 2.0 * w.batch * w.heads * w.seq * w.d_qk
+    # what the PyTorch passes move on top: forward reads xq, xk and writes q, k; backward reads dq, dk and
+    # xq, xk (or the saved q, k) and writes dxq, dxk
+    e = float(w.batch * w.heads * w.seq)
+    recipe_extra = 2.0 * e * w.d_qk * (4 + 6)
+    gbs = bytes_step / (ms_step * 1e-3) / 1e9
+    ff, fb = _chunked_flops(w)
+    result = {
+        "metric": f"causal linear attention with elu(x)+1 applied on load, chunk-wise, fwd+bwd GB/s of algorithmic bytes, "
+                  f"B={w.batch} H={w.heads} N={w.seq} D_qk={w.d_qk} D_v={w.d_v}, 1 MI355X",
+        "value": round(gbs, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {
+            "workload": f"{w.name} from its raw inputs: xq, xk, v, dO randn (seed 0), q = elu(xq) + 1, k = elu(xk) + 1 inside "
+                        f"the kernels; {_chunk_rows(w)}-row chunks",
+            "algorithmic_bytes_per_step": bytes_step,
+            "own_tflops": round((ff + fb) / (ms_step * 1e-3) / 1e12, 1),
+            "median_ms": {"fwd": round(ms_fwd, 4), "bwd": round(ms_bwd, 4), "autograd_step": round(ms_auto, 4)},
+            "pytorch_elu_passes_plus_chunked_operator_autograd_step_ms": round(ms_recipe, 4),
+            "speedup_vs_pytorch_elu_passes": round(ms_recipe / ms_auto, 2),
+            "bytes_the_pytorch_passes_move_on_top": recipe_extra,
+        },
+        "roofline": {"bound": "hbm", "kernel": "all kernels of a chunk-wise step with the feature map applied on load",
+                     "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes_per_step": bytes_step},
+    }
+    print(json.dumps(result))
+    return 0
+
+
 def main() -> int:
     args = _parse()
     if args.gpus != 1:
@@ -401,6 +479,8 @@ def main() -> int:
     dev = torch.device("cuda:0")
     if args.algo == "poly":
         return _bench_poly(torch, args, w, dev)
+    if args.algo == "feature":
+        return _bench_feature(torch, args, w, dev)
     normalised = args.algo.startswith("normalised")
     chunked = args.algo in ("chunked", "normalised-chunked")
     o = _ops(torch, w, "chunked" if chunked else "quadratic", dev)

@@ -37,7 +37,7 @@ SIGNATURES = {
     "fla_linear_attn_chunked_workspace_bytes": ([_i64] * 5, ctypes.c_int64),
     "fla_linear_attn_chunked_fwd": ([_ptr] * 4 + [_i64] * 5 + [_strides] * 4
                                     + [ctypes.c_int, _ptr, ctypes.POINTER(ctypes.c_int32), _ptr, _i64, _ptr], ctypes.c_int),
-    "fla_feature_attn_fwd": ([_ptr] * 4 + [_i64] * 5 + [_strides] * 4
+    "fla_feature_attn_fwd": ([_ptr] * 6 + [_i64] * 5 + [_strides] * 6
                              + [ctypes.c_int, ctypes.c_int, _ptr, ctypes.POINTER(ctypes.c_int32), _ptr, _i64, _ptr], ctypes.c_int),
     "fla_feature_attn_bwd": ([_ptr] * 7 + [_i64] * 5 + [_strides] * 7 + [ctypes.c_int, ctypes.c_int, _ptr, _ptr, _i64, _ptr],
                              ctypes.c_int),

@@ -164,8 +164,9 @@ TriParams make_params(const View &x, const View &y, const View &z, const View &o
     p.eps = 0.f;
     p.poly[0] = p.poly[1] = p.poly[2] = 0.f;
     p.poly_on = 0;
-    p.map_x = p.map_y = p.map_z = p.map_out = 0;
-    p.omap = nullptr;
+    p.map_x = p.map_out = 0;
+    p.xmap_out = nullptr, p.omap = nullptr;
+    p.xo_b = p.xo_h = p.xo_n = 0;
     p.ms_b = p.ms_h = p.ms_n = 0;
     p.vec_x = vec_ok(x, dc), p.vec_y = vec_ok(y, dc), p.vec_z = vec_ok(z, dout), p.vec_out = vec_ok(out, dout);
     return p;
@@ -220,6 +221,63 @@ int64_t chunked_bytes(int64_t B, int64_t H, int64_t N, int64_t dc, int64_t dout)
     return B * H * chunks * padded(dc) * padded(dout) * 6;
 }
 
+// ---- element-wise feature passes, for the shapes and layouts the kernels' own map-on-load does
+// not cover: mode 1 writes dst = phi(src); mode 2 multiplies dst in place by phi'(x) computed from
+// src = phi(x).  Any strides; eight elements per thread where both tensors allow 16-byte accesses.
+template <typename T, bool VEC>
+__global__ __launch_bounds__(256) void feature_pass_kernel(int mode, int fmap, const T *src, int64_t ss_b, int64_t ss_h,
+                                                           int64_t ss_n, T *dst, int64_t ds_b, int64_t ds_h,
+                                                           int64_t ds_n, int H, int64_t N, int D, int64_t total) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= total) return;
+    constexpr int E = VEC ? 8 : 1;
+    const int per_row = D / E;
+    const int64_t row = t / per_row;
+    const int col = (int)(t - row * per_row) * E;
+    const int64_t bh = row / N, n = row - bh * N;
+    const int64_t b = bh / H, h = bh - b * H;
+    const T *sp = src + b * ss_b + h * ss_h + n * ss_n + col;
+    T *dp = dst + b * ds_b + h * ds_h + n * ds_n + col;
+    if constexpr (VEC) {
+        typedef T v8 __attribute__((ext_vector_type(8)));
+        v8 s = *reinterpret_cast<const v8 *>(sp), d;
+        if (mode == 2) d = *reinterpret_cast<const v8 *>(dp);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            const float x = static_cast<float>(s[e]);
+            d[e] = static_cast<T>(mode == 1 ? fla::feature_value(fmap, x)
+                                            : static_cast<float>(d[e]) * fla::feature_slope_from_value(fmap, x));
+        }
+        *reinterpret_cast<v8 *>(dp) = d;
+    } else {
+        const float x = static_cast<float>(*sp);
+        *dp = static_cast<T>(mode == 1 ? fla::feature_value(fmap, x)
+                                       : static_cast<float>(*dp) * fla::feature_slope_from_value(fmap, x));
+    }
+}
+
+int launch_feature_pass(int mode, int fmap, const View &src, const View &dst, int64_t B, int64_t H, int64_t N,
+                        int64_t D, int dtype, void *stream) {
+    if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    const bool vec = vec_ok(src, D) && vec_ok(dst, D);
+    const int64_t total = B * H * N * (vec ? D / 8 : D);
+    const int64_t grid = (total + 255) / 256;
+    if (grid > 0x7fffffffLL) return FLA_ERR_SHAPE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t e;
+#define FLA_FEATURE_PASS(T, V)                                                                                      \
+    fla::launch_kernel(feature_pass_kernel<T, V>, dim3((unsigned)grid), dim3(256), 0, s, mode, fmap,                \
+                       static_cast<const T *>(src.ptr), src.strides[0], src.strides[1], src.strides[2],            \
+                       static_cast<T *>(const_cast<void *>(dst.ptr)), dst.strides[0], dst.strides[1], dst.strides[2], \
+                       (int)H, N, (int)D, total)
+    if (dtype == FLA_DTYPE_BF16)
+        e = vec ? FLA_FEATURE_PASS(__bf16, true) : FLA_FEATURE_PASS(__bf16, false);
+    else
+        e = vec ? FLA_FEATURE_PASS(_Float16, true) : FLA_FEATURE_PASS(_Float16, false);
+#undef FLA_FEATURE_PASS
+    return e == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+}
+
 // ---- chunk-wise evaluation, in three steps per product:
 //   chunk_states: per-chunk Y_c^T Z_c in fp32, then the exclusive running sum over the chunks
 //                 before (lower) / after (upper) each chunk, rounded to the storage dtype;
@@ -233,7 +291,7 @@ bool chunkable(const TriParams &p, int64_t dc, int64_t dout, int64_t N) {
 }
 
 int chunk_states(const View &y, const View &z, int64_t B, int64_t H, int64_t N, int64_t dc, int64_t dout, int upper,
-                 int dtype, float *w, void *state, void *stream, int map_y = 0, int map_z = 0) {
+                 int dtype, float *w, void *state, void *stream, int map_y = 0, const View *ymap_out = nullptr) {
     const int64_t rows = chunk_rows(dc, dout), chunks = (N + rows - 1) / rows, E = padded(dc) * padded(dout);
     hipStream_t s = static_cast<hipStream_t>(stream);
     fla::ChunkStateParams cp;
@@ -242,7 +300,12 @@ int chunk_states(const View &y, const View &z, int64_t B, int64_t H, int64_t N, 
     cp.zs_b = z.strides[0], cp.zs_h = z.strides[1], cp.zs_n = z.strides[2];
     cp.H = (int32_t)H, cp.N = (int32_t)N, cp.BH = (int32_t)(B * H), cp.dc = (int32_t)dc, cp.dout = (int32_t)dout;
     cp.n_chunks = (int32_t)chunks;
-    cp.map_y = map_y, cp.map_z = map_z;
+    cp.map_y = map_y, cp.ymap_out = nullptr;
+    cp.yo_b = cp.yo_h = cp.yo_n = 0;
+    if (map_y) {
+        cp.ymap_out = const_cast<void *>(ymap_out->ptr);
+        cp.yo_b = ymap_out->strides[0], cp.yo_h = ymap_out->strides[1], cp.yo_n = ymap_out->strides[2];
+    }
     if (lookup_state(dtype, dc, dout)(cp, s) != hipSuccess) return FLA_ERR_LAUNCH;
     const hipError_t e = dtype == FLA_DTYPE_BF16
                              ? fla::launch_chunk_scan<__bf16>(w, state, B * H, (int)chunks, E, upper ? 1 : 0, s)
@@ -257,20 +320,10 @@ int chunk_main(TriParams p, int64_t dc, int64_t dout, int dtype, const void *sta
     return e == hipSuccess ? FLA_OK : e == hipErrorNotSupported ? FLA_ERR_UNSUPPORTED : FLA_ERR_LAUNCH;
 }
 
-// Feature maps of one product (fla_feature.h): phi on the operands as they are loaded, and the
-// output multiplied by phi'(omap).  Only the chunk-wise fast-path kernels implement them.
-struct Maps {
-    int x = 0, y = 0, z = 0, out = 0;
-    View omap{nullptr, nullptr};
-    bool any() const { return x || y || z || omap.ptr; }
-};
-
-void set_maps(TriParams &p, const Maps &m) {
-    p.map_x = m.x, p.map_y = m.y, p.map_z = m.z;
-    if (m.omap.ptr) {
-        p.map_out = m.out, p.omap = m.omap.ptr;
-        p.ms_b = m.omap.strides[0], p.ms_h = m.omap.strides[1], p.ms_n = m.omap.strides[2];
-    }
+// Out *= phi'(x) from y = phi(x) held in `y` (Out's shape): the chain rule in the kernel's epilogue
+void set_output_slope(TriParams &p, int fmap, const View &y) {
+    p.map_out = fmap, p.omap = y.ptr;
+    p.ms_b = y.strides[0], p.ms_h = y.strides[1], p.ms_n = y.strides[2];
 }
 
 // Out = mask(X Y^T) Z evaluated chunk-wise; same arguments as run_tri plus the workspace.
@@ -278,35 +331,25 @@ void set_maps(TriParams &p, const Maps &m) {
 // or the sequence is a single chunk.
 int run_tri_chunked(const View &x, const View &y, const View &z, const View &out, int64_t B, int64_t H, int64_t N,
                     int64_t dc, int64_t dout, int upper, int dtype, void *workspace, int64_t workspace_bytes,
-                    void *stream, const Maps &maps = Maps{}) {
+                    void *stream) {
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
     if (dout > 128 && (dc <= 64 || dc > 128)) {
         const View z_hi{static_cast<const char *>(z.ptr) + 128 * 2, z.strides};
         const View out_hi{static_cast<const char *>(out.ptr) + 128 * 2, out.strides};
-        Maps maps_hi = maps;
-        if (maps.omap.ptr) maps_hi.omap.ptr = static_cast<const char *>(maps.omap.ptr) + 128 * 2;
-        if (int rc = run_tri_chunked(x, y, z, out, B, H, N, dc, 128, upper, dtype, workspace, workspace_bytes, stream,
-                                     maps))
+        if (int rc = run_tri_chunked(x, y, z, out, B, H, N, dc, 128, upper, dtype, workspace, workspace_bytes, stream))
             return rc;
         return run_tri_chunked(x, y, z_hi, out_hi, B, H, N, dc, dout - 128, upper, dtype, workspace, workspace_bytes,
-                               stream, maps_hi);
+                               stream);
     }
-    TriParams p = make_params(x, y, z, out, B, H, N, dc, dout, upper);
-    set_maps(p, maps);
-    if (!chunkable(p, dc, dout, N)) {
-        if (!maps.any()) return run_tri(x, y, z, out, B, H, N, dc, dout, upper, dtype, stream);
-        // feature maps exist in the chunk-wise kernel only: a sequence of a single chunk runs it
-        // without a state (the pointer merely selects the kernel; a single chunk never reads it)
-        if (chunk_rows(dc, dout) == 0 || N > chunk_rows(dc, dout) || !fla::fast_path_ok(p)) return FLA_ERR_UNSUPPORTED;
-        return chunk_main(p, dc, dout, dtype, p.x, 0, stream);
-    }
+    const TriParams p = make_params(x, y, z, out, B, H, N, dc, dout, upper);
+    if (!chunkable(p, dc, dout, N)) return run_tri(x, y, z, out, B, H, N, dc, dout, upper, dtype, stream);
     const int64_t rows = chunk_rows(dc, dout), chunks = (N + rows - 1) / rows, E = padded(dc) * padded(dout);
     const int64_t BH = B * H;
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < BH * chunks * E * 6)
         return FLA_ERR_WORKSPACE;
     float *w = static_cast<float *>(workspace);
     void *state = static_cast<char *>(workspace) + BH * chunks * E * 4;
-    if (int rc = chunk_states(y, z, B, H, N, dc, dout, upper, dtype, w, state, stream, maps.y, maps.z)) return rc;
+    if (int rc = chunk_states(y, z, B, H, N, dc, dout, upper, dtype, w, state, stream)) return rc;
     return chunk_main(p, dc, dout, dtype, state, 0, stream);
 }
 
@@ -338,22 +381,29 @@ int64_t chunked_op_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk,
     return m > t ? m : t;
 }
 
-// fmap != 0: q and k are the arguments of the feature map phi, applied as they are loaded
+// fmap != 0 (feature_forward below): q and k hold the arguments xq, xk of the feature map phi, and
+// `mapped` = {phi(xq), phi(xk)} are outputs: the state kernel maps xk as it loads it and writes
+// phi(xk), which the main kernel then reads as its Y operand; the main kernel maps its X rows xq
+// and writes phi(xq).  Only the shared-state fast path does this; *mapped_done says whether it ran.
 int chunked_forward(const View &q, const View &k, const View &v, const View &o, int64_t B, int64_t H, int64_t N,
                     int64_t dqk, int64_t dv, int dtype, void *state_out, int32_t *state_valid, void *workspace,
-                    int64_t workspace_bytes, void *stream, int fmap = 0) {
+                    int64_t workspace_bytes, void *stream, int fmap = 0, const View *mapped = nullptr,
+                    bool *mapped_done = nullptr) {
     if (state_valid) *state_valid = 0;
     const View all[] = {q, k, v, o};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
     if (int rc = check_alias_fwd(q, k, v, o, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
-    TriParams p = make_params(q, k, v, o, B, H, N, dqk, dv, 0);
-    p.map_x = p.map_y = fmap;
-    if (!states_shareable(dqk, dv, N) || !fla::fast_path_ok(p)) {
-        Maps m;
-        m.x = m.y = fmap;
-        return run_tri_chunked(q, k, v, o, B, H, N, dqk, dv, 0, dtype, workspace, workspace_bytes, stream, m);
+    TriParams p = make_params(q, fmap ? mapped[1] : k, v, o, B, H, N, dqk, dv, 0);
+    const bool k_fast = !fmap || fla::fast_path_ok(make_params(q, k, v, o, B, H, N, dqk, dv, 0));  // xk under the state kernel's loads
+    if (!states_shareable(dqk, dv, N) || !fla::fast_path_ok(p) || !k_fast) {
+        if (fmap) return FLA_OK;  // *mapped_done stays false: the caller maps with a pass of its own
+        return run_tri_chunked(q, k, v, o, B, H, N, dqk, dv, 0, dtype, workspace, workspace_bytes, stream);
+    }
+    if (fmap) {
+        p.map_x = fmap, p.xmap_out = const_cast<void *>(mapped[0].ptr);
+        p.xo_b = mapped[0].strides[0], p.xo_h = mapped[0].strides[1], p.xo_n = mapped[0].strides[2];
     }
     const int64_t sb = shared_state_bytes(B, H, N, dqk, dv);
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < sb * (state_out ? 2 : 3))
@@ -361,8 +411,10 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
     if (state_out && reinterpret_cast<uintptr_t>(state_out) % 16 != 0) return FLA_ERR_WORKSPACE;
     float *w = static_cast<float *>(workspace);
     void *state = state_out ? state_out : static_cast<char *>(workspace) + 2 * sb;
-    if (int rc = chunk_states(k, v, B, H, N, dqk, dv, 0, dtype, w, state, stream, fmap, 0)) return rc;
+    if (int rc = chunk_states(k, v, B, H, N, dqk, dv, 0, dtype, w, state, stream, fmap, fmap ? &mapped[1] : nullptr))
+        return rc;
     if (int rc = chunk_main(p, dqk, dv, dtype, state, 0, stream)) return rc;
+    if (mapped_done) *mapped_done = true;
     if (state_out && state_valid) *state_valid = 1;
     return FLA_OK;
 }
@@ -375,25 +427,24 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         if (int rc = check_view(t)) return rc;
     if (int rc = check_alias_bwd(go, q, k, v, nullptr, dq, dk, dvv, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
-    // With a feature map q and k are its arguments: K and Q are mapped wherever they are loaded, and
-    // the gradients with respect to phi(xq), phi(xk) leave multiplied by phi'(xq), phi'(xk).
-    Maps mq, mv, mk;
-    if (fmap) {
-        mq.z = fmap, mq.out = fmap, mq.omap = q;  // dXq = (lower(dO V^T) phi(Xk)) . phi'(Xq)
-        mv.x = mv.y = fmap;                       // dV  = upper(phi(Xk) phi(Xq)^T) dO
-        mk.z = fmap, mk.out = fmap, mk.omap = k;  // dXk = (upper(V dO^T) phi(Xq)) . phi'(Xk)
-    }
+    // fmap != 0: q and k hold y = phi(x) (what the forward pass wrote), and the gradients leave as
+    // gradients with respect to x: dQ and dK are multiplied by phi'(x), computed from y -- in the
+    // kernels' epilogue on the fast path, by a pass of its own after the products otherwise.
     TriParams pq = make_params(go, v, k, dq, B, H, N, dv, dqk, 0);   // dQ = lower(dO V^T) K
     TriParams pv = make_params(k, q, go, dvv, B, H, N, dqk, dv, 1);  // dV = upper(K Q^T) dO
     TriParams pk = make_params(v, go, q, dk, B, H, N, dv, dqk, 1);   // dK = upper(V dO^T) Q
-    set_maps(pq, mq), set_maps(pv, mv), set_maps(pk, mk);
     if (!states_shareable(dqk, dv, N) || !fla::fast_path_ok(pq) || !fla::fast_path_ok(pv) || !fla::fast_path_ok(pk)) {
-        if (int rc = run_tri_chunked(go, v, k, dq, B, H, N, dv, dqk, 0, dtype, workspace, workspace_bytes, stream, mq))
+        if (int rc = run_tri_chunked(go, v, k, dq, B, H, N, dv, dqk, 0, dtype, workspace, workspace_bytes, stream))
             return rc;
-        if (int rc = run_tri_chunked(k, q, go, dvv, B, H, N, dqk, dv, 1, dtype, workspace, workspace_bytes, stream, mv))
+        if (int rc = run_tri_chunked(k, q, go, dvv, B, H, N, dqk, dv, 1, dtype, workspace, workspace_bytes, stream))
             return rc;
-        return run_tri_chunked(v, go, q, dk, B, H, N, dv, dqk, 1, dtype, workspace, workspace_bytes, stream, mk);
+        if (int rc = run_tri_chunked(v, go, q, dk, B, H, N, dv, dqk, 1, dtype, workspace, workspace_bytes, stream))
+            return rc;
+        if (!fmap) return FLA_OK;
+        if (int rc = launch_feature_pass(2, fmap, q, dq, B, H, N, dqk, dtype, stream)) return rc;
+        return launch_feature_pass(2, fmap, k, dk, B, H, N, dqk, dtype, stream);
     }
+    if (fmap) set_output_slope(pq, fmap, q), set_output_slope(pk, fmap, k);
     const int64_t sb = shared_state_bytes(B, H, N, dqk, dv);
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < sb * (state_in ? 3 : 4))
         return FLA_ERR_WORKSPACE;
@@ -402,10 +453,10 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
     const void *state_f = state_in;
     if (!state_f) {
         void *mine = static_cast<char *>(workspace) + 3 * sb;
-        if (int rc = chunk_states(k, v, B, H, N, dqk, dv, 0, dtype, w, mine, stream, fmap, 0)) return rc;
+        if (int rc = chunk_states(k, v, B, H, N, dqk, dv, 0, dtype, w, mine, stream)) return rc;
         state_f = mine;
     }
-    if (int rc = chunk_states(q, go, B, H, N, dqk, dv, 1, dtype, w, state_v, stream, fmap, 0)) return rc;
+    if (int rc = chunk_states(q, go, B, H, N, dqk, dv, 1, dtype, w, state_v, stream)) return rc;
     // One launch for the three products: a workgroup evaluates dQ, dV and dK of its chunk in turn,
     // so q, k, v and dO come from memory once.  dQ reads the forward state [D_v][D_qk] as its own
     // [D_c = D_v][D_o = D_qk] transposed state; dK reads the state of dV transposed.
@@ -909,17 +960,37 @@ int fla_linear_attn_chunked_fwd_static(const void *q, const void *k, const void 
                            nullptr, nullptr, ws, FLA_STATIC_SCRATCH_BYTES, stream);
 }
 
-int fla_feature_attn_fwd(const void *xq, const void *xk, const void *v, void *o, int64_t B, int64_t H, int64_t N,
-                         int64_t D_qk, int64_t D_v, const int64_t *xq_strides, const int64_t *xk_strides,
-                         const int64_t *v_strides, const int64_t *o_strides, int feature_map, int dtype,
+int fla_feature_attn_fwd(const void *xq, const void *xk, const void *v, void *o, void *q_out, void *k_out, int64_t B,
+                         int64_t H, int64_t N, int64_t D_qk, int64_t D_v, const int64_t *xq_strides,
+                         const int64_t *xk_strides, const int64_t *v_strides, const int64_t *o_strides,
+                         const int64_t *q_out_strides, const int64_t *k_out_strides, int feature_map, int dtype,
                          void *state_out, int32_t *state_valid, void *workspace, int64_t workspace_bytes, void *stream) {
     if (state_valid) *state_valid = 0;
     if (int rc = check_common(B, H, N, dtype)) return rc;
     if (D_qk < 1 || D_qk > 256) return FLA_ERR_HEAD_DIM;
     if (D_v < 1 || D_v > 256) return FLA_ERR_V_HEAD_DIM;
     if (feature_map != FLA_MAP_ELU1 && feature_map != FLA_MAP_SOFTPLUS) return FLA_ERR_UNSUPPORTED;
-    return chunked_forward({xq, xq_strides}, {xk, xk_strides}, {v, v_strides}, {o, o_strides}, B, H, N, D_qk, D_v,
-                           dtype, state_out, state_valid, workspace, workspace_bytes, stream, feature_map);
+    const View vxq{xq, xq_strides}, vxk{xk, xk_strides}, vv{v, v_strides}, vo{o, o_strides};
+    const View mapped[2] = {{q_out, q_out_strides}, {k_out, k_out_strides}};
+    const View all[] = {vxq, vxk, vv, vo, mapped[0], mapped[1]};
+    for (const View &t : all)
+        if (int rc = check_view(t)) return rc;
+    {
+        const Span ins[] = {span_of(vxq, B, H, N, D_qk), span_of(vxk, B, H, N, D_qk), span_of(vv, B, H, N, D_v)};
+        const Span outs[] = {span_of(vo, B, H, N, D_v), span_of(mapped[0], B, H, N, D_qk), span_of(mapped[1], B, H, N, D_qk)};
+        if (int rc = check_alias(ins, 3, outs, 3)) return rc;
+    }
+    // the kernels map on load where they can: the state kernel xk, the main kernel its rows of xq
+    bool done = false;
+    if (int rc = chunked_forward(vxq, vxk, vv, vo, B, H, N, D_qk, D_v, dtype, state_out, state_valid, workspace,
+                                 workspace_bytes, stream, feature_map, mapped, &done))
+        return rc;
+    if (done) return FLA_OK;
+    // any other shape or layout: one element-wise pass per operand, then the operator on phi(xq), phi(xk)
+    if (int rc = launch_feature_pass(1, feature_map, vxq, mapped[0], B, H, N, D_qk, dtype, stream)) return rc;
+    if (int rc = launch_feature_pass(1, feature_map, vxk, mapped[1], B, H, N, D_qk, dtype, stream)) return rc;
+    return chunked_forward(mapped[0], mapped[1], vv, vo, B, H, N, D_qk, D_v, dtype, state_out, state_valid, workspace,
+                           workspace_bytes, stream);
 }
 
 int fla_feature_attn_bwd(const void *grad_out, const void *xq, const void *xk, const void *v, void *dxq, void *dxk,
@@ -928,6 +999,7 @@ int fla_feature_attn_bwd(const void *grad_out, const void *xq, const void *xk, c
                          const int64_t *v_strides, const int64_t *dxq_strides, const int64_t *dxk_strides,
                          const int64_t *dv_strides, int feature_map, int dtype, const void *state_in, void *workspace,
                          int64_t workspace_bytes, void *stream) {
+    // (xq, xk name the forward's q_out, k_out here: phi(xq), phi(xk))
     if (int rc = check_common(B, H, N, dtype)) return rc;
     if (D_qk < 1 || D_qk > 256) return FLA_ERR_HEAD_DIM;
     if (D_v < 1 || D_v > 256) return FLA_ERR_V_HEAD_DIM;

@@ -32,7 +32,12 @@ struct ChunkStateParams {
     int32_t H, N, BH;
     int32_t dc, dout;
     int32_t n_chunks;
-    int32_t map_y, map_z;  // feature map applied to Y / Z as the tiles arrive (fla_feature.h), 0: none
+    // Feature map on load (fla_feature.h): map_y != 0 replaces every element of Y by phi(element) as
+    // the tiles arrive, and writes the mapped rows to `ymap_out` (Y's shape, element strides yo_*) so
+    // that the passes after this one read phi(y) instead of mapping again.
+    int32_t map_y;
+    void *ymap_out;
+    int64_t yo_b, yo_h, yo_n;
 };
 
 // LDS footprint of the state kernel: at most half of the CU's 160 KiB, so that two workgroups fit
@@ -125,25 +130,26 @@ __global__ __launch_bounds__(256) void chunk_state_kernel(const ChunkStateParams
         });
         wait_vm<0>();
         __builtin_amdgcn_s_barrier();
-        if (p.map_y | p.map_z) {
-            // feature map on load: rewrite the landed tiles in place; zero padding stays zero
-            auto map_tiles = [&](int map, int region, int row_bytes, int cpr, int width, auto swz) {
-#pragma unroll 1
-                for (int t = 0; t < RT; ++t) {
-                    unsigned char *tile = smem + t * STAGE + region;
-                    const int row0 = r0 + (R * RT + t) * BN;
-#pragma unroll 1
-                    for (int u = tid; u < BN * cpr; u += 256) {
-                        const int r = u / cpr, c = (u - r * cpr) ^ swz(r);
-                        if (row0 + r < N && c * 8 < width) {
-                            u32x4 *ptr = reinterpret_cast<u32x4 *>(tile + r * row_bytes + ((u - r * cpr) << 4));
-                            *ptr = feature_map8<T>(map, *ptr);
-                        }
+        if (p.map_y) {
+            // Feature map on load: every thread rewrites its share of the landed Y tiles in place
+            // (16 bytes at a time; rows beyond the sequence and chunks beyond the true width arrived
+            // as zeros and stay zeros) and stores the mapped values to ymap_out.
+            T *YO = static_cast<T *>(p.ymap_out) + b * p.yo_b + h * p.yo_h;
+#pragma unroll
+            for (int t = 0; t < RT; ++t) {
+                unsigned char *tile = smem + t * STAGE;
+                const int row0 = r0 + (R * RT + t) * BN;
+#pragma unroll
+                for (int v = 0; v < BN * CY / 256; ++v) {
+                    const int u = tid + 256 * v, r = u / CY, pos = u % CY, c = pos ^ swizzle_y<CY>(r);
+                    if (row0 + r < N && c * 8 < p.dc) {
+                        u32x4 *ptr = reinterpret_cast<u32x4 *>(tile + r * RY + (pos << 4));
+                        const u32x4 m = feature_map8<T>(p.map_y, *ptr);
+                        *ptr = m;
+                        *reinterpret_cast<u32x4 *>(YO + (int64_t)(row0 + r) * p.yo_n + c * 8) = m;
                     }
                 }
-            };
-            if (p.map_y) map_tiles(p.map_y, 0, RY, CY, p.dc, [](int r) { return swizzle_y<CY>(r); });
-            if (p.map_z) map_tiles(p.map_z, Y_BYTES, RZ, CZ, p.dout, [](int r) { return swizzle_z<CZ>(r); });
+            }
             __syncthreads();
         }
     };

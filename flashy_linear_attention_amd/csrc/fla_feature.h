@@ -21,10 +21,12 @@ __device__ __forceinline__ float feature_value(int map, float x) {
     return x > 20.f ? x : (x < -10.f ? e : __logf(1.f + e));
 }
 
-// phi'(x) in fp32
-__device__ __forceinline__ float feature_slope(int map, float x) {
-    if (map == kMapElu1) return x > 0.f ? 1.f : __expf(x);
-    return 1.f / (1.f + __expf(-x));  // softplus' = sigmoid
+// phi'(x) in fp32, from y = phi(x) (the value the forward pass left in memory; x itself is not
+// needed again): elu(x) + 1 has slope 1 where y >= 1 and e^x = y below; softplus has slope
+// sigmoid(x) = e^x / (1 + e^x) = 1 - e^{-y}.
+__device__ __forceinline__ float feature_slope_from_value(int map, float y) {
+    if (map == kMapElu1) return y >= 1.f ? 1.f : y;
+    return 1.f - __expf(-y);
 }
 
 // phi on eight packed 16-bit values (one rounding to the storage type)

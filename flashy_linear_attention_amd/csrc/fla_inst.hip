@@ -21,7 +21,7 @@ hipError_t FLA_LAUNCH_NAME(FLA_INST_DTYPE, FLA_INST_DC, FLA_INST_DO)(const TriPa
     // stages) takes the bounds-checked generic kernel
     if (FastConfig<FLA_INST_DC, FLA_INST_DO>::kSupported && fast_path_ok(p))
         return launch_tri_fast<InstT, FLA_INST_DC, FLA_INST_DO>(p, stream);
-    if (p.map_x || p.map_y || p.map_z || p.omap) return hipErrorNotSupported;  // feature maps: fast path only
+    if (p.map_x || p.omap) return hipErrorNotSupported;  // feature maps: fast path only
     return launch_tri<InstT, FLA_INST_DC, FLA_INST_DO>(p, stream);
 }
 

@@ -515,13 +515,24 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         }
         wait_vm<0>();
         __builtin_amdgcn_s_barrier();
-        if (p.map_x) {  // X = phi(x): the fragments are in registers, columns beyond the true width stay zero
+        if (p.map_x) {
+            // X = phi(x): the fragments are in registers (a lane holds eight consecutive columns of
+            // one row per fragment); columns beyond the true width stay zero.  The mapped rows are
+            // written out once, for the passes that need phi(x) later.
+            T *XO = static_cast<T *>(p.xmap_out) + b * p.xo_b + h * p.xo_h;
 #pragma unroll
-            for (int ib = 0; ib < NIB; ++ib)
+            for (int ib = 0; ib < NIB; ++ib) {
+                const int row = i0 + blk[ib] * 32 + l32;
 #pragma unroll
-                for (int kc = 0; kc < KC; ++kc)
-                    if (kc * 16 + 8 * g < p.dc)
-                        xf[ib][kc] = __builtin_bit_cast(V8, feature_map8<T>(p.map_x, __builtin_bit_cast(u32x4, xf[ib][kc])));
+                for (int kc = 0; kc < KC; ++kc) {
+                    const int col = kc * 16 + 8 * g;
+                    if (col < p.dc) {
+                        const u32x4 m = feature_map8<T>(p.map_x, __builtin_bit_cast(u32x4, xf[ib][kc]));
+                        xf[ib][kc] = __builtin_bit_cast(V8, m);
+                        if (row < N) *reinterpret_cast<u32x4 *>(XO + (int64_t)row * p.xo_n + col) = m;
+                    }
+                }
+            }
         }
         pin_x();
         if constexpr (kLateTiles)
@@ -775,30 +786,6 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
         if constexpr (!chunked) issue_tile(q + Cfg::NBUF - 1, prev_off);  // the one tile not yet requested (if any)
         wait_vm<0>();
         __builtin_amdgcn_s_barrier();
-        if constexpr (chunked) {
-            // Feature map on load: the tiles of the diagonal block are all resident now and hold the
-            // raw operand; every thread rewrites its share of the 16-byte units in place.  Rows
-            // beyond the sequence and chunks beyond the true width arrived as zeros and stay zeros.
-            if (p.map_y | p.map_z) {
-                auto map_tiles = [&](int map, int region, int row_bytes, int cpr, int width, auto swz) {
-#pragma unroll 1
-                    for (int t = 0; t < n_diag; ++t) {
-                        unsigned char *tile = smem + t * STAGE + region;
-#pragma unroll 1
-                        for (int u = tid; u < BN * cpr; u += 256) {
-                            const int r = u / cpr, c = (u - r * cpr) ^ swz(r);
-                            if (i0 + t * BN + r < N && c * 8 < width) {
-                                u32x4 *ptr = reinterpret_cast<u32x4 *>(tile + r * row_bytes + ((u - r * cpr) << 4));
-                                *ptr = feature_map8<T>(map, *ptr);
-                            }
-                        }
-                    }
-                };
-                if (p.map_y) map_tiles(p.map_y, 0, RY, CY, p.dc, [](int r) { return swizzle_y<CY>(r); });
-                if (p.map_z) map_tiles(p.map_z, Y_BYTES, RZ, CZ, p.dout, [](int r) { return swizzle_z<CZ>(r); });
-                __syncthreads();
-            }
-        }
 
         const int nsub = (diag_rows + 31) >> 5;  // sub-tiles with at least one valid row
         int blk_min = blk[0], blk_max = blk[0];
@@ -910,8 +897,9 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
     }
     if constexpr (chunked) {
         if (p.omap) {
-            // Out is the gradient with respect to phi(x): multiply by phi'(x) for the gradient with
-            // respect to x.  A lane holds 16 consecutive columns of one row per (row block, column block).
+            // Out is the gradient with respect to y = phi(x): multiply by phi'(x), computed from y, for
+            // the gradient with respect to x.  A lane holds 16 consecutive columns of one row per
+            // (row block, column block).
             const T *M = static_cast<const T *>(p.omap) + b * p.ms_b + h * p.ms_h;
             const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(
                 const_cast<T *>(M), 0, (N - 1) * (int)p.ms_n * 2 + p.dout * 2, 0x00020000);
@@ -927,7 +915,7 @@ __device__ __forceinline__ void tri_fast_body(const TriParams &p, const int wg_i
                         const V8 mv = __builtin_bit_cast(V8, __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0));
 #pragma unroll
                         for (int e = 0; e < 8; ++e)
-                            acc[ib][db][8 * hq + e] *= feature_slope(p.map_out, static_cast<float>(mv[e]));
+                            acc[ib][db][8 * hq + e] *= feature_slope_from_value(p.map_out, static_cast<float>(mv[e]));
                     }
                 }
             }
@@ -1039,7 +1027,7 @@ template <typename T, int DC, int DO>
 hipError_t launch_tri_fast(const TriParams &p, hipStream_t stream) {
     if (p.state)
         return (p.denom || p.poly_on) ? hipErrorNotSupported : launch_tri_fast_variant<T, DC, DO, true, 0>(p, stream);
-    if (p.map_x || p.map_y || p.map_z || p.omap) return hipErrorNotSupported;  // chunk-wise kernel only
+    if (p.map_x || p.omap) return hipErrorNotSupported;  // chunk-wise kernel only
     if (p.poly_on == 2) {  // dual-score walk: built for 32-wide outputs (the argument of the score map)
         if constexpr (DC >= 64 && DO == 32) {
             return p.denom ? hipErrorNotSupported : launch_tri_fast_variant<T, DC, DO, false, kDualFlag>(p, stream);

@@ -73,12 +73,16 @@ struct TriParams {
     // last 32 columns, [DC - 32, DC).
     float poly[3];
     int32_t poly_on;
-    // Feature map on load (chunk-wise fast path only; fla_feature.h): a non-zero map_x / map_y /
-    // map_z replaces every element of that operand by phi(element) as it arrives (zero padding
-    // stays zero).  `omap`, when non-null, is a tensor of Out's shape (element strides ms_*): each
-    // output element is multiplied by phi'(omap element), map_out naming phi -- the chain rule of
-    // a gradient with respect to the argument of phi.
-    int32_t map_x, map_y, map_z, map_out;
+    // Feature map on load (chunk-wise fast path only; fla_feature.h).  map_x != 0: X holds the
+    // argument x of the feature map phi; every element is replaced by phi(x) as the rows arrive
+    // (columns beyond the true width stay zero), and the mapped rows are also written to
+    // `xmap_out` (X's shape, element strides xo_*) for later passes.  `omap`, when non-null, is a
+    // tensor of Out's shape (element strides ms_*) holding y = phi(x): each output element is
+    // multiplied by phi'(x) computed from y, map_out naming phi -- the chain rule of a gradient with
+    // respect to the argument of phi.
+    int32_t map_x, map_out;
+    void *xmap_out;
+    int64_t xo_b, xo_h, xo_n;
     const void *omap;
     int64_t ms_b, ms_h, ms_n;
 };

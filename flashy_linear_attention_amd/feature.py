@@ -5,9 +5,11 @@ flashlinear/test_attn.py:36-40 of the reference):
     FeatureMapLinearAttention.apply(xq, xk, v, "elu1")   ==   LinearAttention.apply(elu(xq) + 1, elu(xk) + 1, v)
 
 with ``"softplus"`` as the other map.  The product is evaluated chunk-wise
-(``LinearAttentionChunked``'s method) and the map is applied while the kernels load xq and xk,
-so phi(xq), phi(xk) are never written to memory and backward returns the gradients with respect
-to xq and xk themselves (``fla_feature_attn_fwd`` / ``fla_feature_attn_bwd``).
+(``LinearAttentionChunked``'s method) and the map is applied while the kernels load xq and xk:
+no pass over memory exists for the map alone.  The kernels leave phi(xq), phi(xk) behind as a
+by-product; autograd keeps those instead of xq, xk, and backward returns the gradients with
+respect to xq and xk themselves, the slope of phi multiplied in before the gradients are stored
+(``fla_feature_attn_fwd`` / ``fla_feature_attn_bwd``).
 """
 
 from __future__ import annotations
@@ -33,8 +35,9 @@ def _map_code(feature: str) -> int:
 
 def feature_attention_fwd(xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, feature: str = "elu1",
                           want_state: bool = False):
-    """``O = tril(phi(xq) phi(xk)^T) v``.  With ``want_state`` returns ``(O, state)``, the running
-    state for :func:`feature_attention_bwd` (None when the shape does not allow sharing it)."""
+    """``(O, q, k)`` with ``O = tril(q k^T) v``, ``q = phi(xq)``, ``k = phi(xk)``.  With ``want_state``
+    returns ``(O, q, k, state)``, ``state`` being the running state for :func:`feature_attention_bwd`
+    (None when the shape does not allow sharing it)."""
     assert xq.shape == xk.shape and v.shape[:3] == xq.shape[:3], "xq, xk: (B,H,N,D_qk); v: (B,H,N,D_v)"
     assert xq.shape[-1] <= 256 and v.shape[-1] <= 256, "Only head_dims <= 256 are supported."
     code = _map_code(feature)
@@ -42,6 +45,8 @@ def feature_attention_fwd(xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, f
     b, h, n, dqk = xq.shape
     dv = v.shape[-1]
     out = torch.empty_like(v, memory_format=torch.contiguous_format)
+    q = torch.empty_like(xq, memory_format=torch.contiguous_format)
+    k = torch.empty_like(xk, memory_format=torch.contiguous_format)
     lib = _lib.load()
     with torch.cuda.device(xq.device):
         sbytes = lib.fla_linear_attn_chunked_state_bytes(b, h, n, dqk, dv) if want_state else 0
@@ -52,23 +57,25 @@ def feature_attention_fwd(xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, f
         _lib.check(
             "fla_feature_attn_fwd",
             lib.fla_feature_attn_fwd(
-                xq.data_ptr(), xk.data_ptr(), v.data_ptr(), out.data_ptr(), b, h, n, dqk, dv,
+                xq.data_ptr(), xk.data_ptr(), v.data_ptr(), out.data_ptr(), q.data_ptr(), k.data_ptr(),
+                b, h, n, dqk, dv,
                 _lib.strides_arg(xq), _lib.strides_arg(xk), _lib.strides_arg(v), _lib.strides_arg(out),
+                _lib.strides_arg(q), _lib.strides_arg(k),
                 code, dtype_code(xq), state.data_ptr() if state is not None else None, ctypes.byref(valid),
                 work.data_ptr(), wbytes, stream_handle(xq.device),
             ),
         )
     if want_state:
-        return out, (state if valid.value else None)
-    return out
+        return out, q, k, (state if valid.value else None)
+    return out, q, k
 
 
-def feature_attention_bwd(grad_output: torch.Tensor, xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor,
+def feature_attention_bwd(grad_output: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                           feature: str = "elu1", state: Optional[torch.Tensor] = None,
                           ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """(dxq, dxk, dv); ``state`` is what the forward call returned (or None)."""
+    """(dxq, dxk, dv) from the forward call's ``q = phi(xq)``, ``k = phi(xk)`` and ``state`` (or None)."""
     code = _map_code(feature)
-    grad_output, xq, xk, v = prepare(grad_output, xq, xk, v)
+    grad_output, xq, xk, v = prepare(grad_output, q, k, v)
     b, h, n, dqk = xq.shape
     dv = v.shape[-1]
     dxq = torch.empty_like(xq, memory_format=torch.contiguous_format)
@@ -99,23 +106,23 @@ class FeatureMapLinearAttention(Function):
     @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.bfloat16)
     def forward(ctx: Any, xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, feature: str = "elu1") -> torch.Tensor:
         if any(ctx.needs_input_grad[:3]):
-            out, state = feature_attention_fwd(xq, xk, v, feature, want_state=True)
+            out, q, k, state = feature_attention_fwd(xq, xk, v, feature, want_state=True)
         else:
-            out, state = feature_attention_fwd(xq, xk, v, feature), None
+            (out, q, k), state = feature_attention_fwd(xq, xk, v, feature), None
         ctx.feature = feature
         ctx.has_state = state is not None
         if state is not None:
-            ctx.save_for_backward(xq, xk, v, state)
+            ctx.save_for_backward(q, k, v, state)
         else:
-            ctx.save_for_backward(xq, xk, v)
+            ctx.save_for_backward(q, k, v)
         return out
 
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx: Any, grad_output: torch.Tensor):
         if ctx.has_state:
-            xq, xk, v, state = ctx.saved_tensors
+            q, k, v, state = ctx.saved_tensors
         else:
-            (xq, xk, v), state = ctx.saved_tensors, None
-        dxq, dxk, dv = feature_attention_bwd(grad_output, xq, xk, v, ctx.feature, state)
+            (q, k, v), state = ctx.saved_tensors, None
+        dxq, dxk, dv = feature_attention_bwd(grad_output, q, k, v, ctx.feature, state)
         return dxq, dxk, dv, None

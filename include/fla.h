@@ -178,31 +178,37 @@ int fla_linear_attn_chunked_bwd(const void *grad_out, const void *q, const void 
  *
  *     O = tril(phi(Xq) phi(Xk)^T) V,
  *
- * evaluated chunk-wise (fla_linear_attn_chunked_fwd/bwd's method) with phi applied as the
- * operands are loaded: phi(xq) and phi(xk) never exist in memory, neither in forward nor in
- * backward, and backward returns the gradients with respect to xq and xk directly,
- *     dXq = (tril(dO V^T) phi(Xk)) . phi'(Xq),    dXk = (tril(dO V^T)^T phi(Xq)) . phi'(Xk)
- * (the chain rule is applied to the accumulators before they are rounded and stored), plus dV.
+ * evaluated chunk-wise (fla_linear_attn_chunked_fwd/bwd's method) with phi applied while the
+ * kernels load xq and xk: the kernel that builds the chunk states maps xk as its tiles arrive,
+ * the main kernel maps its rows of xq, and each writes what it mapped to q_out = phi(xq),
+ * k_out = phi(xk) ((B, H, N, D_qk) in the storage dtype; every element is written) -- a
+ * by-product that replaces xq, xk as what backward needs, so no pass over memory exists for the
+ * map alone.  Backward takes q = q_out, k = k_out and returns the gradients with respect to xq
+ * and xk directly,
+ *     dXq = (tril(dO V^T) K) . phi'(Xq),    dXk = (tril(dO V^T)^T Q) . phi'(Xk),    dV,
+ * the slopes computed from q, k themselves (elu(x) + 1: 1 where y >= 1, else y; softplus:
+ * 1 - e^-y) and multiplied into the accumulators before they are rounded and stored.
  * feature_map: FLA_MAP_ELU1 (elu(x) + 1) or FLA_MAP_SOFTPLUS (log(1 + e^x), the map the
  * reference's tests put in front of its operators, flashlinear/test_attn.py:36-40); phi is
  * evaluated in fp32 and rounded once to the storage dtype.  state_out / state_valid / state_in,
- * workspace: exactly as for fla_linear_attn_chunked_fwd/bwd, same size queries.  Fast-path
- * operands only (16-byte aligned, widths and outer strides multiples of 8 elements), else
- * FLA_ERR_UNSUPPORTED.  No counterpart in the reference: its callers materialise phi(x) with a
- * PyTorch pass before the operator and differentiate through it with another
- * (README.md:27-30 of the reference). */
+ * workspace: exactly as for fla_linear_attn_chunked_fwd/bwd, same size queries.  Shapes and
+ * layouts outside the shared-state fast path (unequal padded head dims, a single chunk,
+ * unaligned operands) run an element-wise pass per operand instead, same results.  No
+ * counterpart in the reference: its callers materialise phi(x) with PyTorch passes before the
+ * operator and differentiate through them with more (README.md:27-30 of the reference). */
 enum fla_feature_map { FLA_MAP_NONE = 0, FLA_MAP_ELU1 = 1, FLA_MAP_SOFTPLUS = 2 };
-int fla_feature_attn_fwd(const void *xq, const void *xk, const void *v, void *o,
+int fla_feature_attn_fwd(const void *xq, const void *xk, const void *v, void *o, void *q_out, void *k_out,
                          int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
                          const int64_t *xq_strides, const int64_t *xk_strides,
                          const int64_t *v_strides, const int64_t *o_strides,
+                         const int64_t *q_out_strides, const int64_t *k_out_strides,
                          int feature_map, int dtype, void *state_out, int32_t *state_valid,
                          void *workspace, int64_t workspace_bytes, void *stream);
-int fla_feature_attn_bwd(const void *grad_out, const void *xq, const void *xk, const void *v,
+int fla_feature_attn_bwd(const void *grad_out, const void *q, const void *k, const void *v,
                          void *dxq, void *dxk, void *dv,
                          int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
-                         const int64_t *go_strides, const int64_t *xq_strides,
-                         const int64_t *xk_strides, const int64_t *v_strides,
+                         const int64_t *go_strides, const int64_t *q_strides,
+                         const int64_t *k_strides, const int64_t *v_strides,
                          const int64_t *dxq_strides, const int64_t *dxk_strides,
                          const int64_t *dv_strides,
                          int feature_map, int dtype, const void *state_in,
