@@ -41,6 +41,11 @@ SIGNATURES = {
                              + [ctypes.c_int, ctypes.c_int, _ptr, ctypes.POINTER(ctypes.c_int32), _ptr, _i64, _ptr], ctypes.c_int),
     "fla_feature_attn_bwd": ([_ptr] * 7 + [_i64] * 5 + [_strides] * 7 + [ctypes.c_int, ctypes.c_int, _ptr, _ptr, _i64, _ptr],
                              ctypes.c_int),
+    "fla_feature_attn_normalised_fwd": ([_ptr] * 7 + [_i64] * 5 + [_strides] * 6
+                                        + [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_int, _ptr, _i64, _ptr],
+                                        ctypes.c_int),
+    "fla_feature_attn_normalised_bwd": ([_ptr] * 9 + [_i64] * 5 + [_strides] * 8
+                                        + [ctypes.c_int, ctypes.c_int, ctypes.c_int, _ptr, _i64, _ptr], ctypes.c_int),
     "fla_linear_attn_chunked_fwd_static": ([_ptr] * 4 + [_i64] * 5 + [_strides] * 4 + [ctypes.c_int, _ptr], ctypes.c_int),
     "fla_linear_attn_chunked_bwd": ([_ptr] * 7 + [_i64] * 5 + [_strides] * 7 + [ctypes.c_int, _ptr, _ptr, _i64, _ptr],
                                     ctypes.c_int),

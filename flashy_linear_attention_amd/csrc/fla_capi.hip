@@ -468,6 +468,35 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
                                                                                                    : FLA_ERR_LAUNCH;
 }
 
+// O = tril(phi(xq) phi(xk)^T) v with mapped = {phi(xq), phi(xk)} as further outputs.  Chunk-wise
+// (chunked != 0): the kernels map on load where they can (the state kernel xk, the main kernel its
+// rows of xq); any other shape or layout, and the quadratic kernels, get one element-wise pass
+// per operand and then the plain operator on phi(xq), phi(xk).
+int feature_forward(const View &vxq, const View &vxk, const View &vv, const View &vo, const View (&mapped)[2], int64_t B,
+                    int64_t H, int64_t N, int64_t dqk, int64_t dv, int fmap, int dtype, int chunked, void *state_out,
+                    int32_t *state_valid, void *workspace, int64_t workspace_bytes, void *stream) {
+    const View all[] = {vxq, vxk, vv, vo, mapped[0], mapped[1]};
+    for (const View &t : all)
+        if (int rc = check_view(t)) return rc;
+    {
+        const Span ins[] = {span_of(vxq, B, H, N, dqk), span_of(vxk, B, H, N, dqk), span_of(vv, B, H, N, dv)};
+        const Span outs[] = {span_of(vo, B, H, N, dv), span_of(mapped[0], B, H, N, dqk), span_of(mapped[1], B, H, N, dqk)};
+        if (int rc = check_alias(ins, 3, outs, 3)) return rc;
+    }
+    if (chunked) {
+        bool done = false;
+        if (int rc = chunked_forward(vxq, vxk, vv, vo, B, H, N, dqk, dv, dtype, state_out, state_valid, workspace,
+                                     workspace_bytes, stream, fmap, mapped, &done))
+            return rc;
+        if (done) return FLA_OK;
+    }
+    if (int rc = launch_feature_pass(1, fmap, vxq, mapped[0], B, H, N, dqk, dtype, stream)) return rc;
+    if (int rc = launch_feature_pass(1, fmap, vxk, mapped[1], B, H, N, dqk, dtype, stream)) return rc;
+    if (!chunked) return run_tri(mapped[0], mapped[1], vv, vo, B, H, N, dqk, dv, 0, dtype, stream);
+    return chunked_forward(mapped[0], mapped[1], vv, vo, B, H, N, dqk, dv, dtype, state_out, state_valid, workspace,
+                           workspace_bytes, stream);
+}
+
 int forward(const View &q, const View &k, const View &v, const View &o, int64_t B, int64_t H, int64_t N,
             int64_t dqk, int64_t dv, int dtype, void *stream) {
     const View all[] = {q, k, v, o};
@@ -584,24 +613,41 @@ int fused_normalised_forward(const View &q, const View &k, const View &v, const 
     return lookup(dtype, dqk, dv - 128)(p1, static_cast<hipStream_t>(stream)) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
 }
 
-int normalised_forward(const View &q, const View &k, const View &v, const View &o, float *denom, int64_t B, int64_t H,
+// fmap != 0: q0, k0 hold the arguments xq, xk of the feature map and mapped = {phi(xq), phi(xk)} are
+// further outputs; the normaliser is that of phi(xq), phi(xk).
+int normalised_forward(const View &q0, const View &k0, const View &v, const View &o, float *denom, int64_t B, int64_t H,
                        int64_t N, int64_t dqk, int64_t dv, float eps, int dtype, int chunked, void *workspace,
-                       int64_t workspace_bytes, void *stream) {
-    const View all[] = {q, k, v, o};
+                       int64_t workspace_bytes, void *stream, int fmap = 0, const View *mapped = nullptr) {
+    const View all[] = {q0, k0, v, o};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
     if (!denom) return FLA_ERR_NULL_POINTER;
-    if (int rc = check_alias_fwd(q, k, v, o, B, H, N, dqk, dv)) return rc;
+    if (int rc = check_alias_fwd(q0, k0, v, o, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
     const NormLayout l = norm_layout(B, H, N, dqk, dv, chunked);
     if ((l.chunks > 1 || l.chunk_bytes > 0) &&
         (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < l.norm_bytes + l.chunk_bytes))
         return FLA_ERR_WORKSPACE;
+    if (fmap && !chunked) {
+        // quadratic product: phi by element-wise passes, then the operator on phi(xq), phi(xk)
+        for (int i = 0; i < 2; ++i)
+            if (int rc = check_view(mapped[i])) return rc;
+        if (int rc = launch_feature_pass(1, fmap, q0, mapped[0], B, H, N, dqk, dtype, stream)) return rc;
+        if (int rc = launch_feature_pass(1, fmap, k0, mapped[1], B, H, N, dqk, dtype, stream)) return rc;
+        return normalised_forward(mapped[0], mapped[1], v, o, denom, B, H, N, dqk, dv, eps, dtype, 0, workspace,
+                                  workspace_bytes, stream);
+    }
+    const View &q = fmap ? mapped[0] : q0, &k = fmap ? mapped[1] : k0;
     if (!chunked) {
         const int rc = fused_normalised_forward(q, k, v, o, denom, B, H, N, dqk, dv, eps, dtype, stream);
         if (rc <= 0) return rc;
     }
-    if (chunked) {
+    if (fmap) {
+        const View both[2] = {mapped[0], mapped[1]};
+        if (int rc = feature_forward(q0, k0, v, o, both, B, H, N, dqk, dv, fmap, dtype, 1, nullptr, nullptr,
+                                     static_cast<char *>(workspace) + l.norm_bytes, l.chunk_bytes, stream))
+            return rc;
+    } else if (chunked) {
         if (int rc = chunked_forward(q, k, v, o, B, H, N, dqk, dv, dtype, nullptr, nullptr,
                                      static_cast<char *>(workspace) + l.norm_bytes, l.chunk_bytes, stream))
             return rc;
@@ -622,7 +668,9 @@ int normalised_forward(const View &q, const View &k, const View &v, const View &
 int normalised_backward(const View &go, const View &q, const View &k, const View &v, const View &o,
                         const float *denom, const View &dq, const View &dk, const View &dvv, int64_t B, int64_t H,
                         int64_t N, int64_t dqk, int64_t dv, int dtype, int chunked, void *workspace,
-                        int64_t workspace_bytes, void *stream) {
+                        int64_t workspace_bytes, void *stream, int fmap = 0) {
+    // fmap != 0: q, k hold phi(xq), phi(xk) and dq, dk leave as gradients with respect to xq, xk (the
+    // slope is multiplied in by the last pass, after the normaliser's own terms have been added)
     const View all[] = {go, q, k, v, o, dq, dk, dvv};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
@@ -660,6 +708,7 @@ int normalised_backward(const View &go, const View &q, const View &k, const View
     p.dq = const_cast<void *>(dq.ptr), p.dqs_b = dq.strides[0], p.dqs_h = dq.strides[1], p.dqs_n = dq.strides[2];
     p.dk = const_cast<void *>(dk.ptr), p.dks_b = dk.strides[0], p.dks_h = dk.strides[1], p.dks_n = dk.strides[2];
     p.vec_dq = vec_ok(dq, dqk), p.vec_dk = vec_ok(dk, dqk);
+    p.fmap = fmap;
     return norm_launch(2, dtype, l.lpr, p, stream) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
 }
 
@@ -970,27 +1019,9 @@ int fla_feature_attn_fwd(const void *xq, const void *xk, const void *v, void *o,
     if (D_qk < 1 || D_qk > 256) return FLA_ERR_HEAD_DIM;
     if (D_v < 1 || D_v > 256) return FLA_ERR_V_HEAD_DIM;
     if (feature_map != FLA_MAP_ELU1 && feature_map != FLA_MAP_SOFTPLUS) return FLA_ERR_UNSUPPORTED;
-    const View vxq{xq, xq_strides}, vxk{xk, xk_strides}, vv{v, v_strides}, vo{o, o_strides};
     const View mapped[2] = {{q_out, q_out_strides}, {k_out, k_out_strides}};
-    const View all[] = {vxq, vxk, vv, vo, mapped[0], mapped[1]};
-    for (const View &t : all)
-        if (int rc = check_view(t)) return rc;
-    {
-        const Span ins[] = {span_of(vxq, B, H, N, D_qk), span_of(vxk, B, H, N, D_qk), span_of(vv, B, H, N, D_v)};
-        const Span outs[] = {span_of(vo, B, H, N, D_v), span_of(mapped[0], B, H, N, D_qk), span_of(mapped[1], B, H, N, D_qk)};
-        if (int rc = check_alias(ins, 3, outs, 3)) return rc;
-    }
-    // the kernels map on load where they can: the state kernel xk, the main kernel its rows of xq
-    bool done = false;
-    if (int rc = chunked_forward(vxq, vxk, vv, vo, B, H, N, D_qk, D_v, dtype, state_out, state_valid, workspace,
-                                 workspace_bytes, stream, feature_map, mapped, &done))
-        return rc;
-    if (done) return FLA_OK;
-    // any other shape or layout: one element-wise pass per operand, then the operator on phi(xq), phi(xk)
-    if (int rc = launch_feature_pass(1, feature_map, vxq, mapped[0], B, H, N, D_qk, dtype, stream)) return rc;
-    if (int rc = launch_feature_pass(1, feature_map, vxk, mapped[1], B, H, N, D_qk, dtype, stream)) return rc;
-    return chunked_forward(mapped[0], mapped[1], vv, vo, B, H, N, D_qk, D_v, dtype, state_out, state_valid, workspace,
-                           workspace_bytes, stream);
+    return feature_forward({xq, xq_strides}, {xk, xk_strides}, {v, v_strides}, {o, o_strides}, mapped, B, H, N, D_qk, D_v,
+                           feature_map, dtype, 1, state_out, state_valid, workspace, workspace_bytes, stream);
 }
 
 int fla_feature_attn_bwd(const void *grad_out, const void *xq, const void *xk, const void *v, void *dxq, void *dxk,
@@ -1021,6 +1052,33 @@ int fla_linear_attn_chunked_bwd(const void *grad_out, const void *q, const void 
     return chunked_backward({grad_out, go_strides}, {q, q_strides}, {k, k_strides}, {v, v_strides}, {dq, dq_strides},
                             {dk, dk_strides}, {dv, dv_strides}, B, H, N, D_qk, D_v, dtype, state_in, workspace,
                             workspace_bytes, stream);
+}
+
+int fla_feature_attn_normalised_fwd(const void *xq, const void *xk, const void *v, void *o, void *q_out, void *k_out,
+                                    float *denom, int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                                    const int64_t *xq_strides, const int64_t *xk_strides, const int64_t *v_strides,
+                                    const int64_t *o_strides, const int64_t *q_out_strides,
+                                    const int64_t *k_out_strides, int feature_map, float eps, int dtype, int chunked,
+                                    void *workspace, int64_t workspace_bytes, void *stream) {
+    if (int rc = check_norm_args(B, H, N, D_qk, D_v, dtype)) return rc;
+    if (feature_map != FLA_MAP_ELU1 && feature_map != FLA_MAP_SOFTPLUS) return FLA_ERR_UNSUPPORTED;
+    const View mapped[2] = {{q_out, q_out_strides}, {k_out, k_out_strides}};
+    return normalised_forward({xq, xq_strides}, {xk, xk_strides}, {v, v_strides}, {o, o_strides}, denom, B, H, N, D_qk,
+                              D_v, eps, dtype, chunked, workspace, workspace_bytes, stream, feature_map, mapped);
+}
+
+int fla_feature_attn_normalised_bwd(const void *grad_out, const void *q, const void *k, const void *v, const void *o,
+                                    const float *denom, void *dxq, void *dxk, void *dv, int64_t B, int64_t H,
+                                    int64_t N, int64_t D_qk, int64_t D_v, const int64_t *go_strides,
+                                    const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
+                                    const int64_t *o_strides, const int64_t *dxq_strides, const int64_t *dxk_strides,
+                                    const int64_t *dv_strides, int feature_map, int dtype, int chunked,
+                                    void *workspace, int64_t workspace_bytes, void *stream) {
+    if (int rc = check_norm_args(B, H, N, D_qk, D_v, dtype)) return rc;
+    if (feature_map != FLA_MAP_ELU1 && feature_map != FLA_MAP_SOFTPLUS) return FLA_ERR_UNSUPPORTED;
+    return normalised_backward({grad_out, go_strides}, {q, q_strides}, {k, k_strides}, {v, v_strides}, {o, o_strides},
+                               denom, {dxq, dxq_strides}, {dxk, dxk_strides}, {dv, dv_strides}, B, H, N, D_qk, D_v,
+                               dtype, chunked, workspace, workspace_bytes, stream, feature_map);
 }
 
 int64_t fla_poly_attn_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t R, int64_t D_v) {

@@ -22,6 +22,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "fla_feature.h"
 #include "fla_tri_kernel.h"
 
 namespace fla {
@@ -43,6 +44,10 @@ struct NormParams {
     int32_t H, N, BH, dqk, dv, n_chunks;
     int32_t vec_q, vec_k, vec_a, vec_b, vec_out, vec_dq, vec_dk;
     float eps;
+    // bwd-post with a feature map (fla_feature.h): q and k hold y = phi(x), and the finished
+    // gradients are multiplied by phi'(x) computed from y -- they leave as gradients with respect
+    // to x.  0: none.
+    int32_t fmap;
 };
 
 template <typename T>
@@ -324,6 +329,18 @@ __global__ __launch_bounds__(256, 2) void norm_bwd_post_kernel(const NormParams 
 #pragma unroll
     for (int r = 0; r < kNormSegRows; ++r)
         dr[r] = load8(D + (int64_t)(row0 + r) * ds_n, row0 + r < p.N, col, p.dqk, vec_d);
+    // with a feature map: the rows of y = phi(x) that belong to the gradient being finished
+    // (q for dq, k for dk), for the slope
+    u32x4 yr[kNormSegRows];
+    if (p.fmap) {
+        const T *Yv = part_dk ? static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h
+                              : static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h;
+        const int64_t ys_n = part_dk ? p.ks_n : p.qs_n;
+        const bool vec_y = VEC || (part_dk ? p.vec_k : p.vec_q) != 0;
+#pragma unroll
+        for (int r = 0; r < kNormSegRows; ++r)
+            yr[r] = load8(Yv + (int64_t)(row0 + r) * ys_n, row0 + r < p.N, col, p.dqk, vec_y);
+    }
     // running sum at the entry of this chunk: chunks before it (k) or after it (dn q)
     float run[8];
     {
@@ -369,6 +386,12 @@ __global__ __launch_bounds__(256, 2) void norm_bwd_post_kernel(const NormParams 
         for (int e = 0; e < 8; ++e) {
             run[e] += (part_dk ? dnr : 1.0f) * sf[e];
             g[e] += (part_dk ? 1.0f : dnr) * run[e];
+        }
+        if (p.fmap) {
+            float yf[8];
+            unpack8<T>(part_dk ? yr[kNormSegRows - 1 - i] : yr[i], yf);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) g[e] *= feature_slope_from_value(p.fmap, yf[e]);
         }
         if (row < p.N) store8<T>(D + (int64_t)row * ds_n, col, p.dqk, vec_d, pack8<T>(g));
     }

@@ -10,6 +10,11 @@ no pass over memory exists for the map alone.  The kernels leave phi(xq), phi(xk
 by-product; autograd keeps those instead of xq, xk, and backward returns the gradients with
 respect to xq and xk themselves, the slope of phi multiplied in before the gradients are stored
 (``fla_feature_attn_fwd`` / ``fla_feature_attn_bwd``).
+
+``FeatureMapLinearAttention.apply(xq, xk, v, feature, True, eps)`` is the normalised operator on
+the same features, ``LinearAttentionNormalised.apply(phi(xq), phi(xk), v, eps, True)``
+(``fla_feature_attn_normalised_fwd`` / ``_bwd``); a seventh argument ``chunked=False`` selects the
+quadratic product kernels there.
 """
 
 from __future__ import annotations
@@ -101,10 +106,78 @@ def feature_attention_bwd(grad_output: torch.Tensor, q: torch.Tensor, k: torch.T
     return dxq, dxk, dvv
 
 
+def feature_attention_normalised_fwd(xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, feature: str = "elu1",
+                                     eps: float = 1e-5, chunked: bool = True):
+    """``(out, q, k, denom)``: the normalised output, ``q = phi(xq)``, ``k = phi(xk)`` and the fp32
+    normaliser (B, H, N)."""
+    assert xq.shape == xk.shape and v.shape[:3] == xq.shape[:3], "xq, xk: (B,H,N,D_qk); v: (B,H,N,D_v)"
+    assert xq.shape[-1] <= 256 and v.shape[-1] <= 256, "Only head_dims <= 256 are supported."
+    code = _map_code(feature)
+    xq, xk, v = prepare(xq, xk, v)
+    b, h, n, dqk = xq.shape
+    dv = v.shape[-1]
+    out = torch.empty_like(v, memory_format=torch.contiguous_format)
+    q = torch.empty_like(xq, memory_format=torch.contiguous_format)
+    k = torch.empty_like(xk, memory_format=torch.contiguous_format)
+    denom = torch.empty(b, h, n, dtype=torch.float32, device=xq.device)
+    lib = _lib.load()
+    with torch.cuda.device(xq.device):
+        nbytes = lib.fla_normalised_workspace_bytes(b, h, n, dqk, dv, int(chunked))
+        work = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=xq.device)
+        _lib.check(
+            "fla_feature_attn_normalised_fwd",
+            lib.fla_feature_attn_normalised_fwd(
+                xq.data_ptr(), xk.data_ptr(), v.data_ptr(), out.data_ptr(), q.data_ptr(), k.data_ptr(), denom.data_ptr(),
+                b, h, n, dqk, dv,
+                _lib.strides_arg(xq), _lib.strides_arg(xk), _lib.strides_arg(v), _lib.strides_arg(out),
+                _lib.strides_arg(q), _lib.strides_arg(k),
+                code, float(eps), dtype_code(xq), int(chunked), work.data_ptr(), nbytes, stream_handle(xq.device),
+            ),
+        )
+    return out, q, k, denom
+
+
+def feature_attention_normalised_bwd(grad_output: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
+                                     out: torch.Tensor, denom: torch.Tensor, feature: str = "elu1",
+                                     chunked: bool = True) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dxq, dxk, dv) from the forward call's ``q``, ``k``, ``out`` and ``denom``."""
+    code = _map_code(feature)
+    grad_output, q, k, v, out = prepare(grad_output, q, k, v, out)
+    assert denom.dtype == torch.float32 and denom.is_contiguous() and denom.shape == q.shape[:3]
+    b, h, n, dqk = q.shape
+    dv = v.shape[-1]
+    dxq = torch.empty_like(q, memory_format=torch.contiguous_format)
+    dxk = torch.empty_like(k, memory_format=torch.contiguous_format)
+    dvv = torch.empty_like(v, memory_format=torch.contiguous_format)
+    lib = _lib.load()
+    with torch.cuda.device(q.device):
+        nbytes = lib.fla_normalised_workspace_bytes(b, h, n, dqk, dv, int(chunked))
+        work = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
+        _lib.check(
+            "fla_feature_attn_normalised_bwd",
+            lib.fla_feature_attn_normalised_bwd(
+                grad_output.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), denom.data_ptr(),
+                dxq.data_ptr(), dxk.data_ptr(), dvv.data_ptr(), b, h, n, dqk, dv,
+                _lib.strides_arg(grad_output), _lib.strides_arg(q), _lib.strides_arg(k), _lib.strides_arg(v),
+                _lib.strides_arg(out), _lib.strides_arg(dxq), _lib.strides_arg(dxk), _lib.strides_arg(dvv),
+                code, dtype_code(q), int(chunked), work.data_ptr(), nbytes, stream_handle(q.device),
+            ),
+        )
+    return dxq, dxk, dvv
+
+
 class FeatureMapLinearAttention(Function):
     @staticmethod
     @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.bfloat16)
-    def forward(ctx: Any, xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, feature: str = "elu1") -> torch.Tensor:
+    def forward(ctx: Any, xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, feature: str = "elu1",
+                normalise: bool = False, eps: float = 1e-5, chunked: bool = True) -> torch.Tensor:
+        ctx.normalise = normalise
+        if normalise:
+            out, q, k, denom = feature_attention_normalised_fwd(xq, xk, v, feature, eps, chunked)
+            ctx.feature, ctx.chunked = feature, chunked
+            ctx.save_for_backward(q, k, v, out, denom)
+            return out
+        assert chunked, "without the normaliser the feature map exists for the chunk-wise product only"
         if any(ctx.needs_input_grad[:3]):
             out, q, k, state = feature_attention_fwd(xq, xk, v, feature, want_state=True)
         else:
@@ -120,9 +193,13 @@ class FeatureMapLinearAttention(Function):
     @staticmethod
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx: Any, grad_output: torch.Tensor):
+        if ctx.normalise:
+            q, k, v, out, denom = ctx.saved_tensors
+            dxq, dxk, dv = feature_attention_normalised_bwd(grad_output, q, k, v, out, denom, ctx.feature, ctx.chunked)
+            return dxq, dxk, dv, None, None, None, None
         if ctx.has_state:
             q, k, v, state = ctx.saved_tensors
         else:
             (q, k, v), state = ctx.saved_tensors, None
         dxq, dxk, dv = feature_attention_bwd(grad_output, q, k, v, ctx.feature, state)
-        return dxq, dxk, dv, None
+        return dxq, dxk, dv, None, None, None, None

@@ -214,6 +214,33 @@ int fla_feature_attn_bwd(const void *grad_out, const void *q, const void *k, con
                          int feature_map, int dtype, const void *state_in,
                          void *workspace, int64_t workspace_bytes, void *stream);
 
+/* The two operators above combined: normalised causal linear attention on q = phi(xq),
+ * k = phi(xk),   out_i = [tril(Q K^T) V]_i / (q_i . (k_0 + ... + k_i) + eps),
+ * arguments as for fla_linear_attn_normalised_fwd/bwd (same workspace size query, `chunked`
+ * selects the product's evaluation) plus the feature map and its by-products q_out, k_out as for
+ * fla_feature_attn_fwd.  With the chunk-wise product the map is applied while the kernels load
+ * xq, xk; with the quadratic kernels by one element-wise pass per operand.  Backward takes
+ * q = q_out, k = k_out and returns gradients with respect to xq, xk: the slope of phi is
+ * multiplied in by the pass that adds the normaliser's own terms.  No counterpart in the
+ * reference (README.md:27-30 of the reference is the recipe this replaces). */
+int fla_feature_attn_normalised_fwd(const void *xq, const void *xk, const void *v, void *o, void *q_out, void *k_out,
+                                    float *denom,
+                                    int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                                    const int64_t *xq_strides, const int64_t *xk_strides,
+                                    const int64_t *v_strides, const int64_t *o_strides,
+                                    const int64_t *q_out_strides, const int64_t *k_out_strides,
+                                    int feature_map, float eps, int dtype, int chunked,
+                                    void *workspace, int64_t workspace_bytes, void *stream);
+int fla_feature_attn_normalised_bwd(const void *grad_out, const void *q, const void *k, const void *v,
+                                    const void *o, const float *denom, void *dxq, void *dxk, void *dv,
+                                    int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                                    const int64_t *go_strides, const int64_t *q_strides,
+                                    const int64_t *k_strides, const int64_t *v_strides,
+                                    const int64_t *o_strides, const int64_t *dxq_strides,
+                                    const int64_t *dxk_strides, const int64_t *dv_strides,
+                                    int feature_map, int dtype, int chunked,
+                                    void *workspace, int64_t workspace_bytes, void *stream);
+
 /* fla_linear_attn_chunked_fwd for callers that cannot allocate device memory or pass a workspace
  * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no
  * counterpart in the reference.  Same arguments and results as fla_linear_attn_chunked_fwd with

@@ -211,3 +211,12 @@ def feature_causal_dot_product_grads(
     times the slope of phi."""
     dq, dk, dv = causal_dot_product_grads(feature_map(xq, kind), feature_map(xk, kind), v, do)
     return dq * feature_map_slope(xq, kind), dk * feature_map_slope(xk, kind), dv
+
+
+def feature_linear_attention_normalised(
+    xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, kind: str, eps: float = 1e-5
+) -> torch.Tensor:
+    """:func:`linear_attention_normalised` on phi(xq), phi(xk): the whole caller-side recipe
+    (feature map, product, normaliser; README.md:27-30 of the reference) as a function of the raw
+    xq, xk.  Differentiable; gradients by autograd."""
+    return linear_attention_normalised(feature_map(xq, kind), feature_map(xk, kind), v, eps=eps)

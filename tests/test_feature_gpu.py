@@ -118,3 +118,35 @@ def test_feature_operator_full_size(name, gpu_device):
     assert_close(f"{name} dXq (CPU oracle)", a.grad[sl], dq_c * naive.feature_map_slope(xqc, "elu1"))
     assert_close(f"{name} dXk (CPU oracle)", b.grad[sl], dk_c * naive.feature_map_slope(xkc, "elu1"))
     assert_close(f"{name} dV (CPU oracle)", c.grad[sl], dv_c)
+
+
+NORMALISED_CASES = [
+    (1, 2, 256, 64, 64),
+    (2, 3, 1024, 128, 128),
+    (1, 2, 1088, 128, 128),
+    (1, 2, 2112, 64, 64),
+    (1, 2, 1000, 64, 64),
+    (1, 2, 768, 256, 64),
+    (1, 1, 200, 96, 32),
+]
+
+
+@pytest.mark.parametrize("chunked", [True, False], ids=["chunked", "quadratic"])
+@pytest.mark.parametrize("kind", ["elu1", "softplus"])
+@pytest.mark.parametrize("dims", NORMALISED_CASES, ids=lambda d: "x".join(map(str, d)))
+def test_feature_normalised_fwd_bwd_vs_oracle(dims, kind, chunked, gpu_device):
+    """The whole caller-side recipe (map, product, normaliser) as one operator.  Gradient
+    tolerances as for the normalised operator (tests/test_normalised_gpu.py): Frobenius-relative
+    <= 1e-2, element bound 5e-2 of the largest magnitude."""
+    xq, xk, v, do = _inputs(dims, torch.bfloat16, seed=sum(dims) + 1)
+    eps = 1e-5
+    a0, b0, c0 = (t.float().requires_grad_(True) for t in (xq, xk, v))
+    want = naive.feature_linear_attention_normalised(a0, b0, c0, kind, eps)
+    want_g = torch.autograd.grad(want, (a0, b0, c0), do.float())
+    a, b, c = (t.to(gpu_device).requires_grad_(True) for t in (xq, xk, v))
+    out = FeatureMapLinearAttention.apply(a, b, c, kind, True, eps, chunked)
+    assert out.dtype == torch.bfloat16 and out.shape == v.shape
+    out.backward(do.to(gpu_device))
+    assert_close("out", out, want.detach())
+    for name, got, w_ in (("dXq", a.grad, want_g[0]), ("dXk", b.grad, want_g[1]), ("dV", c.grad, want_g[2])):
+        assert_close(name, got, w_, tol_fro=1e-2, tol_max=5e-2)
