@@ -86,6 +86,10 @@ def _parse():
                          "Taylor features with the polynomial score map, priced in its own FLOPs; "
                          "feature: the chunk-wise operator on raw xq, xk with elu(x) + 1 applied as the kernels load "
                          "them, next to 'PyTorch elu pass + chunk-wise operator' through autograd in the same run")
+    ap.add_argument("--sweep", action="store_true",
+                    help="instead of one workload: forward + backward of the quadratic kernels over a grid of "
+                         "(B*H, N, D_qk, D_v) off the benchmark shapes, one JSON line with a `sweep` list (what the "
+                         "fixed launch rules give where nobody tuned them)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain device copy of 256 MiB (a known-size reference for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -254,6 +258,51 @@ def _other_workload(torch, name, algo, dev, steps):
     del o
     torch.cuda.empty_cache()
     return rec
+
+
+def _sweep(torch, dev, steps) -> int:
+    """Quadratic forward + backward over a grid of shapes, bf16, inputs drawn on the GPU (q, k
+    uniform in [0.5, 1.5), v and dO normal).  Medians of per-iteration event pairs."""
+    from flashy_linear_attention_amd.kernels import (
+        linear_flash_wrapper_bwd,
+        linear_flash_wrapper_bwd_smallv_hd,
+        linear_flash_wrapper_fwd,
+        linear_flash_wrapper_fwd_smallv_hd,
+    )
+
+    grid = []
+    for d_qk, d_v in ((32, 32), (64, 64), (128, 128), (256, 256), (64, 16), (128, 32), (256, 64), (96, 96), (200, 64)):
+        for n in (512, 1024, 2048, 4096, 8192, 16384):
+            for bh in (8, 32, 128):
+                flops = float(bh) * n * n * (4 * d_qk + 3 * d_v)
+                if flops < 2e10 or flops > 8e12 or bh * n * max(d_qk, d_v) * 2 * 7 > 6e9:
+                    continue
+                grid.append((bh, n, d_qk, d_v, flops))
+    gen = torch.Generator(device=dev).manual_seed(0)
+    out = []
+    for bh, n, d_qk, d_v, flops in grid:
+        q = (torch.rand(1, bh, n, d_qk, device=dev, generator=gen) + 0.5).bfloat16()
+        k = (torch.rand(1, bh, n, d_qk, device=dev, generator=gen) + 0.5).bfloat16()
+        v = torch.randn(1, bh, n, d_v, device=dev, generator=gen).bfloat16()
+        do = torch.randn(1, bh, n, d_v, device=dev, generator=gen).bfloat16()
+        small = d_qk != d_v
+        fwd = (lambda: linear_flash_wrapper_fwd_smallv_hd(q, k, v)) if small else (lambda: linear_flash_wrapper_fwd(q, k, v))
+        bwd = (lambda: linear_flash_wrapper_bwd_smallv_hd(do, q, k, v)) if small else (lambda: linear_flash_wrapper_bwd(do, q, k, v))
+
+        def step():
+            fwd()
+            bwd()
+
+        _settle(torch, step, 0.1)
+        ms_f, ms_b = _median_ms(torch, fwd, steps), _median_ms(torch, bwd, steps)
+        ms_s = _median_ms(torch, step, steps)
+        tf = flops / (ms_s * 1e-3) / 1e12
+        out.append({"BH": bh, "N": n, "D_qk": d_qk, "D_v": d_v, "fwd_ms": round(ms_f, 4), "bwd_ms": round(ms_b, 4),
+                    "step_ms": round(ms_s, 4), "tflops": round(tf, 1), "pct_of_peak": round(100 * tf / PEAK_TFLOPS["bf16"], 1)})
+        del q, k, v, do
+    print(json.dumps({"metric": "causal linear attention fwd+bwd TFLOP/s (causal-counted) over a grid of shapes, bf16, 1 MI355X",
+                      "unit": "TFLOP/s", "steps": steps, "sweep": out}))
+    return 0
 
 
 def _cpu_baseline(torch, w, target_seconds):
@@ -480,6 +529,8 @@ def main() -> int:
 
     w = WORKLOADS[args.workload]
     dev = torch.device("cuda:0")
+    if args.sweep:
+        return _sweep(torch, dev, min(args.steps, 30))
     if args.algo == "poly":
         return _bench_poly(torch, args, w, dev)
     if args.algo == "feature":
