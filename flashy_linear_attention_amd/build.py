@@ -69,8 +69,10 @@ def build(jobs: int | None = None, verbose: bool = True) -> str:
         objs = list(pool.map(_compile_inst, work))
     capi = os.path.join(OBJ_DIR, "fla_capi.o")
     _run([_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, "fla_capi.hip"), "-o", capi])
+    walk = os.path.join(OBJ_DIR, "fla_walk_inst.o")
+    _run([_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, "fla_walk_inst.hip"), "-o", walk])
     tmp = LIB_PATH + ".tmp"
-    _run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, capi, *objs])
+    _run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, capi, walk, *objs])
     os.replace(tmp, LIB_PATH)
     if verbose:
         print(f"built {LIB_PATH} ({os.path.getsize(LIB_PATH) / 1e6:.1f} MB, {len(objs)} kernel objects)")

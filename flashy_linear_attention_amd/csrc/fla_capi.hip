@@ -360,6 +360,47 @@ int run_tri_chunked(const View &x, const View &y, const View &z, const View &out
 // so forward can hand its state to backward, and backward computes one new state instead of
 // three.  Any other shape evaluates each product on its own.
 
+// ---- equal padded head dims up to 64: the walk kernels (fla_chunk_walk.h).  A workgroup walks a
+// segment of 128-row chunks with the running state in registers; segment entry states come from
+// a totals kernel and a scan over the segments.
+struct WalkPlan {
+    bool ok;
+    int D;
+    int64_t n_chunks, seg_chunks, n_seg;
+    int64_t totals_bytes;  // fp32 entry states of the segments (0 with a single segment)
+    int64_t saved_bytes;   // 16-bit state at the entry of every chunk, forward -> backward
+};
+
+WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
+    WalkPlan w{};
+    w.ok = pad_index(dqk) == pad_index(dv) && padded(dqk) <= 64 && N > fla::kWalkRows;
+    if (!w.ok) return w;
+    w.D = (int)padded(dqk);
+    w.n_chunks = (N + fla::kWalkRows - 1) / fla::kWalkRows;
+    // about a thousand workgroups (two resident per CU, two rounds) where the problem has that many chunks
+    const int64_t total = B * H * w.n_chunks;
+    w.seg_chunks = total / 1024 > 1 ? total / 1024 : 1;
+    if (w.seg_chunks > w.n_chunks) w.seg_chunks = w.n_chunks;
+    w.n_seg = (w.n_chunks + w.seg_chunks - 1) / w.seg_chunks;
+    w.totals_bytes = w.n_seg > 1 ? B * H * w.n_seg * w.D * w.D * 4 : 0;
+    w.saved_bytes = B * H * w.n_chunks * w.D * w.D * 2;
+    return w;
+}
+
+// totals of Y^T Z per segment into `totals`, then their exclusive sums over the segments before
+// (reverse == 0) or after (reverse != 0)
+int walk_entry_states(const WalkPlan &w, const View &y, const View &z, int64_t B, int64_t H, int64_t N, int64_t dy,
+                      int64_t dz, int dtype, int reverse, float *totals, hipStream_t s) {
+    fla::WalkTotalsParams tp{};
+    tp.y = y.ptr, tp.z = z.ptr, tp.totals = totals;
+    tp.ys_b = y.strides[0], tp.ys_h = y.strides[1], tp.ys_n = y.strides[2];
+    tp.zs_b = z.strides[0], tp.zs_h = z.strides[1], tp.zs_n = z.strides[2];
+    tp.H = (int32_t)H, tp.N = (int32_t)N, tp.BH = (int32_t)(B * H), tp.dy = (int32_t)dy, tp.dz = (int32_t)dz;
+    tp.n_chunks = (int32_t)w.n_chunks, tp.seg_chunks = (int32_t)w.seg_chunks, tp.n_seg = (int32_t)w.n_seg;
+    if (fla::walk_totals(dtype, w.D, tp, s) != hipSuccess) return FLA_ERR_LAUNCH;
+    return fla::walk_scan(totals, B * H, (int)w.n_seg, w.D * w.D, reverse, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+}
+
 bool states_shareable(int64_t dqk, int64_t dv, int64_t N) {
     if (pad_index(dqk) != pad_index(dv) || padded(dqk) > 128) return false;
     const int rows = chunk_rows(dqk, dv);
@@ -368,6 +409,8 @@ bool states_shareable(int64_t dqk, int64_t dv, int64_t N) {
 
 // bytes of one rounded running state / of the scratch one state computation needs (fp32 chunk states)
 int64_t shared_state_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
+    const WalkPlan w = walk_plan(B, H, N, dqk, dv);
+    if (w.ok) return w.saved_bytes;  // one state per 128-row chunk (also room for the 256-row chunks' states)
     if (!states_shareable(dqk, dv, N)) return 0;
     const int64_t rows = chunk_rows(dqk, dv);
     return B * H * ((N + rows - 1) / rows) * padded(dqk) * padded(dv) * 2;
@@ -395,6 +438,29 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         if (int rc = check_view(t)) return rc;
     if (int rc = check_alias_fwd(q, k, v, o, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    const WalkPlan wp = walk_plan(B, H, N, dqk, dv);
+    if (!fmap && wp.ok && fla::fast_path_ok(make_params(q, k, v, o, B, H, N, dqk, dv, 0))) {
+        if (wp.totals_bytes &&
+            (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.totals_bytes))
+            return FLA_ERR_WORKSPACE;
+        if (state_out && reinterpret_cast<uintptr_t>(state_out) % 16 != 0) return FLA_ERR_WORKSPACE;
+        hipStream_t s = static_cast<hipStream_t>(stream);
+        float *totals = wp.totals_bytes ? static_cast<float *>(workspace) : nullptr;
+        if (totals)
+            if (int rc = walk_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, totals, s)) return rc;
+        fla::WalkParams w{};
+        w.q = q.ptr, w.k = k.ptr, w.v = v.ptr, w.o = const_cast<void *>(o.ptr);
+        w.qs_b = q.strides[0], w.qs_h = q.strides[1], w.qs_n = q.strides[2];
+        w.ks_b = k.strides[0], w.ks_h = k.strides[1], w.ks_n = k.strides[2];
+        w.vs_b = v.strides[0], w.vs_h = v.strides[1], w.vs_n = v.strides[2];
+        w.os_b = o.strides[0], w.os_h = o.strides[1], w.os_n = o.strides[2];
+        w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dqk, w.wv = (int32_t)dv;
+        w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
+        w.init = totals, w.saved = state_out;
+        if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
+        if (state_out && state_valid) *state_valid = 1;
+        return FLA_OK;
+    }
     TriParams p = make_params(q, fmap ? mapped[1] : k, v, o, B, H, N, dqk, dv, 0);
     const bool k_fast = !fmap || fla::fast_path_ok(make_params(q, k, v, o, B, H, N, dqk, dv, 0));  // xk under the state kernel's loads
     if (!states_shareable(dqk, dv, N) || !fla::fast_path_ok(p) || !k_fast) {
@@ -444,6 +510,32 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         if (int rc = launch_feature_pass(2, fmap, q, dq, B, H, N, dqk, dtype, stream)) return rc;
         return launch_feature_pass(2, fmap, k, dk, B, H, N, dqk, dtype, stream);
     }
+    const WalkPlan wp = walk_plan(B, H, N, dqk, dv);
+    if (!fmap && wp.ok && state_in) {  // (the states forward saved are per 128-row chunk: only this path reads them)
+        if (wp.totals_bytes &&
+            (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.totals_bytes))
+            return FLA_ERR_WORKSPACE;
+        if (reinterpret_cast<uintptr_t>(state_in) % 16 != 0) return FLA_ERR_WORKSPACE;
+        hipStream_t s = static_cast<hipStream_t>(stream);
+        float *totals = wp.totals_bytes ? static_cast<float *>(workspace) : nullptr;
+        if (totals)
+            if (int rc = walk_entry_states(wp, q, go, B, H, N, dqk, dv, dtype, 1, totals, s)) return rc;
+        fla::WalkParams w{};
+        w.q = q.ptr, w.k = k.ptr, w.v = v.ptr, w.go = go.ptr;
+        w.dq = const_cast<void *>(dq.ptr), w.dk = const_cast<void *>(dk.ptr), w.dv = const_cast<void *>(dvv.ptr);
+        w.qs_b = q.strides[0], w.qs_h = q.strides[1], w.qs_n = q.strides[2];
+        w.ks_b = k.strides[0], w.ks_h = k.strides[1], w.ks_n = k.strides[2];
+        w.vs_b = v.strides[0], w.vs_h = v.strides[1], w.vs_n = v.strides[2];
+        w.gs_b = go.strides[0], w.gs_h = go.strides[1], w.gs_n = go.strides[2];
+        w.dqs_b = dq.strides[0], w.dqs_h = dq.strides[1], w.dqs_n = dq.strides[2];
+        w.dks_b = dk.strides[0], w.dks_h = dk.strides[1], w.dks_n = dk.strides[2];
+        w.dvs_b = dvv.strides[0], w.dvs_h = dvv.strides[1], w.dvs_n = dvv.strides[2];
+        w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dqk, w.wv = (int32_t)dv;
+        w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
+        w.init = totals, w.saved = const_cast<void *>(state_in);
+        return fla::walk_bwd(dtype, wp.D, w, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+    }
+    if (wp.ok && !fmap) state_in = nullptr;  // not in the 256-row chunks' format: recomputed below
     if (fmap) set_output_slope(pq, fmap, q), set_output_slope(pk, fmap, k);
     const int64_t sb = shared_state_bytes(B, H, N, dqk, dv);
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < sb * (state_in ? 3 : 4))
@@ -1001,7 +1093,14 @@ int fla_linear_attn_chunked_fwd_static(const void *q, const void *k, const void 
     if (int rc = check_common(B, H, N, dtype)) return rc;
     if (D_qk < 1 || D_qk > 256) return FLA_ERR_HEAD_DIM;
     if (D_v < 1 || D_v > 256) return FLA_ERR_V_HEAD_DIM;
-    const int64_t need = chunked_op_workspace_bytes(B, H, N, D_qk, D_v);
+    // what this call's kernels use of the workspace: without a state to hand over, the walk path
+    // needs the segments' entry states only
+    const WalkPlan wp = walk_plan(B, H, N, D_qk, D_v);
+    int64_t need = chunked_op_workspace_bytes(B, H, N, D_qk, D_v);
+    if (wp.ok) {
+        const int64_t other = chunked_bytes(B, H, N, D_qk, D_v);  // operands off the speed path
+        need = wp.totals_bytes > other ? wp.totals_bytes : other;
+    }
     if (need > (int64_t)FLA_STATIC_SCRATCH_BYTES) return FLA_ERR_WORKSPACE;
     void *ws = nullptr;
     if (int rc = static_scratch(&ws)) return rc;

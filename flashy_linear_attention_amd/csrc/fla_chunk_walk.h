@@ -1,0 +1,534 @@
+// Chunk-wise causal linear attention with the running state kept inside the kernel, for equal
+// padded head dims D = 32 or 64 (the long-sequence shapes, which are bound by memory traffic).
+//
+// The chunk-wise evaluation of fla_chunk_state.h / fla_tri_fast.h computes every per-chunk
+// state, writes it in fp32, scans it, writes the running sums in 16 bit and reads them back in
+// each consumer, and its backward reads q, k, v and dO once per product.  Here a workgroup walks
+// a *segment* of consecutive 128-row chunks in sequence order and carries the running state
+//
+//     S = sum over the chunks before of K_c^T V_c      (forward, lower mask: ascending walk)
+//     R = sum over the chunks after  of Q_c^T dO_c     (backward, upper mask: descending walk)
+//
+// in fp32 accumulators; per chunk it is rounded once to the storage type (as before) into 8 KiB
+// of LDS, where the MFMAs of the state products read it.  Every operand tile of a chunk is
+// brought to LDS once and serves all products of that chunk:
+//
+//   forward   O_c  = lower(Q_c K_c^T) V_c   + Q_c S          then S += K_c^T V_c
+//   backward  dQ_c = lower(dO_c V_c^T) K_c  + dO_c S_c^T     (S_c: saved by forward, 16 bit per chunk)
+//             dV_c = upper(K_c Q_c^T) dO_c  + K_c R
+//             dK_c = upper(V_c dO_c^T) Q_c  + V_c R^T        then R += Q_c^T dO_c
+//
+// Segments make the walk parallel: a first kernel adds up K^T V (Q^T dO) over each segment, a
+// small one turns the totals into exclusive prefix (suffix) sums, and each walking workgroup
+// starts from its segment's entry state.  Per step that reads k, v (q, dO) twice and everything
+// else once; no fp32 per-chunk state ever goes to memory.
+//
+// Layout.  An operand tile is 128 rows x D 16-bit values, row-major, the 16-byte chunk index of
+// a row XORed with swizzle_y (fla_tri_fast.h) -- one layout for the 16-byte row reads (MFMA
+// operands with k along the row) and for the transposing column reads (k down the rows).  Wave w
+// of the four owns rows 32 w .. 32 w + 31 of the chunk as the "X rows" of every product; the
+// MFMA operand chaining is that of the other kernels: S^T = Y X^T leaves a lane holding one X
+// row and eight-row groups of Y rows, which is the B operand of Out^T += Z^T P^T.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "fla_launch.h"
+#include "fla_tri_fast.h"
+
+namespace fla {
+
+constexpr int kWalkRows = 128;  // rows per chunk of the walk kernels
+
+struct WalkParams {
+    const void *q, *k, *v, *go;  // operands (go: backward only); (B, H, N, D)
+    void *o, *dq, *dk, *dv;      // results (forward: o; backward: dq, dk, dv)
+    int64_t qs_b, qs_h, qs_n, ks_b, ks_h, ks_n, vs_b, vs_h, vs_n, gs_b, gs_h, gs_n;
+    int64_t os_b, os_h, os_n, dqs_b, dqs_h, dqs_n, dks_b, dks_h, dks_n, dvs_b, dvs_h, dvs_n;
+    int32_t H, N, BH, wqk, wv;   // true widths of q/k and of v (<= D)
+    int32_t n_chunks;            // ceil(N / 128)
+    int32_t seg_chunks, n_seg;   // chunks per segment, segments per (b, h)
+    // entry state of every segment, fp32 [BH][n_seg][D (q/k index)][D (v index)]: sum of K^T V over
+    // the segments before (forward) / of Q^T dO over the segments after (backward); null when
+    // there is a single segment (entry state zero)
+    const float *init;
+    // forward: where the 16-bit state at the entry of every chunk goes, [BH][n_chunks][D][D]
+    // ([q/k index][v index]), or null; backward: the same buffer, read for dQ
+    void *saved;
+};
+
+template <int D>
+struct WalkCfg {
+    static constexpr int C = kWalkRows;
+    static constexpr int RB = D * 2;        // bytes per tile row
+    static constexpr int CR = D / 8;        // 16-byte chunks per row
+    static constexpr int TILE = C * RB;     // bytes per operand tile
+    static constexpr int KC = D / 16;       // 16-wide k chunks of a contraction over D
+    static constexpr int DB = D / 32;       // 32-wide blocks of D
+    static constexpr int RPI = 1024 / RB;   // rows covered by one wave-level 1 KiB load
+    static constexpr int NI = TILE / 4096;  // such loads per wave and tile
+    static constexpr int STATE = D * RB;    // the 16-bit state in LDS
+    static constexpr int NBLK = DB * DB;    // 32 x 32 blocks of the state: block b belongs to wave b
+    static_assert(D == 32 || D == 64, "walk kernels are built for padded head dims 32 and 64");
+    static_assert(NBLK <= 4, "one state block per wave at most");
+};
+
+// ---- LDS tile access (tile: row-major [rows][D], chunk index XOR swizzle_y(row))
+
+// whole 128-row tile HBM -> LDS; rows >= N and chunks beyond the true width arrive as zeros
+template <int D>
+__device__ __forceinline__ void walk_load_tile(u32x4 rsrc, uint32_t lds_tile, int row0, int stride2, int width, int wave,
+                                               int lane) {
+    using W = WalkCfg<D>;
+    const int r = wave * W::RPI + lane / W::CR;
+    const int c = (lane % W::CR) ^ swizzle_y<W::CR>(r);
+    const uint32_t voff = (uint32_t)(r * stride2 + c * 16) + (c * 8 < width ? 0u : kOobOffset);
+    const uint32_t base = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_tile + wave * 1024));
+    u32x4 rs = {(uint32_t)__builtin_amdgcn_readfirstlane((int)rsrc[0]), (uint32_t)__builtin_amdgcn_readfirstlane((int)rsrc[1]),
+                (uint32_t)__builtin_amdgcn_readfirstlane((int)rsrc[2]), (uint32_t)__builtin_amdgcn_readfirstlane((int)rsrc[3])};
+    static_for<0, W::NI>([&](auto u) {
+        constexpr int U = decltype(u)::value;
+        const uint32_t so = (uint32_t)__builtin_amdgcn_readfirstlane((row0 + U * 4 * W::RPI) * stride2);
+        dma_16B_per_lane<U * 4096>(rs, base, voff, so);
+    });
+}
+
+// eight consecutive columns 16 kc + 8 g .. of one row: an MFMA operand with k along the row
+template <typename T, int D>
+__device__ __forceinline__ typename Mma<T>::V8 walk_row_frag(const unsigned char *tile, int row, int kc, int g) {
+    using W = WalkCfg<D>;
+    const int ch = (2 * kc + g) ^ swizzle_y<W::CR>(row);
+    return __builtin_bit_cast(typename Mma<T>::V8, *reinterpret_cast<const u32x4 *>(tile + row * W::RB + (ch << 4)));
+}
+
+__device__ __forceinline__ s16x4 walk_tr_read(const unsigned char *p) {
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
+}
+
+// Column fragment with the output-column permutation of the product kernels: rows R0 + {4g .. 4g+3,
+// 8+4g .. 8+4g+3} (the k order of a rounded S^T accumulator) of the 32 columns of block cb, taken
+// so that MFMA row m = 8a + 4g' + b holds column 16g' + 4a + b -- a lane's 16 accumulator registers
+// are then 16 consecutive output columns.  With `consecutive` the rows are R0 + 8g .. 8g+7 instead
+// (the k order of a row fragment): the transposed read of the state.
+template <typename T, int D>
+__device__ __forceinline__ typename Mma<T>::V8 walk_col_frag_perm(const unsigned char *tile, int R0, int cb, int lane,
+                                                                  bool consecutive) {
+    using W = WalkCfg<D>;
+    const int lam = lane & 15, g = lane >> 5, beta = (lane >> 4) & 1, zc = lam & 3;
+    const int row_lo = R0 + (consecutive ? 8 * g : 4 * g) + (lam >> 2), row_hi = row_lo + (consecutive ? 4 : 8);
+    const int ch = 4 * cb + 2 * (zc & 1) + beta, byte = 8 * (zc >> 1);
+    const s16x4 lo = walk_tr_read(tile + row_lo * W::RB + ((ch ^ swizzle_y<W::CR>(row_lo)) << 4) + byte);
+    const s16x4 hi = walk_tr_read(tile + row_hi * W::RB + ((ch ^ swizzle_y<W::CR>(row_hi)) << 4) + byte);
+    return __builtin_bit_cast(typename Mma<T>::V8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+// Column fragment, plain mapping (lane l32 <-> column 32 cb + l32), rows R0 + {4g.., 8+4g..}: both
+// operands of the state update Y^T Z, whose contraction runs down the rows.
+template <typename T, int D>
+__device__ __forceinline__ typename Mma<T>::V8 walk_col_frag(const unsigned char *tile, int R0, int cb, int lane) {
+    using W = WalkCfg<D>;
+    const int lam = lane & 15, g = lane >> 5, beta = (lane >> 4) & 1;
+    const int row_lo = R0 + 4 * g + (lam >> 2), row_hi = row_lo + 8;
+    const int ch = 4 * cb + 2 * beta + ((lam & 3) >> 1), sub = 8 * (lam & 1);
+    const s16x4 lo = walk_tr_read(tile + row_lo * W::RB + ((ch ^ swizzle_y<W::CR>(row_lo)) << 4) + sub);
+    const s16x4 hi = walk_tr_read(tile + row_hi * W::RB + ((ch ^ swizzle_y<W::CR>(row_hi)) << 4) + sub);
+    return __builtin_bit_cast(typename Mma<T>::V8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+// MFMA row m of a state-product A operand holds output column e_lane(m) of its 32-column block
+// (the permutation of walk_col_frag_perm)
+__device__ __forceinline__ int walk_e_lane(int l32) { return 16 * ((l32 >> 2) & 1) + 4 * (l32 >> 3) + (l32 & 3); }
+
+// ---- one product of a chunk for this wave's 32 X rows:
+//   acc = [state: X_w . State]  +  mask(X_w Y^T) Z        (UPPER: keep row <= column, else row >= column)
+// xt, yt, zt: LDS tiles; sfrag(db, kc): the state's A-operand fragment for output block db, k chunk kc.
+template <typename T, int D, bool UPPER, typename SFrag>
+__device__ __forceinline__ void walk_product(const unsigned char *xt, const unsigned char *yt, const unsigned char *zt,
+                                             int wave, int lane, bool has_state, SFrag &&sfrag,
+                                             f32x16 (&acc)[WalkCfg<D>::DB]) {
+    using W = WalkCfg<D>;
+    using M = Mma<T>;
+    using V8 = typename M::V8;
+    const int l32 = lane & 31, g = lane >> 5;
+    V8 xf[W::KC];
+#pragma unroll
+    for (int kc = 0; kc < W::KC; ++kc) xf[kc] = walk_row_frag<T, D>(xt, 32 * wave + l32, kc, g);
+#pragma unroll
+    for (int db = 0; db < W::DB; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[db][v] = 0.f;
+    if (has_state) {
+#pragma unroll
+        for (int db = 0; db < W::DB; ++db)
+#pragma unroll
+            for (int kc = 0; kc < W::KC; ++kc) acc[db] = M::mma(sfrag(db, kc), xf[kc], acc[db]);
+    }
+    const int s_lo = UPPER ? wave : 0, s_hi = UPPER ? 3 : wave;
+#pragma unroll 1
+    for (int s = s_lo; s <= s_hi; ++s) {
+        f32x16 sc;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) sc[v] = 0.f;
+#pragma unroll
+        for (int kc = 0; kc < W::KC; ++kc) sc = M::mma(walk_row_frag<T, D>(yt, 32 * s + l32, kc, g), xf[kc], sc);
+        if (s == wave) {  // the 32 x 32 block on the diagonal: lane = X row l32, register v = Y row jl
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int jl = 8 * (v / 4) + 4 * g + (v % 4);
+                const bool keep = UPPER ? l32 <= jl : l32 >= jl;
+                sc[v] = keep ? sc[v] : 0.f;
+            }
+        }
+        V8 pf[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[t][e] = static_cast<T>(sc[8 * t + e]);
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int db = 0; db < W::DB; ++db)
+                acc[db] = M::mma(walk_col_frag_perm<T, D>(zt, 32 * s + 16 * t, db, lane, false), pf[t], acc[db]);
+    }
+}
+
+// acc[db][v] = Out[row][32 db + 16 g + v]: two 16-byte stores per block; rows >= N and columns beyond
+// the true width fall outside the buffer resource and are dropped
+template <typename T, int D>
+__device__ __forceinline__ void walk_store(__amdgpu_buffer_rsrc_t rs, int stride2, int width, int row, int g,
+                                           const f32x16 (&acc)[WalkCfg<D>::DB]) {
+    using V8 = typename Mma<T>::V8;
+#pragma unroll
+    for (int db = 0; db < WalkCfg<D>::DB; ++db) {
+#pragma unroll
+        for (int hq = 0; hq < 2; ++hq) {
+            V8 o8;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o8[e] = static_cast<T>(acc[db][8 * hq + e]);
+            const int col = 32 * db + 16 * g + 8 * hq;
+            const uint32_t off = (uint32_t)(row * stride2 + col * 2) + (col < width ? 0u : kOobOffset);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o8), rs, off, 0, 0);
+        }
+    }
+}
+
+// state += Y^T Z over the 128 rows of the tiles, this wave's 32 x 32 block (dbk: block of Y columns,
+// eb: block of Z columns): st[v] = State[32 dbk + 8(v/4) + 4g + v%4][32 eb + l32]
+template <typename T, int D>
+__device__ __forceinline__ void walk_update(const unsigned char *yt, const unsigned char *zt, int dbk, int eb, int lane,
+                                            f32x16 &st) {
+    using M = Mma<T>;
+#pragma unroll
+    for (int ks = 0; ks < kWalkRows / 16; ++ks)
+        st = M::mma(walk_col_frag<T, D>(yt, 16 * ks, dbk, lane), walk_col_frag<T, D>(zt, 16 * ks, eb, lane), st);
+}
+
+// the state rounded to 16 bit into LDS as T[v index][q/k index] (row = 32 eb + l32, four consecutive
+// columns per register group), in the tile layout
+template <typename T, int D>
+__device__ __forceinline__ void walk_state_to_lds(unsigned char *tl, int dbk, int eb, int lane, const f32x16 &st) {
+    using W = WalkCfg<D>;
+    typedef T t4 __attribute__((ext_vector_type(4)));
+    const int l32 = lane & 31, g = lane >> 5, row = 32 * eb + l32;
+#pragma unroll
+    for (int a = 0; a < 4; ++a) {
+        t4 w;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) w[b] = static_cast<T>(st[4 * a + b]);
+        *reinterpret_cast<t4 *>(tl + row * W::RB + (((4 * dbk + a) ^ swizzle_y<W::CR>(row)) << 4) + 8 * g) = w;
+    }
+}
+
+struct WalkSlice {
+    int bh, seg, c_lo, c_hi;  // chunks c_lo .. c_hi - 1
+    bool valid;
+};
+
+// workgroup -> ((b, h), segment): heads of one XCD in sequence, as in the other kernels
+__device__ __forceinline__ WalkSlice walk_slice(const WalkParams &p) {
+    const int wg = blockIdx.x, xcd = wg & 7, slot = wg >> 3;
+    const int hl = slot / p.n_seg, seg = slot - hl * p.n_seg;
+    WalkSlice s;
+    s.bh = hl * 8 + xcd, s.seg = seg;
+    s.c_lo = seg * p.seg_chunks;
+    s.c_hi = s.c_lo + p.seg_chunks < p.n_chunks ? s.c_lo + p.seg_chunks : p.n_chunks;
+    s.valid = s.bh < p.BH && s.c_lo < p.n_chunks;
+    return s;
+}
+
+template <int D>
+__device__ __forceinline__ void walk_load_init(const float *init, int dbk, int eb, int lane, f32x16 &st) {
+    const int l32 = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) st[v] = init ? init[(32 * dbk + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * eb + l32] : 0.f;
+}
+
+// ---- forward: O_c = lower(Q_c K_c^T) V_c + Q_c S, S += K_c^T V_c, chunks ascending
+template <typename T, int D>
+__global__ __launch_bounds__(256, 2) void walk_fwd_kernel(const WalkParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    using W = WalkCfg<D>;
+    using V8 = typename Mma<T>::V8;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    unsigned char *tq = smem, *tk = smem + W::TILE, *tv = smem + 2 * W::TILE, *tl = smem + 3 * W::TILE;
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const WalkSlice sl = walk_slice(p);
+    if (!sl.valid) return;
+    const int b = sl.bh / p.H, h = sl.bh - b * p.H, N = p.N;
+    const T *Q = static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h;
+    const T *K = static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h;
+    const T *V = static_cast<const T *>(p.v) + b * p.vs_b + h * p.vs_h;
+    T *O = static_cast<T *>(p.o) + b * p.os_b + h * p.os_h;
+    const int qs2 = (int)p.qs_n * 2, ks2 = (int)p.ks_n * 2, vs2 = (int)p.vs_n * 2, os2 = (int)p.os_n * 2;
+    const u32x4 rq = make_rsrc(Q, (uint32_t)((N - 1) * qs2 + p.wqk * 2));
+    const u32x4 rk = make_rsrc(K, (uint32_t)((N - 1) * ks2 + p.wqk * 2));
+    const u32x4 rv = make_rsrc(V, (uint32_t)((N - 1) * vs2 + p.wv * 2));
+    const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(O, 0, (N - 1) * os2 + p.wv * 2, 0x00020000);
+
+    const bool has_block = wave < W::NBLK;
+    const int dbk = wave / W::DB, eb = wave % W::DB;
+    f32x16 st;
+    walk_load_init<D>(p.init ? p.init + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D) : nullptr, dbk, eb, lane, st);
+    if (has_block) walk_state_to_lds<T, D>(tl, dbk, eb, lane, st);
+
+#pragma unroll 1
+    for (int c = sl.c_lo; c < sl.c_hi; ++c) {
+        const int row0 = c * kWalkRows;
+        walk_load_tile<D>(rq, lds0, row0, qs2, p.wqk, wave, lane);
+        walk_load_tile<D>(rk, lds0 + W::TILE, row0, ks2, p.wqk, wave, lane);
+        walk_load_tile<D>(rv, lds0 + 2 * W::TILE, row0, vs2, p.wv, wave, lane);
+        wait_vm<0>();
+        __syncthreads();  // the tiles have landed; the state written by the previous iteration is visible
+        f32x16 acc[W::DB];
+        walk_product<T, D, false>(tq, tk, tv, wave, lane, c > 0, [&](int db, int kc) -> V8 {
+            return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g);
+        }, acc);
+        walk_store<T, D>(ro, os2, p.wv, row0 + 32 * wave + l32, g, acc);
+        if (has_block) {
+            if (p.saved) {  // the state at the entry of this chunk, [q/k index][v index], for backward's dQ
+                T *sv = static_cast<T *>(p.saved) + ((int64_t)sl.bh * p.n_chunks + c) * (D * D);
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    sv[(32 * dbk + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * eb + l32] = static_cast<T>(st[v]);
+            }
+            walk_update<T, D>(tk, tv, dbk, eb, lane, st);
+        }
+        __syncthreads();  // every wave is done with the tiles and with the old state
+        if (has_block) walk_state_to_lds<T, D>(tl, dbk, eb, lane, st);
+    }
+#else
+    (void)p;
+#endif
+}
+
+// ---- backward: dQ, dV, dK of a chunk from one set of tiles; R += Q_c^T dO_c, chunks descending
+template <typename T, int D>
+__global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    using W = WalkCfg<D>;
+    using V8 = typename Mma<T>::V8;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    unsigned char *tq = smem, *tk = smem + W::TILE, *tv = smem + 2 * W::TILE, *tg = smem + 3 * W::TILE,
+                  *tl = smem + 4 * W::TILE;
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const WalkSlice sl = walk_slice(p);
+    if (!sl.valid) return;
+    const int b = sl.bh / p.H, h = sl.bh - b * p.H, N = p.N;
+    const T *Q = static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h;
+    const T *K = static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h;
+    const T *V = static_cast<const T *>(p.v) + b * p.vs_b + h * p.vs_h;
+    const T *G = static_cast<const T *>(p.go) + b * p.gs_b + h * p.gs_h;
+    T *DQ = static_cast<T *>(p.dq) + b * p.dqs_b + h * p.dqs_h;
+    T *DK = static_cast<T *>(p.dk) + b * p.dks_b + h * p.dks_h;
+    T *DV = static_cast<T *>(p.dv) + b * p.dvs_b + h * p.dvs_h;
+    const int qs2 = (int)p.qs_n * 2, ks2 = (int)p.ks_n * 2, vs2 = (int)p.vs_n * 2, gs2 = (int)p.gs_n * 2;
+    const int dqs2 = (int)p.dqs_n * 2, dks2 = (int)p.dks_n * 2, dvs2 = (int)p.dvs_n * 2;
+    const u32x4 rq = make_rsrc(Q, (uint32_t)((N - 1) * qs2 + p.wqk * 2));
+    const u32x4 rk = make_rsrc(K, (uint32_t)((N - 1) * ks2 + p.wqk * 2));
+    const u32x4 rv = make_rsrc(V, (uint32_t)((N - 1) * vs2 + p.wv * 2));
+    const u32x4 rg = make_rsrc(G, (uint32_t)((N - 1) * gs2 + p.wv * 2));
+    const __amdgpu_buffer_rsrc_t rdq = __builtin_amdgcn_make_buffer_rsrc(DQ, 0, (N - 1) * dqs2 + p.wqk * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rdk = __builtin_amdgcn_make_buffer_rsrc(DK, 0, (N - 1) * dks2 + p.wqk * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rdv = __builtin_amdgcn_make_buffer_rsrc(DV, 0, (N - 1) * dvs2 + p.wv * 2, 0x00020000);
+
+    const bool has_block = wave < W::NBLK;
+    const int dbk = wave / W::DB, eb = wave % W::DB;
+    f32x16 st;  // R[q/k index][v index]
+    walk_load_init<D>(p.init ? p.init + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D) : nullptr, dbk, eb, lane, st);
+    if (has_block) walk_state_to_lds<T, D>(tl, dbk, eb, lane, st);
+
+#pragma unroll 1
+    for (int c = sl.c_hi - 1; c >= sl.c_lo; --c) {
+        const int row0 = c * kWalkRows;
+        walk_load_tile<D>(rq, lds0, row0, qs2, p.wqk, wave, lane);
+        walk_load_tile<D>(rk, lds0 + W::TILE, row0, ks2, p.wqk, wave, lane);
+        walk_load_tile<D>(rv, lds0 + 2 * W::TILE, row0, vs2, p.wv, wave, lane);
+        walk_load_tile<D>(rg, lds0 + 3 * W::TILE, row0, gs2, p.wv, wave, lane);
+        // dQ's state, S_c[q/k index][v index] as saved by forward: A-operand fragments straight from
+        // memory (row = output column of dQ, eight consecutive v indices)
+        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+            static_cast<T *>(p.saved) + ((int64_t)sl.bh * p.n_chunks + c) * (D * D), 0, D * D * 2, 0x00020000);
+        V8 sfq[W::DB][W::KC];
+        if (c > 0) {
+#pragma unroll
+            for (int db = 0; db < W::DB; ++db)
+#pragma unroll
+                for (int kc = 0; kc < W::KC; ++kc)
+                    sfq[db][kc] = __builtin_bit_cast(V8, __builtin_amdgcn_raw_buffer_load_b128(
+                                                             rs, (uint32_t)(((32 * db + walk_e_lane(l32)) * D + 16 * kc + 8 * g) * 2), 0, 0));
+        }
+        wait_vm<0>();
+        __syncthreads();
+        const int row = row0 + 32 * wave + l32;
+        const bool later = c + 1 < p.n_chunks;  // chunks after this one exist: R is not identically zero
+        f32x16 acc[W::DB];
+        // dQ = lower(dO V^T) K + dO S_c^T
+        walk_product<T, D, false>(tg, tv, tk, wave, lane, c > 0, [&](int db, int kc) -> V8 { return sfq[db][kc]; }, acc);
+        walk_store<T, D>(rdq, dqs2, p.wqk, row, g, acc);
+        // dV = upper(K Q^T) dO + K R: A operand R^T[v index][q/k index] = the LDS copy as it is
+        walk_product<T, D, true>(tk, tq, tg, wave, lane, later, [&](int db, int kc) -> V8 {
+            return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g);
+        }, acc);
+        walk_store<T, D>(rdv, dvs2, p.wv, row, g, acc);
+        // dK = upper(V dO^T) Q + V R^T: A operand R[q/k index][v index] = the LDS copy read transposed
+        walk_product<T, D, true>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
+            return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
+        }, acc);
+        walk_store<T, D>(rdk, dks2, p.wqk, row, g, acc);
+        if (has_block) walk_update<T, D>(tq, tg, dbk, eb, lane, st);
+        __syncthreads();
+        if (has_block) walk_state_to_lds<T, D>(tl, dbk, eb, lane, st);
+    }
+#else
+    (void)p;
+#endif
+}
+
+// ---- segment totals: totals[bh][seg] = sum over the segment's rows of Y^T Z, fp32 [D][D]
+struct WalkTotalsParams {
+    const void *y, *z;
+    int64_t ys_b, ys_h, ys_n, zs_b, zs_h, zs_n;
+    int32_t H, N, BH, dy, dz;
+    int32_t n_chunks, seg_chunks, n_seg;
+    float *totals;
+};
+
+template <typename T, int D>
+__global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    using W = WalkCfg<D>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wg = blockIdx.x, xcd = wg & 7, slot = wg >> 3;
+    const int hl = slot / p.n_seg, seg = slot - hl * p.n_seg, bh = hl * 8 + xcd;
+    const int c_lo = seg * p.seg_chunks;
+    const int c_hi = c_lo + p.seg_chunks < p.n_chunks ? c_lo + p.seg_chunks : p.n_chunks;
+    if (bh >= p.BH || c_lo >= p.n_chunks) return;
+    const int b = bh / p.H, h = bh - b * p.H, N = p.N;
+    const T *Y = static_cast<const T *>(p.y) + b * p.ys_b + h * p.ys_h;
+    const T *Z = static_cast<const T *>(p.z) + b * p.zs_b + h * p.zs_h;
+    const int ys2 = (int)p.ys_n * 2, zs2 = (int)p.zs_n * 2;
+    const u32x4 ry = make_rsrc(Y, (uint32_t)((N - 1) * ys2 + p.dy * 2));
+    const u32x4 rz = make_rsrc(Z, (uint32_t)((N - 1) * zs2 + p.dz * 2));
+    const bool has_block = wave < W::NBLK;
+    const int dbk = wave / W::DB, eb = wave % W::DB;
+    f32x16 st;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) st[v] = 0.f;
+#pragma unroll 1
+    for (int c = c_lo; c < c_hi; ++c) {
+        walk_load_tile<D>(ry, lds0, c * kWalkRows, ys2, p.dy, wave, lane);
+        walk_load_tile<D>(rz, lds0 + W::TILE, c * kWalkRows, zs2, p.dz, wave, lane);
+        wait_vm<0>();
+        __syncthreads();
+        if (has_block) walk_update<T, D>(smem, smem + W::TILE, dbk, eb, lane, st);
+        __syncthreads();
+    }
+    if (has_block) {
+        float *out = p.totals + ((int64_t)bh * p.n_seg + seg) * (D * D);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) out[(32 * dbk + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * eb + l32] = st[v];
+    }
+#else
+    (void)p;
+#endif
+}
+
+// totals[bh][seg][e] -> exclusive sum over the segments before (reverse == 0) / after (reverse != 0), in
+// place.  One thread per pair of elements; the loads of sixteen segments are issued together (a
+// chain of dependent loads, one per segment, would cost a memory latency each).
+// (a template only so that the header can be included by several translation units)
+template <int kUnused = 0>
+__global__ __launch_bounds__(256) void walk_scan_kernel(float *totals, int n_seg, int E, int64_t total2, int reverse) {
+    typedef float f32x2 __attribute__((ext_vector_type(2)));
+    const int64_t i2 = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i2 >= total2) return;
+    const int64_t bh = (i2 * 2) / E, e = i2 * 2 - bh * E;
+    float *pt = totals + bh * n_seg * E + e;
+    const int64_t step = reverse ? -(int64_t)E : (int64_t)E;
+    if (reverse) pt += (int64_t)(n_seg - 1) * E;
+    f32x2 run = {0.f, 0.f};
+    int s = 0;
+    auto batch = [&](auto nn) {
+        constexpr int NB = decltype(nn)::value;
+        for (; s + NB <= n_seg; s += NB) {
+            f32x2 t[NB];
+#pragma unroll
+            for (int u = 0; u < NB; ++u) t[u] = *reinterpret_cast<const f32x2 *>(pt + u * step);
+#pragma unroll
+            for (int u = 0; u < NB; ++u) {
+                *reinterpret_cast<f32x2 *>(pt + u * step) = run;
+                run += t[u];
+            }
+            pt += NB * step;
+        }
+    };
+    batch(std::integral_constant<int, 16>{});
+    batch(std::integral_constant<int, 4>{});
+    batch(std::integral_constant<int, 1>{});
+}
+
+template <typename T, int D>
+hipError_t launch_walk_totals(const WalkTotalsParams &p, hipStream_t stream) {
+    const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
+    if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    constexpr auto kern = walk_totals_kernel<T, D>;
+    constexpr int smem = 2 * WalkCfg<D>::TILE;
+    if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
+    return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+}
+
+inline hipError_t launch_walk_scan(float *totals, int64_t BH, int n_seg, int E, int reverse, hipStream_t stream) {
+    const int64_t total2 = BH * E / 2;
+    return launch_kernel(walk_scan_kernel<0>, dim3((unsigned)((total2 + 255) / 256)), dim3(256), 0, stream, totals, n_seg,
+                         E, total2, reverse);
+}
+
+template <typename T, int D>
+hipError_t launch_walk_fwd(const WalkParams &p, hipStream_t stream) {
+    const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
+    if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    constexpr auto kern = walk_fwd_kernel<T, D>;
+    constexpr int smem = 3 * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
+    if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
+    return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+}
+
+template <typename T, int D>
+hipError_t launch_walk_bwd(const WalkParams &p, hipStream_t stream) {
+    const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
+    if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    constexpr auto kern = walk_bwd_kernel<T, D>;
+    constexpr int smem = 4 * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
+    if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
+    return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+}
+
+}  // namespace fla

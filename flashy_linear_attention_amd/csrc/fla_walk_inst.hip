@@ -1,0 +1,23 @@
+// Instantiations of the walk kernels (fla_chunk_walk.h): both storage types, padded head dims 32 and 64.
+#include "fla_dispatch.h"
+
+namespace fla {
+
+#define FLA_WALK_DISPATCH(fn, ...)                                                       \
+    if (dtype == 0) return D == 32 ? fn<__bf16, 32>(__VA_ARGS__) : fn<__bf16, 64>(__VA_ARGS__); \
+    return D == 32 ? fn<_Float16, 32>(__VA_ARGS__) : fn<_Float16, 64>(__VA_ARGS__)
+
+hipError_t walk_totals(int dtype, int D, const WalkTotalsParams &p, hipStream_t stream) {
+    FLA_WALK_DISPATCH(launch_walk_totals, p, stream);
+}
+hipError_t walk_fwd(int dtype, int D, const WalkParams &p, hipStream_t stream) {
+    FLA_WALK_DISPATCH(launch_walk_fwd, p, stream);
+}
+hipError_t walk_bwd(int dtype, int D, const WalkParams &p, hipStream_t stream) {
+    FLA_WALK_DISPATCH(launch_walk_bwd, p, stream);
+}
+hipError_t walk_scan(float *totals, int64_t BH, int n_seg, int E, int reverse, hipStream_t stream) {
+    return launch_walk_scan(totals, BH, n_seg, E, reverse, stream);
+}
+
+}  // namespace fla

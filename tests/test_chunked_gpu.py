@@ -138,7 +138,8 @@ def test_chunked_operator_workspace_is_checked(gpu_device):
     stream = torch.cuda.current_stream().cuda_stream
     need = lib.fla_linear_attn_chunked_workspace_bytes(1, 2, 1024, 64, 64)
     sbytes = lib.fla_linear_attn_chunked_state_bytes(1, 2, 1024, 64, 64)
-    assert need > 0 and sbytes == 2 * 4 * 64 * 64 * 2
+    assert need > 0 and sbytes == 2 * 8 * 64 * 64 * 2  # one 64 x 64 state per 128-row chunk and head
+    assert lib.fla_linear_attn_chunked_state_bytes(1, 2, 1024, 128, 128) == 2 * 4 * 128 * 128 * 2  # per 256-row chunk
     valid = ctypes.c_int32(7)
     rc = lib.fla_linear_attn_chunked_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), 1, 2, 1024, 64, 64,
                                          st(q), st(k), st(v), st(out), 0, None, ctypes.byref(valid), None, 0, stream)
