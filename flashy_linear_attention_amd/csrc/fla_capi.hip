@@ -382,7 +382,7 @@ WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     w.seg_chunks = total / 1024 > 1 ? total / 1024 : 1;
     if (w.seg_chunks > w.n_chunks) w.seg_chunks = w.n_chunks;
     w.n_seg = (w.n_chunks + w.seg_chunks - 1) / w.seg_chunks;
-    w.totals_bytes = w.n_seg > 1 ? B * H * w.n_seg * w.D * w.D * 4 : 0;
+    w.totals_bytes = B * H * w.n_seg * w.D * w.D * 4;  // (a single segment needs them only with a feature map)
     w.saved_bytes = B * H * w.n_chunks * w.D * w.D * 2;
     return w;
 }
@@ -390,8 +390,13 @@ WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
 // totals of Y^T Z per segment into `totals`, then their exclusive sums over the segments before
 // (reverse == 0) or after (reverse != 0)
 int walk_entry_states(const WalkPlan &w, const View &y, const View &z, int64_t B, int64_t H, int64_t N, int64_t dy,
-                      int64_t dz, int dtype, int reverse, float *totals, hipStream_t s) {
+                      int64_t dz, int dtype, int reverse, float *totals, hipStream_t s, int map_y = 0,
+                      const View *ymap_out = nullptr) {
     fla::WalkTotalsParams tp{};
+    if (map_y) {
+        tp.map_y = map_y, tp.ymap_out = const_cast<void *>(ymap_out->ptr);
+        tp.yo_b = ymap_out->strides[0], tp.yo_h = ymap_out->strides[1], tp.yo_n = ymap_out->strides[2];
+    }
     tp.y = y.ptr, tp.z = z.ptr, tp.totals = totals;
     tp.ys_b = y.strides[0], tp.ys_h = y.strides[1], tp.ys_n = y.strides[2];
     tp.zs_b = z.strides[0], tp.zs_h = z.strides[1], tp.zs_n = z.strides[2];
@@ -439,25 +444,36 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
     if (int rc = check_alias_fwd(q, k, v, o, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
     const WalkPlan wp = walk_plan(B, H, N, dqk, dv);
-    if (!fmap && wp.ok && fla::fast_path_ok(make_params(q, k, v, o, B, H, N, dqk, dv, 0))) {
-        if (wp.totals_bytes &&
+    if (wp.ok && fla::fast_path_ok(make_params(q, k, v, o, B, H, N, dqk, dv, 0)) &&
+        (!fmap || fla::fast_path_ok(make_params(mapped[0], mapped[1], v, o, B, H, N, dqk, dv, 0)))) {
+        // the segments' entry states; with a feature map the same kernel maps xk as it loads it and
+        // writes phi(xk), which the walk then reads (so it runs for a single segment as well)
+        const bool need_totals = wp.n_seg > 1 || fmap;
+        if (need_totals &&
             (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.totals_bytes))
             return FLA_ERR_WORKSPACE;
         if (state_out && reinterpret_cast<uintptr_t>(state_out) % 16 != 0) return FLA_ERR_WORKSPACE;
         hipStream_t s = static_cast<hipStream_t>(stream);
-        float *totals = wp.totals_bytes ? static_cast<float *>(workspace) : nullptr;
+        float *totals = need_totals ? static_cast<float *>(workspace) : nullptr;
         if (totals)
-            if (int rc = walk_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, totals, s)) return rc;
+            if (int rc = walk_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, totals, s, fmap, fmap ? &mapped[1] : nullptr))
+                return rc;
+        const View &kk = fmap ? mapped[1] : k;
         fla::WalkParams w{};
-        w.q = q.ptr, w.k = k.ptr, w.v = v.ptr, w.o = const_cast<void *>(o.ptr);
+        if (fmap) {
+            w.fmap = fmap, w.qmap_out = const_cast<void *>(mapped[0].ptr);
+            w.qo_b = mapped[0].strides[0], w.qo_h = mapped[0].strides[1], w.qo_n = mapped[0].strides[2];
+        }
+        w.q = q.ptr, w.k = kk.ptr, w.v = v.ptr, w.o = const_cast<void *>(o.ptr);
         w.qs_b = q.strides[0], w.qs_h = q.strides[1], w.qs_n = q.strides[2];
-        w.ks_b = k.strides[0], w.ks_h = k.strides[1], w.ks_n = k.strides[2];
+        w.ks_b = kk.strides[0], w.ks_h = kk.strides[1], w.ks_n = kk.strides[2];
         w.vs_b = v.strides[0], w.vs_h = v.strides[1], w.vs_n = v.strides[2];
         w.os_b = o.strides[0], w.os_h = o.strides[1], w.os_n = o.strides[2];
         w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dqk, w.wv = (int32_t)dv;
         w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
-        w.init = totals, w.saved = state_out;
+        w.init = wp.n_seg > 1 ? totals : nullptr, w.saved = state_out;
         if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
+        if (mapped_done) *mapped_done = true;
         if (state_out && state_valid) *state_valid = 1;
         return FLA_OK;
     }
@@ -511,16 +527,17 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         return launch_feature_pass(2, fmap, k, dk, B, H, N, dqk, dtype, stream);
     }
     const WalkPlan wp = walk_plan(B, H, N, dqk, dv);
-    if (!fmap && wp.ok && state_in) {  // (the states forward saved are per 128-row chunk: only this path reads them)
-        if (wp.totals_bytes &&
+    if (wp.ok && state_in) {  // (the states forward saved are per 128-row chunk: only this path reads them)
+        if (wp.n_seg > 1 &&
             (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.totals_bytes))
             return FLA_ERR_WORKSPACE;
         if (reinterpret_cast<uintptr_t>(state_in) % 16 != 0) return FLA_ERR_WORKSPACE;
         hipStream_t s = static_cast<hipStream_t>(stream);
-        float *totals = wp.totals_bytes ? static_cast<float *>(workspace) : nullptr;
+        float *totals = wp.n_seg > 1 ? static_cast<float *>(workspace) : nullptr;
         if (totals)
             if (int rc = walk_entry_states(wp, q, go, B, H, N, dqk, dv, dtype, 1, totals, s)) return rc;
         fla::WalkParams w{};
+        w.fmap = fmap;  // q, k hold phi(x): the slopes come from the LDS tiles
         w.q = q.ptr, w.k = k.ptr, w.v = v.ptr, w.go = go.ptr;
         w.dq = const_cast<void *>(dq.ptr), w.dk = const_cast<void *>(dk.ptr), w.dv = const_cast<void *>(dvv.ptr);
         w.qs_b = q.strides[0], w.qs_h = q.strides[1], w.qs_n = q.strides[2];
@@ -535,7 +552,7 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         w.init = totals, w.saved = const_cast<void *>(state_in);
         return fla::walk_bwd(dtype, wp.D, w, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
     }
-    if (wp.ok && !fmap) state_in = nullptr;  // not in the 256-row chunks' format: recomputed below
+    if (wp.ok) state_in = nullptr;  // not in the 256-row chunks' format: recomputed below
     if (fmap) set_output_slope(pq, fmap, q), set_output_slope(pk, fmap, k);
     const int64_t sb = shared_state_bytes(B, H, N, dqk, dv);
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < sb * (state_in ? 3 : 4))

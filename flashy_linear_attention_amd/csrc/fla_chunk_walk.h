@@ -56,6 +56,14 @@ struct WalkParams {
     // forward: where the 16-bit state at the entry of every chunk goes, [BH][n_chunks][D][D]
     // ([q/k index][v index]), or null; backward: the same buffer, read for dQ
     void *saved;
+    // Feature map (fla_feature.h), 0: none.  Forward: q holds the argument xq of the map phi; the Q
+    // tile is mapped in LDS as it lands and phi(xq) is written to qmap_out (q's shape, element
+    // strides qo_*); k already holds phi(xk) (written by the totals kernel).  Backward: q and k
+    // hold phi(xq), phi(xk), and dQ, dK are multiplied by the slope of phi, computed from those
+    // values in the LDS tiles, before they are rounded and stored.
+    int32_t fmap;
+    void *qmap_out;
+    int64_t qo_b, qo_h, qo_n;
 };
 
 template <int D>
@@ -193,19 +201,51 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
     }
 }
 
+// Every element of the landed tile replaced by phi(element), in place, and the mapped rows written
+// to `out` (rows >= N and chunks beyond the true width arrived as zeros and stay zeros).  The
+// caller synchronises before the tile is read.
+template <typename T, int D>
+__device__ __forceinline__ void walk_map_tile(unsigned char *tile, int fmap, int row0, int N, int width, T *out,
+                                              int64_t out_stride, int tid) {
+    using W = WalkCfg<D>;
+#pragma unroll
+    for (int v = 0; v < kWalkRows * W::CR / 256; ++v) {
+        const int u = tid + 256 * v, r = u / W::CR, pos = u % W::CR, c = pos ^ swizzle_y<W::CR>(r);
+        if (row0 + r < N && c * 8 < width) {
+            u32x4 *ptr = reinterpret_cast<u32x4 *>(tile + r * W::RB + (pos << 4));
+            const u32x4 m = feature_map8<T>(fmap, *ptr);
+            *ptr = m;
+            *reinterpret_cast<u32x4 *>(out + (int64_t)(row0 + r) * out_stride + c * 8) = m;
+        }
+    }
+}
+
 // acc[db][v] = Out[row][32 db + 16 g + v]: two 16-byte stores per block; rows >= N and columns beyond
-// the true width fall outside the buffer resource and are dropped
+// the true width fall outside the buffer resource and are dropped.  With a feature map, `ytile` is
+// the LDS tile holding y = phi(x) for the same rows (tile row `trow`) and Out is multiplied by the
+// slope phi'(x), computed from y, first.
 template <typename T, int D>
 __device__ __forceinline__ void walk_store(__amdgpu_buffer_rsrc_t rs, int stride2, int width, int row, int g,
-                                           const f32x16 (&acc)[WalkCfg<D>::DB]) {
+                                           const f32x16 (&acc)[WalkCfg<D>::DB], int fmap = 0,
+                                           const unsigned char *ytile = nullptr, int trow = 0) {
+    using W = WalkCfg<D>;
     using V8 = typename Mma<T>::V8;
 #pragma unroll
     for (int db = 0; db < WalkCfg<D>::DB; ++db) {
 #pragma unroll
         for (int hq = 0; hq < 2; ++hq) {
+            float f[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) f[e] = acc[db][8 * hq + e];
+            if (fmap) {
+                const int ch = (4 * db + 2 * g + hq) ^ swizzle_y<W::CR>(trow);
+                const V8 y = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4 *>(ytile + trow * W::RB + (ch << 4)));
+#pragma unroll
+                for (int e = 0; e < 8; ++e) f[e] *= feature_slope_from_value(fmap, static_cast<float>(y[e]));
+            }
             V8 o8;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o8[e] = static_cast<T>(acc[db][8 * hq + e]);
+            for (int e = 0; e < 8; ++e) o8[e] = static_cast<T>(f[e]);
             const int col = 32 * db + 16 * g + 8 * hq;
             const uint32_t off = (uint32_t)(row * stride2 + col * 2) + (col < width ? 0u : kOobOffset);
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o8), rs, off, 0, 0);
@@ -302,6 +342,11 @@ __global__ __launch_bounds__(256, 2) void walk_fwd_kernel(const WalkParams p) {
         walk_load_tile<D>(rv, lds0 + 2 * W::TILE, row0, vs2, p.wv, wave, lane);
         wait_vm<0>();
         __syncthreads();  // the tiles have landed; the state written by the previous iteration is visible
+        if (p.fmap) {
+            walk_map_tile<T, D>(tq, p.fmap, row0, N, p.wqk, static_cast<T *>(p.qmap_out) + b * p.qo_b + h * p.qo_h,
+                                p.qo_n, tid);
+            __syncthreads();
+        }
         f32x16 acc[W::DB];
         walk_product<T, D, false>(tq, tk, tv, wave, lane, c > 0, [&](int db, int kc) -> V8 {
             return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g);
@@ -389,7 +434,7 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
         f32x16 acc[W::DB];
         // dQ = lower(dO V^T) K + dO S_c^T
         walk_product<T, D, false>(tg, tv, tk, wave, lane, c > 0, [&](int db, int kc) -> V8 { return sfq[db][kc]; }, acc);
-        walk_store<T, D>(rdq, dqs2, p.wqk, row, g, acc);
+        walk_store<T, D>(rdq, dqs2, p.wqk, row, g, acc, p.fmap, tq, 32 * wave + l32);
         // dV = upper(K Q^T) dO + K R: A operand R^T[v index][q/k index] = the LDS copy as it is
         walk_product<T, D, true>(tk, tq, tg, wave, lane, later, [&](int db, int kc) -> V8 {
             return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g);
@@ -399,7 +444,7 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
         walk_product<T, D, true>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
             return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
         }, acc);
-        walk_store<T, D>(rdk, dks2, p.wqk, row, g, acc);
+        walk_store<T, D>(rdk, dks2, p.wqk, row, g, acc, p.fmap, tk, 32 * wave + l32);
         if (has_block) walk_update<T, D>(tq, tg, dbk, eb, lane, st);
         __syncthreads();
         if (has_block) walk_state_to_lds<T, D>(tl, dbk, eb, lane, st);
@@ -416,6 +461,11 @@ struct WalkTotalsParams {
     int32_t H, N, BH, dy, dz;
     int32_t n_chunks, seg_chunks, n_seg;
     float *totals;
+    // feature map on load: Y holds the argument of the map; every Y tile is mapped in LDS as it lands
+    // and the mapped rows are written to ymap_out (Y's shape, element strides yo_*).  0: none.
+    int32_t map_y;
+    void *ymap_out;
+    int64_t yo_b, yo_h, yo_n;
 };
 
 template <typename T, int D>
@@ -448,6 +498,11 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
         walk_load_tile<D>(rz, lds0 + W::TILE, c * kWalkRows, zs2, p.dz, wave, lane);
         wait_vm<0>();
         __syncthreads();
+        if (p.map_y) {
+            walk_map_tile<T, D>(smem, p.map_y, c * kWalkRows, N, p.dy, static_cast<T *>(p.ymap_out) + b * p.yo_b + h * p.yo_h,
+                                p.yo_n, tid);
+            __syncthreads();
+        }
         if (has_block) walk_update<T, D>(smem, smem + W::TILE, dbk, eb, lane, st);
         __syncthreads();
     }
