@@ -492,19 +492,37 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
     f32x16 st;
 #pragma unroll
     for (int v = 0; v < 16; ++v) st[v] = 0.f;
+    // two sets of tiles: the loads of chunk c + 1 are in flight while chunk c is multiplied
+    auto load_chunk = [&](int c, int buf) {
+        walk_load_tile<D>(ry, lds0 + buf * 2 * W::TILE, c * kWalkRows, ys2, p.dy, wave, lane);
+        walk_load_tile<D>(rz, lds0 + buf * 2 * W::TILE + W::TILE, c * kWalkRows, zs2, p.dz, wave, lane);
+    };
+    load_chunk(c_lo, 0);
 #pragma unroll 1
     for (int c = c_lo; c < c_hi; ++c) {
-        walk_load_tile<D>(ry, lds0, c * kWalkRows, ys2, p.dy, wave, lane);
-        walk_load_tile<D>(rz, lds0 + W::TILE, c * kWalkRows, zs2, p.dz, wave, lane);
-        wait_vm<0>();
-        __syncthreads();
+        const int buf = (c - c_lo) & 1;
+        unsigned char *ty = smem + buf * 2 * W::TILE, *tz = ty + W::TILE;
+        const bool more = c + 1 < c_hi;
+        if (more) load_chunk(c + 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
+        // this wave's loads of chunk c have landed: only those of chunk c + 1 may still be in flight
+        // (the mapped rows' stores of a feature map share the counter: then everything is awaited)
+        if (more && !p.map_y)
+            wait_vm<2 * W::NI>();
+        else
+            wait_vm<0>();
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
         if (p.map_y) {
-            walk_map_tile<T, D>(smem, p.map_y, c * kWalkRows, N, p.dy, static_cast<T *>(p.ymap_out) + b * p.yo_b + h * p.yo_h,
+            walk_map_tile<T, D>(ty, p.map_y, c * kWalkRows, N, p.dy, static_cast<T *>(p.ymap_out) + b * p.yo_b + h * p.yo_h,
                                 p.yo_n, tid);
-            __syncthreads();
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the rewritten tile is in LDS
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
         }
-        if (has_block) walk_update<T, D>(smem, smem + W::TILE, dbk, eb, lane, st);
-        __syncthreads();
+        if (has_block) walk_update<T, D>(ty, tz, dbk, eb, lane, st);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS reads of the set are done
+        __builtin_amdgcn_s_barrier();
     }
     if (has_block) {
         float *out = p.totals + ((int64_t)bh * p.n_seg + seg) * (D * D);
@@ -555,7 +573,7 @@ hipError_t launch_walk_totals(const WalkTotalsParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     constexpr auto kern = walk_totals_kernel<T, D>;
-    constexpr int smem = 2 * WalkCfg<D>::TILE;
+    constexpr int smem = 4 * WalkCfg<D>::TILE;
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
     return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
 }
