@@ -360,25 +360,35 @@ int run_tri_chunked(const View &x, const View &y, const View &z, const View &out
 // so forward can hand its state to backward, and backward computes one new state instead of
 // three.  Any other shape evaluates each product on its own.
 
-// ---- equal padded head dims up to 64: the walk kernels (fla_chunk_walk.h).  A workgroup walks a
-// segment of 128-row chunks with the running state in registers; segment entry states come from
-// a totals kernel and a scan over the segments.
+// ---- equal padded head dims up to 128: the walk kernels (fla_chunk_walk.h).  A workgroup walks a
+// segment of chunks (128 rows, 64 at D = 128) with the running state in registers; segment entry
+// states come from a totals kernel and a scan over the segments.
+//   D <= 64: forward saves the 16-bit state at the entry of every chunk, and one backward kernel
+//            computes dQ, dV and dK of a chunk from one set of tiles;
+//   D = 128 (`split`): a per-chunk state would cost as much traffic as an operand, so forward hands
+//            over its segments' fp32 entry states only; backward is a forward-direction walk for dQ
+//            (from those entry states, transposed) and a reverse walk for dK and dV whose
+//            workgroups (one per CU, two sets of tiles) cover two segments each.
 struct WalkPlan {
-    bool ok;
-    int D;
+    bool ok, split;
+    int D, rows;
     int64_t n_chunks, seg_chunks, n_seg;
     int64_t totals_bytes;  // fp32 entry states of the segments (0 with a single segment)
-    int64_t saved_bytes;   // 16-bit state at the entry of every chunk, forward -> backward
+    int64_t saved_bytes;   // what forward hands to backward: per-chunk 16-bit states / split: the entry states
+    int64_t bwd_seg_chunks, bwd_n_seg;  // split: segments of the dK/dV walk (pairs of the segments above)
 };
 
 constexpr int64_t kWalkWorkgroups = 512;
 
 WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     WalkPlan w{};
-    w.ok = pad_index(dqk) == pad_index(dv) && padded(dqk) <= 64 && N > fla::kWalkRows;
-    if (!w.ok) return w;
+    if (pad_index(dqk) != pad_index(dv) || padded(dqk) > 128) return w;
     w.D = (int)padded(dqk);
-    w.n_chunks = (N + fla::kWalkRows - 1) / fla::kWalkRows;
+    w.rows = fla::walk_rows(w.D);
+    w.split = w.D > 64;
+    w.ok = N > (w.split ? 256 : w.rows);  // (D = 128: up to 256 rows one diagonal block of the quadratic kernel does it)
+    if (!w.ok) return w;
+    w.n_chunks = (N + w.rows - 1) / w.rows;
     // as many workgroups as are resident at once, two per CU (measured at B H = 16, N = 32768, D = 64:
     // 256 / 512 / 1024 / 2048 workgroups give 0.265 / 0.231 / 0.243 / 0.268 ms per forward + backward)
     const int64_t total = B * H * w.n_chunks;
@@ -386,7 +396,9 @@ WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     if (w.seg_chunks > w.n_chunks) w.seg_chunks = w.n_chunks;
     w.n_seg = (w.n_chunks + w.seg_chunks - 1) / w.seg_chunks;
     w.totals_bytes = B * H * w.n_seg * w.D * w.D * 4;  // (a single segment needs them only with a feature map)
-    w.saved_bytes = B * H * w.n_chunks * w.D * w.D * 2;
+    w.saved_bytes = w.split ? w.totals_bytes : B * H * w.n_chunks * w.D * w.D * 2;
+    w.bwd_seg_chunks = 2 * w.seg_chunks;
+    w.bwd_n_seg = (w.n_chunks + w.bwd_seg_chunks - 1) / w.bwd_seg_chunks;
     return w;
 }
 
@@ -418,10 +430,11 @@ bool states_shareable(int64_t dqk, int64_t dv, int64_t N) {
 // bytes of one rounded running state / of the scratch one state computation needs (fp32 chunk states)
 int64_t shared_state_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     const WalkPlan w = walk_plan(B, H, N, dqk, dv);
-    if (w.ok) return w.saved_bytes;  // one state per 128-row chunk (also room for the 256-row chunks' states)
-    if (!states_shareable(dqk, dv, N)) return 0;
+    if (w.ok && !w.split) return w.saved_bytes;  // one state per 128-row chunk (also room for the 256-row chunks' states)
+    if (!states_shareable(dqk, dv, N)) return w.ok ? w.saved_bytes : 0;
     const int64_t rows = chunk_rows(dqk, dv);
-    return B * H * ((N + rows - 1) / rows) * padded(dqk) * padded(dv) * 2;
+    const int64_t per_chunk = B * H * ((N + rows - 1) / rows) * padded(dqk) * padded(dv) * 2;
+    return w.ok && w.saved_bytes > per_chunk ? w.saved_bytes : per_chunk;  // (split: either path's state fits)
 }
 
 int64_t chunked_op_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
@@ -447,17 +460,20 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
     if (int rc = check_alias_fwd(q, k, v, o, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
     const WalkPlan wp = walk_plan(B, H, N, dqk, dv);
-    if (wp.ok && fla::fast_path_ok(make_params(q, k, v, o, B, H, N, dqk, dv, 0)) &&
+    // (the split kernels take no feature map: those calls go through the 256-row chunks below)
+    if (wp.ok && !(wp.split && fmap) && fla::fast_path_ok(make_params(q, k, v, o, B, H, N, dqk, dv, 0)) &&
         (!fmap || fla::fast_path_ok(make_params(mapped[0], mapped[1], v, o, B, H, N, dqk, dv, 0)))) {
         // the segments' entry states; with a feature map the same kernel maps xk as it loads it and
         // writes phi(xk), which the walk then reads (so it runs for a single segment as well)
         const bool need_totals = wp.n_seg > 1 || fmap;
-        if (need_totals &&
+        // split: the entry states are what backward gets, so they are computed in place in state_out
+        const bool in_state = wp.split && state_out;
+        if (need_totals && !in_state &&
             (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.totals_bytes))
             return FLA_ERR_WORKSPACE;
         if (state_out && reinterpret_cast<uintptr_t>(state_out) % 16 != 0) return FLA_ERR_WORKSPACE;
         hipStream_t s = static_cast<hipStream_t>(stream);
-        float *totals = need_totals ? static_cast<float *>(workspace) : nullptr;
+        float *totals = need_totals ? static_cast<float *>(in_state ? state_out : workspace) : nullptr;
         if (totals)
             if (int rc = walk_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, totals, s, fmap, fmap ? &mapped[1] : nullptr))
                 return rc;
@@ -474,7 +490,8 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         w.os_b = o.strides[0], w.os_h = o.strides[1], w.os_n = o.strides[2];
         w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dqk, w.wv = (int32_t)dv;
         w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
-        w.init = wp.n_seg > 1 ? totals : nullptr, w.saved = state_out;
+        w.init = wp.n_seg > 1 ? totals : nullptr, w.saved = wp.split ? nullptr : state_out;
+        w.init_n_seg = (int32_t)wp.n_seg, w.init_mul = 1;
         if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
         if (mapped_done) *mapped_done = true;
         if (state_out && state_valid) *state_valid = 1;
@@ -530,7 +547,45 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         return launch_feature_pass(2, fmap, k, dk, B, H, N, dqk, dtype, stream);
     }
     const WalkPlan wp = walk_plan(B, H, N, dqk, dv);
-    if (wp.ok && state_in) {  // (the states forward saved are per 128-row chunk: only this path reads them)
+    const bool walk = wp.ok && state_in && !(wp.split && fmap);  // (what forward saved is in this path's format)
+    if (walk && wp.split) {
+        if (wp.n_seg > 1 &&
+            (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.totals_bytes))
+            return FLA_ERR_WORKSPACE;
+        if (reinterpret_cast<uintptr_t>(state_in) % 16 != 0) return FLA_ERR_WORKSPACE;
+        hipStream_t s = static_cast<hipStream_t>(stream);
+        float *totals = wp.n_seg > 1 ? static_cast<float *>(workspace) : nullptr;
+        if (totals)
+            if (int rc = walk_entry_states(wp, q, go, B, H, N, dqk, dv, dtype, 1, totals, s)) return rc;
+        // dQ = lower(dO V^T) K + dO S^T: the forward walk over (dO, V, K), its states V^T K = S^T
+        fla::WalkParams w{};
+        w.q = go.ptr, w.k = v.ptr, w.v = k.ptr, w.o = const_cast<void *>(dq.ptr);
+        w.qs_b = go.strides[0], w.qs_h = go.strides[1], w.qs_n = go.strides[2];
+        w.ks_b = v.strides[0], w.ks_h = v.strides[1], w.ks_n = v.strides[2];
+        w.vs_b = k.strides[0], w.vs_h = k.strides[1], w.vs_n = k.strides[2];
+        w.os_b = dq.strides[0], w.os_h = dq.strides[1], w.os_n = dq.strides[2];
+        w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dv, w.wv = (int32_t)dqk;
+        w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
+        w.init = wp.n_seg > 1 ? static_cast<const float *>(state_in) : nullptr;
+        w.init_n_seg = (int32_t)wp.n_seg, w.init_mul = 1, w.init_transposed = 1;
+        if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
+        // dV, dK: the reverse walk; a workgroup covers two of the segments the totals were taken over
+        // and enters with the sum over the segments after its second one
+        fla::WalkParams r{};
+        r.q = q.ptr, r.k = k.ptr, r.v = v.ptr, r.go = go.ptr;
+        r.dk = const_cast<void *>(dk.ptr), r.dv = const_cast<void *>(dvv.ptr);
+        r.qs_b = q.strides[0], r.qs_h = q.strides[1], r.qs_n = q.strides[2];
+        r.ks_b = k.strides[0], r.ks_h = k.strides[1], r.ks_n = k.strides[2];
+        r.vs_b = v.strides[0], r.vs_h = v.strides[1], r.vs_n = v.strides[2];
+        r.gs_b = go.strides[0], r.gs_h = go.strides[1], r.gs_n = go.strides[2];
+        r.dks_b = dk.strides[0], r.dks_h = dk.strides[1], r.dks_n = dk.strides[2];
+        r.dvs_b = dvv.strides[0], r.dvs_h = dvv.strides[1], r.dvs_n = dvv.strides[2];
+        r.H = (int32_t)H, r.N = (int32_t)N, r.BH = (int32_t)(B * H), r.wqk = (int32_t)dqk, r.wv = (int32_t)dv;
+        r.n_chunks = (int32_t)wp.n_chunks, r.seg_chunks = (int32_t)wp.bwd_seg_chunks, r.n_seg = (int32_t)wp.bwd_n_seg;
+        r.init = totals, r.init_n_seg = (int32_t)wp.n_seg, r.init_mul = 2, r.init_add = 1;
+        return fla::walk_dkdv(dtype, wp.D, r, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+    }
+    if (walk) {  // (the states forward saved are per 128-row chunk: only this path reads them)
         if (wp.n_seg > 1 &&
             (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.totals_bytes))
             return FLA_ERR_WORKSPACE;
@@ -553,9 +608,10 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dqk, w.wv = (int32_t)dv;
         w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
         w.init = totals, w.saved = const_cast<void *>(state_in);
+        w.init_n_seg = (int32_t)wp.n_seg, w.init_mul = 1;
         return fla::walk_bwd(dtype, wp.D, w, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
     }
-    if (wp.ok) state_in = nullptr;  // not in the 256-row chunks' format: recomputed below
+    if (wp.ok && !(wp.split && fmap)) state_in = nullptr;  // not in the 256-row chunks' format: recomputed below
     if (fmap) set_output_slope(pq, fmap, q), set_output_slope(pk, fmap, k);
     const int64_t sb = shared_state_bytes(B, H, N, dqk, dv);
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < sb * (state_in ? 3 : 4))

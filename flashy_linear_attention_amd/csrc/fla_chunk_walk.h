@@ -39,7 +39,8 @@
 
 namespace fla {
 
-constexpr int kWalkRows = 128;  // rows per chunk of the walk kernels
+// rows per chunk of the walk kernels: 128, or 64 at D = 128 (tiles and state must share the LDS)
+constexpr int walk_rows(int D) { return D <= 64 ? 128 : 64; }
 
 struct WalkParams {
     const void *q, *k, *v, *go;  // operands (go: backward only); (B, H, N, D)
@@ -47,12 +48,15 @@ struct WalkParams {
     int64_t qs_b, qs_h, qs_n, ks_b, ks_h, ks_n, vs_b, vs_h, vs_n, gs_b, gs_h, gs_n;
     int64_t os_b, os_h, os_n, dqs_b, dqs_h, dqs_n, dks_b, dks_h, dks_n, dvs_b, dvs_h, dvs_n;
     int32_t H, N, BH, wqk, wv;   // true widths of q/k and of v (<= D)
-    int32_t n_chunks;            // ceil(N / 128)
+    int32_t n_chunks;            // ceil(N / rows per chunk)
     int32_t seg_chunks, n_seg;   // chunks per segment, segments per (b, h)
-    // entry state of every segment, fp32 [BH][n_seg][D (q/k index)][D (v index)]: sum of K^T V over
-    // the segments before (forward) / of Q^T dO over the segments after (backward); null when
-    // there is a single segment (entry state zero)
+    // entry state of every segment, fp32 [BH][init_n_seg][D (q/k index)][D (v index)]: sum of K^T V
+    // over the segments before (forward) / of Q^T dO over the segments after (backward); null when
+    // there is a single segment (entry state zero).  Segment s of this launch starts from entry
+    // min(s * init_mul + init_add, init_n_seg - 1): the totals may be kept over finer segments than
+    // the walk's.  init_transposed: the buffer holds the transposed matrices ([v index][q/k index]).
     const float *init;
+    int32_t init_n_seg, init_mul, init_add, init_transposed;
     // forward: where the 16-bit state at the entry of every chunk goes, [BH][n_chunks][D][D]
     // ([q/k index][v index]), or null; backward: the same buffer, read for dQ
     void *saved;
@@ -68,7 +72,7 @@ struct WalkParams {
 
 template <int D>
 struct WalkCfg {
-    static constexpr int C = kWalkRows;
+    static constexpr int C = walk_rows(D);  // rows per chunk
     static constexpr int RB = D * 2;        // bytes per tile row
     static constexpr int CR = D / 8;        // 16-byte chunks per row
     static constexpr int TILE = C * RB;     // bytes per operand tile
@@ -77,9 +81,25 @@ struct WalkCfg {
     static constexpr int RPI = 1024 / RB;   // rows covered by one wave-level 1 KiB load
     static constexpr int NI = TILE / 4096;  // such loads per wave and tile
     static constexpr int STATE = D * RB;    // the 16-bit state in LDS
-    static constexpr int NBLK = DB * DB;    // 32 x 32 blocks of the state: block b belongs to wave b
-    static_assert(D == 32 || D == 64, "walk kernels are built for padded head dims 32 and 64");
-    static_assert(NBLK <= 4, "one state block per wave at most");
+    static constexpr int NBLK = DB * DB;    // 32 x 32 blocks of the state: block b belongs to wave b % 4
+    static constexpr int NBW = (NBLK + 3) / 4;  // state blocks per wave
+    // a wave owns one 32-row block of the chunk as the X rows of every product, and -- with fewer
+    // than four such blocks -- one part of the output columns
+    static constexpr int NRB = C / 32;      // row blocks per chunk
+    static constexpr int NCH = 4 / NRB;     // column parts
+    static constexpr int DBW = DB / NCH;    // 32-wide output blocks per wave
+    static_assert(D == 32 || D == 64 || D == 128, "walk kernels are built for padded head dims 32, 64 and 128");
+    static_assert(NRB * NCH == 4 && DBW * NCH == DB, "four waves tile the chunk's rows and output columns");
+};
+
+// state block i of wave `wave`: (block of q/k indices, block of v indices); the v block is the
+// same for all blocks of a wave
+template <int D>
+struct WalkBlock {
+    using W = WalkCfg<D>;
+    __device__ static __forceinline__ bool valid(int wave, int i) { return wave + 4 * i < W::NBLK; }
+    __device__ static __forceinline__ int dbk(int wave, int i) { return (wave + 4 * i) / W::DB; }
+    __device__ static __forceinline__ int eb(int wave) { return wave % W::DB; }
 };
 
 // ---- LDS tile access (tile: row-major [rows][D], chunk index XOR swizzle_y(row))
@@ -148,31 +168,34 @@ __device__ __forceinline__ typename Mma<T>::V8 walk_col_frag(const unsigned char
 // (the permutation of walk_col_frag_perm)
 __device__ __forceinline__ int walk_e_lane(int l32) { return 16 * ((l32 >> 2) & 1) + 4 * (l32 >> 3) + (l32 & 3); }
 
-// ---- one product of a chunk for this wave's 32 X rows:
+// ---- one product of a chunk for this wave's 32 X rows (row block rb = wave % NRB) and its part of
+// the output columns (blocks db0 .. db0 + DBW - 1, db0 = (wave / NRB) * DBW):
 //   acc = [state: X_w . State]  +  mask(X_w Y^T) Z        (UPPER: keep row <= column, else row >= column)
 // xt, yt, zt: LDS tiles; sfrag(db, kc): the state's A-operand fragment for output block db, k chunk kc.
+// (With several column parts the waves of one row block each compute the same scores.)
 template <typename T, int D, bool UPPER, typename SFrag>
 __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsigned char *yt, const unsigned char *zt,
                                              int wave, int lane, bool has_state, SFrag &&sfrag,
-                                             f32x16 (&acc)[WalkCfg<D>::DB]) {
+                                             f32x16 (&acc)[WalkCfg<D>::DBW]) {
     using W = WalkCfg<D>;
     using M = Mma<T>;
     using V8 = typename M::V8;
     const int l32 = lane & 31, g = lane >> 5;
+    const int rb = W::NCH == 1 ? wave : wave % W::NRB, db0 = W::NCH == 1 ? 0 : (wave / W::NRB) * W::DBW;
     V8 xf[W::KC];
 #pragma unroll
-    for (int kc = 0; kc < W::KC; ++kc) xf[kc] = walk_row_frag<T, D>(xt, 32 * wave + l32, kc, g);
+    for (int kc = 0; kc < W::KC; ++kc) xf[kc] = walk_row_frag<T, D>(xt, 32 * rb + l32, kc, g);
 #pragma unroll
-    for (int db = 0; db < W::DB; ++db)
+    for (int i = 0; i < W::DBW; ++i)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[db][v] = 0.f;
+        for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
     if (has_state) {
 #pragma unroll
-        for (int db = 0; db < W::DB; ++db)
+        for (int i = 0; i < W::DBW; ++i)
 #pragma unroll
-            for (int kc = 0; kc < W::KC; ++kc) acc[db] = M::mma(sfrag(db, kc), xf[kc], acc[db]);
+            for (int kc = 0; kc < W::KC; ++kc) acc[i] = M::mma(sfrag(db0 + i, kc), xf[kc], acc[i]);
     }
-    const int s_lo = UPPER ? wave : 0, s_hi = UPPER ? 3 : wave;
+    const int s_lo = UPPER ? rb : 0, s_hi = UPPER ? W::NRB - 1 : rb;
 #pragma unroll 1
     for (int s = s_lo; s <= s_hi; ++s) {
         f32x16 sc;
@@ -180,7 +203,7 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
         for (int v = 0; v < 16; ++v) sc[v] = 0.f;
 #pragma unroll
         for (int kc = 0; kc < W::KC; ++kc) sc = M::mma(walk_row_frag<T, D>(yt, 32 * s + l32, kc, g), xf[kc], sc);
-        if (s == wave) {  // the 32 x 32 block on the diagonal: lane = X row l32, register v = Y row jl
+        if (s == rb) {  // the 32 x 32 block on the diagonal: lane = X row l32, register v = Y row jl
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int jl = 8 * (v / 4) + 4 * g + (v % 4);
@@ -196,8 +219,8 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int db = 0; db < W::DB; ++db)
-                acc[db] = M::mma(walk_col_frag_perm<T, D>(zt, 32 * s + 16 * t, db, lane, false), pf[t], acc[db]);
+            for (int i = 0; i < W::DBW; ++i)
+                acc[i] = M::mma(walk_col_frag_perm<T, D>(zt, 32 * s + 16 * t, db0 + i, lane, false), pf[t], acc[i]);
     }
 }
 
@@ -209,7 +232,7 @@ __device__ __forceinline__ void walk_map_tile(unsigned char *tile, int fmap, int
                                               int64_t out_stride, int tid) {
     using W = WalkCfg<D>;
 #pragma unroll
-    for (int v = 0; v < kWalkRows * W::CR / 256; ++v) {
+    for (int v = 0; v < W::C * W::CR / 256; ++v) {
         const int u = tid + 256 * v, r = u / W::CR, pos = u % W::CR, c = pos ^ swizzle_y<W::CR>(r);
         if (row0 + r < N && c * 8 < width) {
             u32x4 *ptr = reinterpret_cast<u32x4 *>(tile + r * W::RB + (pos << 4));
@@ -220,23 +243,24 @@ __device__ __forceinline__ void walk_map_tile(unsigned char *tile, int fmap, int
     }
 }
 
-// acc[db][v] = Out[row][32 db + 16 g + v]: two 16-byte stores per block; rows >= N and columns beyond
-// the true width fall outside the buffer resource and are dropped.  With a feature map, `ytile` is
-// the LDS tile holding y = phi(x) for the same rows (tile row `trow`) and Out is multiplied by the
-// slope phi'(x), computed from y, first.
+// acc[i][v] = Out[row][32 (db0 + i) + 16 g + v]: two 16-byte stores per block; rows >= N and columns
+// beyond the true width fall outside the buffer resource and are dropped.  With a feature map,
+// `ytile` is the LDS tile holding y = phi(x) for the same rows (tile row `trow`) and Out is
+// multiplied by the slope phi'(x), computed from y, first.
 template <typename T, int D>
-__device__ __forceinline__ void walk_store(__amdgpu_buffer_rsrc_t rs, int stride2, int width, int row, int g,
-                                           const f32x16 (&acc)[WalkCfg<D>::DB], int fmap = 0,
+__device__ __forceinline__ void walk_store(__amdgpu_buffer_rsrc_t rs, int stride2, int width, int row, int g, int db0,
+                                           const f32x16 (&acc)[WalkCfg<D>::DBW], int fmap = 0,
                                            const unsigned char *ytile = nullptr, int trow = 0) {
     using W = WalkCfg<D>;
     using V8 = typename Mma<T>::V8;
 #pragma unroll
-    for (int db = 0; db < WalkCfg<D>::DB; ++db) {
+    for (int i = 0; i < W::DBW; ++i) {
+        const int db = db0 + i;
 #pragma unroll
         for (int hq = 0; hq < 2; ++hq) {
             float f[8];
 #pragma unroll
-            for (int e = 0; e < 8; ++e) f[e] = acc[db][8 * hq + e];
+            for (int e = 0; e < 8; ++e) f[e] = acc[i][8 * hq + e];
             if (fmap) {
                 const int ch = (4 * db + 2 * g + hq) ^ swizzle_y<W::CR>(trow);
                 const V8 y = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4 *>(ytile + trow * W::RB + (ch << 4)));
@@ -253,30 +277,44 @@ __device__ __forceinline__ void walk_store(__amdgpu_buffer_rsrc_t rs, int stride
     }
 }
 
-// state += Y^T Z over the 128 rows of the tiles, this wave's 32 x 32 block (dbk: block of Y columns,
-// eb: block of Z columns): st[v] = State[32 dbk + 8(v/4) + 4g + v%4][32 eb + l32]
+// state += Y^T Z over the rows of the tiles, this wave's 32 x 32 blocks (block i: Y columns of block
+// dbk(i), Z columns of block eb): st[i][v] = State[32 dbk(i) + 8(v/4) + 4g + v%4][32 eb + l32]
 template <typename T, int D>
-__device__ __forceinline__ void walk_update(const unsigned char *yt, const unsigned char *zt, int dbk, int eb, int lane,
-                                            f32x16 &st) {
+__device__ __forceinline__ void walk_update(const unsigned char *yt, const unsigned char *zt, int wave, int lane,
+                                            f32x16 (&st)[WalkCfg<D>::NBW]) {
+    using W = WalkCfg<D>;
     using M = Mma<T>;
+    using B = WalkBlock<D>;
+    if (!B::valid(wave, 0)) return;
 #pragma unroll
-    for (int ks = 0; ks < kWalkRows / 16; ++ks)
-        st = M::mma(walk_col_frag<T, D>(yt, 16 * ks, dbk, lane), walk_col_frag<T, D>(zt, 16 * ks, eb, lane), st);
+    for (int ks = 0; ks < W::C / 16; ++ks) {
+        const typename M::V8 zf = walk_col_frag<T, D>(zt, 16 * ks, B::eb(wave), lane);
+#pragma unroll
+        for (int i = 0; i < W::NBW; ++i)
+            if (B::valid(wave, i)) st[i] = M::mma(walk_col_frag<T, D>(yt, 16 * ks, B::dbk(wave, i), lane), zf, st[i]);
+    }
 }
 
 // the state rounded to 16 bit into LDS as T[v index][q/k index] (row = 32 eb + l32, four consecutive
 // columns per register group), in the tile layout
 template <typename T, int D>
-__device__ __forceinline__ void walk_state_to_lds(unsigned char *tl, int dbk, int eb, int lane, const f32x16 &st) {
+__device__ __forceinline__ void walk_state_to_lds(unsigned char *tl, int wave, int lane,
+                                                  const f32x16 (&st)[WalkCfg<D>::NBW]) {
     using W = WalkCfg<D>;
+    using B = WalkBlock<D>;
     typedef T t4 __attribute__((ext_vector_type(4)));
-    const int l32 = lane & 31, g = lane >> 5, row = 32 * eb + l32;
+    const int l32 = lane & 31, g = lane >> 5, row = 32 * B::eb(wave) + l32;
 #pragma unroll
-    for (int a = 0; a < 4; ++a) {
-        t4 w;
+    for (int i = 0; i < W::NBW; ++i) {
+        if (!B::valid(wave, i)) continue;
+        const int dbk = B::dbk(wave, i);
 #pragma unroll
-        for (int b = 0; b < 4; ++b) w[b] = static_cast<T>(st[4 * a + b]);
-        *reinterpret_cast<t4 *>(tl + row * W::RB + (((4 * dbk + a) ^ swizzle_y<W::CR>(row)) << 4) + 8 * g) = w;
+        for (int a = 0; a < 4; ++a) {
+            t4 w;
+#pragma unroll
+            for (int b = 0; b < 4; ++b) w[b] = static_cast<T>(st[i][4 * a + b]);
+            *reinterpret_cast<t4 *>(tl + row * W::RB + (((4 * dbk + a) ^ swizzle_y<W::CR>(row)) << 4) + 8 * g) = w;
+        }
     }
 }
 
@@ -297,24 +335,46 @@ __device__ __forceinline__ WalkSlice walk_slice(const WalkParams &p) {
     return s;
 }
 
+// this wave's blocks of the entry state of segment sl.seg (zeros without an init buffer)
 template <int D>
-__device__ __forceinline__ void walk_load_init(const float *init, int dbk, int eb, int lane, f32x16 &st) {
+__device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSlice &sl, int wave, int lane,
+                                               f32x16 (&st)[WalkCfg<D>::NBW]) {
+    using W = WalkCfg<D>;
+    using B = WalkBlock<D>;
     const int l32 = lane & 31, g = lane >> 5;
+    const float *init = nullptr;
+    if (p.init) {
+        int idx = sl.seg * p.init_mul + p.init_add;
+        idx = idx < p.init_n_seg - 1 ? idx : p.init_n_seg - 1;
+        init = p.init + ((int64_t)sl.bh * p.init_n_seg + idx) * (D * D);
+    }
 #pragma unroll
-    for (int v = 0; v < 16; ++v) st[v] = init ? init[(32 * dbk + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * eb + l32] : 0.f;
+    for (int i = 0; i < W::NBW; ++i) {
+        const int dbk = B::dbk(wave, i), eb = B::eb(wave);
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int r = 32 * dbk + 8 * (v / 4) + 4 * g + (v % 4), c = 32 * eb + l32;
+            st[i][v] = init && B::valid(wave, i) ? (p.init_transposed ? init[c * D + r] : init[r * D + c]) : 0.f;
+        }
+    }
 }
 
-// ---- forward: O_c = lower(Q_c K_c^T) V_c + Q_c S, S += K_c^T V_c, chunks ascending
+// ---- one product with its running state, chunks ascending:
+//   O_c = lower(Q_c K_c^T) V_c + Q_c S, then S += K_c^T V_c
+// (forward as named; dQ of the split backward with q <- dO, k <- V, v <- K, o <- dQ and the entry
+// states read transposed)
 template <typename T, int D>
 __global__ __launch_bounds__(256, 2) void walk_fwd_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
     using V8 = typename Mma<T>::V8;
+    using B = WalkBlock<D>;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     unsigned char *tq = smem, *tk = smem + W::TILE, *tv = smem + 2 * W::TILE, *tl = smem + 3 * W::TILE;
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rb = W::NCH == 1 ? wave : wave % W::NRB, db0 = W::NCH == 1 ? 0 : (wave / W::NRB) * W::DBW;
     const WalkSlice sl = walk_slice(p);
     if (!sl.valid) return;
     const int b = sl.bh / p.H, h = sl.bh - b * p.H, N = p.N;
@@ -328,15 +388,13 @@ __global__ __launch_bounds__(256, 2) void walk_fwd_kernel(const WalkParams p) {
     const u32x4 rv = make_rsrc(V, (uint32_t)((N - 1) * vs2 + p.wv * 2));
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(O, 0, (N - 1) * os2 + p.wv * 2, 0x00020000);
 
-    const bool has_block = wave < W::NBLK;
-    const int dbk = wave / W::DB, eb = wave % W::DB;
-    f32x16 st;
-    walk_load_init<D>(p.init ? p.init + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D) : nullptr, dbk, eb, lane, st);
-    if (has_block) walk_state_to_lds<T, D>(tl, dbk, eb, lane, st);
+    f32x16 st[W::NBW];
+    walk_load_init<D>(p, sl, wave, lane, st);
+    walk_state_to_lds<T, D>(tl, wave, lane, st);
 
 #pragma unroll 1
     for (int c = sl.c_lo; c < sl.c_hi; ++c) {
-        const int row0 = c * kWalkRows;
+        const int row0 = c * W::C;
         walk_load_tile<D>(rq, lds0, row0, qs2, p.wqk, wave, lane);
         walk_load_tile<D>(rk, lds0 + W::TILE, row0, ks2, p.wqk, wave, lane);
         walk_load_tile<D>(rv, lds0 + 2 * W::TILE, row0, vs2, p.wv, wave, lane);
@@ -347,22 +405,25 @@ __global__ __launch_bounds__(256, 2) void walk_fwd_kernel(const WalkParams p) {
                                 p.qo_n, tid);
             __syncthreads();
         }
-        f32x16 acc[W::DB];
+        f32x16 acc[W::DBW];
         walk_product<T, D, false>(tq, tk, tv, wave, lane, c > 0, [&](int db, int kc) -> V8 {
             return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g);
         }, acc);
-        walk_store<T, D>(ro, os2, p.wv, row0 + 32 * wave + l32, g, acc);
-        if (has_block) {
-            if (p.saved) {  // the state at the entry of this chunk, [q/k index][v index], for backward's dQ
-                T *sv = static_cast<T *>(p.saved) + ((int64_t)sl.bh * p.n_chunks + c) * (D * D);
+        walk_store<T, D>(ro, os2, p.wv, row0 + 32 * rb + l32, g, db0, acc);
+        if (p.saved) {  // the state at the entry of this chunk, [q/k index][v index], for backward's dQ
+            T *sv = static_cast<T *>(p.saved) + ((int64_t)sl.bh * p.n_chunks + c) * (D * D);
 #pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    sv[(32 * dbk + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * eb + l32] = static_cast<T>(st[v]);
-            }
-            walk_update<T, D>(tk, tv, dbk, eb, lane, st);
+            for (int i = 0; i < W::NBW; ++i)
+                if (B::valid(wave, i)) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        sv[(32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * B::eb(wave) + l32] =
+                            static_cast<T>(st[i][v]);
+                }
         }
+        walk_update<T, D>(tk, tv, wave, lane, st);
         __syncthreads();  // every wave is done with the tiles and with the old state
-        if (has_block) walk_state_to_lds<T, D>(tl, dbk, eb, lane, st);
+        walk_state_to_lds<T, D>(tl, wave, lane, st);
     }
 #else
     (void)p;
@@ -375,6 +436,7 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
     using V8 = typename Mma<T>::V8;
+    static_assert(W::NCH == 1, "the fused backward keeps dQ's state fragments of all output blocks in registers");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     unsigned char *tq = smem, *tk = smem + W::TILE, *tv = smem + 2 * W::TILE, *tg = smem + 3 * W::TILE,
@@ -401,15 +463,13 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
     const __amdgpu_buffer_rsrc_t rdk = __builtin_amdgcn_make_buffer_rsrc(DK, 0, (N - 1) * dks2 + p.wqk * 2, 0x00020000);
     const __amdgpu_buffer_rsrc_t rdv = __builtin_amdgcn_make_buffer_rsrc(DV, 0, (N - 1) * dvs2 + p.wv * 2, 0x00020000);
 
-    const bool has_block = wave < W::NBLK;
-    const int dbk = wave / W::DB, eb = wave % W::DB;
-    f32x16 st;  // R[q/k index][v index]
-    walk_load_init<D>(p.init ? p.init + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D) : nullptr, dbk, eb, lane, st);
-    if (has_block) walk_state_to_lds<T, D>(tl, dbk, eb, lane, st);
+    f32x16 st[W::NBW];  // R[q/k index][v index]
+    walk_load_init<D>(p, sl, wave, lane, st);
+    walk_state_to_lds<T, D>(tl, wave, lane, st);
 
 #pragma unroll 1
     for (int c = sl.c_hi - 1; c >= sl.c_lo; --c) {
-        const int row0 = c * kWalkRows;
+        const int row0 = c * W::C;
         walk_load_tile<D>(rq, lds0, row0, qs2, p.wqk, wave, lane);
         walk_load_tile<D>(rk, lds0 + W::TILE, row0, ks2, p.wqk, wave, lane);
         walk_load_tile<D>(rv, lds0 + 2 * W::TILE, row0, vs2, p.wv, wave, lane);
@@ -431,23 +491,108 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
         __syncthreads();
         const int row = row0 + 32 * wave + l32;
         const bool later = c + 1 < p.n_chunks;  // chunks after this one exist: R is not identically zero
-        f32x16 acc[W::DB];
+        f32x16 acc[W::DBW];
         // dQ = lower(dO V^T) K + dO S_c^T
         walk_product<T, D, false>(tg, tv, tk, wave, lane, c > 0, [&](int db, int kc) -> V8 { return sfq[db][kc]; }, acc);
-        walk_store<T, D>(rdq, dqs2, p.wqk, row, g, acc, p.fmap, tq, 32 * wave + l32);
+        walk_store<T, D>(rdq, dqs2, p.wqk, row, g, 0, acc, p.fmap, tq, 32 * wave + l32);
         // dV = upper(K Q^T) dO + K R: A operand R^T[v index][q/k index] = the LDS copy as it is
         walk_product<T, D, true>(tk, tq, tg, wave, lane, later, [&](int db, int kc) -> V8 {
             return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g);
         }, acc);
-        walk_store<T, D>(rdv, dvs2, p.wv, row, g, acc);
+        walk_store<T, D>(rdv, dvs2, p.wv, row, g, 0, acc);
         // dK = upper(V dO^T) Q + V R^T: A operand R[q/k index][v index] = the LDS copy read transposed
         walk_product<T, D, true>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
             return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
         }, acc);
-        walk_store<T, D>(rdk, dks2, p.wqk, row, g, acc, p.fmap, tk, 32 * wave + l32);
-        if (has_block) walk_update<T, D>(tq, tg, dbk, eb, lane, st);
+        walk_store<T, D>(rdk, dks2, p.wqk, row, g, 0, acc, p.fmap, tk, 32 * wave + l32);
+        walk_update<T, D>(tq, tg, wave, lane, st);
         __syncthreads();
-        if (has_block) walk_state_to_lds<T, D>(tl, dbk, eb, lane, st);
+        walk_state_to_lds<T, D>(tl, wave, lane, st);
+    }
+#else
+    (void)p;
+#endif
+}
+
+// ---- backward without saved per-chunk states, dV and dK: chunks descending, R += Q_c^T dO_c.  One
+// workgroup per CU with two sets of tiles: the loads of the next chunk are in flight while this
+// one is multiplied.  (dQ is a walk_fwd_kernel launch over dO, V, K.)
+template <typename T, int D>
+__global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    using W = WalkCfg<D>;
+    using V8 = typename Mma<T>::V8;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    unsigned char *tl = smem + 8 * W::TILE;
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rb = W::NCH == 1 ? wave : wave % W::NRB, db0 = W::NCH == 1 ? 0 : (wave / W::NRB) * W::DBW;
+    const WalkSlice sl = walk_slice(p);
+    if (!sl.valid) return;
+    const int b = sl.bh / p.H, h = sl.bh - b * p.H, N = p.N;
+    const T *Q = static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h;
+    const T *K = static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h;
+    const T *V = static_cast<const T *>(p.v) + b * p.vs_b + h * p.vs_h;
+    const T *G = static_cast<const T *>(p.go) + b * p.gs_b + h * p.gs_h;
+    T *DK = static_cast<T *>(p.dk) + b * p.dks_b + h * p.dks_h;
+    T *DV = static_cast<T *>(p.dv) + b * p.dvs_b + h * p.dvs_h;
+    const int qs2 = (int)p.qs_n * 2, ks2 = (int)p.ks_n * 2, vs2 = (int)p.vs_n * 2, gs2 = (int)p.gs_n * 2;
+    const int dks2 = (int)p.dks_n * 2, dvs2 = (int)p.dvs_n * 2;
+    const u32x4 rq = make_rsrc(Q, (uint32_t)((N - 1) * qs2 + p.wqk * 2));
+    const u32x4 rk = make_rsrc(K, (uint32_t)((N - 1) * ks2 + p.wqk * 2));
+    const u32x4 rv = make_rsrc(V, (uint32_t)((N - 1) * vs2 + p.wv * 2));
+    const u32x4 rg = make_rsrc(G, (uint32_t)((N - 1) * gs2 + p.wv * 2));
+    const __amdgpu_buffer_rsrc_t rdk = __builtin_amdgcn_make_buffer_rsrc(DK, 0, (N - 1) * dks2 + p.wqk * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rdv = __builtin_amdgcn_make_buffer_rsrc(DV, 0, (N - 1) * dvs2 + p.wv * 2, 0x00020000);
+
+    f32x16 st[W::NBW];  // R[q/k index][v index]
+    walk_load_init<D>(p, sl, wave, lane, st);
+    walk_state_to_lds<T, D>(tl, wave, lane, st);
+
+    auto load_chunk = [&](int c, int buf) {
+        const uint32_t base = lds0 + buf * 4 * W::TILE;
+        const int row0 = c * W::C;
+        walk_load_tile<D>(rq, base, row0, qs2, p.wqk, wave, lane);
+        walk_load_tile<D>(rk, base + W::TILE, row0, ks2, p.wqk, wave, lane);
+        walk_load_tile<D>(rv, base + 2 * W::TILE, row0, vs2, p.wv, wave, lane);
+        walk_load_tile<D>(rg, base + 3 * W::TILE, row0, gs2, p.wv, wave, lane);
+    };
+    load_chunk(sl.c_hi - 1, 0);
+#pragma unroll 1
+    for (int c = sl.c_hi - 1; c >= sl.c_lo; --c) {
+        const int buf = (sl.c_hi - 1 - c) & 1;
+        unsigned char *tq = smem + buf * 4 * W::TILE, *tk = tq + W::TILE, *tv = tq + 2 * W::TILE, *tg = tq + 3 * W::TILE;
+        const bool more = c > sl.c_lo;
+        if (more) load_chunk(c - 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
+        // this wave's loads of chunk c have landed when at most the loads issued after them are
+        // outstanding (the stores of the previous chunk were issued before those)
+        if (more)
+            wait_vm<4 * W::NI>();
+        else
+            wait_vm<0>();
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's part of the state is in LDS
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        const int row = c * W::C + 32 * rb + l32;
+        const bool later = c + 1 < p.n_chunks;  // chunks after this one exist: R is not identically zero
+        f32x16 acc[W::DBW];
+        // dV = upper(K Q^T) dO + K R: A operand R^T[v index][q/k index] = the LDS copy as it is
+        walk_product<T, D, true>(tk, tq, tg, wave, lane, later, [&](int db, int kc) -> V8 {
+            return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g);
+        }, acc);
+        walk_store<T, D>(rdv, dvs2, p.wv, row, g, db0, acc);
+        // dK = upper(V dO^T) Q + V R^T: A operand R[q/k index][v index] = the LDS copy read transposed
+        walk_product<T, D, true>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
+            return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
+        }, acc);
+        walk_store<T, D>(rdk, dks2, p.wqk, row, g, db0, acc);
+        walk_update<T, D>(tq, tg, wave, lane, st);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS reads of the tiles and of the state are done
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        walk_state_to_lds<T, D>(tl, wave, lane, st);
     }
 #else
     (void)p;
@@ -487,15 +632,16 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
     const int ys2 = (int)p.ys_n * 2, zs2 = (int)p.zs_n * 2;
     const u32x4 ry = make_rsrc(Y, (uint32_t)((N - 1) * ys2 + p.dy * 2));
     const u32x4 rz = make_rsrc(Z, (uint32_t)((N - 1) * zs2 + p.dz * 2));
-    const bool has_block = wave < W::NBLK;
-    const int dbk = wave / W::DB, eb = wave % W::DB;
-    f32x16 st;
+    using B = WalkBlock<D>;
+    f32x16 st[W::NBW];
 #pragma unroll
-    for (int v = 0; v < 16; ++v) st[v] = 0.f;
+    for (int i = 0; i < W::NBW; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) st[i][v] = 0.f;
     // two sets of tiles: the loads of chunk c + 1 are in flight while chunk c is multiplied
     auto load_chunk = [&](int c, int buf) {
-        walk_load_tile<D>(ry, lds0 + buf * 2 * W::TILE, c * kWalkRows, ys2, p.dy, wave, lane);
-        walk_load_tile<D>(rz, lds0 + buf * 2 * W::TILE + W::TILE, c * kWalkRows, zs2, p.dz, wave, lane);
+        walk_load_tile<D>(ry, lds0 + buf * 2 * W::TILE, c * W::C, ys2, p.dy, wave, lane);
+        walk_load_tile<D>(rz, lds0 + buf * 2 * W::TILE + W::TILE, c * W::C, zs2, p.dz, wave, lane);
     };
     load_chunk(c_lo, 0);
 #pragma unroll 1
@@ -513,22 +659,25 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         if (p.map_y) {
-            walk_map_tile<T, D>(ty, p.map_y, c * kWalkRows, N, p.dy, static_cast<T *>(p.ymap_out) + b * p.yo_b + h * p.yo_h,
+            walk_map_tile<T, D>(ty, p.map_y, c * W::C, N, p.dy, static_cast<T *>(p.ymap_out) + b * p.yo_b + h * p.yo_h,
                                 p.yo_n, tid);
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the rewritten tile is in LDS
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
         }
-        if (has_block) walk_update<T, D>(ty, tz, dbk, eb, lane, st);
+        walk_update<T, D>(ty, tz, wave, lane, st);
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS reads of the set are done
         __builtin_amdgcn_s_barrier();
     }
-    if (has_block) {
-        float *out = p.totals + ((int64_t)bh * p.n_seg + seg) * (D * D);
+    float *out = p.totals + ((int64_t)bh * p.n_seg + seg) * (D * D);
 #pragma unroll
-        for (int v = 0; v < 16; ++v) out[(32 * dbk + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * eb + l32] = st[v];
-    }
+    for (int i = 0; i < W::NBW; ++i)
+        if (B::valid(wave, i)) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                out[(32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * B::eb(wave) + l32] = st[i][v];
+        }
 #else
     (void)p;
 #endif
@@ -600,6 +749,17 @@ hipError_t launch_walk_bwd(const WalkParams &p, hipStream_t stream) {
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     constexpr auto kern = walk_bwd_kernel<T, D>;
     constexpr int smem = 4 * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
+    if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
+    return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+}
+
+template <typename T, int D>
+hipError_t launch_walk_dkdv(const WalkParams &p, hipStream_t stream) {
+    const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
+    if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    constexpr auto kern = walk_dkdv_kernel<T, D>;
+    constexpr int smem = 8 * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
+    static_assert(smem <= 160 * 1024, "two sets of tiles and the state must fit the LDS of a CU");
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
     return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
 }

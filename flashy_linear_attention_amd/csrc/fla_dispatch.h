@@ -40,9 +40,11 @@ FLA_FOR_EACH_DIM_PAIR(FLA_DECLARE)
     hipError_t FLA_CBATCH_NAME(1, d)(const TriBatch &b, int count, hipStream_t stream);
 FLA_DECLARE_BATCH(32) FLA_DECLARE_BATCH(64) FLA_DECLARE_BATCH(128) FLA_DECLARE_BATCH(256)
 #undef FLA_DECLARE_BATCH
-// walk kernels (fla_chunk_walk.h), dtype 0 bf16 / 1 f16, padded head dim D = 32 or 64
+// walk kernels (fla_chunk_walk.h), dtype 0 bf16 / 1 f16, padded head dim D = 32, 64 or 128
+// (walk_bwd: 32 and 64; walk_dkdv: 128)
 hipError_t walk_totals(int dtype, int D, const WalkTotalsParams &p, hipStream_t stream);
 hipError_t walk_fwd(int dtype, int D, const WalkParams &p, hipStream_t stream);
 hipError_t walk_bwd(int dtype, int D, const WalkParams &p, hipStream_t stream);
+hipError_t walk_dkdv(int dtype, int D, const WalkParams &p, hipStream_t stream);
 hipError_t walk_scan(float *totals, int64_t BH, int n_seg, int E, int reverse, hipStream_t stream);
 }  // namespace fla

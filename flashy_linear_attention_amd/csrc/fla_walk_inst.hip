@@ -1,4 +1,5 @@
-// Instantiations of the walk kernels (fla_chunk_walk.h): both storage types, padded head dims 32 and 64.
+// Instantiations of the walk kernels (fla_chunk_walk.h): both storage types, padded head dims 32, 64 and 128
+// (128: no fused backward -- dQ is a forward-direction walk, dK and dV a kernel of their own).
 #include "fla_dispatch.h"
 
 namespace fla {
@@ -7,14 +8,23 @@ namespace fla {
     if (dtype == 0) return D == 32 ? fn<__bf16, 32>(__VA_ARGS__) : fn<__bf16, 64>(__VA_ARGS__); \
     return D == 32 ? fn<_Float16, 32>(__VA_ARGS__) : fn<_Float16, 64>(__VA_ARGS__)
 
+hipError_t walk_bwd(int dtype, int D, const WalkParams &p, hipStream_t stream) {
+    if (D == 128) return hipErrorNotSupported;
+    FLA_WALK_DISPATCH(launch_walk_bwd, p, stream);
+}
+#define FLA_WALK_DISPATCH3(fn, ...)                                                                 \
+    if (D == 128) return dtype == 0 ? fn<__bf16, 128>(__VA_ARGS__) : fn<_Float16, 128>(__VA_ARGS__); \
+    FLA_WALK_DISPATCH(fn, __VA_ARGS__)
+
+hipError_t walk_dkdv(int dtype, int D, const WalkParams &p, hipStream_t stream) {
+    if (D != 128) return hipErrorNotSupported;
+    return dtype == 0 ? launch_walk_dkdv<__bf16, 128>(p, stream) : launch_walk_dkdv<_Float16, 128>(p, stream);
+}
 hipError_t walk_totals(int dtype, int D, const WalkTotalsParams &p, hipStream_t stream) {
-    FLA_WALK_DISPATCH(launch_walk_totals, p, stream);
+    FLA_WALK_DISPATCH3(launch_walk_totals, p, stream);
 }
 hipError_t walk_fwd(int dtype, int D, const WalkParams &p, hipStream_t stream) {
-    FLA_WALK_DISPATCH(launch_walk_fwd, p, stream);
-}
-hipError_t walk_bwd(int dtype, int D, const WalkParams &p, hipStream_t stream) {
-    FLA_WALK_DISPATCH(launch_walk_bwd, p, stream);
+    FLA_WALK_DISPATCH3(launch_walk_fwd, p, stream);
 }
 hipError_t walk_scan(float *totals, int64_t BH, int n_seg, int E, int reverse, hipStream_t stream) {
     return launch_walk_scan(totals, BH, n_seg, E, reverse, stream);
