@@ -363,22 +363,24 @@ int run_tri_chunked(const View &x, const View &y, const View &z, const View &out
 // ---- equal padded head dims up to 128: the walk kernels (fla_chunk_walk.h).  A workgroup walks a
 // segment of chunks (128 rows, 64 at D = 128) with the running state in registers; segment entry
 // states come from a totals kernel and a scan over the segments.
-//   D <= 64: forward saves the 16-bit state at the entry of every chunk, and one backward kernel
-//            computes dQ, dV and dK of a chunk from one set of tiles;
-//   D = 128 (`split`): a per-chunk state would cost as much traffic as an operand, so forward hands
-//            over its segments' fp32 entry states only; backward is a forward-direction walk for dQ
-//            (from those entry states, transposed) and a reverse walk for dK and dV whose
-//            workgroups (one per CU, two sets of tiles) cover two segments each.
+//   D <= 64: two workgroups per CU; forward saves the 16-bit state at the entry of every chunk, and
+//            one backward kernel computes dQ, dV and dK of a chunk from one set of tiles;
+//   D = 128 (`split`): one workgroup per CU with two sets of tiles.  A per-chunk state would cost as
+//            much traffic as an operand, so forward hands over its segments' fp32 entry states
+//            only; backward is a forward-direction walk for dQ (from those entry states,
+//            transposed) and a reverse walk for dK and dV.  The totals kernel keeps two workgroups
+//            per CU busy on a part of the sequence only (the last segment's total is never
+//            needed), so it works on `m` finer segments per walk segment.
 struct WalkPlan {
     bool ok, split;
     int D, rows;
-    int64_t n_chunks, seg_chunks, n_seg;
-    int64_t totals_bytes;  // fp32 entry states of the segments (0 with a single segment)
-    int64_t saved_bytes;   // what forward hands to backward: per-chunk 16-bit states / split: the entry states
-    int64_t bwd_seg_chunks, bwd_n_seg;  // split: segments of the dK/dV walk (pairs of the segments above)
+    int64_t n_chunks, seg_chunks, n_seg;  // the walks' segments
+    int64_t m;                            // totals: finer segments per walk segment (seg_chunks / m chunks each)
+    int64_t fine_bytes;                   // fp32 totals of the finer segments
+    int64_t entry_bytes;                  // fp32 entry states of the walk segments (in place over the totals when m == 1)
+    int64_t work_bytes;                   // workspace of one direction: totals, and entry states when m > 1
+    int64_t saved_bytes;                  // what forward hands to backward: per-chunk 16-bit states / split: the entry states
 };
-
-constexpr int64_t kWalkWorkgroups = 512;
 
 WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     WalkPlan w{};
@@ -389,36 +391,49 @@ WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     w.ok = N > (w.split ? 256 : w.rows);  // (D = 128: up to 256 rows one diagonal block of the quadratic kernel does it)
     if (!w.ok) return w;
     w.n_chunks = (N + w.rows - 1) / w.rows;
-    // as many workgroups as are resident at once, two per CU (measured at B H = 16, N = 32768, D = 64:
+    // as many workgroups as are resident at once (measured at B H = 16, N = 32768, D = 64, two per CU:
     // 256 / 512 / 1024 / 2048 workgroups give 0.265 / 0.231 / 0.243 / 0.268 ms per forward + backward)
-    const int64_t total = B * H * w.n_chunks;
-    w.seg_chunks = total / kWalkWorkgroups > 1 ? total / kWalkWorkgroups : 1;
-    if (w.seg_chunks > w.n_chunks) w.seg_chunks = w.n_chunks;
+    const int64_t target = w.split ? 256 : 512, total = B * H * w.n_chunks;
+    w.seg_chunks = total / target > 1 ? total / target : 1;
+    w.m = !w.split ? 1 : w.seg_chunks >= 4 ? 4 : w.seg_chunks >= 2 ? 2 : 1;
+    w.seg_chunks = (w.seg_chunks + w.m - 1) / w.m * w.m;
+    if (w.seg_chunks >= w.n_chunks) w.seg_chunks = w.n_chunks, w.m = 1;  // a single segment: no totals
     w.n_seg = (w.n_chunks + w.seg_chunks - 1) / w.seg_chunks;
-    w.totals_bytes = B * H * w.n_seg * w.D * w.D * 4;  // (a single segment needs them only with a feature map)
-    w.saved_bytes = w.split ? w.totals_bytes : B * H * w.n_chunks * w.D * w.D * 2;
-    w.bwd_seg_chunks = 2 * w.seg_chunks;
-    w.bwd_n_seg = (w.n_chunks + w.bwd_seg_chunks - 1) / w.bwd_seg_chunks;
+    w.entry_bytes = B * H * w.n_seg * w.D * w.D * 4;
+    w.fine_bytes = w.entry_bytes * w.m;
+    w.work_bytes = w.fine_bytes + (w.m > 1 ? w.entry_bytes : 0);  // (a single segment needs them only with a feature map)
+    w.saved_bytes = w.split ? w.entry_bytes : B * H * w.n_chunks * w.D * w.D * 2;
     return w;
 }
 
-// totals of Y^T Z per segment into `totals`, then their exclusive sums over the segments before
-// (reverse == 0) or after (reverse != 0)
+// totals of Y^T Z over the finer segments into `work`, then the walk segments' entry states: their
+// sums over the segments before (reverse == 0) or after (reverse != 0), written to `entry` (null:
+// behind the totals in `work`, or over them when m == 1).  Returns where the entry states are.
 int walk_entry_states(const WalkPlan &w, const View &y, const View &z, int64_t B, int64_t H, int64_t N, int64_t dy,
-                      int64_t dz, int dtype, int reverse, float *totals, hipStream_t s, int map_y = 0,
-                      const View *ymap_out = nullptr) {
+                      int64_t dz, int dtype, int reverse, void *work, float *entry, const float **where, hipStream_t s,
+                      int map_y = 0, const View *ymap_out = nullptr) {
     fla::WalkTotalsParams tp{};
     if (map_y) {
         tp.map_y = map_y, tp.ymap_out = const_cast<void *>(ymap_out->ptr);
         tp.yo_b = ymap_out->strides[0], tp.yo_h = ymap_out->strides[1], tp.yo_n = ymap_out->strides[2];
     }
+    float *totals = static_cast<float *>(work);
+    if (!entry) entry = w.m == 1 ? totals : reinterpret_cast<float *>(static_cast<char *>(work) + w.fine_bytes);
     tp.y = y.ptr, tp.z = z.ptr, tp.totals = totals;
     tp.ys_b = y.strides[0], tp.ys_h = y.strides[1], tp.ys_n = y.strides[2];
     tp.zs_b = z.strides[0], tp.zs_h = z.strides[1], tp.zs_n = z.strides[2];
     tp.H = (int32_t)H, tp.N = (int32_t)N, tp.BH = (int32_t)(B * H), tp.dy = (int32_t)dy, tp.dz = (int32_t)dz;
-    tp.n_chunks = (int32_t)w.n_chunks, tp.seg_chunks = (int32_t)w.seg_chunks, tp.n_seg = (int32_t)w.n_seg;
+    const int64_t n_fine = w.n_seg * w.m;
+    tp.n_chunks = (int32_t)w.n_chunks, tp.seg_chunks = (int32_t)(w.seg_chunks / w.m), tp.n_seg = (int32_t)n_fine;
+    // the total of the walk's last segment (first, walking in reverse) is under no sum; a feature map
+    // is applied by this kernel, which then has to visit every row
+    tp.seg_lo = reverse && !map_y ? (int32_t)w.m : 0;
+    tp.seg_hi = (int32_t)(!reverse && !map_y ? n_fine - w.m : n_fine);
     if (fla::walk_totals(dtype, w.D, tp, s) != hipSuccess) return FLA_ERR_LAUNCH;
-    return fla::walk_scan(totals, B * H, (int)w.n_seg, w.D * w.D, reverse, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+    *where = entry;
+    return fla::walk_scan(totals, entry, B * H, (int)w.n_seg, (int)w.m, w.D * w.D, reverse, s) == hipSuccess
+               ? FLA_OK
+               : FLA_ERR_LAUNCH;
 }
 
 bool states_shareable(int64_t dqk, int64_t dv, int64_t N) {
@@ -439,7 +454,10 @@ int64_t shared_state_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t
 
 int64_t chunked_op_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     const int64_t shared = shared_state_bytes(B, H, N, dqk, dv);
-    if (shared) return shared * 4;  // fp32 chunk states (2x) + two rounded states (backward without a saved one)
+    if (shared) {  // fp32 chunk states (2x) + two rounded states (backward without a saved one); the walk's totals
+        const WalkPlan w = walk_plan(B, H, N, dqk, dv);
+        return w.ok && w.work_bytes > shared * 4 ? w.work_bytes : shared * 4;
+    }
     int64_t m = chunked_bytes(B, H, N, dqk, dv);
     const int64_t t = chunked_bytes(B, H, N, dv, dqk);
     return m > t ? m : t;
@@ -466,16 +484,20 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         // the segments' entry states; with a feature map the same kernel maps xk as it loads it and
         // writes phi(xk), which the walk then reads (so it runs for a single segment as well)
         const bool need_totals = wp.n_seg > 1 || fmap;
-        // split: the entry states are what backward gets, so they are computed in place in state_out
+        // split: the entry states are what backward gets, so the scan writes them to state_out
+        // (m == 1: the totals themselves are computed there, and no workspace is used)
         const bool in_state = wp.split && state_out;
-        if (need_totals && !in_state &&
-            (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.totals_bytes))
+        if (need_totals && !(in_state && wp.m == 1) &&
+            (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 ||
+             workspace_bytes < (in_state ? wp.fine_bytes : wp.work_bytes)))
             return FLA_ERR_WORKSPACE;
         if (state_out && reinterpret_cast<uintptr_t>(state_out) % 16 != 0) return FLA_ERR_WORKSPACE;
         hipStream_t s = static_cast<hipStream_t>(stream);
-        float *totals = need_totals ? static_cast<float *>(in_state ? state_out : workspace) : nullptr;
-        if (totals)
-            if (int rc = walk_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, totals, s, fmap, fmap ? &mapped[1] : nullptr))
+        const float *entry = nullptr;
+        if (need_totals)
+            if (int rc = walk_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, in_state && wp.m == 1 ? state_out : workspace,
+                                           in_state ? static_cast<float *>(state_out) : nullptr, &entry, s, fmap,
+                                           fmap ? &mapped[1] : nullptr))
                 return rc;
         const View &kk = fmap ? mapped[1] : k;
         fla::WalkParams w{};
@@ -490,8 +512,7 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         w.os_b = o.strides[0], w.os_h = o.strides[1], w.os_n = o.strides[2];
         w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dqk, w.wv = (int32_t)dv;
         w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
-        w.init = wp.n_seg > 1 ? totals : nullptr, w.saved = wp.split ? nullptr : state_out;
-        w.init_n_seg = (int32_t)wp.n_seg, w.init_mul = 1;
+        w.init = wp.n_seg > 1 ? entry : nullptr, w.saved = wp.split ? nullptr : state_out;
         if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
         if (mapped_done) *mapped_done = true;
         if (state_out && state_valid) *state_valid = 1;
@@ -550,13 +571,13 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
     const bool walk = wp.ok && state_in && !(wp.split && fmap);  // (what forward saved is in this path's format)
     if (walk && wp.split) {
         if (wp.n_seg > 1 &&
-            (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.totals_bytes))
+            (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.work_bytes))
             return FLA_ERR_WORKSPACE;
         if (reinterpret_cast<uintptr_t>(state_in) % 16 != 0) return FLA_ERR_WORKSPACE;
         hipStream_t s = static_cast<hipStream_t>(stream);
-        float *totals = wp.n_seg > 1 ? static_cast<float *>(workspace) : nullptr;
-        if (totals)
-            if (int rc = walk_entry_states(wp, q, go, B, H, N, dqk, dv, dtype, 1, totals, s)) return rc;
+        const float *entry = nullptr;
+        if (wp.n_seg > 1)
+            if (int rc = walk_entry_states(wp, q, go, B, H, N, dqk, dv, dtype, 1, workspace, nullptr, &entry, s)) return rc;
         // dQ = lower(dO V^T) K + dO S^T: the forward walk over (dO, V, K), its states V^T K = S^T
         fla::WalkParams w{};
         w.q = go.ptr, w.k = v.ptr, w.v = k.ptr, w.o = const_cast<void *>(dq.ptr);
@@ -566,11 +587,9 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         w.os_b = dq.strides[0], w.os_h = dq.strides[1], w.os_n = dq.strides[2];
         w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dv, w.wv = (int32_t)dqk;
         w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
-        w.init = wp.n_seg > 1 ? static_cast<const float *>(state_in) : nullptr;
-        w.init_n_seg = (int32_t)wp.n_seg, w.init_mul = 1, w.init_transposed = 1;
+        w.init = wp.n_seg > 1 ? static_cast<const float *>(state_in) : nullptr, w.init_transposed = 1;
         if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
-        // dV, dK: the reverse walk; a workgroup covers two of the segments the totals were taken over
-        // and enters with the sum over the segments after its second one
+        // dV, dK: the reverse walk over the same segments
         fla::WalkParams r{};
         r.q = q.ptr, r.k = k.ptr, r.v = v.ptr, r.go = go.ptr;
         r.dk = const_cast<void *>(dk.ptr), r.dv = const_cast<void *>(dvv.ptr);
@@ -581,19 +600,19 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         r.dks_b = dk.strides[0], r.dks_h = dk.strides[1], r.dks_n = dk.strides[2];
         r.dvs_b = dvv.strides[0], r.dvs_h = dvv.strides[1], r.dvs_n = dvv.strides[2];
         r.H = (int32_t)H, r.N = (int32_t)N, r.BH = (int32_t)(B * H), r.wqk = (int32_t)dqk, r.wv = (int32_t)dv;
-        r.n_chunks = (int32_t)wp.n_chunks, r.seg_chunks = (int32_t)wp.bwd_seg_chunks, r.n_seg = (int32_t)wp.bwd_n_seg;
-        r.init = totals, r.init_n_seg = (int32_t)wp.n_seg, r.init_mul = 2, r.init_add = 1;
+        r.n_chunks = (int32_t)wp.n_chunks, r.seg_chunks = (int32_t)wp.seg_chunks, r.n_seg = (int32_t)wp.n_seg;
+        r.init = entry;
         return fla::walk_dkdv(dtype, wp.D, r, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
     }
     if (walk) {  // (the states forward saved are per 128-row chunk: only this path reads them)
         if (wp.n_seg > 1 &&
-            (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.totals_bytes))
+            (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.work_bytes))
             return FLA_ERR_WORKSPACE;
         if (reinterpret_cast<uintptr_t>(state_in) % 16 != 0) return FLA_ERR_WORKSPACE;
         hipStream_t s = static_cast<hipStream_t>(stream);
-        float *totals = wp.n_seg > 1 ? static_cast<float *>(workspace) : nullptr;
-        if (totals)
-            if (int rc = walk_entry_states(wp, q, go, B, H, N, dqk, dv, dtype, 1, totals, s)) return rc;
+        const float *entry = nullptr;
+        if (wp.n_seg > 1)
+            if (int rc = walk_entry_states(wp, q, go, B, H, N, dqk, dv, dtype, 1, workspace, nullptr, &entry, s)) return rc;
         fla::WalkParams w{};
         w.fmap = fmap;  // q, k hold phi(x): the slopes come from the LDS tiles
         w.q = q.ptr, w.k = k.ptr, w.v = v.ptr, w.go = go.ptr;
@@ -607,8 +626,7 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         w.dvs_b = dvv.strides[0], w.dvs_h = dvv.strides[1], w.dvs_n = dvv.strides[2];
         w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dqk, w.wv = (int32_t)dv;
         w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
-        w.init = totals, w.saved = const_cast<void *>(state_in);
-        w.init_n_seg = (int32_t)wp.n_seg, w.init_mul = 1;
+        w.init = entry, w.saved = const_cast<void *>(state_in);
         return fla::walk_bwd(dtype, wp.D, w, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
     }
     if (wp.ok && !(wp.split && fmap)) state_in = nullptr;  // not in the 256-row chunks' format: recomputed below
@@ -1175,7 +1193,7 @@ int fla_linear_attn_chunked_fwd_static(const void *q, const void *k, const void 
     int64_t need = chunked_op_workspace_bytes(B, H, N, D_qk, D_v);
     if (wp.ok) {
         const int64_t other = chunked_bytes(B, H, N, D_qk, D_v);  // operands off the speed path
-        need = wp.totals_bytes > other ? wp.totals_bytes : other;
+        need = wp.work_bytes > other ? wp.work_bytes : other;
     }
     if (need > (int64_t)FLA_STATIC_SCRATCH_BYTES) return FLA_ERR_WORKSPACE;
     void *ws = nullptr;

@@ -50,13 +50,12 @@ struct WalkParams {
     int32_t H, N, BH, wqk, wv;   // true widths of q/k and of v (<= D)
     int32_t n_chunks;            // ceil(N / rows per chunk)
     int32_t seg_chunks, n_seg;   // chunks per segment, segments per (b, h)
-    // entry state of every segment, fp32 [BH][init_n_seg][D (q/k index)][D (v index)]: sum of K^T V
-    // over the segments before (forward) / of Q^T dO over the segments after (backward); null when
-    // there is a single segment (entry state zero).  Segment s of this launch starts from entry
-    // min(s * init_mul + init_add, init_n_seg - 1): the totals may be kept over finer segments than
-    // the walk's.  init_transposed: the buffer holds the transposed matrices ([v index][q/k index]).
+    // entry state of every segment, fp32 [BH][n_seg][D (q/k index)][D (v index)]: sum of K^T V over
+    // the segments before (forward) / of Q^T dO over the segments after (backward); null when
+    // there is a single segment (entry state zero).  init_transposed: the buffer holds the
+    // transposed matrices ([v index][q/k index]).
     const float *init;
-    int32_t init_n_seg, init_mul, init_add, init_transposed;
+    int32_t init_transposed;
     // forward: where the 16-bit state at the entry of every chunk goes, [BH][n_chunks][D][D]
     // ([q/k index][v index]), or null; backward: the same buffer, read for dQ
     void *saved;
@@ -343,11 +342,7 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
     using B = WalkBlock<D>;
     const int l32 = lane & 31, g = lane >> 5;
     const float *init = nullptr;
-    if (p.init) {
-        int idx = sl.seg * p.init_mul + p.init_add;
-        idx = idx < p.init_n_seg - 1 ? idx : p.init_n_seg - 1;
-        init = p.init + ((int64_t)sl.bh * p.init_n_seg + idx) * (D * D);
-    }
+    if (p.init) init = p.init + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D);
 #pragma unroll
     for (int i = 0; i < W::NBW; ++i) {
         const int dbk = B::dbk(wave, i), eb = B::eb(wave);
@@ -363,15 +358,18 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
 //   O_c = lower(Q_c K_c^T) V_c + Q_c S, then S += K_c^T V_c
 // (forward as named; dQ of the split backward with q <- dO, k <- V, v <- K, o <- dQ and the entry
 // states read transposed)
-template <typename T, int D>
-__global__ __launch_bounds__(256, 2) void walk_fwd_kernel(const WalkParams p) {
+// DOUBLE: one workgroup per CU with two sets of tiles -- the loads of the next chunk are in flight
+// while this one is multiplied (no feature map in this variant).
+template <typename T, int D, bool DOUBLE>
+__global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
     using V8 = typename Mma<T>::V8;
     using B = WalkBlock<D>;
+    constexpr int SETS = DOUBLE ? 2 : 1;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
-    unsigned char *tq = smem, *tk = smem + W::TILE, *tv = smem + 2 * W::TILE, *tl = smem + 3 * W::TILE;
+    unsigned char *tl = smem + SETS * 3 * W::TILE;
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int rb = W::NCH == 1 ? wave : wave % W::NRB, db0 = W::NCH == 1 ? 0 : (wave / W::NRB) * W::DBW;
@@ -392,18 +390,38 @@ __global__ __launch_bounds__(256, 2) void walk_fwd_kernel(const WalkParams p) {
     walk_load_init<D>(p, sl, wave, lane, st);
     walk_state_to_lds<T, D>(tl, wave, lane, st);
 
+    auto load_chunk = [&](int c, int buf) {
+        const uint32_t base = lds0 + buf * 3 * W::TILE;
+        walk_load_tile<D>(rq, base, c * W::C, qs2, p.wqk, wave, lane);
+        walk_load_tile<D>(rk, base + W::TILE, c * W::C, ks2, p.wqk, wave, lane);
+        walk_load_tile<D>(rv, base + 2 * W::TILE, c * W::C, vs2, p.wv, wave, lane);
+    };
+    if constexpr (DOUBLE) load_chunk(sl.c_lo, 0);
 #pragma unroll 1
     for (int c = sl.c_lo; c < sl.c_hi; ++c) {
-        const int row0 = c * W::C;
-        walk_load_tile<D>(rq, lds0, row0, qs2, p.wqk, wave, lane);
-        walk_load_tile<D>(rk, lds0 + W::TILE, row0, ks2, p.wqk, wave, lane);
-        walk_load_tile<D>(rv, lds0 + 2 * W::TILE, row0, vs2, p.wv, wave, lane);
-        wait_vm<0>();
-        __syncthreads();  // the tiles have landed; the state written by the previous iteration is visible
-        if (p.fmap) {
-            walk_map_tile<T, D>(tq, p.fmap, row0, N, p.wqk, static_cast<T *>(p.qmap_out) + b * p.qo_b + h * p.qo_h,
-                                p.qo_n, tid);
-            __syncthreads();
+        const int row0 = c * W::C, buf = DOUBLE ? (c - sl.c_lo) & 1 : 0;
+        unsigned char *tq = smem + buf * 3 * W::TILE, *tk = tq + W::TILE, *tv = tq + 2 * W::TILE;
+        if constexpr (DOUBLE) {
+            const bool more = c + 1 < sl.c_hi;
+            if (more) load_chunk(c + 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
+            // this wave's loads of chunk c have landed when at most the loads issued after them are
+            // outstanding (the stores of the previous chunk were issued before those)
+            if (more)
+                wait_vm<3 * W::NI>();
+            else
+                wait_vm<0>();
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's part of the state is in LDS
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        } else {
+            load_chunk(c, 0);
+            wait_vm<0>();
+            __syncthreads();  // the tiles have landed; the state written by the previous iteration is visible
+            if (p.fmap) {
+                walk_map_tile<T, D>(tq, p.fmap, row0, N, p.wqk, static_cast<T *>(p.qmap_out) + b * p.qo_b + h * p.qo_h,
+                                    p.qo_n, tid);
+                __syncthreads();
+            }
         }
         f32x16 acc[W::DBW];
         walk_product<T, D, false>(tq, tk, tv, wave, lane, c > 0, [&](int db, int kc) -> V8 {
@@ -422,7 +440,14 @@ __global__ __launch_bounds__(256, 2) void walk_fwd_kernel(const WalkParams p) {
                 }
         }
         walk_update<T, D>(tk, tv, wave, lane, st);
-        __syncthreads();  // every wave is done with the tiles and with the old state
+        if constexpr (DOUBLE) {
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS reads of the tiles and of the state are done
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+        } else {
+            __syncthreads();  // every wave is done with the tiles and with the old state
+        }
         walk_state_to_lds<T, D>(tl, wave, lane, st);
     }
 #else
@@ -605,6 +630,7 @@ struct WalkTotalsParams {
     int64_t ys_b, ys_h, ys_n, zs_b, zs_h, zs_n;
     int32_t H, N, BH, dy, dz;
     int32_t n_chunks, seg_chunks, n_seg;
+    int32_t seg_lo, seg_hi;  // only segments seg_lo .. seg_hi - 1 are needed (the others' totals stay unwritten)
     float *totals;
     // feature map on load: Y holds the argument of the map; every Y tile is mapped in LDS as it lands
     // and the mapped rows are written to ymap_out (Y's shape, element strides yo_*).  0: none.
@@ -625,7 +651,12 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
     const int hl = slot / p.n_seg, seg = slot - hl * p.n_seg, bh = hl * 8 + xcd;
     const int c_lo = seg * p.seg_chunks;
     const int c_hi = c_lo + p.seg_chunks < p.n_chunks ? c_lo + p.seg_chunks : p.n_chunks;
-    if (bh >= p.BH || c_lo >= p.n_chunks) return;
+    if (bh >= p.BH || seg < p.seg_lo || seg >= p.seg_hi) return;
+    if (c_lo >= p.n_chunks) {  // a segment beyond the end of the sequence: its total is zero
+        float *out = p.totals + ((int64_t)bh * p.n_seg + seg) * (D * D);
+        for (int i = tid; i < D * D; i += 256) out[i] = 0.f;
+        return;
+    }
     const int b = bh / p.H, h = bh - b * p.H, N = p.N;
     const T *Y = static_cast<const T *>(p.y) + b * p.ys_b + h * p.ys_h;
     const T *Z = static_cast<const T *>(p.z) + b * p.zs_b + h * p.zs_h;
@@ -683,38 +714,62 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
 #endif
 }
 
-// totals[bh][seg][e] -> exclusive sum over the segments before (reverse == 0) / after (reverse != 0), in
-// place.  One thread per pair of elements; the loads of sixteen segments are issued together (a
-// chain of dependent loads, one per segment, would cost a memory latency each).
+// Entry states of the walk's segments from the totals of finer segments, `m` of them per walk
+// segment: entry[bh][s][e] = sum of totals[bh][f][e] over f < s m (reverse == 0) or f >= (s + 1) m
+// (reverse != 0).  Only the totals under those sums are read.  entry may be totals when m == 1 (a
+// thread reads an element before it writes it).  One thread per pair of elements; the loads of up
+// to sixteen segments are issued together (a chain of dependent loads would cost a memory latency
+// each).
 // (a template only so that the header can be included by several translation units)
 template <int kUnused = 0>
-__global__ __launch_bounds__(256) void walk_scan_kernel(float *totals, int n_seg, int E, int64_t total2, int reverse) {
+__global__ __launch_bounds__(256) void walk_scan_kernel(const float *totals, float *entry, int n_seg, int m, int E,
+                                                        int64_t total2, int reverse) {
     typedef float f32x2 __attribute__((ext_vector_type(2)));
     const int64_t i2 = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i2 >= total2) return;
     const int64_t bh = (i2 * 2) / E, e = i2 * 2 - bh * E;
-    float *pt = totals + bh * n_seg * E + e;
+    const int n_fine = n_seg * m;
+    const float *pt = totals + bh * n_fine * E + e;
+    float *pe = entry + bh * n_seg * E + e;
     const int64_t step = reverse ? -(int64_t)E : (int64_t)E;
-    if (reverse) pt += (int64_t)(n_seg - 1) * E;
+    if (reverse) pt += (int64_t)(n_fine - 1) * E, pe += (int64_t)(n_seg - 1) * E;
     f32x2 run = {0.f, 0.f};
-    int s = 0;
-    auto batch = [&](auto nn) {
-        constexpr int NB = decltype(nn)::value;
-        for (; s + NB <= n_seg; s += NB) {
-            f32x2 t[NB];
+    if (m == 1) {
+        int s = 0;
+        auto batch = [&](auto nn) {
+            constexpr int NB = decltype(nn)::value;
+            for (; s + NB <= n_seg - 1; s += NB) {
+                f32x2 t[NB];
 #pragma unroll
-            for (int u = 0; u < NB; ++u) t[u] = *reinterpret_cast<const f32x2 *>(pt + u * step);
+                for (int u = 0; u < NB; ++u) t[u] = *reinterpret_cast<const f32x2 *>(pt + u * step);
 #pragma unroll
-            for (int u = 0; u < NB; ++u) {
-                *reinterpret_cast<f32x2 *>(pt + u * step) = run;
-                run += t[u];
+                for (int u = 0; u < NB; ++u) {
+                    *reinterpret_cast<f32x2 *>(pe + u * step) = run;
+                    run += t[u];
+                }
+                pt += NB * step, pe += NB * step;
             }
-            pt += NB * step;
+        };
+        batch(std::integral_constant<int, 16>{});
+        batch(std::integral_constant<int, 4>{});
+        batch(std::integral_constant<int, 1>{});
+        *reinterpret_cast<f32x2 *>(pe) = run;  // the last segment in walking order: its own total is not needed
+        return;
+    }
+    for (int s = 0; s < n_seg; ++s) {
+        *reinterpret_cast<f32x2 *>(pe) = run;
+        pe += step;
+        if (s == n_seg - 1) break;
+        for (int u0 = 0; u0 < m; u0 += 4) {
+            f32x2 t[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+                t[u] = u0 + u < m ? *reinterpret_cast<const f32x2 *>(pt + (u0 + u) * step) : f32x2{0.f, 0.f};
+#pragma unroll
+            for (int u = 0; u < 4; ++u) run += t[u];
         }
-    };
-    batch(std::integral_constant<int, 16>{});
-    batch(std::integral_constant<int, 4>{});
-    batch(std::integral_constant<int, 1>{});
+        pt += m * step;
+    }
 }
 
 template <typename T, int D>
@@ -727,18 +782,22 @@ hipError_t launch_walk_totals(const WalkTotalsParams &p, hipStream_t stream) {
     return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
 }
 
-inline hipError_t launch_walk_scan(float *totals, int64_t BH, int n_seg, int E, int reverse, hipStream_t stream) {
+inline hipError_t launch_walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, int m, int E, int reverse,
+                                   hipStream_t stream) {
     const int64_t total2 = BH * E / 2;
-    return launch_kernel(walk_scan_kernel<0>, dim3((unsigned)((total2 + 255) / 256)), dim3(256), 0, stream, totals, n_seg,
-                         E, total2, reverse);
+    if (m < 1 || (m > 1 && entry == totals)) return hipErrorInvalidValue;
+    return launch_kernel(walk_scan_kernel<0>, dim3((unsigned)((total2 + 255) / 256)), dim3(256), 0, stream, totals, entry,
+                         n_seg, m, E, total2, reverse);
 }
 
 template <typename T, int D>
 hipError_t launch_walk_fwd(const WalkParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-    constexpr auto kern = walk_fwd_kernel<T, D>;
-    constexpr int smem = 3 * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
+    constexpr bool kDouble = D > 64;  // (the plan's workgroup count must match: one per CU when double)
+    if (kDouble && p.fmap) return hipErrorNotSupported;
+    constexpr auto kern = walk_fwd_kernel<T, D, kDouble>;
+    constexpr int smem = (kDouble ? 6 : 3) * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
     return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
 }

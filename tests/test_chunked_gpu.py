@@ -26,6 +26,12 @@ CASES = [
     (1, 1, 512, 128, 256),
     (1, 2, 576, 48, 48),
     (1, 1, 1024, 32, 32),
+    # several chunks per walking workgroup with a ragged last segment: D = 128 with two and with four
+    # finer total segments per walk segment, padded widths, and D = 64
+    (2, 8, 2450, 128, 128),
+    (2, 8, 4136, 128, 128),
+    (1, 4, 1500, 104, 120),
+    (8, 8, 2100, 64, 64),
 ]
 
 
