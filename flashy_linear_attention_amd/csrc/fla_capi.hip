@@ -478,8 +478,7 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
     if (int rc = check_alias_fwd(q, k, v, o, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
     const WalkPlan wp = walk_plan(B, H, N, dqk, dv);
-    // (the split kernels take no feature map: those calls go through the 256-row chunks below)
-    if (wp.ok && !(wp.split && fmap) && fla::fast_path_ok(make_params(q, k, v, o, B, H, N, dqk, dv, 0)) &&
+    if (wp.ok && fla::fast_path_ok(make_params(q, k, v, o, B, H, N, dqk, dv, 0)) &&
         (!fmap || fla::fast_path_ok(make_params(mapped[0], mapped[1], v, o, B, H, N, dqk, dv, 0)))) {
         // the segments' entry states; with a feature map the same kernel maps xk as it loads it and
         // writes phi(xk), which the walk then reads (so it runs for a single segment as well)
@@ -568,7 +567,7 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         return launch_feature_pass(2, fmap, k, dk, B, H, N, dqk, dtype, stream);
     }
     const WalkPlan wp = walk_plan(B, H, N, dqk, dv);
-    const bool walk = wp.ok && state_in && !(wp.split && fmap);  // (what forward saved is in this path's format)
+    const bool walk = wp.ok && state_in;  // (what forward saved is in this path's format)
     if (walk && wp.split) {
         if (wp.n_seg > 1 &&
             (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.work_bytes))
@@ -588,6 +587,10 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dv, w.wv = (int32_t)dqk;
         w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
         w.init = wp.n_seg > 1 ? static_cast<const float *>(state_in) : nullptr, w.init_transposed = 1;
+        if (fmap) {  // q holds phi(xq): dQ leaves multiplied by the slope computed from it
+            w.fmap = fmap, w.slope_y = q.ptr;
+            w.sy_b = q.strides[0], w.sy_h = q.strides[1], w.sy_n = q.strides[2];
+        }
         if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
         // dV, dK: the reverse walk over the same segments
         fla::WalkParams r{};
@@ -601,7 +604,7 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         r.dvs_b = dvv.strides[0], r.dvs_h = dvv.strides[1], r.dvs_n = dvv.strides[2];
         r.H = (int32_t)H, r.N = (int32_t)N, r.BH = (int32_t)(B * H), r.wqk = (int32_t)dqk, r.wv = (int32_t)dv;
         r.n_chunks = (int32_t)wp.n_chunks, r.seg_chunks = (int32_t)wp.seg_chunks, r.n_seg = (int32_t)wp.n_seg;
-        r.init = entry;
+        r.init = entry, r.fmap = fmap;  // (dK: the slope from phi(xk) in the K tile)
         return fla::walk_dkdv(dtype, wp.D, r, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
     }
     if (walk) {  // (the states forward saved are per 128-row chunk: only this path reads them)
@@ -629,7 +632,7 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         w.init = entry, w.saved = const_cast<void *>(state_in);
         return fla::walk_bwd(dtype, wp.D, w, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
     }
-    if (wp.ok && !(wp.split && fmap)) state_in = nullptr;  // not in the 256-row chunks' format: recomputed below
+    if (wp.ok) state_in = nullptr;  // not in the 256-row chunks' format: recomputed below
     if (fmap) set_output_slope(pq, fmap, q), set_output_slope(pk, fmap, k);
     const int64_t sb = shared_state_bytes(B, H, N, dqk, dv);
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < sb * (state_in ? 3 : 4))

@@ -67,6 +67,11 @@ struct WalkParams {
     int32_t fmap;
     void *qmap_out;
     int64_t qo_b, qo_h, qo_n;
+    // walk_fwd_kernel run as the dQ walk of the split backward (q <- dO, k <- V, v <- K, o <- dQ) with
+    // a feature map: slope_y holds phi(xq) (o's shape, element strides sy_*) and the result is
+    // multiplied by the slope of phi computed from it; null: none.
+    const void *slope_y;
+    int64_t sy_b, sy_h, sy_n;
 };
 
 template <int D>
@@ -242,14 +247,14 @@ __device__ __forceinline__ void walk_map_tile(unsigned char *tile, int fmap, int
     }
 }
 
-// acc[i][v] = Out[row][32 (db0 + i) + 16 g + v]: two 16-byte stores per block; rows >= N and columns
-// beyond the true width fall outside the buffer resource and are dropped.  With a feature map,
-// `ytile` is the LDS tile holding y = phi(x) for the same rows (tile row `trow`) and Out is
-// multiplied by the slope phi'(x), computed from y, first.
+// acc[i][v] = Out[row][32 (db0 + i) + 16 g + v] rounded to the storage type: pk[i][hq] = columns
+// 32 (db0 + i) + 16 g + 8 hq .. + 7.  With a feature map, `ytile` is the LDS tile holding
+// y = phi(x) for the same rows (tile row `trow`) and Out is multiplied by the slope phi'(x),
+// computed from y, first.
 template <typename T, int D>
-__device__ __forceinline__ void walk_store(__amdgpu_buffer_rsrc_t rs, int stride2, int width, int row, int g, int db0,
-                                           const f32x16 (&acc)[WalkCfg<D>::DBW], int fmap = 0,
-                                           const unsigned char *ytile = nullptr, int trow = 0) {
+__device__ __forceinline__ void walk_pack(const f32x16 (&acc)[WalkCfg<D>::DBW], int g, int db0,
+                                          u32x4 (&pk)[WalkCfg<D>::DBW][2], int fmap = 0,
+                                          const unsigned char *ytile = nullptr, int trow = 0) {
     using W = WalkCfg<D>;
     using V8 = typename Mma<T>::V8;
 #pragma unroll
@@ -269,11 +274,33 @@ __device__ __forceinline__ void walk_store(__amdgpu_buffer_rsrc_t rs, int stride
             V8 o8;
 #pragma unroll
             for (int e = 0; e < 8; ++e) o8[e] = static_cast<T>(f[e]);
-            const int col = 32 * db + 16 * g + 8 * hq;
-            const uint32_t off = (uint32_t)(row * stride2 + col * 2) + (col < width ? 0u : kOobOffset);
-            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, o8), rs, off, 0, 0);
+            pk[i][hq] = __builtin_bit_cast(u32x4, o8);
         }
     }
+}
+
+// two 16-byte stores per block; rows >= N and columns beyond the true width fall outside the
+// buffer resource and are dropped
+template <int D>
+__device__ __forceinline__ void walk_store_packed(__amdgpu_buffer_rsrc_t rs, int stride2, int width, int row, int g,
+                                                  int db0, const u32x4 (&pk)[WalkCfg<D>::DBW][2]) {
+#pragma unroll
+    for (int i = 0; i < WalkCfg<D>::DBW; ++i)
+#pragma unroll
+        for (int hq = 0; hq < 2; ++hq) {
+            const int col = 32 * (db0 + i) + 16 * g + 8 * hq;
+            const uint32_t off = (uint32_t)(row * stride2 + col * 2) + (col < width ? 0u : kOobOffset);
+            __builtin_amdgcn_raw_buffer_store_b128(pk[i][hq], rs, off, 0, 0);
+        }
+}
+
+template <typename T, int D>
+__device__ __forceinline__ void walk_store(__amdgpu_buffer_rsrc_t rs, int stride2, int width, int row, int g, int db0,
+                                           const f32x16 (&acc)[WalkCfg<D>::DBW], int fmap = 0,
+                                           const unsigned char *ytile = nullptr, int trow = 0) {
+    u32x4 pk[WalkCfg<D>::DBW][2];
+    walk_pack<T, D>(acc, g, db0, pk, fmap, ytile, trow);
+    walk_store_packed<D>(rs, stride2, width, row, g, db0, pk);
 }
 
 // state += Y^T Z over the rows of the tiles, this wave's 32 x 32 blocks (block i: Y columns of block
@@ -359,7 +386,10 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
 // (forward as named; dQ of the split backward with q <- dO, k <- V, v <- K, o <- dQ and the entry
 // states read transposed)
 // DOUBLE: one workgroup per CU with two sets of tiles -- the loads of the next chunk are in flight
-// while this one is multiplied (no feature map in this variant).
+// while this one is multiplied.  (Holding a chunk's results back and storing them after the next
+// chunk's tiles have been awaited, so that the wait for the tiles never includes fresh stores,
+// measured 20 % slower: the stores then compete with the loads in flight instead of filling the
+// gap after them.)
 template <typename T, int D, bool DOUBLE>
 __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -401,6 +431,22 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
     for (int c = sl.c_lo; c < sl.c_hi; ++c) {
         const int row0 = c * W::C, buf = DOUBLE ? (c - sl.c_lo) & 1 : 0;
         unsigned char *tq = smem + buf * 3 * W::TILE, *tk = tq + W::TILE, *tv = tq + 2 * W::TILE;
+        const int row = row0 + 32 * rb + l32;
+        // dQ walk with a feature map: this lane's values of phi(xq) under its accumulator registers,
+        // requested before the tiles so that they have arrived with them
+        V8 ys[W::DBW][2];
+        if (p.slope_y) {
+            const T *yrow = static_cast<const T *>(p.slope_y) + b * p.sy_b + h * p.sy_h + (int64_t)(row < N ? row : 0) * p.sy_n;
+#pragma unroll
+            for (int i = 0; i < W::DBW; ++i)
+#pragma unroll
+                for (int hq = 0; hq < 2; ++hq) {
+                    const int col = 32 * (db0 + i) + 16 * g + 8 * hq;
+                    u32x4 raw = {0u, 0u, 0u, 0u};
+                    if (col < p.wv) raw = *reinterpret_cast<const u32x4 *>(yrow + col);
+                    ys[i][hq] = __builtin_bit_cast(V8, raw);
+                }
+        }
         if constexpr (DOUBLE) {
             const bool more = c + 1 < sl.c_hi;
             if (more) load_chunk(c + 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
@@ -413,11 +459,18 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's part of the state is in LDS
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
+            if (p.fmap && p.qmap_out) {
+                walk_map_tile<T, D>(tq, p.fmap, row0, N, p.wqk, static_cast<T *>(p.qmap_out) + b * p.qo_b + h * p.qo_h,
+                                    p.qo_n, tid);
+                __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the rewritten tile is in LDS
+                __builtin_amdgcn_s_barrier();
+                asm volatile("" ::: "memory");
+            }
         } else {
             load_chunk(c, 0);
             wait_vm<0>();
             __syncthreads();  // the tiles have landed; the state written by the previous iteration is visible
-            if (p.fmap) {
+            if (p.fmap && p.qmap_out) {
                 walk_map_tile<T, D>(tq, p.fmap, row0, N, p.wqk, static_cast<T *>(p.qmap_out) + b * p.qo_b + h * p.qo_h,
                                     p.qo_n, tid);
                 __syncthreads();
@@ -427,7 +480,14 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
         walk_product<T, D, false>(tq, tk, tv, wave, lane, c > 0, [&](int db, int kc) -> V8 {
             return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g);
         }, acc);
-        walk_store<T, D>(ro, os2, p.wv, row0 + 32 * rb + l32, g, db0, acc);
+        if (p.slope_y) {
+#pragma unroll
+            for (int i = 0; i < W::DBW; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    acc[i][v] *= feature_slope_from_value(p.fmap, static_cast<float>(ys[i][v / 8][v % 8]));
+        }
+        walk_store<T, D>(ro, os2, p.wv, row, g, db0, acc);
         if (p.saved) {  // the state at the entry of this chunk, [q/k index][v index], for backward's dQ
             T *sv = static_cast<T *>(p.saved) + ((int64_t)sl.bh * p.n_chunks + c) * (D * D);
 #pragma unroll
@@ -611,7 +671,7 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
         walk_product<T, D, true>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
             return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
         }, acc);
-        walk_store<T, D>(rdk, dks2, p.wqk, row, g, db0, acc);
+        walk_store<T, D>(rdk, dks2, p.wqk, row, g, db0, acc, p.fmap, tk, 32 * rb + l32);
         walk_update<T, D>(tq, tg, wave, lane, st);
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS reads of the tiles and of the state are done
@@ -795,7 +855,6 @@ hipError_t launch_walk_fwd(const WalkParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     constexpr bool kDouble = D > 64;  // (the plan's workgroup count must match: one per CU when double)
-    if (kDouble && p.fmap) return hipErrorNotSupported;
     constexpr auto kern = walk_fwd_kernel<T, D, kDouble>;
     constexpr int smem = (kDouble ? 6 : 3) * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
