@@ -51,8 +51,8 @@ HBM_PEAK_GBS = 8000.0
 PROFILED_TRAFFIC = {
     ("C3", "quadratic"): (2.426e9, "profiles/tri_xyt_z_fast_kernels_C3_pmc.md"),
     # chunk-wise: all kernels of a step
-    ("C3", "chunked"): (3.605e9, "profiles/chunked_C3_C5_kernel_trace_pmc.md"),
-    ("C5", "chunked"): (1.573e9, "profiles/chunked_C3_C5_kernel_trace_pmc.md"),
+    ("C3", "chunked"): (2.367e9, "profiles/chunked_C3_C5_kernel_trace_pmc.md"),
+    ("C5", "chunked"): (1.146e9, "profiles/chunked_C3_C5_kernel_trace_pmc.md"),
 }
 # MFMA operations the dominant kernel issues over those of its product-units (rocprofv3
 # SQ_INSTS_VALU_MFMA_MOPS_BF16 x 512 FLOPs; the excess is the 32 x 32 blocks on the diagonal)
@@ -166,6 +166,9 @@ def _pad(d):
 
 
 def _chunk_rows(w):
+    """Rows per chunk of the kernels this workload's chunk-wise step runs."""
+    if _pad(w.d_qk) == _pad(w.d_v) and _pad(w.d_qk) <= 128:  # the walk kernels
+        return 128 if _pad(w.d_qk) <= 64 else 64
     return 256 if (w.d_qk // 2 + w.d_v <= 192 and w.d_v // 2 + w.d_qk <= 192) else 128
 
 
@@ -706,7 +709,7 @@ def main() -> int:
         gbs = bytes_step / (ms_step * 1e-3) / 1e9
         result["roofline"] = {
             "bound": "hbm",
-            "kernel": "all kernels of a chunk-wise step (chunk states and their running sums, diagonal blocks + state product)",
+            "kernel": "all kernels of a chunk-wise step (segment totals and their running sums, the walks over the chunks)",
             "achieved": round(gbs, 1),
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
