@@ -552,13 +552,14 @@ def main() -> int:
             linear_attention_normalised_fwd,
         )
 
-        norm_out, norm_denom = linear_attention_normalised_fwd(q, k, v, 1e-5, chunked)
+        # (chunk-wise: forward hands its running state to backward, as the autograd Function does)
+        norm_out, norm_denom, norm_state = linear_attention_normalised_fwd(q, k, v, 1e-5, chunked, want_state=True)
 
         def fwd(q_, k_, v_):
-            return linear_attention_normalised_fwd(q_, k_, v_, 1e-5, chunked)
+            return linear_attention_normalised_fwd(q_, k_, v_, 1e-5, chunked, want_state=chunked)
 
         def bwd(do_, q_, k_, v_):
-            return linear_attention_normalised_bwd(do_, q_, k_, v_, norm_out, norm_denom, chunked)
+            return linear_attention_normalised_bwd(do_, q_, k_, v_, norm_out, norm_denom, chunked, norm_state)
 
         qa, ka, va = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
 

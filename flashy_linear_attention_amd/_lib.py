@@ -12,7 +12,7 @@ import threading
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libfla_gfx950.so")
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 FLA_DTYPE_BF16 = 0
 FLA_DTYPE_F16 = 1
@@ -42,10 +42,11 @@ SIGNATURES = {
     "fla_feature_attn_bwd": ([_ptr] * 7 + [_i64] * 5 + [_strides] * 7 + [ctypes.c_int, ctypes.c_int, _ptr, _ptr, _i64, _ptr],
                              ctypes.c_int),
     "fla_feature_attn_normalised_fwd": ([_ptr] * 7 + [_i64] * 5 + [_strides] * 6
-                                        + [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_int, _ptr, _i64, _ptr],
+                                        + [ctypes.c_int, ctypes.c_float, ctypes.c_int, ctypes.c_int, _ptr,
+                                           ctypes.POINTER(ctypes.c_int32), _ptr, _i64, _ptr],
                                         ctypes.c_int),
     "fla_feature_attn_normalised_bwd": ([_ptr] * 9 + [_i64] * 5 + [_strides] * 8
-                                        + [ctypes.c_int, ctypes.c_int, ctypes.c_int, _ptr, _i64, _ptr], ctypes.c_int),
+                                        + [ctypes.c_int, ctypes.c_int, ctypes.c_int, _ptr, _ptr, _i64, _ptr], ctypes.c_int),
     "fla_linear_attn_chunked_fwd_static": ([_ptr] * 4 + [_i64] * 5 + [_strides] * 4 + [ctypes.c_int, _ptr], ctypes.c_int),
     "fla_linear_attn_chunked_bwd": ([_ptr] * 7 + [_i64] * 5 + [_strides] * 7 + [ctypes.c_int, _ptr, _ptr, _i64, _ptr],
                                     ctypes.c_int),
@@ -56,9 +57,10 @@ SIGNATURES = {
                           + [ctypes.POINTER(ctypes.c_float), ctypes.c_int, _ptr, _i64, _ptr], ctypes.c_int),
     "fla_normalised_workspace_bytes": ([_i64] * 5 + [ctypes.c_int], ctypes.c_int64),
     "fla_linear_attn_normalised_fwd": ([_ptr] * 5 + [_i64] * 5 + [_strides] * 4
-                                       + [ctypes.c_float, ctypes.c_int, ctypes.c_int, _ptr, _i64, _ptr], ctypes.c_int),
+                                       + [ctypes.c_float, ctypes.c_int, ctypes.c_int, _ptr, ctypes.POINTER(ctypes.c_int32),
+                                          _ptr, _i64, _ptr], ctypes.c_int),
     "fla_linear_attn_normalised_bwd": ([_ptr] * 9 + [_i64] * 5 + [_strides] * 8
-                                       + [ctypes.c_int, ctypes.c_int, _ptr, _i64, _ptr], ctypes.c_int),
+                                       + [ctypes.c_int, ctypes.c_int, _ptr, _ptr, _i64, _ptr], ctypes.c_int),
 }
 
 _lock = threading.Lock()

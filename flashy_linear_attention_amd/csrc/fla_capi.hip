@@ -436,6 +436,32 @@ int walk_entry_states(const WalkPlan &w, const View &y, const View &z, int64_t B
                : FLA_ERR_LAUNCH;
 }
 
+// The normaliser's terms handed to the walk kernels (fla_chunk_walk.h, WalkParams::denom ...).
+struct WalkNorm {
+    float *denom;     // forward: receives n
+    float eps;
+    const float *dn;  // backward: dn_i = -(g_i . out_i) / n_i (and the grad_out operand holds g / n)
+    void *vec;        // scratch, 2 * walk_vec_bytes(): zc, rc
+    bool fused;       // out: the kernels took the terms (false: the caller runs the passes of fla_norm.h)
+    bool dk_pending;  // out: ... all but dK's sum over later rows (and dK's slope, with a feature map)
+};
+
+int64_t walk_vec_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
+    const WalkPlan w = walk_plan(B, H, N, dqk, dv);
+    return w.ok ? B * H * w.n_chunks * w.D * 4 : 0;
+}
+
+// out[bh][c] = sum over the rows before (reverse: after) chunk c of w[row] y[row] (w null: y[row])
+int walk_chunk_vectors(const WalkPlan &wp, const View &y, int64_t width, const float *w, int reverse, float *out,
+                       int64_t B, int64_t H, int64_t N, int dtype, hipStream_t s) {
+    fla::WalkVecParams vp{};
+    vp.y = y.ptr, vp.ys_b = y.strides[0], vp.ys_h = y.strides[1], vp.ys_n = y.strides[2];
+    vp.w = w, vp.H = (int32_t)H, vp.N = (int32_t)N, vp.width = (int32_t)width, vp.n_chunks = (int32_t)wp.n_chunks;
+    vp.out = out;
+    if (fla::walk_vec_sums(dtype, wp.D, vp, B * H, s) != hipSuccess) return FLA_ERR_LAUNCH;
+    return fla::walk_scan(out, out, B * H, (int)wp.n_chunks, 1, wp.D, reverse, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+}
+
 bool states_shareable(int64_t dqk, int64_t dv, int64_t N) {
     if (pad_index(dqk) != pad_index(dv) || padded(dqk) > 128) return false;
     const int rows = chunk_rows(dqk, dv);
@@ -456,7 +482,7 @@ int64_t chunked_op_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk,
     const int64_t shared = shared_state_bytes(B, H, N, dqk, dv);
     if (shared) {  // fp32 chunk states (2x) + two rounded states (backward without a saved one); the walk's totals
         const WalkPlan w = walk_plan(B, H, N, dqk, dv);
-        return w.ok && w.work_bytes > shared * 4 ? w.work_bytes : shared * 4;
+        return w.ok && w.work_bytes * 2 > shared * 4 ? w.work_bytes * 2 : shared * 4;
     }
     int64_t m = chunked_bytes(B, H, N, dqk, dv);
     const int64_t t = chunked_bytes(B, H, N, dv, dqk);
@@ -470,8 +496,9 @@ int64_t chunked_op_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk,
 int chunked_forward(const View &q, const View &k, const View &v, const View &o, int64_t B, int64_t H, int64_t N,
                     int64_t dqk, int64_t dv, int dtype, void *state_out, int32_t *state_valid, void *workspace,
                     int64_t workspace_bytes, void *stream, int fmap = 0, const View *mapped = nullptr,
-                    bool *mapped_done = nullptr) {
+                    bool *mapped_done = nullptr, WalkNorm *nx = nullptr) {
     if (state_valid) *state_valid = 0;
+    if (nx) nx->fused = nx->dk_pending = false;
     const View all[] = {q, k, v, o};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
@@ -512,6 +539,12 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dqk, w.wv = (int32_t)dv;
         w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
         w.init = wp.n_seg > 1 ? entry : nullptr, w.saved = wp.split ? nullptr : state_out;
+        if (nx) {  // the normaliser inside the walk: zc = running sum of k at the entry of every chunk
+            float *zc = static_cast<float *>(nx->vec);
+            if (int rc = walk_chunk_vectors(wp, kk, dqk, nullptr, 0, zc, B, H, N, dtype, s)) return rc;
+            w.denom = nx->denom, w.eps = nx->eps, w.zc = zc;
+            nx->fused = true;
+        }
         if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
         if (mapped_done) *mapped_done = true;
         if (state_out && state_valid) *state_valid = 1;
@@ -543,7 +576,9 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
 
 int chunked_backward(const View &go, const View &q, const View &k, const View &v, const View &dq, const View &dk,
                      const View &dvv, int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv, int dtype,
-                     const void *state_in, void *workspace, int64_t workspace_bytes, void *stream, int fmap = 0) {
+                     const void *state_in, void *workspace, int64_t workspace_bytes, void *stream, int fmap = 0,
+                     WalkNorm *nx = nullptr) {
+    if (nx) nx->fused = nx->dk_pending = false;
     const View all[] = {go, q, k, v, dq, dk, dvv};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
@@ -555,6 +590,8 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
     TriParams pq = make_params(go, v, k, dq, B, H, N, dv, dqk, 0);   // dQ = lower(dO V^T) K
     TriParams pv = make_params(k, q, go, dvv, B, H, N, dqk, dv, 1);  // dV = upper(K Q^T) dO
     TriParams pk = make_params(v, go, q, dk, B, H, N, dv, dqk, 1);   // dK = upper(V dO^T) Q
+    // (with the normaliser's terms still to be added by the caller, so is the slope)
+    const int fmap_late = nx ? 0 : fmap;
     if (!states_shareable(dqk, dv, N) || !fla::fast_path_ok(pq) || !fla::fast_path_ok(pv) || !fla::fast_path_ok(pk)) {
         if (int rc = run_tri_chunked(go, v, k, dq, B, H, N, dv, dqk, 0, dtype, workspace, workspace_bytes, stream))
             return rc;
@@ -562,21 +599,38 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
             return rc;
         if (int rc = run_tri_chunked(v, go, q, dk, B, H, N, dv, dqk, 1, dtype, workspace, workspace_bytes, stream))
             return rc;
-        if (!fmap) return FLA_OK;
+        if (!fmap_late) return FLA_OK;
         if (int rc = launch_feature_pass(2, fmap, q, dq, B, H, N, dqk, dtype, stream)) return rc;
         return launch_feature_pass(2, fmap, k, dk, B, H, N, dqk, dtype, stream);
     }
     const WalkPlan wp = walk_plan(B, H, N, dqk, dv);
-    const bool walk = wp.ok && state_in;  // (what forward saved is in this path's format)
+    // (what forward saved is in this path's format; the split path's entry states are cheap to recompute)
+    const bool walk = wp.ok && (state_in || wp.split);
     if (walk && wp.split) {
-        if (wp.n_seg > 1 &&
-            (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.work_bytes))
+        // workspace: totals and entry states of Q^T dO; behind them those of K^T V when forward's are not given
+        if (wp.n_seg > 1 && (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 ||
+                             workspace_bytes < wp.work_bytes * (state_in ? 1 : 2)))
             return FLA_ERR_WORKSPACE;
-        if (reinterpret_cast<uintptr_t>(state_in) % 16 != 0) return FLA_ERR_WORKSPACE;
+        if (state_in && reinterpret_cast<uintptr_t>(state_in) % 16 != 0) return FLA_ERR_WORKSPACE;
         hipStream_t s = static_cast<hipStream_t>(stream);
         const float *entry = nullptr;
-        if (wp.n_seg > 1)
+        if (wp.n_seg > 1) {
+            if (!state_in) {
+                const float *fwd_entry = nullptr;
+                if (int rc = walk_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, static_cast<char *>(workspace) + wp.work_bytes,
+                                               nullptr, &fwd_entry, s))
+                    return rc;
+                state_in = fwd_entry;
+            }
             if (int rc = walk_entry_states(wp, q, go, B, H, N, dqk, dv, dtype, 1, workspace, nullptr, &entry, s)) return rc;
+        }
+        float *zc = nullptr, *rcv = nullptr;
+        if (nx) {  // zc: running sum of k at the entry of every chunk; rc: sum of dn_i q_i over the rows after it
+            zc = static_cast<float *>(nx->vec);
+            rcv = reinterpret_cast<float *>(static_cast<char *>(nx->vec) + walk_vec_bytes(B, H, N, dqk, dv));
+            if (int rc = walk_chunk_vectors(wp, q, dqk, nx->dn, 1, rcv, B, H, N, dtype, s)) return rc;
+            if (int rc = walk_chunk_vectors(wp, k, dqk, nullptr, 0, zc, B, H, N, dtype, s)) return rc;
+        }
         // dQ = lower(dO V^T) K + dO S^T: the forward walk over (dO, V, K), its states V^T K = S^T
         fla::WalkParams w{};
         w.q = go.ptr, w.k = v.ptr, w.v = k.ptr, w.o = const_cast<void *>(dq.ptr);
@@ -591,6 +645,7 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
             w.fmap = fmap, w.slope_y = q.ptr;
             w.sy_b = q.strides[0], w.sy_h = q.strides[1], w.sy_n = q.strides[2];
         }
+        if (nx) w.dn = nx->dn, w.zc = zc, nx->fused = true;  // dQ's term of the normaliser inside its walk
         if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
         // dV, dK: the reverse walk over the same segments
         fla::WalkParams r{};
@@ -605,6 +660,7 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         r.H = (int32_t)H, r.N = (int32_t)N, r.BH = (int32_t)(B * H), r.wqk = (int32_t)dqk, r.wv = (int32_t)dv;
         r.n_chunks = (int32_t)wp.n_chunks, r.seg_chunks = (int32_t)wp.seg_chunks, r.n_seg = (int32_t)wp.n_seg;
         r.init = entry, r.fmap = fmap;  // (dK: the slope from phi(xk) in the K tile)
+        if (nx) r.dn = nx->dn, r.rc = rcv;  // dK's terms
         return fla::walk_dkdv(dtype, wp.D, r, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
     }
     if (walk) {  // (the states forward saved are per 128-row chunk: only this path reads them)
@@ -630,10 +686,18 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dqk, w.wv = (int32_t)dv;
         w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
         w.init = entry, w.saved = const_cast<void *>(state_in);
+        if (nx) {
+            const int64_t vb = walk_vec_bytes(B, H, N, dqk, dv);
+            float *zc = static_cast<float *>(nx->vec), *rcv = reinterpret_cast<float *>(static_cast<char *>(nx->vec) + vb);
+            if (int rc = walk_chunk_vectors(wp, k, dqk, nullptr, 0, zc, B, H, N, dtype, s)) return rc;
+            if (int rc = walk_chunk_vectors(wp, q, dqk, nx->dn, 1, rcv, B, H, N, dtype, s)) return rc;
+            w.dn = nx->dn, w.zc = zc, w.rc = rcv;
+            nx->fused = true;
+        }
         return fla::walk_bwd(dtype, wp.D, w, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
     }
     if (wp.ok) state_in = nullptr;  // not in the 256-row chunks' format: recomputed below
-    if (fmap) set_output_slope(pq, fmap, q), set_output_slope(pk, fmap, k);
+    if (fmap_late) set_output_slope(pq, fmap, q), set_output_slope(pk, fmap, k);
     const int64_t sb = shared_state_bytes(B, H, N, dqk, dv);
     if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < sb * (state_in ? 3 : 4))
         return FLA_ERR_WORKSPACE;
@@ -663,7 +727,8 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
 // per operand and then the plain operator on phi(xq), phi(xk).
 int feature_forward(const View &vxq, const View &vxk, const View &vv, const View &vo, const View (&mapped)[2], int64_t B,
                     int64_t H, int64_t N, int64_t dqk, int64_t dv, int fmap, int dtype, int chunked, void *state_out,
-                    int32_t *state_valid, void *workspace, int64_t workspace_bytes, void *stream) {
+                    int32_t *state_valid, void *workspace, int64_t workspace_bytes, void *stream,
+                    WalkNorm *nx = nullptr) {
     const View all[] = {vxq, vxk, vv, vo, mapped[0], mapped[1]};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
@@ -675,7 +740,7 @@ int feature_forward(const View &vxq, const View &vxk, const View &vv, const View
     if (chunked) {
         bool done = false;
         if (int rc = chunked_forward(vxq, vxk, vv, vo, B, H, N, dqk, dv, dtype, state_out, state_valid, workspace,
-                                     workspace_bytes, stream, fmap, mapped, &done))
+                                     workspace_bytes, stream, fmap, mapped, &done, nx))
             return rc;
         if (done) return FLA_OK;
     }
@@ -683,7 +748,7 @@ int feature_forward(const View &vxq, const View &vxk, const View &vv, const View
     if (int rc = launch_feature_pass(1, fmap, vxk, mapped[1], B, H, N, dqk, dtype, stream)) return rc;
     if (!chunked) return run_tri(mapped[0], mapped[1], vv, vo, B, H, N, dqk, dv, 0, dtype, stream);
     return chunked_forward(mapped[0], mapped[1], vv, vo, B, H, N, dqk, dv, dtype, state_out, state_valid, workspace,
-                           workspace_bytes, stream);
+                           workspace_bytes, stream, 0, nullptr, nullptr, nx);
 }
 
 int forward(const View &q, const View &k, const View &v, const View &o, int64_t B, int64_t H, int64_t N,
@@ -733,7 +798,8 @@ int backward(const View &go, const View &q, const View &k, const View &v, const 
 struct NormLayout {
     int lpr;
     int64_t chunks, sums_bytes, do_bytes, dn_bytes;
-    int64_t norm_bytes;   // the normaliser's own scratch: dO, dn, two sets of chunk sums
+    int64_t vec_bytes;    // chunk-wise walk kernels: one set of per-chunk running vectors (two are kept)
+    int64_t norm_bytes;   // the normaliser's own scratch: dO, dn, two sets of chunk sums, two sets of vectors
     int64_t chunk_bytes;  // behind it: scratch of the chunk-wise product evaluation (0 when quadratic)
 };
 
@@ -746,7 +812,8 @@ NormLayout norm_layout(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv,
     l.do_bytes = (B * H * N * dv * 2 + 15) / 16 * 16;
     l.dn_bytes = (B * H * N * 4 + 15) / 16 * 16;
     l.sums_bytes = (l.sums_bytes + 15) / 16 * 16;
-    l.norm_bytes = l.do_bytes + l.dn_bytes + 2 * l.sums_bytes;
+    l.vec_bytes = chunked ? walk_vec_bytes(B, H, N, dqk, dv) : 0;
+    l.norm_bytes = l.do_bytes + l.dn_bytes + 2 * l.sums_bytes + 2 * l.vec_bytes;
     l.chunk_bytes = chunked ? chunked_op_workspace_bytes(B, H, N, dqk, dv) : 0;
     return l;
 }
@@ -806,7 +873,9 @@ int fused_normalised_forward(const View &q, const View &k, const View &v, const 
 // further outputs; the normaliser is that of phi(xq), phi(xk).
 int normalised_forward(const View &q0, const View &k0, const View &v, const View &o, float *denom, int64_t B, int64_t H,
                        int64_t N, int64_t dqk, int64_t dv, float eps, int dtype, int chunked, void *workspace,
-                       int64_t workspace_bytes, void *stream, int fmap = 0, const View *mapped = nullptr) {
+                       int64_t workspace_bytes, void *stream, int fmap = 0, const View *mapped = nullptr,
+                       void *state_out = nullptr, int32_t *state_valid = nullptr) {
+    if (state_valid) *state_valid = 0;
     const View all[] = {q0, k0, v, o};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
@@ -826,6 +895,9 @@ int normalised_forward(const View &q0, const View &k0, const View &v, const View
         return normalised_forward(mapped[0], mapped[1], v, o, denom, B, H, N, dqk, dv, eps, dtype, 0, workspace,
                                   workspace_bytes, stream);
     }
+    // chunk-wise walk kernels compute n and divide by it themselves
+    WalkNorm nx{denom, eps, nullptr,
+                workspace ? static_cast<char *>(workspace) + l.do_bytes + l.dn_bytes + 2 * l.sums_bytes : nullptr, false, false};
     const View &q = fmap ? mapped[0] : q0, &k = fmap ? mapped[1] : k0;
     if (!chunked) {
         const int rc = fused_normalised_forward(q, k, v, o, denom, B, H, N, dqk, dv, eps, dtype, stream);
@@ -833,13 +905,16 @@ int normalised_forward(const View &q0, const View &k0, const View &v, const View
     }
     if (fmap) {
         const View both[2] = {mapped[0], mapped[1]};
-        if (int rc = feature_forward(q0, k0, v, o, both, B, H, N, dqk, dv, fmap, dtype, 1, nullptr, nullptr,
-                                     static_cast<char *>(workspace) + l.norm_bytes, l.chunk_bytes, stream))
+        if (int rc = feature_forward(q0, k0, v, o, both, B, H, N, dqk, dv, fmap, dtype, 1, state_out, state_valid,
+                                     static_cast<char *>(workspace) + l.norm_bytes, l.chunk_bytes, stream, &nx))
             return rc;
+        if (nx.fused) return FLA_OK;
     } else if (chunked) {
-        if (int rc = chunked_forward(q, k, v, o, B, H, N, dqk, dv, dtype, nullptr, nullptr,
-                                     static_cast<char *>(workspace) + l.norm_bytes, l.chunk_bytes, stream))
+        if (int rc = chunked_forward(q, k, v, o, B, H, N, dqk, dv, dtype, state_out, state_valid,
+                                     static_cast<char *>(workspace) + l.norm_bytes, l.chunk_bytes, stream, 0, nullptr,
+                                     nullptr, &nx))
             return rc;
+        if (nx.fused) return FLA_OK;
     } else if (int rc = run_tri(q, k, v, o, B, H, N, dqk, dv, 0, dtype, stream)) {
         return rc;
     }
@@ -857,7 +932,7 @@ int normalised_forward(const View &q0, const View &k0, const View &v, const View
 int normalised_backward(const View &go, const View &q, const View &k, const View &v, const View &o,
                         const float *denom, const View &dq, const View &dk, const View &dvv, int64_t B, int64_t H,
                         int64_t N, int64_t dqk, int64_t dv, int dtype, int chunked, void *workspace,
-                        int64_t workspace_bytes, void *stream, int fmap = 0) {
+                        int64_t workspace_bytes, void *stream, int fmap = 0, const void *state_in = nullptr) {
     // fmap != 0: q, k hold phi(xq), phi(xk) and dq, dk leave as gradients with respect to xq, xk (the
     // slope is multiplied in by the last pass, after the normaliser's own terms have been added)
     const View all[] = {go, q, k, v, o, dq, dk, dvv};
@@ -886,10 +961,13 @@ int normalised_backward(const View &go, const View &q, const View &k, const View
     p.out = dO, p.os_b = do_strides[0], p.os_h = do_strides[1], p.os_n = do_strides[2], p.vec_out = vec_ok(dOv, dv);
     if (norm_launch(1, dtype, l.lpr, p, stream) != hipSuccess) return FLA_ERR_LAUNCH;
     // gradients of the unnormalised product
+    WalkNorm nx{nullptr, 0.f, dn, ws + l.do_bytes + l.dn_bytes + 2 * l.sums_bytes, false, false};
     if (chunked) {
-        if (int rc = chunked_backward(dOv, q, k, v, dq, dk, dvv, B, H, N, dqk, dv, dtype, nullptr, ws + l.norm_bytes,
-                                      l.chunk_bytes, stream))
+        // the walk kernels add the normaliser's terms (and apply the slope of a feature map) themselves
+        if (int rc = chunked_backward(dOv, q, k, v, dq, dk, dvv, B, H, N, dqk, dv, dtype, state_in, ws + l.norm_bytes,
+                                      l.chunk_bytes, stream, fmap, &nx))
             return rc;
+        if (nx.fused && !nx.dk_pending) return FLA_OK;
     } else if (int rc = backward_products(dOv, q, k, v, dq, dk, dvv, B, H, N, dqk, dv, dtype, stream)) {
         return rc;
     }
@@ -898,6 +976,7 @@ int normalised_backward(const View &go, const View &q, const View &k, const View
     p.dk = const_cast<void *>(dk.ptr), p.dks_b = dk.strides[0], p.dks_h = dk.strides[1], p.dks_n = dk.strides[2];
     p.vec_dq = vec_ok(dq, dqk), p.vec_dk = vec_ok(dk, dqk);
     p.fmap = fmap;
+    p.only_dk = nx.fused && nx.dk_pending;  // (dq is complete, slope included)
     return norm_launch(2, dtype, l.lpr, p, stream) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
 }
 
@@ -1255,12 +1334,15 @@ int fla_feature_attn_normalised_fwd(const void *xq, const void *xk, const void *
                                     const int64_t *xq_strides, const int64_t *xk_strides, const int64_t *v_strides,
                                     const int64_t *o_strides, const int64_t *q_out_strides,
                                     const int64_t *k_out_strides, int feature_map, float eps, int dtype, int chunked,
-                                    void *workspace, int64_t workspace_bytes, void *stream) {
+                                    void *state_out, int32_t *state_valid, void *workspace, int64_t workspace_bytes,
+                                    void *stream) {
+    if (state_valid) *state_valid = 0;
     if (int rc = check_norm_args(B, H, N, D_qk, D_v, dtype)) return rc;
     if (feature_map != FLA_MAP_ELU1 && feature_map != FLA_MAP_SOFTPLUS) return FLA_ERR_UNSUPPORTED;
     const View mapped[2] = {{q_out, q_out_strides}, {k_out, k_out_strides}};
     return normalised_forward({xq, xq_strides}, {xk, xk_strides}, {v, v_strides}, {o, o_strides}, denom, B, H, N, D_qk,
-                              D_v, eps, dtype, chunked, workspace, workspace_bytes, stream, feature_map, mapped);
+                              D_v, eps, dtype, chunked, workspace, workspace_bytes, stream, feature_map, mapped,
+                              state_out, state_valid);
 }
 
 int fla_feature_attn_normalised_bwd(const void *grad_out, const void *q, const void *k, const void *v, const void *o,
@@ -1269,12 +1351,12 @@ int fla_feature_attn_normalised_bwd(const void *grad_out, const void *q, const v
                                     const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
                                     const int64_t *o_strides, const int64_t *dxq_strides, const int64_t *dxk_strides,
                                     const int64_t *dv_strides, int feature_map, int dtype, int chunked,
-                                    void *workspace, int64_t workspace_bytes, void *stream) {
+                                    const void *state_in, void *workspace, int64_t workspace_bytes, void *stream) {
     if (int rc = check_norm_args(B, H, N, D_qk, D_v, dtype)) return rc;
     if (feature_map != FLA_MAP_ELU1 && feature_map != FLA_MAP_SOFTPLUS) return FLA_ERR_UNSUPPORTED;
     return normalised_backward({grad_out, go_strides}, {q, q_strides}, {k, k_strides}, {v, v_strides}, {o, o_strides},
                                denom, {dxq, dxq_strides}, {dxk, dxk_strides}, {dv, dv_strides}, B, H, N, D_qk, D_v,
-                               dtype, chunked, workspace, workspace_bytes, stream, feature_map);
+                               dtype, chunked, workspace, workspace_bytes, stream, feature_map, state_in);
 }
 
 int64_t fla_poly_attn_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t R, int64_t D_v) {
@@ -1314,11 +1396,13 @@ int64_t fla_normalised_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t 
 int fla_linear_attn_normalised_fwd(const void *q, const void *k, const void *v, void *o, float *denom, int64_t B,
                                    int64_t H, int64_t N, int64_t D_qk, int64_t D_v, const int64_t *q_strides,
                                    const int64_t *k_strides, const int64_t *v_strides, const int64_t *o_strides,
-                                   float eps, int dtype, int chunked, void *workspace, int64_t workspace_bytes,
-                                   void *stream) {
+                                   float eps, int dtype, int chunked, void *state_out, int32_t *state_valid,
+                                   void *workspace, int64_t workspace_bytes, void *stream) {
+    if (state_valid) *state_valid = 0;
     if (int rc = check_norm_args(B, H, N, D_qk, D_v, dtype)) return rc;
     return normalised_forward({q, q_strides}, {k, k_strides}, {v, v_strides}, {o, o_strides}, denom, B, H, N, D_qk,
-                              D_v, eps, dtype, chunked, workspace, workspace_bytes, stream);
+                              D_v, eps, dtype, chunked, workspace, workspace_bytes, stream, 0, nullptr, state_out,
+                              state_valid);
 }
 
 int fla_linear_attn_normalised_bwd(const void *grad_out, const void *q, const void *k, const void *v, const void *o,
@@ -1326,12 +1410,12 @@ int fla_linear_attn_normalised_bwd(const void *grad_out, const void *q, const vo
                                    int64_t N, int64_t D_qk, int64_t D_v, const int64_t *go_strides,
                                    const int64_t *q_strides, const int64_t *k_strides, const int64_t *v_strides,
                                    const int64_t *o_strides, const int64_t *dq_strides, const int64_t *dk_strides,
-                                   const int64_t *dv_strides, int dtype, int chunked, void *workspace,
-                                   int64_t workspace_bytes, void *stream) {
+                                   const int64_t *dv_strides, int dtype, int chunked, const void *state_in,
+                                   void *workspace, int64_t workspace_bytes, void *stream) {
     if (int rc = check_norm_args(B, H, N, D_qk, D_v, dtype)) return rc;
     return normalised_backward({grad_out, go_strides}, {q, q_strides}, {k, k_strides}, {v, v_strides},
                                {o, o_strides}, denom, {dq, dq_strides}, {dk, dk_strides}, {dv, dv_strides}, B, H, N,
-                               D_qk, D_v, dtype, chunked, workspace, workspace_bytes, stream);
+                               D_qk, D_v, dtype, chunked, workspace, workspace_bytes, stream, 0, state_in);
 }
 
 }  // extern "C"

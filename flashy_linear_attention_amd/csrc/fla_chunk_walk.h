@@ -72,6 +72,16 @@ struct WalkParams {
     // multiplied by the slope of phi computed from it; null: none.
     const void *slope_y;
     int64_t sy_b, sy_h, sy_n;
+    // The normaliser n_i = q_i . (k_0 + ... + k_i) + eps fused into the walks (null pointers: off).
+    // Forward (denom, zc): n_i = sum of row i's masked scores + q_i . zc_c; the result is divided by
+    // n_i and n goes to denom.  Backward, with dn_i = -(g_i . out_i) / n_i and dO = g / n prepared by
+    // the caller: dQ's scores get + dn_i and its result + dn_i zc_c (dn, zc); dK's scores get + dn_i
+    // (i: the dO row) and its result + rc_c (dn, rc).
+    float *denom;     // fp32 [BH][N]
+    float eps;
+    const float *zc;  // fp32 [BH][n_chunks][D]: sum of k over the rows before chunk c
+    const float *dn;  // fp32 [BH][N]
+    const float *rc;  // fp32 [BH][n_chunks][D]: sum of dn_i q_i over the rows after chunk c
 };
 
 template <int D>
@@ -85,6 +95,8 @@ struct WalkCfg {
     static constexpr int RPI = 1024 / RB;   // rows covered by one wave-level 1 KiB load
     static constexpr int NI = TILE / 4096;  // such loads per wave and tile
     static constexpr int STATE = D * RB;    // the 16-bit state in LDS
+    static constexpr int VEC = 3 * 1024;    // per set of tiles: zc, rc, dn of the chunk (fp32, 1 KiB each)
+    static constexpr int NID = C / 64;      // wave-level 256-byte loads of a chunk's dn
     static constexpr int NBLK = DB * DB;    // 32 x 32 blocks of the state: block b belongs to wave b % 4
     static constexpr int NBW = (NBLK + 3) / 4;  // state blocks per wave
     // a wave owns one 32-row block of the chunk as the X rows of every product, and -- with fewer
@@ -172,15 +184,67 @@ __device__ __forceinline__ typename Mma<T>::V8 walk_col_frag(const unsigned char
 // (the permutation of walk_col_frag_perm)
 __device__ __forceinline__ int walk_e_lane(int l32) { return 16 * ((l32 >> 2) & 1) + 4 * (l32 >> 3) + (l32 & 3); }
 
+// ---- small fp32 vectors of a chunk HBM -> LDS (every wave issues them, to the same place)
+template <int LDS_IMM>
+__device__ __forceinline__ void dma_4B_per_lane(u32x4 rsrc, uint32_t lds_base, uint32_t voffset, uint32_t soffset) {
+    asm volatile("s_add_u32 m0, %0, %4\n\ts_nop 0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                 :
+                 : "s"(lds_base), "v"(voffset), "s"(rsrc), "s"(soffset), "n"(LDS_IMM)
+                 : "memory", "m0", "scc");
+}
+__device__ __forceinline__ u32x4 walk_uniform_rsrc(const void *base, uint32_t bytes) {
+    const u32x4 r = make_rsrc(base, bytes);
+    return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)r[0]), (uint32_t)__builtin_amdgcn_readfirstlane((int)r[1]),
+                 (uint32_t)__builtin_amdgcn_readfirstlane((int)r[2]), (uint32_t)__builtin_amdgcn_readfirstlane((int)r[3])};
+}
+// D floats (16-byte aligned) to lds_dst: one load, lanes beyond D / 4 write zeros (1 KiB is written)
+template <int D>
+__device__ __forceinline__ void walk_load_vec(const float *src, uint32_t lds_dst, int lane) {
+    dma_16B_per_lane<0>(walk_uniform_rsrc(src, D * 4), (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_dst),
+                        (uint32_t)lane * 16, 0);
+}
+// rows row0 .. row0 + C - 1 of a vector of N floats (zeros past the end) to lds_dst
+template <int D>
+__device__ __forceinline__ void walk_load_rows(const float *vec, int row0, int N, uint32_t lds_dst, int lane) {
+    const u32x4 rs = walk_uniform_rsrc(vec + row0, (uint32_t)(N - row0) * 4);
+    const uint32_t base = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_dst);
+    static_for<0, WalkCfg<D>::NID>([&](auto u) {
+        constexpr int U = decltype(u)::value;
+        dma_4B_per_lane<U * 256>(rs, base, (uint32_t)lane * 4 + U * 256, 0);
+    });
+}
+
+// acc[i][v] += scale * vec[32 (db0 + i) + 16 g + v] (vec: fp32 in LDS)
+template <int D>
+__device__ __forceinline__ void walk_add_vec(f32x16 (&acc)[WalkCfg<D>::DBW], float scale, const float *vec, int db0, int g) {
+    typedef float f32x4 __attribute__((ext_vector_type(4)));  // (declared again below, for the products)
+#pragma unroll
+    for (int i = 0; i < WalkCfg<D>::DBW; ++i)
+#pragma unroll
+        for (int a = 0; a < 4; ++a) {
+            const f32x4 z = *reinterpret_cast<const f32x4 *>(vec + 32 * (db0 + i) + 16 * g + 4 * a);
+#pragma unroll
+            for (int b = 0; b < 4; ++b) acc[i][4 * a + b] += scale * z[b];
+        }
+}
+
 // ---- one product of a chunk for this wave's 32 X rows (row block rb = wave % NRB) and its part of
 // the output columns (blocks db0 .. db0 + DBW - 1, db0 = (wave / NRB) * DBW):
 //   acc = [state: X_w . State]  +  mask(X_w Y^T) Z        (UPPER: keep row <= column, else row >= column)
 // xt, yt, zt: LDS tiles; sfrag(db, kc): the state's A-operand fragment for output block db, k chunk kc.
 // (With several column parts the waves of one row block each compute the same scores.)
-template <typename T, int D, bool UPPER, typename SFrag>
+// EX (the normaliser's terms): 1: ex = sum of this row's masked scores + x_row . exv (exv: D floats in
+// LDS); 2: every score gets + ex (a value per X row, i.e. per lane) before the mask; 3: every
+// score gets + exv[its Y row] (exv: one float per tile row, in LDS).
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+struct WalkNoRows {
+    __device__ __forceinline__ f32x4 operator()(int, int) const { return f32x4{0.f, 0.f, 0.f, 0.f}; }
+};
+template <typename T, int D, bool UPPER, int EX = 0, typename SFrag, typename YRows = WalkNoRows>
 __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsigned char *yt, const unsigned char *zt,
                                              int wave, int lane, bool has_state, SFrag &&sfrag,
-                                             f32x16 (&acc)[WalkCfg<D>::DBW]) {
+                                             f32x16 (&acc)[WalkCfg<D>::DBW], float *ex = nullptr,
+                                             const float *exv = nullptr, YRows &&yrows = WalkNoRows{}) {
     using W = WalkCfg<D>;
     using M = Mma<T>;
     using V8 = typename M::V8;
@@ -189,6 +253,17 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
     V8 xf[W::KC];
 #pragma unroll
     for (int kc = 0; kc < W::KC; ++kc) xf[kc] = walk_row_frag<T, D>(xt, 32 * rb + l32, kc, g);
+    float rsum = 0.f;
+    if constexpr (EX == 1) {
+#pragma unroll
+        for (int kc = 0; kc < W::KC; ++kc)
+#pragma unroll
+            for (int a = 0; a < 2; ++a) {
+                const f32x4 z = *reinterpret_cast<const f32x4 *>(exv + 16 * kc + 8 * g + 4 * a);
+#pragma unroll
+                for (int b = 0; b < 4; ++b) rsum += static_cast<float>(xf[kc][4 * a + b]) * z[b];
+            }
+    }
 #pragma unroll
     for (int i = 0; i < W::DBW; ++i)
 #pragma unroll
@@ -207,6 +282,18 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
         for (int v = 0; v < 16; ++v) sc[v] = 0.f;
 #pragma unroll
         for (int kc = 0; kc < W::KC; ++kc) sc = M::mma(walk_row_frag<T, D>(yt, 32 * s + l32, kc, g), xf[kc], sc);
+        if constexpr (EX == 2) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) sc[v] += *ex;
+        }
+        if constexpr (EX == 3) {
+#pragma unroll
+            for (int a = 0; a < 4; ++a) {
+                const f32x4 y = yrows(s, a);
+#pragma unroll
+                for (int b = 0; b < 4; ++b) sc[4 * a + b] += y[b];
+            }
+        }
         if (s == rb) {  // the 32 x 32 block on the diagonal: lane = X row l32, register v = Y row jl
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
@@ -214,6 +301,10 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
                 const bool keep = UPPER ? l32 <= jl : l32 >= jl;
                 sc[v] = keep ? sc[v] : 0.f;
             }
+        }
+        if constexpr (EX == 1) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) rsum += sc[v];
         }
         V8 pf[2];
 #pragma unroll
@@ -226,6 +317,7 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
             for (int i = 0; i < W::DBW; ++i)
                 acc[i] = M::mma(walk_col_frag_perm<T, D>(zt, 32 * s + 16 * t, db0 + i, lane, false), pf[t], acc[i]);
     }
+    if constexpr (EX == 1) *ex = rsum + __shfl_xor(rsum, 32, 64);  // the two lanes of a row hold half the columns each
 }
 
 // Every element of the landed tile replaced by phi(element), in place, and the mapped rows written
@@ -371,13 +463,33 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
     const float *init = nullptr;
     if (p.init) init = p.init + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D);
 #pragma unroll
-    for (int i = 0; i < W::NBW; ++i) {
-        const int dbk = B::dbk(wave, i), eb = B::eb(wave);
+    for (int i = 0; i < W::NBW; ++i)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int r = 32 * dbk + 8 * (v / 4) + 4 * g + (v % 4), c = 32 * eb + l32;
-            st[i][v] = init && B::valid(wave, i) ? (p.init_transposed ? init[c * D + r] : init[r * D + c]) : 0.f;
-        }
+        for (int v = 0; v < 16; ++v) st[i][v] = 0.f;
+    if (!init) return;
+    // st[i][v] = State[r = 32 dbk(i) + 8 (v/4) + 4g + v%4][c = 32 eb + l32]: element r D + c of the
+    // buffer, or c D + r when it holds the transposed matrices (then four consecutive floats per v/4)
+    const int c = 32 * B::eb(wave) + l32;
+    if (p.init_transposed) {
+        typedef float f32x4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int i = 0; i < W::NBW; ++i)
+            if (B::valid(wave, i)) {
+#pragma unroll
+                for (int a = 0; a < 4; ++a) {
+                    const f32x4 t = *reinterpret_cast<const f32x4 *>(init + c * D + 32 * B::dbk(wave, i) + 8 * a + 4 * g);
+#pragma unroll
+                    for (int b = 0; b < 4; ++b) st[i][4 * a + b] = t[b];
+                }
+            }
+    } else {
+#pragma unroll
+        for (int i = 0; i < W::NBW; ++i)
+            if (B::valid(wave, i)) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    st[i][v] = init[(32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + c];
+            }
     }
 }
 
@@ -390,7 +502,8 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
 // chunk's tiles have been awaited, so that the wait for the tiles never includes fresh stores,
 // measured 20 % slower: the stores then compete with the loads in flight instead of filling the
 // gap after them.)
-template <typename T, int D, bool DOUBLE>
+// NORM: the instantiation that takes the normaliser's terms (WalkParams::denom / dn).
+template <typename T, int D, bool DOUBLE, bool NORM>
 __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
@@ -400,6 +513,7 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     unsigned char *tl = smem + SETS * 3 * W::TILE;
+    unsigned char *xv = tl + W::STATE;  // per set: zc, (unused), dn of the chunk
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int rb = W::NCH == 1 ? wave : wave % W::NRB, db0 = W::NCH == 1 ? 0 : (wave / W::NRB) * W::DBW;
@@ -425,7 +539,13 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
         walk_load_tile<D>(rq, base, c * W::C, qs2, p.wqk, wave, lane);
         walk_load_tile<D>(rk, base + W::TILE, c * W::C, ks2, p.wqk, wave, lane);
         walk_load_tile<D>(rv, base + 2 * W::TILE, c * W::C, vs2, p.wv, wave, lane);
+        const uint32_t xbase = lds0 + SETS * 3 * W::TILE + W::STATE + buf * W::VEC;
+        if constexpr (NORM) {
+            walk_load_vec<D>(p.zc + ((int64_t)sl.bh * p.n_chunks + c) * D, xbase, lane);
+            if (p.dn) walk_load_rows<D>(p.dn + (int64_t)sl.bh * N, c * W::C, N, xbase + 2048, lane);
+        }
     };
+    const int n_extra = NORM ? 1 + (p.dn ? W::NID : 0) : 0;  // loads per chunk and wave beyond the tiles
     if constexpr (DOUBLE) load_chunk(sl.c_lo, 0);
 #pragma unroll 1
     for (int c = sl.c_lo; c < sl.c_hi; ++c) {
@@ -452,10 +572,14 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
             if (more) load_chunk(c + 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
             // this wave's loads of chunk c have landed when at most the loads issued after them are
             // outstanding (the stores of the previous chunk were issued before those)
-            if (more)
-                wait_vm<3 * W::NI>();
-            else
+            if (!more)
                 wait_vm<0>();
+            else if (n_extra == 0)
+                wait_vm<3 * W::NI>();
+            else if (n_extra == 1)
+                wait_vm<3 * W::NI + 1>();
+            else
+                wait_vm<3 * W::NI + 1 + W::NID>();
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's part of the state is in LDS
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
@@ -477,9 +601,25 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
             }
         }
         f32x16 acc[W::DBW];
-        walk_product<T, D, false>(tq, tk, tv, wave, lane, c > 0, [&](int db, int kc) -> V8 {
-            return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g);
-        }, acc);
+        const float *vz = reinterpret_cast<const float *>(xv + buf * W::VEC);
+        const float *vd = reinterpret_cast<const float *>(xv + buf * W::VEC + 2048);
+        auto sfrag = [&](int db, int kc) -> V8 { return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g); };
+        if (NORM && p.denom) {  // forward with the normaliser: n = masked row sum + q . zc + eps
+            float tot;
+            walk_product<T, D, false, 1>(tq, tk, tv, wave, lane, c > 0, sfrag, acc, &tot, vz);
+            const float n = tot + p.eps, inv = 1.0f / n;
+#pragma unroll
+            for (int i = 0; i < W::DBW; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][v] *= inv;
+            if (db0 == 0 && g == 0 && row < N) p.denom[(int64_t)sl.bh * N + row] = n;
+        } else if (NORM && p.dn) {  // dQ with the normaliser's term: scores + dn_i, result + dn_i zc
+            float ax = vd[32 * rb + l32];
+            walk_product<T, D, false, 2>(tq, tk, tv, wave, lane, c > 0, sfrag, acc, &ax);
+            walk_add_vec<D>(acc, ax, vz, db0, g);
+        } else {
+            walk_product<T, D, false>(tq, tk, tv, wave, lane, c > 0, sfrag, acc);
+        }
         if (p.slope_y) {
 #pragma unroll
             for (int i = 0; i < W::DBW; ++i)
@@ -516,7 +656,7 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
 }
 
 // ---- backward: dQ, dV, dK of a chunk from one set of tiles; R += Q_c^T dO_c, chunks descending
-template <typename T, int D>
+template <typename T, int D, bool NORM>
 __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
@@ -526,6 +666,8 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     unsigned char *tq = smem, *tk = smem + W::TILE, *tv = smem + 2 * W::TILE, *tg = smem + 3 * W::TILE,
                   *tl = smem + 4 * W::TILE;
+    const float *vz = reinterpret_cast<const float *>(tl + W::STATE), *vr = vz + 256, *vd = vz + 512;
+    const uint32_t xbase = lds0 + 4 * W::TILE + W::STATE;
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const WalkSlice sl = walk_slice(p);
@@ -559,6 +701,11 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
         walk_load_tile<D>(rk, lds0 + W::TILE, row0, ks2, p.wqk, wave, lane);
         walk_load_tile<D>(rv, lds0 + 2 * W::TILE, row0, vs2, p.wv, wave, lane);
         walk_load_tile<D>(rg, lds0 + 3 * W::TILE, row0, gs2, p.wv, wave, lane);
+        if constexpr (NORM) {  // the normaliser's terms: zc, rc of this chunk and its rows of dn
+            walk_load_vec<D>(p.zc + ((int64_t)sl.bh * p.n_chunks + c) * D, xbase, lane);
+            walk_load_vec<D>(p.rc + ((int64_t)sl.bh * p.n_chunks + c) * D, xbase + 1024, lane);
+            walk_load_rows<D>(p.dn + (int64_t)sl.bh * N, row0, N, xbase + 2048, lane);
+        }
         // dQ's state, S_c[q/k index][v index] as saved by forward: A-operand fragments straight from
         // memory (row = output column of dQ, eight consecutive v indices)
         const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
@@ -577,8 +724,15 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
         const int row = row0 + 32 * wave + l32;
         const bool later = c + 1 < p.n_chunks;  // chunks after this one exist: R is not identically zero
         f32x16 acc[W::DBW];
-        // dQ = lower(dO V^T) K + dO S_c^T
-        walk_product<T, D, false>(tg, tv, tk, wave, lane, c > 0, [&](int db, int kc) -> V8 { return sfq[db][kc]; }, acc);
+        // dQ = lower(dO V^T) K + dO S_c^T  (normaliser: scores + dn_i, result + dn_i zc)
+        if constexpr (NORM) {
+            float ax = vd[32 * wave + l32];
+            walk_product<T, D, false, 2>(tg, tv, tk, wave, lane, c > 0, [&](int db, int kc) -> V8 { return sfq[db][kc]; },
+                                         acc, &ax);
+            walk_add_vec<D>(acc, ax, vz, 0, g);
+        } else {
+            walk_product<T, D, false>(tg, tv, tk, wave, lane, c > 0, [&](int db, int kc) -> V8 { return sfq[db][kc]; }, acc);
+        }
         walk_store<T, D>(rdq, dqs2, p.wqk, row, g, 0, acc, p.fmap, tq, 32 * wave + l32);
         // dV = upper(K Q^T) dO + K R: A operand R^T[v index][q/k index] = the LDS copy as it is
         walk_product<T, D, true>(tk, tq, tg, wave, lane, later, [&](int db, int kc) -> V8 {
@@ -586,9 +740,19 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
         }, acc);
         walk_store<T, D>(rdv, dvs2, p.wv, row, g, 0, acc);
         // dK = upper(V dO^T) Q + V R^T: A operand R[q/k index][v index] = the LDS copy read transposed
-        walk_product<T, D, true>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
-            return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
-        }, acc);
+        // (normaliser: scores + dn_i with i the dO row, result + rc)
+        if constexpr (NORM) {
+            walk_product<T, D, true, 3>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
+                return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
+            }, acc, nullptr, nullptr, [&](int s, int a) -> f32x4 {
+                return *reinterpret_cast<const f32x4 *>(vd + 32 * s + 8 * a + 4 * g);
+            });
+            walk_add_vec<D>(acc, 1.0f, vr, 0, g);
+        } else {
+            walk_product<T, D, true>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
+                return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
+            }, acc);
+        }
         walk_store<T, D>(rdk, dks2, p.wqk, row, g, 0, acc, p.fmap, tk, 32 * wave + l32);
         walk_update<T, D>(tq, tg, wave, lane, st);
         __syncthreads();
@@ -602,7 +766,11 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
 // ---- backward without saved per-chunk states, dV and dK: chunks descending, R += Q_c^T dO_c.  One
 // workgroup per CU with two sets of tiles: the loads of the next chunk are in flight while this
 // one is multiplied.  (dQ is a walk_fwd_kernel launch over dO, V, K.)
-template <typename T, int D>
+// NORM: dK with the normaliser's terms (scores + dn_i, i the dO row; result + rc).  Tiles and state
+// fill the LDS at D = 128, so the chunk's dn and this wave's columns of rc travel in registers: a
+// lane loads one value of each, a chunk ahead and after the tiles' loads, and the values are
+// handed round within the wave when the chunk's turn comes.
+template <typename T, int D, bool NORM>
 __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
@@ -643,17 +811,44 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
         walk_load_tile<D>(rv, base + 2 * W::TILE, row0, vs2, p.wv, wave, lane);
         walk_load_tile<D>(rg, base + 3 * W::TILE, row0, gs2, p.wv, wave, lane);
     };
+    static_assert(!NORM || W::C == 64, "one dn value per lane covers a chunk of 64 rows");
+    float nxt_dn = 0.f, nxt_rc = 0.f;
+    auto load_vecs = [&](int c) {  // lane l: dn of row l of chunk c, rc of column 32 db0 + l
+        if constexpr (NORM) {
+            const int row = c * W::C + lane;
+            nxt_dn = row < N ? p.dn[(int64_t)sl.bh * N + row] : 0.f;
+            nxt_rc = p.rc[((int64_t)sl.bh * p.n_chunks + c) * D + 32 * db0 + lane];
+        }
+    };
     load_chunk(sl.c_hi - 1, 0);
+    load_vecs(sl.c_hi - 1);
 #pragma unroll 1
     for (int c = sl.c_hi - 1; c >= sl.c_lo; --c) {
         const int buf = (sl.c_hi - 1 - c) & 1;
         unsigned char *tq = smem + buf * 4 * W::TILE, *tk = tq + W::TILE, *tv = tq + 2 * W::TILE, *tg = tq + 3 * W::TILE;
         const bool more = c > sl.c_lo;
-        if (more) load_chunk(c - 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
+        // this chunk's vectors, from the lanes that loaded them: dnv[a][b] = dn of tile row 8 a + 4 g + b,
+        // rcv[i][v] = rc of column 32 (db0 + i) + 16 g + v
+        f32x4 dnv[8];
+        f32x16 rcv[W::DBW];
+        if constexpr (NORM) {
+#pragma unroll
+            for (int a8 = 0; a8 < 8; ++a8)
+#pragma unroll
+                for (int b4 = 0; b4 < 4; ++b4) dnv[a8][b4] = __shfl(nxt_dn, 8 * a8 + 4 * g + b4, 64);
+#pragma unroll
+            for (int i = 0; i < W::DBW; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) rcv[i][v] = __shfl(nxt_rc, 32 * i + 16 * g + v, 64);
+        }
+        if (more) {
+            load_chunk(c - 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
+            load_vecs(c - 1);
+        }
         // this wave's loads of chunk c have landed when at most the loads issued after them are
         // outstanding (the stores of the previous chunk were issued before those)
         if (more)
-            wait_vm<4 * W::NI>();
+            wait_vm<4 * W::NI + (NORM ? 2 : 0)>();
         else
             wait_vm<0>();
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's part of the state is in LDS
@@ -668,9 +863,17 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
         }, acc);
         walk_store<T, D>(rdv, dvs2, p.wv, row, g, db0, acc);
         // dK = upper(V dO^T) Q + V R^T: A operand R[q/k index][v index] = the LDS copy read transposed
-        walk_product<T, D, true>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
-            return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
-        }, acc);
+        if constexpr (NORM) {
+            walk_product<T, D, true, 3>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
+                return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
+            }, acc, nullptr, nullptr, [&](int s, int a4) -> f32x4 { return s == 0 ? dnv[a4] : dnv[4 + a4]; });
+#pragma unroll
+            for (int i = 0; i < W::DBW; ++i) acc[i] += rcv[i];
+        } else {
+            walk_product<T, D, true>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
+                return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
+            }, acc);
+        }
         walk_store<T, D>(rdk, dks2, p.wqk, row, g, db0, acc, p.fmap, tk, 32 * rb + l32);
         walk_update<T, D>(tq, tg, wave, lane, st);
         asm volatile("" ::: "memory");
@@ -832,6 +1035,58 @@ __global__ __launch_bounds__(256) void walk_scan_kernel(const float *totals, flo
     }
 }
 
+// ---- per-chunk column sums for the normaliser's running vectors: out[bh][c][col] = sum over the
+// rows of chunk c of w[row] y[row][col] (w null: plain sums); fp32.  A scan over the chunks
+// (walk_scan_kernel, m = 1) then gives zc (y = k, prefix) or rc (y = q, w = dn, suffix).
+struct WalkVecParams {
+    const void *y;
+    int64_t ys_b, ys_h, ys_n;
+    const float *w;  // [BH][N] or null
+    int32_t H, N, width, n_chunks;
+    float *out;      // [BH][n_chunks][D]
+};
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void walk_vec_sums_kernel(const WalkVecParams p) {
+    using W = WalkCfg<D>;
+    using V8 = typename Mma<T>::V8;
+    constexpr int SLOTS = 256 / W::CR;  // rows visited at a time
+    __shared__ float part[SLOTS][D];
+    const int tid = threadIdx.x, pos = tid % W::CR, slot = tid / W::CR;
+    const int c = blockIdx.x, bh = blockIdx.y, b = bh / p.H, h = bh - b * p.H;
+    const T *Y = static_cast<const T *>(p.y) + b * p.ys_b + h * p.ys_h;
+    float acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    if (pos * 8 < p.width) {
+#pragma unroll 4
+        for (int r = slot; r < W::C; r += SLOTS) {
+            const int row = c * W::C + r;
+            if (row < p.N) {
+                const V8 y = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4 *>(Y + (int64_t)row * p.ys_n + pos * 8));
+                const float w = p.w ? p.w[(int64_t)bh * p.N + row] : 1.0f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[e] += w * static_cast<float>(y[e]);
+            }
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 8; ++e) part[slot][pos * 8 + e] = acc[e];
+    __syncthreads();
+    if (tid < D) {
+        float t = 0.f;
+#pragma unroll
+        for (int u = 0; u < SLOTS; ++u) t += part[u][tid];
+        p.out[((int64_t)bh * p.n_chunks + c) * D + tid] = t;
+    }
+}
+
+template <typename T, int D>
+hipError_t launch_walk_vec_sums(const WalkVecParams &p, int64_t BH, hipStream_t stream) {
+    if (BH > 65535) return hipErrorInvalidConfiguration;
+    return launch_kernel(walk_vec_sums_kernel<T, D>, dim3((unsigned)p.n_chunks, (unsigned)BH), dim3(256), 0, stream, p);
+}
+
 template <typename T, int D>
 hipError_t launch_walk_totals(const WalkTotalsParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
@@ -855,8 +1110,15 @@ hipError_t launch_walk_fwd(const WalkParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     constexpr bool kDouble = D > 64;  // (the plan's workgroup count must match: one per CU when double)
-    constexpr auto kern = walk_fwd_kernel<T, D, kDouble>;
     constexpr int smem = (kDouble ? 6 : 3) * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
+    if (p.denom || p.dn) {  // the normaliser's terms: its vectors live behind the state
+        if (!p.zc) return hipErrorInvalidValue;
+        constexpr auto kern = walk_fwd_kernel<T, D, kDouble, true>;
+        constexpr int smem_n = smem + (kDouble ? 2 : 1) * WalkCfg<D>::VEC;
+        if (hipError_t e = ensure_dynamic_lds<kern>(smem_n)) return e;
+        return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem_n, stream, p);
+    }
+    constexpr auto kern = walk_fwd_kernel<T, D, kDouble, false>;
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
     return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
 }
@@ -865,8 +1127,15 @@ template <typename T, int D>
 hipError_t launch_walk_bwd(const WalkParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-    constexpr auto kern = walk_bwd_kernel<T, D>;
     constexpr int smem = 4 * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
+    if (p.dn) {
+        if (!p.zc || !p.rc) return hipErrorInvalidValue;
+        constexpr auto kern = walk_bwd_kernel<T, D, true>;
+        constexpr int smem_n = smem + WalkCfg<D>::VEC;
+        if (hipError_t e = ensure_dynamic_lds<kern>(smem_n)) return e;
+        return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem_n, stream, p);
+    }
+    constexpr auto kern = walk_bwd_kernel<T, D, false>;
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
     return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
 }
@@ -875,9 +1144,15 @@ template <typename T, int D>
 hipError_t launch_walk_dkdv(const WalkParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-    constexpr auto kern = walk_dkdv_kernel<T, D>;
     constexpr int smem = 8 * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
     static_assert(smem <= 160 * 1024, "two sets of tiles and the state must fit the LDS of a CU");
+    if (p.dn) {
+        if (!p.rc) return hipErrorInvalidValue;
+        constexpr auto kern = walk_dkdv_kernel<T, D, true>;
+        if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
+        return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+    }
+    constexpr auto kern = walk_dkdv_kernel<T, D, false>;
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
     return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
 }

@@ -48,6 +48,7 @@ struct NormParams {
     // gradients are multiplied by phi'(x) computed from y -- they leave as gradients with respect
     // to x.  0: none.
     int32_t fmap;
+    int32_t only_dk;  // bwd-post: only the dk half (dq is complete)
 };
 
 template <typename T>
@@ -305,7 +306,7 @@ __global__ __launch_bounds__(256, 2) void norm_bwd_post_kernel(const NormParams 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int li = lane % LPR, seg = wave * G::RPS + lane / LPR;
     const int chunk = blockIdx.x, bh = blockIdx.y;
-    const bool part_dk = blockIdx.z != 0;
+    const bool part_dk = blockIdx.z != 0 || p.only_dk;
     const int b = bh / p.H, h = bh - b * p.H;
     // the scanned operand (k for dq, q for dk) and the gradient that is updated
     const T *S = part_dk ? static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h
@@ -424,7 +425,7 @@ hipError_t launch_norm_lpr(int which, const NormParams &p, hipStream_t s) {
         if (hipError_t e = launch_kernel(norm_chunk_sums_kernel<T, LPR, VEC, true>, grid, dim3(256), 0, s, p)) return e;
         if (hipError_t e = launch_norm_scan(p, LPR * 8, true, s)) return e;
     }
-    return launch_kernel(norm_bwd_post_kernel<T, LPR, VEC>, dim3(grid.x, grid.y, 2), dim3(256), 0, s, p);
+    return launch_kernel(norm_bwd_post_kernel<T, LPR, VEC>, dim3(grid.x, grid.y, p.only_dk ? 1 : 2), dim3(256), 0, s, p);
 }
 
 // lpr from norm_lanes_per_row; vec: every operand of this call qualifies for 16-byte accesses

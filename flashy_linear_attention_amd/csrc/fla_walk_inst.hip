@@ -26,6 +26,9 @@ hipError_t walk_totals(int dtype, int D, const WalkTotalsParams &p, hipStream_t 
 hipError_t walk_fwd(int dtype, int D, const WalkParams &p, hipStream_t stream) {
     FLA_WALK_DISPATCH3(launch_walk_fwd, p, stream);
 }
+hipError_t walk_vec_sums(int dtype, int D, const WalkVecParams &p, int64_t BH, hipStream_t stream) {
+    FLA_WALK_DISPATCH3(launch_walk_vec_sums, p, BH, stream);
+}
 hipError_t walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, int m, int E, int reverse,
                      hipStream_t stream) {
     return launch_walk_scan(totals, entry, BH, n_seg, m, E, reverse, stream);

@@ -107,9 +107,9 @@ def feature_attention_bwd(grad_output: torch.Tensor, q: torch.Tensor, k: torch.T
 
 
 def feature_attention_normalised_fwd(xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, feature: str = "elu1",
-                                     eps: float = 1e-5, chunked: bool = True):
+                                     eps: float = 1e-5, chunked: bool = True, want_state: bool = False):
     """``(out, q, k, denom)``: the normalised output, ``q = phi(xq)``, ``k = phi(xk)`` and the fp32
-    normaliser (B, H, N)."""
+    normaliser (B, H, N); with ``want_state`` also what the chunk-wise forward hands to backward (or None)."""
     assert xq.shape == xk.shape and v.shape[:3] == xq.shape[:3], "xq, xk: (B,H,N,D_qk); v: (B,H,N,D_v)"
     assert xq.shape[-1] <= 256 and v.shape[-1] <= 256, "Only head_dims <= 256 are supported."
     code = _map_code(feature)
@@ -124,6 +124,9 @@ def feature_attention_normalised_fwd(xq: torch.Tensor, xk: torch.Tensor, v: torc
     with torch.cuda.device(xq.device):
         nbytes = lib.fla_normalised_workspace_bytes(b, h, n, dqk, dv, int(chunked))
         work = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=xq.device)
+        sbytes = lib.fla_linear_attn_chunked_state_bytes(b, h, n, dqk, dv) if (want_state and chunked) else 0
+        state = torch.empty(sbytes, dtype=torch.uint8, device=xq.device) if sbytes else None
+        valid = ctypes.c_int32(0)
         _lib.check(
             "fla_feature_attn_normalised_fwd",
             lib.fla_feature_attn_normalised_fwd(
@@ -131,16 +134,20 @@ def feature_attention_normalised_fwd(xq: torch.Tensor, xk: torch.Tensor, v: torc
                 b, h, n, dqk, dv,
                 _lib.strides_arg(xq), _lib.strides_arg(xk), _lib.strides_arg(v), _lib.strides_arg(out),
                 _lib.strides_arg(q), _lib.strides_arg(k),
-                code, float(eps), dtype_code(xq), int(chunked), work.data_ptr(), nbytes, stream_handle(xq.device),
+                code, float(eps), dtype_code(xq), int(chunked), state.data_ptr() if state is not None else None,
+                ctypes.byref(valid), work.data_ptr(), nbytes, stream_handle(xq.device),
             ),
         )
+    if want_state:
+        return out, q, k, denom, (state if valid.value else None)
     return out, q, k, denom
 
 
 def feature_attention_normalised_bwd(grad_output: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor,
                                      out: torch.Tensor, denom: torch.Tensor, feature: str = "elu1",
-                                     chunked: bool = True) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """(dxq, dxk, dv) from the forward call's ``q``, ``k``, ``out`` and ``denom``."""
+                                     chunked: bool = True,
+                                     state: torch.Tensor = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dxq, dxk, dv) from the forward call's ``q``, ``k``, ``out`` and ``denom`` (and ``state``, if any)."""
     code = _map_code(feature)
     grad_output, q, k, v, out = prepare(grad_output, q, k, v, out)
     assert denom.dtype == torch.float32 and denom.is_contiguous() and denom.shape == q.shape[:3]
@@ -160,7 +167,8 @@ def feature_attention_normalised_bwd(grad_output: torch.Tensor, q: torch.Tensor,
                 dxq.data_ptr(), dxk.data_ptr(), dvv.data_ptr(), b, h, n, dqk, dv,
                 _lib.strides_arg(grad_output), _lib.strides_arg(q), _lib.strides_arg(k), _lib.strides_arg(v),
                 _lib.strides_arg(out), _lib.strides_arg(dxq), _lib.strides_arg(dxk), _lib.strides_arg(dvv),
-                code, dtype_code(q), int(chunked), work.data_ptr(), nbytes, stream_handle(q.device),
+                code, dtype_code(q), int(chunked), state.data_ptr() if state is not None else None, work.data_ptr(),
+                nbytes, stream_handle(q.device),
             ),
         )
     return dxq, dxk, dvv
@@ -173,9 +181,12 @@ class FeatureMapLinearAttention(Function):
                 normalise: bool = False, eps: float = 1e-5, chunked: bool = True) -> torch.Tensor:
         ctx.normalise = normalise
         if normalise:
-            out, q, k, denom = feature_attention_normalised_fwd(xq, xk, v, feature, eps, chunked)
+            want = bool(chunked) and any(ctx.needs_input_grad[:3])
+            out, q, k, denom, state = feature_attention_normalised_fwd(xq, xk, v, feature, eps, chunked, want_state=True) \
+                if want else (*feature_attention_normalised_fwd(xq, xk, v, feature, eps, chunked), None)
             ctx.feature, ctx.chunked = feature, chunked
-            ctx.save_for_backward(q, k, v, out, denom)
+            ctx.has_state = state is not None
+            ctx.save_for_backward(*((q, k, v, out, denom) + ((state,) if state is not None else ())))
             return out
         assert chunked, "without the normaliser the feature map exists for the chunk-wise product only"
         if any(ctx.needs_input_grad[:3]):
@@ -194,8 +205,10 @@ class FeatureMapLinearAttention(Function):
     @torch.amp.custom_bwd(device_type="cuda")
     def backward(ctx: Any, grad_output: torch.Tensor):
         if ctx.normalise:
-            q, k, v, out, denom = ctx.saved_tensors
-            dxq, dxk, dv = feature_attention_normalised_bwd(grad_output, q, k, v, out, denom, ctx.feature, ctx.chunked)
+            q, k, v, out, denom = ctx.saved_tensors[:5]
+            state = ctx.saved_tensors[5] if ctx.has_state else None
+            dxq, dxk, dv = feature_attention_normalised_bwd(grad_output, q, k, v, out, denom, ctx.feature, ctx.chunked,
+                                                            state)
             return dxq, dxk, dv, None, None, None, None
         if ctx.has_state:
             q, k, v, state = ctx.saved_tensors

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 1
+#define FLA_ABI_VERSION 2
 
 enum fla_dtype { FLA_DTYPE_BF16 = 0, FLA_DTYPE_F16 = 1 };
 
@@ -230,6 +230,7 @@ int fla_feature_attn_normalised_fwd(const void *xq, const void *xk, const void *
                                     const int64_t *v_strides, const int64_t *o_strides,
                                     const int64_t *q_out_strides, const int64_t *k_out_strides,
                                     int feature_map, float eps, int dtype, int chunked,
+                                    void *state_out, int32_t *state_valid,
                                     void *workspace, int64_t workspace_bytes, void *stream);
 int fla_feature_attn_normalised_bwd(const void *grad_out, const void *q, const void *k, const void *v,
                                     const void *o, const float *denom, void *dxq, void *dxk, void *dv,
@@ -238,7 +239,7 @@ int fla_feature_attn_normalised_bwd(const void *grad_out, const void *q, const v
                                     const int64_t *k_strides, const int64_t *v_strides,
                                     const int64_t *o_strides, const int64_t *dxq_strides,
                                     const int64_t *dxk_strides, const int64_t *dv_strides,
-                                    int feature_map, int dtype, int chunked,
+                                    int feature_map, int dtype, int chunked, const void *state_in,
                                     void *workspace, int64_t workspace_bytes, void *stream);
 
 /* fla_linear_attn_chunked_fwd for callers that cannot allocate device memory or pass a workspace
@@ -306,7 +307,12 @@ int fla_poly_attn_bwd(const void *grad_out, const void *xq, const void *xk, cons
  * (1..256).  `chunked` != 0 evaluates the products chunk-wise (fla_linear_attn_chunked_fwd/bwd's
  * method) instead of with the quadratic kernels.  `workspace`: at least
  * fla_normalised_workspace_bytes() bytes (same `chunked`) of 16-byte aligned device memory,
- * scratch.  B*H must not exceed 65535.  No counterpart in the reference's kernels; replaces the caller-side recipe and its
+ * scratch.  state_out / state_valid / state_in: with `chunked`, what the chunk-wise forward hands to
+ * its backward, exactly as for fla_linear_attn_chunked_fwd/bwd (size:
+ * fla_linear_attn_chunked_state_bytes(); any of them may be null, backward then works without);
+ * ignored otherwise.  With `chunked` and equal padded head dims up to 128 the normaliser and
+ * its gradient terms are computed inside the chunk-wise kernels rather than by passes of their
+ * own.  B*H must not exceed 65535.  No counterpart in the reference's kernels; replaces the caller-side recipe and its
  * autograd graph (a cumsum, two elementwise products, a row sum and a division, each a full
  * pass over memory, forward and backward). */
 int64_t fla_normalised_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v, int chunked);
@@ -315,6 +321,7 @@ int fla_linear_attn_normalised_fwd(const void *q, const void *k, const void *v, 
                                    const int64_t *q_strides, const int64_t *k_strides,
                                    const int64_t *v_strides, const int64_t *o_strides,
                                    float eps, int dtype, int chunked,
+                                   void *state_out, int32_t *state_valid,
                                    void *workspace, int64_t workspace_bytes, void *stream);
 int fla_linear_attn_normalised_bwd(const void *grad_out, const void *q, const void *k, const void *v,
                                    const void *o, const float *denom, void *dq, void *dk, void *dv,
@@ -323,7 +330,7 @@ int fla_linear_attn_normalised_bwd(const void *grad_out, const void *q, const vo
                                    const int64_t *k_strides, const int64_t *v_strides,
                                    const int64_t *o_strides, const int64_t *dq_strides,
                                    const int64_t *dk_strides, const int64_t *dv_strides,
-                                   int dtype, int chunked,
+                                   int dtype, int chunked, const void *state_in,
                                    void *workspace, int64_t workspace_bytes, void *stream);
 
 #ifdef __cplusplus

@@ -88,17 +88,17 @@ def test_c_abi_validation_codes():
     assert t(A[0], A[1], A[2], A[3], 1, 2, 64, 32, 32, S, S, S, S, 1, 5, None) == -2
     nf = lib.fla_linear_attn_normalised_fwd
     eps = ctypes.c_float(1e-5)
-    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 64, 32, 32, S, S, S, S, eps, 9, 0, None, 0, None) == -2
-    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 64, 257, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -3
-    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 64, 32, 0, S, S, S, S, eps, 0, 0, None, 0, None) == -4
-    assert nf(A[0], A[1], A[2], A[3], A[4], 300, 300, 64, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -5   # B H > 65535
-    assert nf(A[0], A[1], A[2], A[3], None, 1, 2, 64, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -1    # denom
-    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 64, 32, 32, S, S, BAD_S, S, eps, 0, 0, None, 0, None) == -6
-    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 4096, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -9     # chunk sums need workspace
-    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 0, 64, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == 0
+    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 64, 32, 32, S, S, S, S, eps, 9, 0, None, None, None, 0, None) == -2
+    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 64, 257, 32, S, S, S, S, eps, 0, 0, None, None, None, 0, None) == -3
+    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 64, 32, 0, S, S, S, S, eps, 0, 0, None, None, None, 0, None) == -4
+    assert nf(A[0], A[1], A[2], A[3], A[4], 300, 300, 64, 32, 32, S, S, S, S, eps, 0, 0, None, None, None, 0, None) == -5   # B H > 65535
+    assert nf(A[0], A[1], A[2], A[3], None, 1, 2, 64, 32, 32, S, S, S, S, eps, 0, 0, None, None, None, 0, None) == -1    # denom
+    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 64, 32, 32, S, S, BAD_S, S, eps, 0, 0, None, None, None, 0, None) == -6
+    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 2, 4096, 32, 32, S, S, S, S, eps, 0, 0, None, None, None, 0, None) == -9     # chunk sums need workspace
+    assert nf(A[0], A[1], A[2], A[3], A[4], 1, 0, 64, 32, 32, S, S, S, S, eps, 0, 0, None, None, None, 0, None) == 0
     nb = lib.fla_linear_attn_normalised_bwd
-    assert nb(A[0], A[1], A[2], A[3], A[4], A[5], A[6], A[7], A[8], 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, 0, None, 0, None) == -9
-    assert nb(A[0], A[1], A[2], A[3], A[4], None, A[6], A[7], A[8], 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, 1, A[9], 1 << 30, None) == -1
+    assert nb(A[0], A[1], A[2], A[3], A[4], A[5], A[6], A[7], A[8], 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, 0, None, None, 0, None) == -9
+    assert nb(A[0], A[1], A[2], A[3], A[4], None, A[6], A[7], A[8], 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, 1, None, A[9], 1 << 30, None) == -1
     assert lib.fla_normalised_workspace_bytes(1, 2, 64, 32, 32, 0) >= 2 * 64 * 32 * 2 + 2 * 64 * 4
     assert lib.fla_normalised_workspace_bytes(1, 2, 64, 300, 32, 0) == 0
     assert (lib.fla_normalised_workspace_bytes(1, 2, 4096, 64, 64, 1)
@@ -136,10 +136,10 @@ def test_c_abi_rejects_outputs_that_overlap_inputs():
     assert cb(g, q, k, v, dq, dk, v, 1, 2, 64, 32, 32, S, S, S, S, S, S, S, 0, None, None, 0, None) == -10
     eps = ctypes.c_float(1e-5)
     nf = lib.fla_linear_attn_normalised_fwd
-    assert nf(q, k, v, k, A[8], 1, 2, 64, 32, 32, S, S, S, S, eps, 0, 0, None, 0, None) == -10
+    assert nf(q, k, v, k, A[8], 1, 2, 64, 32, 32, S, S, S, S, eps, 0, 0, None, None, None, 0, None) == -10
     nb = lib.fla_linear_attn_normalised_bwd
     # the forward's output is an input of backward: a gradient must not land on it
-    assert nb(g, q, k, v, o, A[8], dq, o, dv, 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, 0, A[9], 1 << 30, None) == -10
+    assert nb(g, q, k, v, o, A[8], dq, o, dv, 1, 2, 64, 32, 32, S, S, S, S, S, S, S, S, 0, 0, None, A[9], 1 << 30, None) == -10
     coef = (ctypes.c_float * 3)(0.0, 0.0, 0.5)
     pf = lib.fla_poly_attn_fwd
     assert pf(q, k, v, v, None, 1, 2, 64, 16, 32, S, S, S, S, coef, eps, 0, None) == -10

@@ -158,14 +158,14 @@ def test_normalised_workspace_is_checked(gpu_device):
     assert need > 0
     rc = lib.fla_linear_attn_normalised_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                             denom.data_ptr(), 1, 2, 1024, 64, 64, st(q), st(k), st(v), st(out),
-                                            ctypes.c_float(1e-5), 0, 0, None, 0, stream)
+                                            ctypes.c_float(1e-5), 0, 0, None, None, None, 0, stream)
     assert rc == -9  # FLA_ERR_WORKSPACE: several chunks need the chunk sums
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     work = torch.empty(need, dtype=torch.uint8, device=gpu_device)
     rc = lib.fla_linear_attn_normalised_bwd(dy.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                                             denom.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
                                             1, 2, 1024, 64, 64, st(dy), st(q), st(k), st(v), st(out), st(dq), st(dk),
-                                            st(dv), 0, 0, work.data_ptr(), need - 1, stream)
+                                            st(dv), 0, 0, None, work.data_ptr(), need - 1, stream)
     assert rc == -9
     torch.cuda.synchronize()
 
