@@ -170,11 +170,14 @@ def test_normalised_workspace_is_checked(gpu_device):
     torch.cuda.synchronize()
 
 
-@pytest.mark.parametrize("dims", [(2, 2, 1536, 128, 128), (1, 2, 2304, 64, 64), (1, 2, 1024, 256, 64), (1, 1, 256, 64, 64)],
+@pytest.mark.parametrize("dims", [(2, 2, 1536, 128, 128), (1, 2, 2304, 64, 64), (1, 2, 1024, 256, 64), (1, 1, 256, 64, 64),
+                                  (2, 8, 2450, 128, 128), (8, 8, 2100, 64, 64), (1, 4, 1500, 104, 120), (1, 3, 777, 32, 24)],
                          ids=lambda d: "x".join(map(str, d)))
 def test_normalised_with_chunkwise_product(dims, gpu_device):
-    """chunked=True: the product goes through the chunk states, the normaliser passes are the
-    same; parity against the oracle as for the quadratic product."""
+    """chunked=True: equal padded head dims up to 128 form the normaliser and its gradient terms
+    inside the chunk-wise walk kernels (ragged last chunks and segments, several chunks per
+    workgroup, padded widths among the cases), other shapes run the chunk states and the normaliser
+    passes; parity against the oracle as for the quadratic product."""
     bs, nh, sq, dqk, dv = dims
     q, k, v, dy = reference_style_inputs(bs, nh, sq, dqk, dv, torch.bfloat16, seed=sum(dims) + 1)
     want_o, _, want_dq, want_dk, want_dv = _oracle(q, k, v, dy, 1e-5)
@@ -184,3 +187,22 @@ def test_normalised_with_chunkwise_product(dims, gpu_device):
     assert_close("out", out, want_o)
     for name, got, want in (("dQ", qg.grad, want_dq), ("dK", kg.grad, want_dk), ("dV", vg.grad, want_dv)):
         assert_close(name, got, want, tol_fro=1e-2, tol_max=5e-2)
+
+
+@pytest.mark.parametrize("dims", [(2, 3, 1280, 128, 128), (2, 3, 1280, 64, 64)], ids=lambda d: "x".join(map(str, d)))
+def test_normalised_chunkwise_backward_with_and_without_the_forward_state(dims, gpu_device):
+    """Backward given what the chunk-wise forward saved, and backward without it, both match the oracle;
+    forward returns the same output and normaliser either way."""
+    bs, nh, sq, dqk, dv = dims
+    q, k, v, dy = reference_style_inputs(bs, nh, sq, dqk, dv, torch.bfloat16, seed=77)
+    want_o, want_n, want_dq, want_dk, want_dv = _oracle(q, k, v, dy, 1e-5)
+    q, k, v, dy = (t.to(gpu_device) for t in (q, k, v, dy))
+    out, denom, state = linear_attention_normalised_fwd(q, k, v, 1e-5, True, want_state=True)
+    out2, denom2 = linear_attention_normalised_fwd(q, k, v, 1e-5, True)
+    assert state is not None and torch.equal(out, out2) and torch.equal(denom, denom2)
+    assert_close("out", out, want_o)
+    assert_close("n", denom, want_n.reshape(denom.shape), tol_fro=1e-4, tol_max=1e-3)
+    for st in (state, None):
+        got = linear_attention_normalised_bwd(dy, q, k, v, out, denom, True, st)
+        for name, g, w in zip(("dQ", "dK", "dV"), got, (want_dq, want_dk, want_dv)):
+            assert_close(f"{name} ({'with' if st is not None else 'without'} state)", g, w, tol_fro=1e-2, tol_max=5e-2)
