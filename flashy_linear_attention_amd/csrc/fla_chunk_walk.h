@@ -502,8 +502,8 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
 // chunk's tiles have been awaited, so that the wait for the tiles never includes fresh stores,
 // measured 20 % slower: the stores then compete with the loads in flight instead of filling the
 // gap after them.)
-// NORM: the instantiation that takes the normaliser's terms (WalkParams::denom / dn).
-template <typename T, int D, bool DOUBLE, bool NORM>
+// NORM: the instantiations that take the normaliser's terms: 1 forward (WalkParams::denom), 2 dQ (dn).
+template <typename T, int D, bool DOUBLE, int NORM>
 __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
@@ -542,10 +542,10 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
         const uint32_t xbase = lds0 + SETS * 3 * W::TILE + W::STATE + buf * W::VEC;
         if constexpr (NORM) {
             walk_load_vec<D>(p.zc + ((int64_t)sl.bh * p.n_chunks + c) * D, xbase, lane);
-            if (p.dn) walk_load_rows<D>(p.dn + (int64_t)sl.bh * N, c * W::C, N, xbase + 2048, lane);
+            if constexpr (NORM == 2) walk_load_rows<D>(p.dn + (int64_t)sl.bh * N, c * W::C, N, xbase + 2048, lane);
         }
     };
-    const int n_extra = NORM ? 1 + (p.dn ? W::NID : 0) : 0;  // loads per chunk and wave beyond the tiles
+    constexpr int n_extra = NORM == 0 ? 0 : NORM == 1 ? 1 : 1 + W::NID;  // loads per chunk and wave beyond the tiles
     if constexpr (DOUBLE) load_chunk(sl.c_lo, 0);
 #pragma unroll 1
     for (int c = sl.c_lo; c < sl.c_hi; ++c) {
@@ -572,14 +572,10 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
             if (more) load_chunk(c + 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
             // this wave's loads of chunk c have landed when at most the loads issued after them are
             // outstanding (the stores of the previous chunk were issued before those)
-            if (!more)
-                wait_vm<0>();
-            else if (n_extra == 0)
-                wait_vm<3 * W::NI>();
-            else if (n_extra == 1)
-                wait_vm<3 * W::NI + 1>();
+            if (more)
+                wait_vm<3 * W::NI + n_extra>();
             else
-                wait_vm<3 * W::NI + 1 + W::NID>();
+                wait_vm<0>();
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's part of the state is in LDS
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
@@ -604,7 +600,7 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
         const float *vz = reinterpret_cast<const float *>(xv + buf * W::VEC);
         const float *vd = reinterpret_cast<const float *>(xv + buf * W::VEC + 2048);
         auto sfrag = [&](int db, int kc) -> V8 { return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g); };
-        if (NORM && p.denom) {  // forward with the normaliser: n = masked row sum + q . zc + eps
+        if constexpr (NORM == 1) {  // forward with the normaliser: n = masked row sum + q . zc + eps
             float tot;
             walk_product<T, D, false, 1>(tq, tk, tv, wave, lane, c > 0, sfrag, acc, &tot, vz);
             const float n = tot + p.eps, inv = 1.0f / n;
@@ -613,7 +609,7 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[i][v] *= inv;
             if (db0 == 0 && g == 0 && row < N) p.denom[(int64_t)sl.bh * N + row] = n;
-        } else if (NORM && p.dn) {  // dQ with the normaliser's term: scores + dn_i, result + dn_i zc
+        } else if constexpr (NORM == 2) {  // dQ with the normaliser's term: scores + dn_i, result + dn_i zc
             float ax = vd[32 * rb + l32];
             walk_product<T, D, false, 2>(tq, tk, tv, wave, lane, c > 0, sfrag, acc, &ax);
             walk_add_vec<D>(acc, ax, vz, db0, g);
@@ -769,7 +765,8 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
 // NORM: dK with the normaliser's terms (scores + dn_i, i the dO row; result + rc).  Tiles and state
 // fill the LDS at D = 128, so the chunk's dn and this wave's columns of rc travel in registers: a
 // lane loads one value of each, a chunk ahead and after the tiles' loads, and the values are
-// handed round within the wave when the chunk's turn comes.
+// handed round within the wave (ds_bpermute: 64 per chunk, about 30 clocks each -- 28 us of a 207 us
+// launch at B H = 128, N = 4096) when the chunk's turn comes.
 template <typename T, int D, bool NORM>
 __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -812,12 +809,21 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
         walk_load_tile<D>(rg, base + 3 * W::TILE, row0, gs2, p.wv, wave, lane);
     };
     static_assert(!NORM || W::C == 64, "one dn value per lane covers a chunk of 64 rows");
+    // The two loads go out as inline assembly, like the tiles': a load the compiler knows of would be
+    // awaited with vmcnt(0) at its first use (loads and stores may complete out of order among each
+    // other, so it cannot count past the stores issued in between), and the previous chunk's stores
+    // with it.  Here the values are needed after the wait for the tiles, which covers every older load.
     float nxt_dn = 0.f, nxt_rc = 0.f;
+    u32x4 rs_dn = {0u, 0u, 0u, 0u}, rs_rc = {0u, 0u, 0u, 0u};
+    if constexpr (NORM) {
+        rs_dn = walk_uniform_rsrc(p.dn + (int64_t)sl.bh * N, (uint32_t)N * 4);  // (rows past the end read as zero)
+        rs_rc = walk_uniform_rsrc(p.rc + (int64_t)sl.bh * p.n_chunks * D, (uint32_t)p.n_chunks * D * 4);
+    }
     auto load_vecs = [&](int c) {  // lane l: dn of row l of chunk c, rc of column 32 db0 + l
         if constexpr (NORM) {
-            const int row = c * W::C + lane;
-            nxt_dn = row < N ? p.dn[(int64_t)sl.bh * N + row] : 0.f;
-            nxt_rc = p.rc[((int64_t)sl.bh * p.n_chunks + c) * D + 32 * db0 + lane];
+            const uint32_t off_dn = (uint32_t)(c * W::C + lane) * 4, off_rc = (uint32_t)(c * D + 32 * db0 + lane) * 4;
+            asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "+v"(nxt_dn) : "v"(off_dn), "s"(rs_dn) : "memory");
+            asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "+v"(nxt_rc) : "v"(off_rc), "s"(rs_rc) : "memory");
         }
     };
     load_chunk(sl.c_hi - 1, 0);
@@ -827,11 +833,19 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
         const int buf = (sl.c_hi - 1 - c) & 1;
         unsigned char *tq = smem + buf * 4 * W::TILE, *tk = tq + W::TILE, *tv = tq + 2 * W::TILE, *tg = tq + 3 * W::TILE;
         const bool more = c > sl.c_lo;
+        if (more) load_chunk(c - 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
+        // this wave's loads of chunk c have landed when at most the loads issued after them are
+        // outstanding (the stores of the previous chunk were issued before those)
+        if (more)
+            wait_vm<4 * W::NI>();
+        else
+            wait_vm<0>();
         // this chunk's vectors, from the lanes that loaded them: dnv[a][b] = dn of tile row 8 a + 4 g + b,
-        // rcv[i][v] = rc of column 32 (db0 + i) + 16 g + v
+        // rcv[i][v] = rc of column 32 (db0 + i) + 16 g + v; then the next chunk's loads
         f32x4 dnv[8];
         f32x16 rcv[W::DBW];
         if constexpr (NORM) {
+            asm volatile("" : "+v"(nxt_dn), "+v"(nxt_rc));  // (the values as they are after the wait)
 #pragma unroll
             for (int a8 = 0; a8 < 8; ++a8)
 #pragma unroll
@@ -840,17 +854,9 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
             for (int i = 0; i < W::DBW; ++i)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) rcv[i][v] = __shfl(nxt_rc, 32 * i + 16 * g + v, 64);
+            asm volatile("" ::"v"(dnv[7]), "v"(rcv[W::DBW - 1]));  // (handed round before the registers are loaded again)
+            if (more) load_vecs(c - 1);
         }
-        if (more) {
-            load_chunk(c - 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
-            load_vecs(c - 1);
-        }
-        // this wave's loads of chunk c have landed when at most the loads issued after them are
-        // outstanding (the stores of the previous chunk were issued before those)
-        if (more)
-            wait_vm<4 * W::NI + (NORM ? 2 : 0)>();
-        else
-            wait_vm<0>();
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's part of the state is in LDS
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
@@ -1113,12 +1119,17 @@ hipError_t launch_walk_fwd(const WalkParams &p, hipStream_t stream) {
     constexpr int smem = (kDouble ? 6 : 3) * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
     if (p.denom || p.dn) {  // the normaliser's terms: its vectors live behind the state
         if (!p.zc) return hipErrorInvalidValue;
-        constexpr auto kern = walk_fwd_kernel<T, D, kDouble, true>;
         constexpr int smem_n = smem + (kDouble ? 2 : 1) * WalkCfg<D>::VEC;
+        if (p.denom) {
+            constexpr auto kern = walk_fwd_kernel<T, D, kDouble, 1>;
+            if (hipError_t e = ensure_dynamic_lds<kern>(smem_n)) return e;
+            return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem_n, stream, p);
+        }
+        constexpr auto kern = walk_fwd_kernel<T, D, kDouble, 2>;
         if (hipError_t e = ensure_dynamic_lds<kern>(smem_n)) return e;
         return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem_n, stream, p);
     }
-    constexpr auto kern = walk_fwd_kernel<T, D, kDouble, false>;
+    constexpr auto kern = walk_fwd_kernel<T, D, kDouble, 0>;
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
     return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
 }
