@@ -459,7 +459,7 @@ int walk_chunk_vectors(const WalkPlan &wp, const View &y, int64_t width, const f
     vp.w = w, vp.H = (int32_t)H, vp.N = (int32_t)N, vp.width = (int32_t)width, vp.n_chunks = (int32_t)wp.n_chunks;
     vp.out = out;
     if (fla::walk_vec_sums(dtype, wp.D, vp, B * H, s) != hipSuccess) return FLA_ERR_LAUNCH;
-    return fla::walk_scan(out, out, B * H, (int)wp.n_chunks, 1, wp.D, reverse, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+    return fla::walk_vec_scan(out, B * H, (int)wp.n_chunks, wp.D, reverse, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
 }
 
 bool states_shareable(int64_t dqk, int64_t dv, int64_t N) {

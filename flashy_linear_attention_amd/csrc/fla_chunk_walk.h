@@ -1043,7 +1043,7 @@ __global__ __launch_bounds__(256) void walk_scan_kernel(const float *totals, flo
 
 // ---- per-chunk column sums for the normaliser's running vectors: out[bh][c][col] = sum over the
 // rows of chunk c of w[row] y[row][col] (w null: plain sums); fp32.  A scan over the chunks
-// (walk_scan_kernel, m = 1) then gives zc (y = k, prefix) or rc (y = q, w = dn, suffix).
+// (walk_vec_scan_kernel) then gives zc (y = k, prefix) or rc (y = q, w = dn, suffix).
 struct WalkVecParams {
     const void *y;
     int64_t ys_b, ys_h, ys_n;
@@ -1085,6 +1085,52 @@ __global__ __launch_bounds__(256) void walk_vec_sums_kernel(const WalkVecParams 
         for (int u = 0; u < SLOTS; ++u) t += part[u][tid];
         p.out[((int64_t)bh * p.n_chunks + c) * D + tid] = t;
     }
+}
+
+// ---- exclusive prefix (reverse: suffix) sums over the chunks of the vectors above, in place:
+// v[bh][c][col] <- sum of v[bh][c'][col] over c' < c (c' > c).  There are few columns and many
+// chunks, so the chunks of a (b, h) are split over sixteen thread groups: each adds up its range,
+// the ranges' sums are scanned in LDS, and each group writes its range's running sums.
+// (a template only so that the header can be included by several translation units)
+template <int kUnused = 0>
+__global__ __launch_bounds__(256) void walk_vec_scan_kernel(float *v, int n_chunks, int D, int reverse) {
+    __shared__ float part[16][16];
+    const int j = threadIdx.x & 15, grp = threadIdx.x >> 4;  // column within the block's 16, range of chunks
+    const int bh = blockIdx.y, col = blockIdx.x * 16 + j;
+    const int per = (n_chunks + 15) / 16;
+    float *base = v + (int64_t)bh * n_chunks * D + col;
+    // walking order: position t = 0 .. n_chunks - 1 is chunk t, or chunk n_chunks - 1 - t in reverse
+    const int t0 = grp * per, t1 = t0 + per < n_chunks ? t0 + per : n_chunks;
+    auto chunk_of = [&](int t) { return reverse ? n_chunks - 1 - t : t; };
+    float sum = 0.f;
+    for (int t = t0; t < t1; t += 8) {
+        float x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = t + u < t1 ? base[(int64_t)chunk_of(t + u) * D] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) sum += x[u];
+    }
+    part[grp][j] = sum;
+    __syncthreads();
+    float run = 0.f;
+    for (int g2 = 0; g2 < grp; ++g2) run += part[g2][j];
+    for (int t = t0; t < t1; t += 8) {
+        float x[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) x[u] = t + u < t1 ? base[(int64_t)chunk_of(t + u) * D] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+            if (t + u < t1) {
+                base[(int64_t)chunk_of(t + u) * D] = run;
+                run += x[u];
+            }
+    }
+}
+
+inline hipError_t launch_walk_vec_scan(float *v, int64_t BH, int n_chunks, int D, int reverse, hipStream_t stream) {
+    if (BH > 65535 || D % 16 != 0) return hipErrorInvalidConfiguration;
+    return launch_kernel(walk_vec_scan_kernel<0>, dim3((unsigned)(D / 16), (unsigned)BH), dim3(256), 0, stream, v, n_chunks,
+                         D, reverse);
 }
 
 template <typename T, int D>
