@@ -469,13 +469,20 @@ bool states_shareable(int64_t dqk, int64_t dv, int64_t N) {
 }
 
 // bytes of one rounded running state / of the scratch one state computation needs (fp32 chunk states)
-int64_t shared_state_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
+int64_t state_core_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     const WalkPlan w = walk_plan(B, H, N, dqk, dv);
     if (w.ok && !w.split) return w.saved_bytes;  // one state per 128-row chunk (also room for the 256-row chunks' states)
     if (!states_shareable(dqk, dv, N)) return w.ok ? w.saved_bytes : 0;
     const int64_t rows = chunk_rows(dqk, dv);
     const int64_t per_chunk = B * H * ((N + rows - 1) / rows) * padded(dqk) * padded(dv) * 2;
     return w.ok && w.saved_bytes > per_chunk ? w.saved_bytes : per_chunk;  // (split: either path's state fits)
+}
+
+// The buffer forward's state goes to: the states above and, behind them, room for the running sums of
+// k at the entry of every chunk, which the normalised forward leaves there for its backward.
+int64_t shared_state_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
+    const int64_t core = state_core_bytes(B, H, N, dqk, dv);
+    return core ? core + walk_vec_bytes(B, H, N, dqk, dv) : 0;
 }
 
 int64_t chunked_op_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
@@ -540,7 +547,9 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
         w.init = wp.n_seg > 1 ? entry : nullptr, w.saved = wp.split ? nullptr : state_out;
         if (nx) {  // the normaliser inside the walk: zc = running sum of k at the entry of every chunk
-            float *zc = static_cast<float *>(nx->vec);
+            // (kept behind the state, when there is one, for backward)
+            float *zc = state_out ? reinterpret_cast<float *>(static_cast<char *>(state_out) + state_core_bytes(B, H, N, dqk, dv))
+                                  : static_cast<float *>(nx->vec);
             if (int rc = walk_chunk_vectors(wp, kk, dqk, nullptr, 0, zc, B, H, N, dtype, s)) return rc;
             w.denom = nx->denom, w.eps = nx->eps, w.zc = zc;
             nx->fused = true;
@@ -606,6 +615,10 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
     const WalkPlan wp = walk_plan(B, H, N, dqk, dv);
     // (what forward saved is in this path's format; the split path's entry states are cheap to recompute)
     const bool walk = wp.ok && (state_in || wp.split);
+    // the normalised forward left zc behind its state
+    const float *zc_saved = nx && state_in ? reinterpret_cast<const float *>(static_cast<const char *>(state_in) +
+                                                                           state_core_bytes(B, H, N, dqk, dv))
+                                           : nullptr;
     if (walk && wp.split) {
         // workspace: totals and entry states of Q^T dO; behind them those of K^T V when forward's are not given
         if (wp.n_seg > 1 && (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 ||
@@ -629,7 +642,8 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
             zc = static_cast<float *>(nx->vec);
             rcv = reinterpret_cast<float *>(static_cast<char *>(nx->vec) + walk_vec_bytes(B, H, N, dqk, dv));
             if (int rc = walk_chunk_vectors(wp, q, dqk, nx->dn, 1, rcv, B, H, N, dtype, s)) return rc;
-            if (int rc = walk_chunk_vectors(wp, k, dqk, nullptr, 0, zc, B, H, N, dtype, s)) return rc;
+            if (zc_saved) zc = const_cast<float *>(zc_saved);
+            else if (int rc = walk_chunk_vectors(wp, k, dqk, nullptr, 0, zc, B, H, N, dtype, s)) return rc;
         }
         // dQ = lower(dO V^T) K + dO S^T: the forward walk over (dO, V, K), its states V^T K = S^T
         fla::WalkParams w{};
@@ -689,7 +703,8 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         if (nx) {
             const int64_t vb = walk_vec_bytes(B, H, N, dqk, dv);
             float *zc = static_cast<float *>(nx->vec), *rcv = reinterpret_cast<float *>(static_cast<char *>(nx->vec) + vb);
-            if (int rc = walk_chunk_vectors(wp, k, dqk, nullptr, 0, zc, B, H, N, dtype, s)) return rc;
+            if (zc_saved) zc = const_cast<float *>(zc_saved);
+            else if (int rc = walk_chunk_vectors(wp, k, dqk, nullptr, 0, zc, B, H, N, dtype, s)) return rc;
             if (int rc = walk_chunk_vectors(wp, q, dqk, nx->dn, 1, rcv, B, H, N, dtype, s)) return rc;
             w.dn = nx->dn, w.zc = zc, w.rc = rcv;
             nx->fused = true;

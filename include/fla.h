@@ -309,7 +309,9 @@ int fla_poly_attn_bwd(const void *grad_out, const void *xq, const void *xk, cons
  * fla_normalised_workspace_bytes() bytes (same `chunked`) of 16-byte aligned device memory,
  * scratch.  state_out / state_valid / state_in: with `chunked`, what the chunk-wise forward hands to
  * its backward, exactly as for fla_linear_attn_chunked_fwd/bwd (size:
- * fla_linear_attn_chunked_state_bytes(); any of them may be null, backward then works without);
+ * fla_linear_attn_chunked_state_bytes(); any of them may be null, backward then works without;
+ * state_in must be what THIS operator's forward wrote for the same inputs -- behind the product's
+ * state it carries the running sums of k, which the plain chunk-wise forward does not write);
  * ignored otherwise.  With `chunked` and equal padded head dims up to 128 the normaliser and
  * its gradient terms are computed inside the chunk-wise kernels rather than by passes of their
  * own.  B*H must not exceed 65535.  No counterpart in the reference's kernels; replaces the caller-side recipe and its
