@@ -54,3 +54,45 @@ def test_replayed_graph_equals_eager(dims, fwd, bwd, gpu_device):
         assert torch.equal(g_out, want_out), f"replay {replay}: O differs"
         for name, got, w in zip(("dQ", "dK", "dV"), (g_dq, g_dk, g_dv), want):
             assert torch.equal(got, w), f"replay {replay}: {name} differs"
+
+
+@pytest.mark.parametrize("dims,normalised", [((2, 4, 2048, 64, 64), False), ((1, 8, 2048, 128, 128), False),
+                                             ((2, 4, 2048, 64, 64), True), ((1, 8, 2048, 128, 128), True)],
+                         ids=["d64", "d128", "d64-normalised", "d128-normalised"])
+def test_replayed_graph_of_the_chunkwise_operators_equals_eager(dims, normalised, gpu_device):
+    """The chunk-wise walk kernels (totals, scan, walks; with the normaliser also the vector sums and
+    the dO pass), forward handing its state to backward: captured once, replayed on fresh inputs."""
+    from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
+    from flashy_linear_attention_amd.normalised import linear_attention_normalised_bwd, linear_attention_normalised_fwd
+
+    bs, nh, sq, dqk, dv = dims
+    static = [t.to(gpu_device) for t in reference_style_inputs(bs, nh, sq, dqk, dv, torch.bfloat16, seed=0)]
+    q, k, v, do = static
+
+    def step():
+        if normalised:
+            out, denom, state = linear_attention_normalised_fwd(q, k, v, 1e-5, True, want_state=True)
+            return (out,) + tuple(linear_attention_normalised_bwd(do, q, k, v, out, denom, True, state))
+        out, state = linear_attention_chunked_fwd(q, k, v, want_state=True)
+        return (out,) + tuple(linear_attention_chunked_bwd(do, q, k, v, state))
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        got = step()
+    for replay in range(3):
+        fresh = [t.to(gpu_device) for t in reference_style_inputs(bs, nh, sq, dqk, dv, torch.bfloat16, seed=20 + replay)]
+        for dst, src in zip(static, fresh):
+            dst.copy_(src)
+        graph.replay()
+        torch.cuda.synchronize()
+        want = step()  # eager work between replays, on the same inputs
+        torch.cuda.synchronize()
+        for name, g, w in zip(("out", "dQ", "dK", "dV"), got, want):
+            assert torch.equal(g, w), f"replay {replay}: {name} differs"
