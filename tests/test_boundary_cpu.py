@@ -198,3 +198,26 @@ def test_synthetic_workloads_have_the_stated_shapes_and_features():
     assert (q1 > 0).all() and (k1 > 0).all() and q1.dtype == torch.float16
     q2, *_ = make_inputs(WORKLOADS["C2"], batch=1, heads=2, seq=64)
     assert torch.equal(q1, q2)
+
+
+def test_chunkwise_state_and_workspace_sizes():
+    """The size queries are host arithmetic on the chunk-wise plan (no GPU): values derived by hand.
+    State = what forward hands to backward (D <= 64: a 16-bit D x D state per 128-row chunk; D = 128:
+    the fp32 entry state of every walk segment, or the 16-bit states of the 256-row chunks if those
+    are larger) plus an fp32 vector of D per chunk for the normalised operator."""
+    lib = _lib.load()
+    sb = lib.fla_linear_attn_chunked_state_bytes
+    # B H = 128, N = 4096, D = 128: 16 chunks of 256 rows x 32 KiB > 2 segments x 64 KiB; 64 chunks of 64 rows
+    assert sb(4, 32, 4096, 128, 128) == 128 * 16 * 128 * 128 * 2 + 128 * 64 * 128 * 4
+    # B H = 16, N = 32768, D = 64: 256 chunks of 128 rows
+    assert sb(1, 16, 32768, 64, 64) == 16 * 256 * 64 * 64 * 2 + 16 * 256 * 64 * 4
+    # ragged: N = 2450 at D = 128 is 39 chunks of 64 rows in 20 walk segments of 2; ten 256-row chunks are less
+    assert sb(2, 8, 2450, 128, 128) == 16 * 20 * 128 * 128 * 4 + 16 * 39 * 128 * 4
+    assert sb(1, 1, 300, 32, 32) == 3 * 32 * 32 * 2 + 3 * 32 * 4
+    # nothing to hand over: unequal padded head dims, a single chunk
+    assert sb(4, 16, 4096, 256, 64) == 0 and sb(1, 2, 256, 128, 128) == 0 and sb(1, 2, 128, 64, 64) == 0
+    ws = lib.fla_linear_attn_chunked_workspace_bytes
+    for shape in [(4, 32, 4096, 128, 128), (1, 16, 32768, 64, 64), (2, 8, 2450, 128, 128), (1, 4, 1500, 104, 120)]:
+        assert ws(*shape) >= 4 * (sb(*shape) - shape[0] * shape[1] * 4)  # room for the 256-row path's four buffers
+        assert lib.fla_normalised_workspace_bytes(*shape, 1) > ws(*shape)
+    assert ws(4, 16, 4096, 256, 64) > 0 and ws(1, 2, 256, 128, 128) == 0
