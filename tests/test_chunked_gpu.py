@@ -159,3 +159,33 @@ def test_chunked_operator_workspace_is_checked(gpu_device):
                                          st(dq), st(dk), st(dv), 0, None, work.data_ptr(), 3 * sbytes, stream)
     assert rc == -9  # without a saved state the call needs room for four
     torch.cuda.synchronize()
+
+
+@pytest.mark.parametrize("dims", [(2, 4, 1664, 64, 64), (2, 4, 1664, 128, 128), (1, 3, 1100, 40, 56)],
+                         ids=lambda d: "x".join(map(str, d)))
+def test_chunked_on_strided_operands(dims, gpu_device):
+    """(B, N, H, D) storage viewed as (B, H, N, D), and rows padded to a wider pitch: the chunk-wise
+    kernels honour every operand's own strides, so the results equal those on contiguous copies bit
+    for bit (outputs and gradients come back contiguous either way)."""
+    from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
+
+    bs, nh, sq, dqk, dv = dims
+    q, k, v, dy = (t.to(gpu_device) for t in reference_style_inputs(bs, nh, sq, dqk, dv, torch.bfloat16, seed=5))
+
+    def bnhd(t):
+        return t.transpose(1, 2).contiguous().transpose(1, 2)
+
+    def pitched(t):
+        wide = torch.zeros(*t.shape[:-1], t.shape[-1] + 24, dtype=t.dtype, device=t.device)
+        wide[..., : t.shape[-1]] = t
+        return wide[..., : t.shape[-1]]
+
+    want_o, state = linear_attention_chunked_fwd(q, k, v, want_state=True)
+    want_g = linear_attention_chunked_bwd(dy, q, k, v, state)
+    for name, f in (("(B, N, H, D) storage", bnhd), ("padded rows", pitched)):
+        qs, ks, vs, ds = f(q), f(k), f(v), f(dy)
+        assert not qs.is_contiguous()
+        out, st = linear_attention_chunked_fwd(qs, ks, vs, want_state=True)
+        assert torch.equal(out, want_o), f"{name}: O differs"
+        for gname, g, w in zip(("dQ", "dK", "dV"), linear_attention_chunked_bwd(ds, qs, ks, vs, st), want_g):
+            assert torch.equal(g, w), f"{name}: {gname} differs"
