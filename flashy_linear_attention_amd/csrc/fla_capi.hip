@@ -223,7 +223,7 @@ int64_t chunked_bytes(int64_t B, int64_t H, int64_t N, int64_t dc, int64_t dout)
 
 // ---- element-wise feature passes, for the shapes and layouts the kernels' own map-on-load does
 // not cover: mode 1 writes dst = phi(src); mode 2 multiplies dst in place by phi'(x) computed from
-// src = phi(x).  Any strides; eight elements per thread where both tensors allow 16-byte accesses.
+// src = phi(x); mode 3 adds src to dst in place (fp32 sum, one rounding).  Any strides; eight elements per thread where both tensors allow 16-byte accesses.
 template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void feature_pass_kernel(int mode, int fmap, const T *src, int64_t ss_b, int64_t ss_h,
                                                            int64_t ss_n, T *dst, int64_t ds_b, int64_t ds_h,
@@ -241,18 +241,20 @@ __global__ __launch_bounds__(256) void feature_pass_kernel(int mode, int fmap, c
     if constexpr (VEC) {
         typedef T v8 __attribute__((ext_vector_type(8)));
         v8 s = *reinterpret_cast<const v8 *>(sp), d;
-        if (mode == 2) d = *reinterpret_cast<const v8 *>(dp);
+        if (mode != 1) d = *reinterpret_cast<const v8 *>(dp);
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
             const float x = static_cast<float>(s[e]);
-            d[e] = static_cast<T>(mode == 1 ? fla::feature_value(fmap, x)
-                                            : static_cast<float>(d[e]) * fla::feature_slope_from_value(fmap, x));
+            d[e] = static_cast<T>(mode == 1   ? fla::feature_value(fmap, x)
+                                  : mode == 2 ? static_cast<float>(d[e]) * fla::feature_slope_from_value(fmap, x)
+                                              : static_cast<float>(d[e]) + x);
         }
         *reinterpret_cast<v8 *>(dp) = d;
     } else {
         const float x = static_cast<float>(*sp);
-        *dp = static_cast<T>(mode == 1 ? fla::feature_value(fmap, x)
-                                       : static_cast<float>(*dp) * fla::feature_slope_from_value(fmap, x));
+        *dp = static_cast<T>(mode == 1   ? fla::feature_value(fmap, x)
+                             : mode == 2 ? static_cast<float>(*dp) * fla::feature_slope_from_value(fmap, x)
+                                         : static_cast<float>(*dp) + x);
     }
 }
 
@@ -469,10 +471,37 @@ bool states_shareable(int64_t dqk, int64_t dv, int64_t N) {
 }
 
 // bytes of one rounded running state / of the scratch one state computation needs (fp32 chunk states)
+// ---- D_qk in (128, 256] with D_v <= 128 (the small-V operator's shapes).  The scores are a sum over
+// the two 128-column halves of q and k and everything is linear in them:
+//     O  = tril(Q_0 K_0^T) V + tril(Q_1 K_1^T) V        dV = the same sum of the halves' dV
+//     dQ_h = tril(dO V^T) K_h                           dK_h = triu(V dO^T) Q_h
+// so each half runs the D = 128 walk kernels on column views of q, k, dq, dk (v and dO are padded
+// with zeros in LDS, never in memory); the second half's O and dV go to a scratch tensor and one
+// element-wise pass adds them.  Forward hands over both halves' entry states.
+struct WidePlan {
+    bool ok;
+    WalkPlan wp;         // the plan of a 128 / 128 problem of the same B, H, N
+    int64_t temp_bytes;  // the second half's O (forward) or dV (backward), contiguous (B, H, N, D_v)
+};
+
+WidePlan wide_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
+    WidePlan w{};
+    if (dqk <= 128 || dqk > 256 || dv > 128) return w;
+    w.wp = walk_plan(B, H, N, 128, 128);
+    w.ok = w.wp.ok;
+    w.temp_bytes = (B * H * N * dv * 2 + 255) / 256 * 256;
+    return w;
+}
+
+View column_half(const View &t, int h) { return View{static_cast<const char *>(t.ptr) + h * 128 * 2, t.strides}; }
+
 int64_t state_core_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     const WalkPlan w = walk_plan(B, H, N, dqk, dv);
     if (w.ok && !w.split) return w.saved_bytes;  // one state per 128-row chunk (also room for the 256-row chunks' states)
-    if (!states_shareable(dqk, dv, N)) return w.ok ? w.saved_bytes : 0;
+    if (!states_shareable(dqk, dv, N)) {
+        const WidePlan wide = wide_plan(B, H, N, dqk, dv);
+        return wide.ok ? 2 * wide.wp.entry_bytes : w.ok ? w.saved_bytes : 0;
+    }
     const int64_t rows = chunk_rows(dqk, dv);
     const int64_t per_chunk = B * H * ((N + rows - 1) / rows) * padded(dqk) * padded(dv) * 2;
     return w.ok && w.saved_bytes > per_chunk ? w.saved_bytes : per_chunk;  // (split: either path's state fits)
@@ -485,15 +514,107 @@ int64_t shared_state_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t
     return core ? core + walk_vec_bytes(B, H, N, dqk, dv) : 0;
 }
 
+// workspace of the two-halves evaluation: the scratch tensor, then totals and entry states of one
+// half at a time (two sets in backward: Q^T dO, and K^T V when forward's entry states are not given)
+int64_t wide_workspace_bytes(const WidePlan &w) { return w.temp_bytes + 2 * w.wp.work_bytes; }
+
 int64_t chunked_op_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     const int64_t shared = shared_state_bytes(B, H, N, dqk, dv);
     if (shared) {  // fp32 chunk states (2x) + two rounded states (backward without a saved one); the walk's totals
         const WalkPlan w = walk_plan(B, H, N, dqk, dv);
-        return w.ok && w.work_bytes * 2 > shared * 4 ? w.work_bytes * 2 : shared * 4;
+        if (w.ok || states_shareable(dqk, dv, N)) return w.ok && w.work_bytes * 2 > shared * 4 ? w.work_bytes * 2 : shared * 4;
     }
     int64_t m = chunked_bytes(B, H, N, dqk, dv);
     const int64_t t = chunked_bytes(B, H, N, dv, dqk);
-    return m > t ? m : t;
+    if (t > m) m = t;
+    const WidePlan wide = wide_plan(B, H, N, dqk, dv);
+    if (wide.ok && wide_workspace_bytes(wide) > m) m = wide_workspace_bytes(wide);
+    return m;
+}
+
+// the walk that computes out = lower(x y^T) z + x S with S += y^T z (fla::walk_fwd_kernel's roles)
+fla::WalkParams lower_walk_params(const WalkPlan &wp, const View &x, const View &y, const View &z, const View &out,
+                                  int64_t B, int64_t H, int64_t N, int64_t wxy, int64_t wz, const float *entry) {
+    fla::WalkParams w{};
+    w.q = x.ptr, w.k = y.ptr, w.v = z.ptr, w.o = const_cast<void *>(out.ptr);
+    w.qs_b = x.strides[0], w.qs_h = x.strides[1], w.qs_n = x.strides[2];
+    w.ks_b = y.strides[0], w.ks_h = y.strides[1], w.ks_n = y.strides[2];
+    w.vs_b = z.strides[0], w.vs_h = z.strides[1], w.vs_n = z.strides[2];
+    w.os_b = out.strides[0], w.os_h = out.strides[1], w.os_n = out.strides[2];
+    w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)wxy, w.wv = (int32_t)wz;
+    w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
+    w.init = wp.n_seg > 1 ? entry : nullptr;
+    return w;
+}
+
+bool wide_fast_path(const View &q, const View &k, const View &v, const View &o, int64_t B, int64_t H, int64_t N,
+                    int64_t dqk, int64_t dv) {
+    return fla::fast_path_ok(make_params(q, k, v, o, B, H, N, 128, dv, 0)) &&
+           fla::fast_path_ok(make_params(column_half(q, 1), column_half(k, 1), v, o, B, H, N, dqk - 128, dv, 0));
+}
+
+int wide_forward(const WidePlan &wide, const View &q, const View &k, const View &v, const View &o, int64_t B, int64_t H,
+                 int64_t N, int64_t dqk, int64_t dv, int dtype, void *state_out, void *workspace, hipStream_t s) {
+    const WalkPlan &wp = wide.wp;
+    char *ws = static_cast<char *>(workspace);
+    const int64_t temp_strides[4] = {H * N * dv, N * dv, dv, 1};
+    const View temp{ws, temp_strides};
+    for (int h = 0; h < 2; ++h) {
+        const View qh = column_half(q, h), kh = column_half(k, h);
+        const int64_t wqk = h == 0 ? 128 : dqk - 128;
+        const float *entry = nullptr;
+        if (wp.n_seg > 1) {
+            float *keep = state_out ? reinterpret_cast<float *>(static_cast<char *>(state_out) + h * wp.entry_bytes) : nullptr;
+            void *work = keep && wp.m == 1 ? static_cast<void *>(keep) : static_cast<void *>(ws + wide.temp_bytes);
+            if (int rc = walk_entry_states(wp, kh, v, B, H, N, wqk, dv, dtype, 0, work, keep, &entry, s)) return rc;
+        }
+        const fla::WalkParams w = lower_walk_params(wp, qh, kh, v, h == 0 ? o : temp, B, H, N, wqk, dv, entry);
+        if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
+    }
+    return launch_feature_pass(3, 0, temp, o, B, H, N, dv, dtype, s);
+}
+
+int wide_backward(const WidePlan &wide, const View &go, const View &q, const View &k, const View &v, const View &dq,
+                  const View &dk, const View &dvv, int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv, int dtype,
+                  const void *state_in, void *workspace, hipStream_t s) {
+    const WalkPlan &wp = wide.wp;
+    char *ws = static_cast<char *>(workspace);
+    const int64_t temp_strides[4] = {H * N * dv, N * dv, dv, 1};
+    const View temp{ws, temp_strides};
+    for (int h = 0; h < 2; ++h) {
+        const View qh = column_half(q, h), kh = column_half(k, h), dqh = column_half(dq, h), dkh = column_half(dk, h);
+        const int64_t wqk = h == 0 ? 128 : dqk - 128;
+        const float *fwd_entry = nullptr, *entry = nullptr;
+        if (wp.n_seg > 1) {
+            if (state_in)
+                fwd_entry = reinterpret_cast<const float *>(static_cast<const char *>(state_in) + h * wp.entry_bytes);
+            else if (int rc = walk_entry_states(wp, kh, v, B, H, N, wqk, dv, dtype, 0, ws + wide.temp_bytes + wp.work_bytes,
+                                                nullptr, &fwd_entry, s))
+                return rc;
+            if (int rc = walk_entry_states(wp, qh, go, B, H, N, wqk, dv, dtype, 1, ws + wide.temp_bytes, nullptr, &entry, s))
+                return rc;
+        }
+        // dQ_h = lower(dO V^T) K_h + dO S_h^T: the forward walk over (dO, V, K_h)
+        fla::WalkParams w = lower_walk_params(wp, go, v, kh, dqh, B, H, N, dv, wqk, fwd_entry);
+        w.init_transposed = 1;
+        if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
+        // dV (this half's part) and dK_h: the reverse walk
+        const View &dvh = h == 0 ? dvv : temp;
+        fla::WalkParams r{};
+        r.q = qh.ptr, r.k = kh.ptr, r.v = v.ptr, r.go = go.ptr;
+        r.dk = const_cast<void *>(dkh.ptr), r.dv = const_cast<void *>(dvh.ptr);
+        r.qs_b = qh.strides[0], r.qs_h = qh.strides[1], r.qs_n = qh.strides[2];
+        r.ks_b = kh.strides[0], r.ks_h = kh.strides[1], r.ks_n = kh.strides[2];
+        r.vs_b = v.strides[0], r.vs_h = v.strides[1], r.vs_n = v.strides[2];
+        r.gs_b = go.strides[0], r.gs_h = go.strides[1], r.gs_n = go.strides[2];
+        r.dks_b = dkh.strides[0], r.dks_h = dkh.strides[1], r.dks_n = dkh.strides[2];
+        r.dvs_b = dvh.strides[0], r.dvs_h = dvh.strides[1], r.dvs_n = dvh.strides[2];
+        r.H = (int32_t)H, r.N = (int32_t)N, r.BH = (int32_t)(B * H), r.wqk = (int32_t)wqk, r.wv = (int32_t)dv;
+        r.n_chunks = (int32_t)wp.n_chunks, r.seg_chunks = (int32_t)wp.seg_chunks, r.n_seg = (int32_t)wp.n_seg;
+        r.init = entry;
+        if (fla::walk_dkdv(dtype, wp.D, r, s) != hipSuccess) return FLA_ERR_LAUNCH;
+    }
+    return launch_feature_pass(3, 0, temp, dvv, B, H, N, dv, dtype, s);
 }
 
 // fmap != 0 (feature_forward below): q and k hold the arguments xq, xk of the feature map phi, and
@@ -511,6 +632,19 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         if (int rc = check_view(t)) return rc;
     if (int rc = check_alias_fwd(q, k, v, o, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    if (!fmap && !nx) {
+        const WidePlan wide = wide_plan(B, H, N, dqk, dv);
+        if (wide.ok && wide_fast_path(q, k, v, o, B, H, N, dqk, dv)) {
+            if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wide_workspace_bytes(wide))
+                return FLA_ERR_WORKSPACE;
+            if (state_out && reinterpret_cast<uintptr_t>(state_out) % 16 != 0) return FLA_ERR_WORKSPACE;
+            if (int rc = wide_forward(wide, q, k, v, o, B, H, N, dqk, dv, dtype, state_out, workspace,
+                                      static_cast<hipStream_t>(stream)))
+                return rc;
+            if (state_out && state_valid) *state_valid = 1;
+            return FLA_OK;
+        }
+    }
     const WalkPlan wp = walk_plan(B, H, N, dqk, dv);
     if (wp.ok && fla::fast_path_ok(make_params(q, k, v, o, B, H, N, dqk, dv, 0)) &&
         (!fmap || fla::fast_path_ok(make_params(mapped[0], mapped[1], v, o, B, H, N, dqk, dv, 0)))) {
@@ -599,6 +733,16 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
     TriParams pq = make_params(go, v, k, dq, B, H, N, dv, dqk, 0);   // dQ = lower(dO V^T) K
     TriParams pv = make_params(k, q, go, dvv, B, H, N, dqk, dv, 1);  // dV = upper(K Q^T) dO
     TriParams pk = make_params(v, go, q, dk, B, H, N, dv, dqk, 1);   // dK = upper(V dO^T) Q
+    if (!fmap && !nx) {
+        const WidePlan wide = wide_plan(B, H, N, dqk, dv);
+        if (wide.ok && wide_fast_path(q, k, v, go, B, H, N, dqk, dv) && wide_fast_path(dq, dk, dvv, dvv, B, H, N, dqk, dv)) {
+            if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wide_workspace_bytes(wide))
+                return FLA_ERR_WORKSPACE;
+            if (state_in && reinterpret_cast<uintptr_t>(state_in) % 16 != 0) return FLA_ERR_WORKSPACE;
+            return wide_backward(wide, go, q, k, v, dq, dk, dvv, B, H, N, dqk, dv, dtype, state_in, workspace,
+                                 static_cast<hipStream_t>(stream));
+        }
+    }
     // (with the normaliser's terms still to be added by the caller, so is the slope)
     const int fmap_late = nx ? 0 : fmap;
     if (!states_shareable(dqk, dv, N) || !fla::fast_path_ok(pq) || !fla::fast_path_ok(pv) || !fla::fast_path_ok(pk)) {

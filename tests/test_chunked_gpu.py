@@ -32,6 +32,10 @@ CASES = [
     (2, 8, 4136, 128, 128),
     (1, 4, 1500, 104, 120),
     (8, 8, 2100, 64, 64),
+    # D_qk in (128, 256] with D_v <= 128: two 128-column halves of q and k through the D = 128 walk kernels
+    (2, 4, 1300, 256, 64),
+    (1, 2, 1024, 200, 128),
+    (2, 8, 2450, 136, 24),
 ]
 
 
@@ -125,8 +129,8 @@ def test_chunked_backward_with_and_without_the_forward_state(gpu_device):
     for name, got, other, w in zip(("dQ", "dK", "dV"), with_state, without, want):
         assert_close(name, got, w)
         assert_close(name + " (no saved state)", other, w)
-    # widths that differ after padding (small V), and a single chunk: no shared state
-    q2, k2, v2, _ = (t.to(gpu_device) for t in reference_style_inputs(1, 2, 1024, 256, 64, torch.bfloat16, seed=32))
+    # a value head dim wider than the query / key one, and a single chunk: no shared state
+    q2, k2, v2, _ = (t.to(gpu_device) for t in reference_style_inputs(1, 2, 1024, 64, 256, torch.bfloat16, seed=32))
     assert linear_attention_chunked_fwd(q2, k2, v2, want_state=True)[1] is None
     assert linear_attention_chunked_fwd(q[:, :, :256], k[:, :, :256], v[:, :, :256], want_state=True)[1] is None
 
@@ -189,3 +193,20 @@ def test_chunked_on_strided_operands(dims, gpu_device):
         assert torch.equal(out, want_o), f"{name}: O differs"
         for gname, g, w in zip(("dQ", "dK", "dV"), linear_attention_chunked_bwd(ds, qs, ks, vs, st), want_g):
             assert torch.equal(g, w), f"{name}: {gname} differs"
+
+
+def test_chunked_small_v_state_hand_over(gpu_device):
+    """D_qk = 256, D_v = 64: forward hands both halves' entry states to backward; backward without
+    them recomputes; both match the oracle."""
+    from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
+
+    q, k, v, dy = (t.to(gpu_device) for t in reference_style_inputs(2, 8, 4200, 256, 64, torch.bfloat16, seed=41))
+    out, state = linear_attention_chunked_fwd(q, k, v, want_state=True)
+    assert state is not None and torch.equal(out, linear_attention_chunked_fwd(q, k, v))
+    assert_close("O", out, naive.causal_dot_product(q.float().cpu(), k.float().cpu(), v.float().cpu()))
+    want = naive.causal_dot_product_grads(q.float().cpu(), k.float().cpu(), v.float().cpu(), dy.float().cpu())
+    with_state = linear_attention_chunked_bwd(dy, q, k, v, state)
+    without = linear_attention_chunked_bwd(dy, q, k, v, None)
+    for name, a, b, w in zip(("dQ", "dK", "dV"), with_state, without, want):
+        assert torch.equal(a, b), f"{name}: recomputed entry states give different gradients"
+        assert_close(name, a, w)
