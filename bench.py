@@ -169,6 +169,8 @@ def _chunk_rows(w):
     """Rows per chunk of the kernels this workload's chunk-wise step runs."""
     if _pad(w.d_qk) == _pad(w.d_v) and _pad(w.d_qk) <= 128:  # the walk kernels
         return 128 if _pad(w.d_qk) <= 64 else 64
+    if 128 < w.d_qk <= 256 and w.d_v <= 128:  # two 128-column halves of q, k through the D = 128 walk kernels
+        return 64
     return 256 if (w.d_qk // 2 + w.d_v <= 192 and w.d_v // 2 + w.d_qk <= 192) else 128
 
 
