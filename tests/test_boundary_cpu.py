@@ -214,10 +214,12 @@ def test_chunkwise_state_and_workspace_sizes():
     # ragged: N = 2450 at D = 128 is 39 chunks of 64 rows in 20 walk segments of 2; ten 256-row chunks are less
     assert sb(2, 8, 2450, 128, 128) == 16 * 20 * 128 * 128 * 4 + 16 * 39 * 128 * 4
     assert sb(1, 1, 300, 32, 32) == 3 * 32 * 32 * 2 + 3 * 32 * 4
-    # nothing to hand over: unequal padded head dims, a single chunk
-    assert sb(4, 16, 4096, 256, 64) == 0 and sb(1, 2, 256, 128, 128) == 0 and sb(1, 2, 128, 64, 64) == 0
+    # D_qk = 256, D_v = 64: the fp32 entry states of both 128-column halves, 4 walk segments per (b, h)
+    assert sb(4, 16, 4096, 256, 64) == 2 * 64 * 4 * 128 * 128 * 4
+    # nothing to hand over: a value head dim wider than the query / key one, a single chunk
+    assert sb(4, 16, 4096, 64, 256) == 0 and sb(1, 2, 256, 128, 128) == 0 and sb(1, 2, 128, 64, 64) == 0
     ws = lib.fla_linear_attn_chunked_workspace_bytes
     for shape in [(4, 32, 4096, 128, 128), (1, 16, 32768, 64, 64), (2, 8, 2450, 128, 128), (1, 4, 1500, 104, 120)]:
         assert ws(*shape) >= 4 * (sb(*shape) - shape[0] * shape[1] * 4)  # room for the 256-row path's four buffers
         assert lib.fla_normalised_workspace_bytes(*shape, 1) > ws(*shape)
-    assert ws(4, 16, 4096, 256, 64) > 0 and ws(1, 2, 256, 128, 128) == 0
+    assert ws(4, 16, 4096, 256, 64) > 0 and ws(4, 16, 4096, 64, 256) > 0 and ws(1, 2, 256, 128, 128) == 0
