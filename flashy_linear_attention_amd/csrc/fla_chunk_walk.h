@@ -1,34 +1,49 @@
 // Chunk-wise causal linear attention with the running state kept inside the kernel, for equal
-// padded head dims D = 32 or 64 (the long-sequence shapes, which are bound by memory traffic).
+// padded head dims D = 32, 64 or 128 (shapes bound by memory traffic, not by the matrix units).
 //
 // The chunk-wise evaluation of fla_chunk_state.h / fla_tri_fast.h computes every per-chunk
 // state, writes it in fp32, scans it, writes the running sums in 16 bit and reads them back in
 // each consumer, and its backward reads q, k, v and dO once per product.  Here a workgroup walks
-// a *segment* of consecutive 128-row chunks in sequence order and carries the running state
+// a *segment* of consecutive chunks in sequence order and carries the running state
 //
 //     S = sum over the chunks before of K_c^T V_c      (forward, lower mask: ascending walk)
 //     R = sum over the chunks after  of Q_c^T dO_c     (backward, upper mask: descending walk)
 //
-// in fp32 accumulators; per chunk it is rounded once to the storage type (as before) into 8 KiB
-// of LDS, where the MFMAs of the state products read it.  Every operand tile of a chunk is
-// brought to LDS once and serves all products of that chunk:
+// in fp32 accumulators; per chunk it is rounded once to the storage type (as before) into LDS,
+// where the MFMAs of the state products read it.  Every operand tile of a chunk is brought to
+// LDS once and serves all products of that chunk:
 //
 //   forward   O_c  = lower(Q_c K_c^T) V_c   + Q_c S          then S += K_c^T V_c
-//   backward  dQ_c = lower(dO_c V_c^T) K_c  + dO_c S_c^T     (S_c: saved by forward, 16 bit per chunk)
+//   backward  dQ_c = lower(dO_c V_c^T) K_c  + dO_c S_c^T
 //             dV_c = upper(K_c Q_c^T) dO_c  + K_c R
 //             dK_c = upper(V_c dO_c^T) Q_c  + V_c R^T        then R += Q_c^T dO_c
 //
-// Segments make the walk parallel: a first kernel adds up K^T V (Q^T dO) over each segment, a
-// small one turns the totals into exclusive prefix (suffix) sums, and each walking workgroup
-// starts from its segment's entry state.  Per step that reads k, v (q, dO) twice and everything
-// else once; no fp32 per-chunk state ever goes to memory.
+// Segments make the walk parallel: a first kernel adds up K^T V (Q^T dO) over segments, a small
+// one turns the totals into each segment's entry state (exclusive prefix / suffix sums), and
+// each walking workgroup starts from its segment's entry state.  No fp32 per-chunk state ever
+// goes to memory.
 //
-// Layout.  An operand tile is 128 rows x D 16-bit values, row-major, the 16-byte chunk index of
+//   D <= 64: 128-row chunks, two workgroups per CU.  Forward saves the 16-bit state at the entry
+//            of every chunk (S_c), and ONE backward kernel (walk_bwd_kernel) computes dQ, dV and
+//            dK of a chunk from one set of tiles.
+//   D = 128: tiles and state must share the 160 KiB of LDS: 64-row chunks, one workgroup per CU
+//            with two sets of tiles (the next chunk's loads are in flight while this one is
+//            multiplied).  A saved per-chunk state would cost as much traffic as an operand, so
+//            forward hands over its segments' fp32 entry states only and backward is split: dQ is
+//            the forward walk over (dO, V, K), whose states V^T K start from the transposed entry
+//            states, and walk_dkdv_kernel is the reverse walk for dV and dK.
+//
+// Options of the walks: an element-wise feature map applied to q, k as they are loaded, with its
+// slope multiplied into dQ, dK (WalkParams::fmap); the normaliser of linear attention and its
+// gradient terms as rank-one additions to the products (WalkParams::denom ...).
+//
+// Layout.  An operand tile is C rows x D 16-bit values, row-major, the 16-byte chunk index of
 // a row XORed with swizzle_y (fla_tri_fast.h) -- one layout for the 16-byte row reads (MFMA
-// operands with k along the row) and for the transposing column reads (k down the rows).  Wave w
-// of the four owns rows 32 w .. 32 w + 31 of the chunk as the "X rows" of every product; the
-// MFMA operand chaining is that of the other kernels: S^T = Y X^T leaves a lane holding one X
-// row and eight-row groups of Y rows, which is the B operand of Out^T += Z^T P^T.
+// operands with k along the row) and for the transposing column reads (k down the rows).  A wave
+// owns one 32-row block of the chunk as the "X rows" of every product (and, at D = 128, one half
+// of the output columns; the two waves of a row block then form the same scores); the MFMA
+// operand chaining is that of the other kernels: S^T = Y X^T leaves a lane holding one X row
+// and eight-row groups of Y rows, which is the B operand of Out^T += Z^T P^T.
 #pragma once
 
 #include <hip/hip_runtime.h>
