@@ -49,7 +49,7 @@ def _static(lib, q, k, v, out):
 
 def test_static_scratch_entry_point_matches_the_workspace_one(gpu_device):
     lib = _lib.load()
-    w = WORKLOADS["C5"]  # D = 64, 256-row chunks
+    w = WORKLOADS["C5"]  # D = 64: the scratch holds the segments' totals and entry states
     # first a problem of many chunks, then a smaller one whose states land on the first one's
     for case, (heads, seq) in enumerate(((6, 4096), (3, 1280))):
         q, k, v, _ = (t.to(gpu_device) for t in make_inputs(w, seed=11 + case, batch=1, heads=heads, seq=seq))
@@ -76,3 +76,22 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit(gpu_device):
     rc = lib.fla_linear_attn_chunked_fwd_static(*fake, b, h, n, d, d, s, s, s, s, 0, _stream())
     assert rc == -9, lib.fla_strerror(rc)
     torch.cuda.synchronize()
+
+
+def test_static_scratch_entry_point_at_other_widths(gpu_device):
+    """D = 128 (two sets of tiles, finer total segments) and D_qk = 256 / D_v = 64 (two halves and a
+    scratch tensor for the second half's output), after the calls above have used the array."""
+    from helpers import reference_style_inputs
+
+    lib = _lib.load()
+    for case, dims in enumerate(((1, 4, 2048, 128, 128), (1, 2, 1024, 256, 64), (1, 3, 700, 128, 128))):
+        q, k, v, _ = (t.to(gpu_device) for t in reference_style_inputs(*dims, torch.bfloat16, seed=90 + case))
+        want, nbytes = _with_workspace(lib, q, k, v)
+        assert 0 < nbytes <= STATIC_BYTES
+        out = torch.full_like(v, float("nan"))
+        before = torch.cuda.memory_allocated()
+        rc = _static(lib, q, k, v, out)
+        assert rc == 0, lib.fla_strerror(rc)
+        assert torch.cuda.memory_allocated() == before
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"{dims}: static-scratch result differs from the workspace one"
