@@ -123,14 +123,31 @@ struct WalkCfg {
     static_assert(NRB * NCH == 4 && DBW * NCH == DB, "four waves tile the chunk's rows and output columns");
 };
 
-// state block i of wave `wave`: (block of q/k indices, block of v indices); the v block is the
-// same for all blocks of a wave
-template <int D>
-struct WalkBlock {
+// The 32 x 32 blocks of the state that hold anything: NQ blocks of q/k indices (its rows), NV of v
+// indices (its columns).  All D / 32 of each by default; the D = 128 kernels are also built for
+// operands of at most 64 true columns on one side (NQ or NV = 2: the other blocks would hold the
+// zeros the tiles are padded with, and the MFMAs on them are left out).
+// State block i of wave `wave` is block wave + 4 i of the NQ x NV: (dbk, eb) = (block of q/k
+// indices, block of v indices); the v block is the same for all blocks of a wave.
+template <int D, int NQ = D / 32, int NV = D / 32>
+struct WalkExt {
+    static_assert(NQ >= 1 && NQ <= D / 32 && NV >= 1 && NV <= D / 32 && (4 % NV == 0 || NV % 4 == 0), "block counts");
+    static constexpr int nq = NQ, nv = NV;
+    static constexpr int SLOTS = (NQ * NV + 3) / 4;  // state blocks per wave
+    static constexpr int KQ = 2 * NQ, KV = 2 * NV;   // 16-wide k chunks over the q/k side, the v side
+    __device__ static __forceinline__ bool valid(int wave, int i) { return wave + 4 * i < NQ * NV; }
+    __device__ static __forceinline__ int dbk(int wave, int i) { return (wave + 4 * i) / NV; }
+    __device__ static __forceinline__ int eb(int wave) { return wave % NV; }
+};
+
+// Output blocks of a product whose result has NOB blocks that hold anything: with two column parts
+// (D = 128) each part takes half of them -- PER blocks from block db0(wave).
+template <int D, int NOB>
+struct WalkOut {
     using W = WalkCfg<D>;
-    __device__ static __forceinline__ bool valid(int wave, int i) { return wave + 4 * i < W::NBLK; }
-    __device__ static __forceinline__ int dbk(int wave, int i) { return (wave + 4 * i) / W::DB; }
-    __device__ static __forceinline__ int eb(int wave) { return wave % W::DB; }
+    static_assert(NOB % W::NCH == 0, "the column parts share the output blocks evenly");
+    static constexpr int PER = NOB / W::NCH;
+    __device__ static __forceinline__ int db0(int wave) { return W::NCH == 1 ? 0 : (wave / W::NRB) * PER; }
 };
 
 // ---- LDS tile access (tile: row-major [rows][D], chunk index XOR swizzle_y(row))
@@ -255,7 +272,9 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 struct WalkNoRows {
     __device__ __forceinline__ f32x4 operator()(int, int) const { return f32x4{0.f, 0.f, 0.f, 0.f}; }
 };
-template <typename T, int D, bool UPPER, int EX = 0, typename SFrag, typename YRows = WalkNoRows>
+// KCL: 16-wide k chunks of the contraction X Y^T that hold anything; NOB: output blocks that do.
+template <typename T, int D, bool UPPER, int EX = 0, int KCL = WalkCfg<D>::KC, int NOB = WalkCfg<D>::DB, typename SFrag,
+          typename YRows = WalkNoRows>
 __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsigned char *yt, const unsigned char *zt,
                                              int wave, int lane, bool has_state, SFrag &&sfrag,
                                              f32x16 (&acc)[WalkCfg<D>::DBW], float *ex = nullptr,
@@ -263,15 +282,16 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
     using W = WalkCfg<D>;
     using M = Mma<T>;
     using V8 = typename M::V8;
+    constexpr int PER = WalkOut<D, NOB>::PER;
     const int l32 = lane & 31, g = lane >> 5;
-    const int rb = W::NCH == 1 ? wave : wave % W::NRB, db0 = W::NCH == 1 ? 0 : (wave / W::NRB) * W::DBW;
-    V8 xf[W::KC];
+    const int rb = W::NCH == 1 ? wave : wave % W::NRB, db0 = WalkOut<D, NOB>::db0(wave);
+    V8 xf[KCL];
 #pragma unroll
-    for (int kc = 0; kc < W::KC; ++kc) xf[kc] = walk_row_frag<T, D>(xt, 32 * rb + l32, kc, g);
+    for (int kc = 0; kc < KCL; ++kc) xf[kc] = walk_row_frag<T, D>(xt, 32 * rb + l32, kc, g);
     float rsum = 0.f;
     if constexpr (EX == 1) {
 #pragma unroll
-        for (int kc = 0; kc < W::KC; ++kc)
+        for (int kc = 0; kc < KCL; ++kc)
 #pragma unroll
             for (int a = 0; a < 2; ++a) {
                 const f32x4 z = *reinterpret_cast<const f32x4 *>(exv + 16 * kc + 8 * g + 4 * a);
@@ -285,9 +305,9 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
         for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
     if (has_state) {
 #pragma unroll
-        for (int i = 0; i < W::DBW; ++i)
+        for (int i = 0; i < PER; ++i)
 #pragma unroll
-            for (int kc = 0; kc < W::KC; ++kc) acc[i] = M::mma(sfrag(db0 + i, kc), xf[kc], acc[i]);
+            for (int kc = 0; kc < KCL; ++kc) acc[i] = M::mma(sfrag(db0 + i, kc), xf[kc], acc[i]);
     }
     const int s_lo = UPPER ? rb : 0, s_hi = UPPER ? W::NRB - 1 : rb;
 #pragma unroll 1
@@ -296,7 +316,7 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
 #pragma unroll
         for (int v = 0; v < 16; ++v) sc[v] = 0.f;
 #pragma unroll
-        for (int kc = 0; kc < W::KC; ++kc) sc = M::mma(walk_row_frag<T, D>(yt, 32 * s + l32, kc, g), xf[kc], sc);
+        for (int kc = 0; kc < KCL; ++kc) sc = M::mma(walk_row_frag<T, D>(yt, 32 * s + l32, kc, g), xf[kc], sc);
         if constexpr (EX == 2) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) sc[v] += *ex;
@@ -329,7 +349,7 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
 #pragma unroll
         for (int t = 0; t < 2; ++t)
 #pragma unroll
-            for (int i = 0; i < W::DBW; ++i)
+            for (int i = 0; i < PER; ++i)
                 acc[i] = M::mma(walk_col_frag_perm<T, D>(zt, 32 * s + 16 * t, db0 + i, lane, false), pf[t], acc[i]);
     }
     if constexpr (EX == 1) *ex = rsum + __shfl_xor(rsum, 32, 64);  // the two lanes of a row hold half the columns each
@@ -358,14 +378,14 @@ __device__ __forceinline__ void walk_map_tile(unsigned char *tile, int fmap, int
 // 32 (db0 + i) + 16 g + 8 hq .. + 7.  With a feature map, `ytile` is the LDS tile holding
 // y = phi(x) for the same rows (tile row `trow`) and Out is multiplied by the slope phi'(x),
 // computed from y, first.
-template <typename T, int D>
+template <typename T, int D, int PER = WalkCfg<D>::DBW>
 __device__ __forceinline__ void walk_pack(const f32x16 (&acc)[WalkCfg<D>::DBW], int g, int db0,
                                           u32x4 (&pk)[WalkCfg<D>::DBW][2], int fmap = 0,
                                           const unsigned char *ytile = nullptr, int trow = 0) {
     using W = WalkCfg<D>;
     using V8 = typename Mma<T>::V8;
 #pragma unroll
-    for (int i = 0; i < W::DBW; ++i) {
+    for (int i = 0; i < PER; ++i) {
         const int db = db0 + i;
 #pragma unroll
         for (int hq = 0; hq < 2; ++hq) {
@@ -388,11 +408,11 @@ __device__ __forceinline__ void walk_pack(const f32x16 (&acc)[WalkCfg<D>::DBW], 
 
 // two 16-byte stores per block; rows >= N and columns beyond the true width fall outside the
 // buffer resource and are dropped
-template <int D>
+template <int D, int PER = WalkCfg<D>::DBW>
 __device__ __forceinline__ void walk_store_packed(__amdgpu_buffer_rsrc_t rs, int stride2, int width, int row, int g,
                                                   int db0, const u32x4 (&pk)[WalkCfg<D>::DBW][2]) {
 #pragma unroll
-    for (int i = 0; i < WalkCfg<D>::DBW; ++i)
+    for (int i = 0; i < PER; ++i)
 #pragma unroll
         for (int hq = 0; hq < 2; ++hq) {
             const int col = 32 * (db0 + i) + 16 * g + 8 * hq;
@@ -401,44 +421,43 @@ __device__ __forceinline__ void walk_store_packed(__amdgpu_buffer_rsrc_t rs, int
         }
 }
 
-template <typename T, int D>
+// (PER: the blocks of acc that are this wave's -- the others belong to another wave or hold nothing)
+template <typename T, int D, int PER = WalkCfg<D>::DBW>
 __device__ __forceinline__ void walk_store(__amdgpu_buffer_rsrc_t rs, int stride2, int width, int row, int g, int db0,
                                            const f32x16 (&acc)[WalkCfg<D>::DBW], int fmap = 0,
                                            const unsigned char *ytile = nullptr, int trow = 0) {
     u32x4 pk[WalkCfg<D>::DBW][2];
-    walk_pack<T, D>(acc, g, db0, pk, fmap, ytile, trow);
-    walk_store_packed<D>(rs, stride2, width, row, g, db0, pk);
+    walk_pack<T, D, PER>(acc, g, db0, pk, fmap, ytile, trow);
+    walk_store_packed<D, PER>(rs, stride2, width, row, g, db0, pk);
 }
 
 // state += Y^T Z over the rows of the tiles, this wave's 32 x 32 blocks (block i: Y columns of block
 // dbk(i), Z columns of block eb): st[i][v] = State[32 dbk(i) + 8(v/4) + 4g + v%4][32 eb + l32]
-template <typename T, int D>
+template <typename T, int D, typename B = WalkExt<D>>
 __device__ __forceinline__ void walk_update(const unsigned char *yt, const unsigned char *zt, int wave, int lane,
                                             f32x16 (&st)[WalkCfg<D>::NBW]) {
     using W = WalkCfg<D>;
     using M = Mma<T>;
-    using B = WalkBlock<D>;
     if (!B::valid(wave, 0)) return;
 #pragma unroll
     for (int ks = 0; ks < W::C / 16; ++ks) {
         const typename M::V8 zf = walk_col_frag<T, D>(zt, 16 * ks, B::eb(wave), lane);
 #pragma unroll
-        for (int i = 0; i < W::NBW; ++i)
+        for (int i = 0; i < B::SLOTS; ++i)
             if (B::valid(wave, i)) st[i] = M::mma(walk_col_frag<T, D>(yt, 16 * ks, B::dbk(wave, i), lane), zf, st[i]);
     }
 }
 
 // the state rounded to 16 bit into LDS as T[v index][q/k index] (row = 32 eb + l32, four consecutive
 // columns per register group), in the tile layout
-template <typename T, int D>
+template <typename T, int D, typename B = WalkExt<D>>
 __device__ __forceinline__ void walk_state_to_lds(unsigned char *tl, int wave, int lane,
                                                   const f32x16 (&st)[WalkCfg<D>::NBW]) {
     using W = WalkCfg<D>;
-    using B = WalkBlock<D>;
     typedef T t4 __attribute__((ext_vector_type(4)));
     const int l32 = lane & 31, g = lane >> 5, row = 32 * B::eb(wave) + l32;
 #pragma unroll
-    for (int i = 0; i < W::NBW; ++i) {
+    for (int i = 0; i < B::SLOTS; ++i) {
         if (!B::valid(wave, i)) continue;
         const int dbk = B::dbk(wave, i);
 #pragma unroll
@@ -469,11 +488,10 @@ __device__ __forceinline__ WalkSlice walk_slice(const WalkParams &p) {
 }
 
 // this wave's blocks of the entry state of segment sl.seg (zeros without an init buffer)
-template <int D>
+template <int D, typename B = WalkExt<D>>
 __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSlice &sl, int wave, int lane,
                                                f32x16 (&st)[WalkCfg<D>::NBW]) {
     using W = WalkCfg<D>;
-    using B = WalkBlock<D>;
     const int l32 = lane & 31, g = lane >> 5;
     const float *init = nullptr;
     if (p.init) init = p.init + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D);
@@ -488,7 +506,7 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
     if (p.init_transposed) {
         typedef float f32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
-        for (int i = 0; i < W::NBW; ++i)
+        for (int i = 0; i < B::SLOTS; ++i)
             if (B::valid(wave, i)) {
 #pragma unroll
                 for (int a = 0; a < 4; ++a) {
@@ -499,7 +517,7 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
             }
     } else {
 #pragma unroll
-        for (int i = 0; i < W::NBW; ++i)
+        for (int i = 0; i < B::SLOTS; ++i)
             if (B::valid(wave, i)) {
 #pragma unroll
                 for (int v = 0; v < 16; ++v)
@@ -518,12 +536,15 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
 // measured 20 % slower: the stores then compete with the loads in flight instead of filling the
 // gap after them.)
 // NORM: the instantiations that take the normaliser's terms: 1 forward (WalkParams::denom), 2 dQ (dn).
-template <typename T, int D, bool DOUBLE, int NORM>
+// NQ, NV: blocks of the state [q/k index][v index] that hold anything (WalkExt).
+template <typename T, int D, bool DOUBLE, int NORM, int NQ = D / 32, int NV = D / 32>
 __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
     using V8 = typename Mma<T>::V8;
-    using B = WalkBlock<D>;
+    using B = WalkExt<D, NQ, NV>;
+    using OB = WalkOut<D, NV>;  // the result is as wide as v
+    static_assert(NORM == 0 || (NQ == W::DB && NV == W::DB), "the normaliser's variants are built for full widths");
     constexpr int SETS = DOUBLE ? 2 : 1;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -531,7 +552,7 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
     unsigned char *xv = tl + W::STATE;  // per set: zc, (unused), dn of the chunk
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int rb = W::NCH == 1 ? wave : wave % W::NRB, db0 = W::NCH == 1 ? 0 : (wave / W::NRB) * W::DBW;
+    const int rb = W::NCH == 1 ? wave : wave % W::NRB, db0 = OB::db0(wave);
     const WalkSlice sl = walk_slice(p);
     if (!sl.valid) return;
     const int b = sl.bh / p.H, h = sl.bh - b * p.H, N = p.N;
@@ -546,8 +567,8 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(O, 0, (N - 1) * os2 + p.wv * 2, 0x00020000);
 
     f32x16 st[W::NBW];
-    walk_load_init<D>(p, sl, wave, lane, st);
-    walk_state_to_lds<T, D>(tl, wave, lane, st);
+    walk_load_init<D, B>(p, sl, wave, lane, st);
+    walk_state_to_lds<T, D, B>(tl, wave, lane, st);
 
     auto load_chunk = [&](int c, int buf) {
         const uint32_t base = lds0 + buf * 3 * W::TILE;
@@ -617,7 +638,7 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
         auto sfrag = [&](int db, int kc) -> V8 { return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g); };
         if constexpr (NORM == 1) {  // forward with the normaliser: n = masked row sum + q . zc + eps
             float tot;
-            walk_product<T, D, false, 1>(tq, tk, tv, wave, lane, c > 0, sfrag, acc, &tot, vz);
+            walk_product<T, D, false, 1, B::KQ, NV>(tq, tk, tv, wave, lane, c > 0, sfrag, acc, &tot, vz);
             const float n = tot + p.eps, inv = 1.0f / n;
 #pragma unroll
             for (int i = 0; i < W::DBW; ++i)
@@ -626,10 +647,10 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
             if (db0 == 0 && g == 0 && row < N) p.denom[(int64_t)sl.bh * N + row] = n;
         } else if constexpr (NORM == 2) {  // dQ with the normaliser's term: scores + dn_i, result + dn_i zc
             float ax = vd[32 * rb + l32];
-            walk_product<T, D, false, 2>(tq, tk, tv, wave, lane, c > 0, sfrag, acc, &ax);
+            walk_product<T, D, false, 2, B::KQ, NV>(tq, tk, tv, wave, lane, c > 0, sfrag, acc, &ax);
             walk_add_vec<D>(acc, ax, vz, db0, g);
         } else {
-            walk_product<T, D, false>(tq, tk, tv, wave, lane, c > 0, sfrag, acc);
+            walk_product<T, D, false, 0, B::KQ, NV>(tq, tk, tv, wave, lane, c > 0, sfrag, acc);
         }
         if (p.slope_y) {
 #pragma unroll
@@ -638,11 +659,11 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
                 for (int v = 0; v < 16; ++v)
                     acc[i][v] *= feature_slope_from_value(p.fmap, static_cast<float>(ys[i][v / 8][v % 8]));
         }
-        walk_store<T, D>(ro, os2, p.wv, row, g, db0, acc);
+        walk_store<T, D, OB::PER>(ro, os2, p.wv, row, g, db0, acc);
         if (p.saved) {  // the state at the entry of this chunk, [q/k index][v index], for backward's dQ
             T *sv = static_cast<T *>(p.saved) + ((int64_t)sl.bh * p.n_chunks + c) * (D * D);
 #pragma unroll
-            for (int i = 0; i < W::NBW; ++i)
+            for (int i = 0; i < B::SLOTS; ++i)
                 if (B::valid(wave, i)) {
 #pragma unroll
                     for (int v = 0; v < 16; ++v)
@@ -650,7 +671,7 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
                             static_cast<T>(st[i][v]);
                 }
         }
-        walk_update<T, D>(tk, tv, wave, lane, st);
+        walk_update<T, D, B>(tk, tv, wave, lane, st);
         if constexpr (DOUBLE) {
             asm volatile("" ::: "memory");
             __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS reads of the tiles and of the state are done
@@ -659,7 +680,7 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
         } else {
             __syncthreads();  // every wave is done with the tiles and with the old state
         }
-        walk_state_to_lds<T, D>(tl, wave, lane, st);
+        walk_state_to_lds<T, D, B>(tl, wave, lane, st);
     }
 #else
     (void)p;
@@ -782,7 +803,7 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
 // lane loads one value of each, a chunk ahead and after the tiles' loads, and the values are
 // handed round within the wave (ds_bpermute: 64 per chunk, about 30 clocks each -- 28 us of a 207 us
 // launch at B H = 128, N = 4096) when the chunk's turn comes.
-template <typename T, int D, bool NORM>
+template <typename T, int D, bool NORM, int NQ = D / 32, int NV = D / 32>
 __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
@@ -792,7 +813,11 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
     unsigned char *tl = smem + 8 * W::TILE;
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int rb = W::NCH == 1 ? wave : wave % W::NRB, db0 = W::NCH == 1 ? 0 : (wave / W::NRB) * W::DBW;
+    using B = WalkExt<D, NQ, NV>;   // R [q/k index][v index]
+    using OV = WalkOut<D, NV>;      // dV is as wide as v,
+    using OQ = WalkOut<D, NQ>;      // dK as q and k
+    static_assert(!NORM || (NQ == W::DB && NV == W::DB), "the normaliser's variant is built for full widths");
+    const int rb = W::NCH == 1 ? wave : wave % W::NRB, db0 = OQ::db0(wave);  // (db0: dK's, and rc's columns)
     const WalkSlice sl = walk_slice(p);
     if (!sl.valid) return;
     const int b = sl.bh / p.H, h = sl.bh - b * p.H, N = p.N;
@@ -812,8 +837,8 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
     const __amdgpu_buffer_rsrc_t rdv = __builtin_amdgcn_make_buffer_rsrc(DV, 0, (N - 1) * dvs2 + p.wv * 2, 0x00020000);
 
     f32x16 st[W::NBW];  // R[q/k index][v index]
-    walk_load_init<D>(p, sl, wave, lane, st);
-    walk_state_to_lds<T, D>(tl, wave, lane, st);
+    walk_load_init<D, B>(p, sl, wave, lane, st);
+    walk_state_to_lds<T, D, B>(tl, wave, lane, st);
 
     auto load_chunk = [&](int c, int buf) {
         const uint32_t base = lds0 + buf * 4 * W::TILE;
@@ -879,10 +904,10 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
         const bool later = c + 1 < p.n_chunks;  // chunks after this one exist: R is not identically zero
         f32x16 acc[W::DBW];
         // dV = upper(K Q^T) dO + K R: A operand R^T[v index][q/k index] = the LDS copy as it is
-        walk_product<T, D, true>(tk, tq, tg, wave, lane, later, [&](int db, int kc) -> V8 {
+        walk_product<T, D, true, 0, B::KQ, NV>(tk, tq, tg, wave, lane, later, [&](int db, int kc) -> V8 {
             return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g);
         }, acc);
-        walk_store<T, D>(rdv, dvs2, p.wv, row, g, db0, acc);
+        walk_store<T, D, OV::PER>(rdv, dvs2, p.wv, row, g, OV::db0(wave), acc);
         // dK = upper(V dO^T) Q + V R^T: A operand R[q/k index][v index] = the LDS copy read transposed
         if constexpr (NORM) {
             walk_product<T, D, true, 3>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
@@ -891,17 +916,17 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
 #pragma unroll
             for (int i = 0; i < W::DBW; ++i) acc[i] += rcv[i];
         } else {
-            walk_product<T, D, true>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
+            walk_product<T, D, true, 0, B::KV, NQ>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
                 return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
             }, acc);
         }
-        walk_store<T, D>(rdk, dks2, p.wqk, row, g, db0, acc, p.fmap, tk, 32 * rb + l32);
-        walk_update<T, D>(tq, tg, wave, lane, st);
+        walk_store<T, D, OQ::PER>(rdk, dks2, p.wqk, row, g, db0, acc, p.fmap, tk, 32 * rb + l32);
+        walk_update<T, D, B>(tq, tg, wave, lane, st);
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS reads of the tiles and of the state are done
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        walk_state_to_lds<T, D>(tl, wave, lane, st);
+        walk_state_to_lds<T, D, B>(tl, wave, lane, st);
     }
 #else
     (void)p;
@@ -923,7 +948,7 @@ struct WalkTotalsParams {
     int64_t yo_b, yo_h, yo_n;
 };
 
-template <typename T, int D>
+template <typename T, int D, int NQ = D / 32, int NV = D / 32>
 __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
@@ -947,7 +972,7 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
     const int ys2 = (int)p.ys_n * 2, zs2 = (int)p.zs_n * 2;
     const u32x4 ry = make_rsrc(Y, (uint32_t)((N - 1) * ys2 + p.dy * 2));
     const u32x4 rz = make_rsrc(Z, (uint32_t)((N - 1) * zs2 + p.dz * 2));
-    using B = WalkBlock<D>;
+    using B = WalkExt<D, NQ, NV>;  // (blocks outside it stay unwritten: no walk of the same extent reads them)
     f32x16 st[W::NBW];
 #pragma unroll
     for (int i = 0; i < W::NBW; ++i)
@@ -980,14 +1005,14 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
         }
-        walk_update<T, D>(ty, tz, wave, lane, st);
+        walk_update<T, D, B>(ty, tz, wave, lane, st);
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS reads of the set are done
         __builtin_amdgcn_s_barrier();
     }
     float *out = p.totals + ((int64_t)bh * p.n_seg + seg) * (D * D);
 #pragma unroll
-    for (int i = 0; i < W::NBW; ++i)
+    for (int i = 0; i < B::SLOTS; ++i)
         if (B::valid(wave, i)) {
 #pragma unroll
             for (int v = 0; v < 16; ++v)
@@ -1158,8 +1183,15 @@ template <typename T, int D>
 hipError_t launch_walk_totals(const WalkTotalsParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-    constexpr auto kern = walk_totals_kernel<T, D>;
     constexpr int smem = 4 * WalkCfg<D>::TILE;
+    if constexpr (D == 128) {
+        if (p.dy > 64 && p.dz <= 64) {  // z of at most 64 true columns: the state's other v blocks hold zeros
+            constexpr auto kern = walk_totals_kernel<T, D, 4, 2>;
+            if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
+            return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+        }
+    }
+    constexpr auto kern = walk_totals_kernel<T, D>;
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
     return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
 }
@@ -1189,6 +1221,20 @@ hipError_t launch_walk_fwd(const WalkParams &p, hipStream_t stream) {
         constexpr auto kern = walk_fwd_kernel<T, D, kDouble, 2>;
         if (hipError_t e = ensure_dynamic_lds<kern>(smem_n)) return e;
         return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem_n, stream, p);
+    }
+    if constexpr (D == 128) {
+        // operands of at most 64 true columns on one side (the halves of a wide q / k against a narrow v):
+        // the kernels that leave out the blocks of padding
+        if (!p.fmap && !p.slope_y && p.wqk > 64 && p.wv <= 64) {
+            constexpr auto kern = walk_fwd_kernel<T, D, kDouble, 0, 4, 2>;
+            if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
+            return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+        }
+        if (!p.fmap && !p.slope_y && p.wqk <= 64 && p.wv > 64) {
+            constexpr auto kern = walk_fwd_kernel<T, D, kDouble, 0, 2, 4>;
+            if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
+            return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+        }
     }
     constexpr auto kern = walk_fwd_kernel<T, D, kDouble, 0>;
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
@@ -1223,6 +1269,13 @@ hipError_t launch_walk_dkdv(const WalkParams &p, hipStream_t stream) {
         constexpr auto kern = walk_dkdv_kernel<T, D, true>;
         if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
         return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+    }
+    if constexpr (D == 128) {
+        if (!p.fmap && p.wqk > 64 && p.wv <= 64) {
+            constexpr auto kern = walk_dkdv_kernel<T, D, false, 4, 2>;
+            if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
+            return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+        }
     }
     constexpr auto kern = walk_dkdv_kernel<T, D, false>;
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
