@@ -135,7 +135,8 @@ struct WalkExt {
     static constexpr int nq = NQ, nv = NV;
     static constexpr int SLOTS = (NQ * NV + 3) / 4;  // state blocks per wave
     static constexpr int KQ = 2 * NQ, KV = 2 * NV;   // 16-wide k chunks over the q/k side, the v side
-    __device__ static __forceinline__ bool valid(int wave, int i) { return wave + 4 * i < NQ * NV; }
+    // (with a multiple of four blocks every slot of every wave holds one: known at compile time)
+    __device__ static __forceinline__ bool valid(int wave, int i) { return (NQ * NV) % 4 == 0 || wave + 4 * i < NQ * NV; }
     __device__ static __forceinline__ int dbk(int wave, int i) { return (wave + 4 * i) / NV; }
     __device__ static __forceinline__ int eb(int wave) { return wave % NV; }
 };
@@ -536,8 +537,9 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
 // measured 20 % slower: the stores then compete with the loads in flight instead of filling the
 // gap after them.)
 // NORM: the instantiations that take the normaliser's terms: 1 forward (WalkParams::denom), 2 dQ (dn).
+// FM: the instantiations that know of feature maps (WalkParams::fmap, slope_y); the others ignore both.
 // NQ, NV: blocks of the state [q/k index][v index] that hold anything (WalkExt).
-template <typename T, int D, bool DOUBLE, int NORM, int NQ = D / 32, int NV = D / 32>
+template <typename T, int D, bool DOUBLE, int NORM, bool FM, int NQ = D / 32, int NV = D / 32>
 __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
@@ -555,6 +557,8 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
     const int rb = W::NCH == 1 ? wave : wave % W::NRB, db0 = OB::db0(wave);
     const WalkSlice sl = walk_slice(p);
     if (!sl.valid) return;
+    const int fmap = FM ? p.fmap : 0;
+    const void *slope_y = FM ? p.slope_y : nullptr;
     const int b = sl.bh / p.H, h = sl.bh - b * p.H, N = p.N;
     const T *Q = static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h;
     const T *K = static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h;
@@ -591,8 +595,8 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
         // dQ walk with a feature map: this lane's values of phi(xq) under its accumulator registers,
         // requested before the tiles so that they have arrived with them
         V8 ys[W::DBW][2];
-        if (p.slope_y) {
-            const T *yrow = static_cast<const T *>(p.slope_y) + b * p.sy_b + h * p.sy_h + (int64_t)(row < N ? row : 0) * p.sy_n;
+        if (slope_y) {
+            const T *yrow = static_cast<const T *>(slope_y) + b * p.sy_b + h * p.sy_h + (int64_t)(row < N ? row : 0) * p.sy_n;
 #pragma unroll
             for (int i = 0; i < W::DBW; ++i)
 #pragma unroll
@@ -615,8 +619,8 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
             __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's part of the state is in LDS
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
-            if (p.fmap && p.qmap_out) {
-                walk_map_tile<T, D>(tq, p.fmap, row0, N, p.wqk, static_cast<T *>(p.qmap_out) + b * p.qo_b + h * p.qo_h,
+            if (fmap && p.qmap_out) {
+                walk_map_tile<T, D>(tq, fmap, row0, N, p.wqk, static_cast<T *>(p.qmap_out) + b * p.qo_b + h * p.qo_h,
                                     p.qo_n, tid);
                 __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the rewritten tile is in LDS
                 __builtin_amdgcn_s_barrier();
@@ -626,8 +630,8 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
             load_chunk(c, 0);
             wait_vm<0>();
             __syncthreads();  // the tiles have landed; the state written by the previous iteration is visible
-            if (p.fmap && p.qmap_out) {
-                walk_map_tile<T, D>(tq, p.fmap, row0, N, p.wqk, static_cast<T *>(p.qmap_out) + b * p.qo_b + h * p.qo_h,
+            if (fmap && p.qmap_out) {
+                walk_map_tile<T, D>(tq, fmap, row0, N, p.wqk, static_cast<T *>(p.qmap_out) + b * p.qo_b + h * p.qo_h,
                                     p.qo_n, tid);
                 __syncthreads();
             }
@@ -652,15 +656,15 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
         } else {
             walk_product<T, D, false, 0, B::KQ, NV>(tq, tk, tv, wave, lane, c > 0, sfrag, acc);
         }
-        if (p.slope_y) {
+        if (slope_y) {
 #pragma unroll
             for (int i = 0; i < W::DBW; ++i)
 #pragma unroll
                 for (int v = 0; v < 16; ++v)
-                    acc[i][v] *= feature_slope_from_value(p.fmap, static_cast<float>(ys[i][v / 8][v % 8]));
+                    acc[i][v] *= feature_slope_from_value(fmap, static_cast<float>(ys[i][v / 8][v % 8]));
         }
         walk_store<T, D, OB::PER>(ro, os2, p.wv, row, g, db0, acc);
-        if (p.saved) {  // the state at the entry of this chunk, [q/k index][v index], for backward's dQ
+        if (!DOUBLE && p.saved) {  // the state at the entry of this chunk, [q/k index][v index], for backward's dQ
             T *sv = static_cast<T *>(p.saved) + ((int64_t)sl.bh * p.n_chunks + c) * (D * D);
 #pragma unroll
             for (int i = 0; i < B::SLOTS; ++i)
@@ -1204,41 +1208,38 @@ inline hipError_t launch_walk_scan(const float *totals, float *entry, int64_t BH
                          n_seg, m, E, total2, reverse);
 }
 
+template <auto kern>
+hipError_t launch_walk_kernel(int64_t grid, int smem, const WalkParams &p, hipStream_t stream) {
+    if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
+    return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+}
+
 template <typename T, int D>
 hipError_t launch_walk_fwd(const WalkParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     constexpr bool kDouble = D > 64;  // (the plan's workgroup count must match: one per CU when double)
     constexpr int smem = (kDouble ? 6 : 3) * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
+    const bool fm = p.fmap || p.slope_y;
     if (p.denom || p.dn) {  // the normaliser's terms: its vectors live behind the state
         if (!p.zc) return hipErrorInvalidValue;
         constexpr int smem_n = smem + (kDouble ? 2 : 1) * WalkCfg<D>::VEC;
-        if (p.denom) {
-            constexpr auto kern = walk_fwd_kernel<T, D, kDouble, 1>;
-            if (hipError_t e = ensure_dynamic_lds<kern>(smem_n)) return e;
-            return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem_n, stream, p);
-        }
-        constexpr auto kern = walk_fwd_kernel<T, D, kDouble, 2>;
-        if (hipError_t e = ensure_dynamic_lds<kern>(smem_n)) return e;
-        return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem_n, stream, p);
+        if (p.denom)
+            return fm ? launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 1, true>>(grid, smem_n, p, stream)
+                      : launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 1, false>>(grid, smem_n, p, stream);
+        return fm ? launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 2, true>>(grid, smem_n, p, stream)
+                  : launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 2, false>>(grid, smem_n, p, stream);
     }
+    if (fm) return launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, true>>(grid, smem, p, stream);
     if constexpr (D == 128) {
         // operands of at most 64 true columns on one side (the halves of a wide q / k against a narrow v):
         // the kernels that leave out the blocks of padding
-        if (!p.fmap && !p.slope_y && p.wqk > 64 && p.wv <= 64) {
-            constexpr auto kern = walk_fwd_kernel<T, D, kDouble, 0, 4, 2>;
-            if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-            return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
-        }
-        if (!p.fmap && !p.slope_y && p.wqk <= 64 && p.wv > 64) {
-            constexpr auto kern = walk_fwd_kernel<T, D, kDouble, 0, 2, 4>;
-            if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-            return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
-        }
+        if (p.wqk > 64 && p.wv <= 64)
+            return launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, false, 4, 2>>(grid, smem, p, stream);
+        if (p.wqk <= 64 && p.wv > 64)
+            return launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, false, 2, 4>>(grid, smem, p, stream);
     }
-    constexpr auto kern = walk_fwd_kernel<T, D, kDouble, 0>;
-    if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-    return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+    return launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, false>>(grid, smem, p, stream);
 }
 
 template <typename T, int D>
