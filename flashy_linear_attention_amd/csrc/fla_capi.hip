@@ -381,7 +381,8 @@ struct WalkPlan {
     int64_t fine_bytes;                   // fp32 totals of the finer segments
     int64_t entry_bytes;                  // fp32 entry states of the walk segments (in place over the totals when m == 1)
     int64_t work_bytes;                   // workspace of one direction: totals, and entry states when m > 1
-    int64_t saved_bytes;                  // what forward hands to backward: per-chunk 16-bit states / split: the entry states
+    int64_t saved_bytes;                  // what forward hands to backward: per-chunk 16-bit states / split: the entry
+                                          // states and, behind them, the state after the last chunk of every (b, h)
 };
 
 WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
@@ -404,7 +405,7 @@ WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     w.entry_bytes = B * H * w.n_seg * w.D * w.D * 4;
     w.fine_bytes = w.entry_bytes * w.m;
     w.work_bytes = w.fine_bytes + (w.m > 1 ? w.entry_bytes : 0);  // (a single segment needs them only with a feature map)
-    w.saved_bytes = w.split ? w.entry_bytes : B * H * w.n_chunks * w.D * w.D * 2;
+    w.saved_bytes = w.split ? w.entry_bytes + B * H * w.D * w.D * 4 : B * H * w.n_chunks * w.D * w.D * 2;
     return w;
 }
 
@@ -680,6 +681,7 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dqk, w.wv = (int32_t)dv;
         w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
         w.init = wp.n_seg > 1 ? entry : nullptr, w.saved = wp.split ? nullptr : state_out;
+        if (in_state) w.total_out = reinterpret_cast<float *>(static_cast<char *>(state_out) + wp.entry_bytes);
         if (nx) {  // the normaliser inside the walk: zc = running sum of k at the entry of every chunk
             // (kept behind the state, when there is one, for backward)
             float *zc = state_out ? reinterpret_cast<float *>(static_cast<char *>(state_out) + state_core_bytes(B, H, N, dqk, dv))
@@ -771,6 +773,8 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         if (state_in && reinterpret_cast<uintptr_t>(state_in) % 16 != 0) return FLA_ERR_WORKSPACE;
         hipStream_t s = static_cast<hipStream_t>(stream);
         const float *entry = nullptr;
+        // with forward's states at hand (and neither a feature map nor the normaliser): one reverse walk
+        const bool one_walk = state_in && !fmap && !nx;
         if (wp.n_seg > 1) {
             if (!state_in) {
                 const float *fwd_entry = nullptr;
@@ -788,6 +792,24 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
             if (int rc = walk_chunk_vectors(wp, q, dqk, nx->dn, 1, rcv, B, H, N, dtype, s)) return rc;
             if (zc_saved) zc = const_cast<float *>(zc_saved);
             else if (int rc = walk_chunk_vectors(wp, k, dqk, nullptr, 0, zc, B, H, N, dtype, s)) return rc;
+        }
+        if (one_walk) {
+            fla::WalkParams r{};
+            r.q = q.ptr, r.k = k.ptr, r.v = v.ptr, r.go = go.ptr;
+            r.dq = const_cast<void *>(dq.ptr), r.dk = const_cast<void *>(dk.ptr), r.dv = const_cast<void *>(dvv.ptr);
+            r.qs_b = q.strides[0], r.qs_h = q.strides[1], r.qs_n = q.strides[2];
+            r.ks_b = k.strides[0], r.ks_h = k.strides[1], r.ks_n = k.strides[2];
+            r.vs_b = v.strides[0], r.vs_h = v.strides[1], r.vs_n = v.strides[2];
+            r.gs_b = go.strides[0], r.gs_h = go.strides[1], r.gs_n = go.strides[2];
+            r.dqs_b = dq.strides[0], r.dqs_h = dq.strides[1], r.dqs_n = dq.strides[2];
+            r.dks_b = dk.strides[0], r.dks_h = dk.strides[1], r.dks_n = dk.strides[2];
+            r.dvs_b = dvv.strides[0], r.dvs_h = dvv.strides[1], r.dvs_n = dvv.strides[2];
+            r.H = (int32_t)H, r.N = (int32_t)N, r.BH = (int32_t)(B * H), r.wqk = (int32_t)dqk, r.wv = (int32_t)dv;
+            r.n_chunks = (int32_t)wp.n_chunks, r.seg_chunks = (int32_t)wp.seg_chunks, r.n_seg = (int32_t)wp.n_seg;
+            r.init = entry;
+            r.xinit = static_cast<const float *>(state_in);
+            r.xtotal = reinterpret_cast<const float *>(static_cast<const char *>(state_in) + wp.entry_bytes);
+            return fla::walk_bwd_rev(dtype, wp.D, r, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
         }
         // dQ = lower(dO V^T) K + dO S^T: the forward walk over (dO, V, K), its states V^T K = S^T
         fla::WalkParams w{};

@@ -97,6 +97,11 @@ struct WalkParams {
     const float *zc;  // fp32 [BH][n_chunks][D]: sum of k over the rows before chunk c
     const float *dn;  // fp32 [BH][N]
     const float *rc;  // fp32 [BH][n_chunks][D]: sum of dn_i q_i over the rows after chunk c
+    // Forward, D = 128: where the state after the last chunk of every (b, h) goes, fp32 [BH][D][D]
+    // ([q/k index][v index]), or null.  walk_bwd_rev_kernel: that buffer (xtotal) and forward's entry
+    // states (xinit, the layout of `init`, not transposed; may be null with a single segment).
+    float *total_out;
+    const float *xinit, *xtotal;
 };
 
 template <int D>
@@ -273,6 +278,23 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 struct WalkNoRows {
     __device__ __forceinline__ f32x4 operator()(int, int) const { return f32x4{0.f, 0.f, 0.f, 0.f}; }
 };
+// N operand fragments read from LDS and consumed in order, the read of fragment j + DEPTH issued
+// before fragment j is used: use(j, fragment) for j = 0 .. N-1 with read(j + DEPTH) ahead of it.  The
+// scheduling barriers keep the compiler from moving a read down to its use again (which it does when
+// registers are scarce, and every MFMA then waits out the whole latency of its own LDS read).
+template <int N, int DEPTH, typename V8, typename Read, typename Use>
+__device__ __forceinline__ void walk_pipe(Read &&read, Use &&use) {
+    V8 buf[N];
+    static_for<0, (DEPTH < N ? DEPTH : N)>([&](auto j) { buf[decltype(j)::value] = read(j); });
+    static_for<0, N>([&](auto j) {
+        constexpr int J = decltype(j)::value;
+        if constexpr (J + DEPTH < N) buf[J + DEPTH] = read(std::integral_constant<int, J + DEPTH>{});
+        __builtin_amdgcn_sched_barrier(0);
+        use(j, buf[J]);
+    });
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 // KCL: 16-wide k chunks of the contraction X Y^T that hold anything; NOB: output blocks that do.
 template <typename T, int D, bool UPPER, int EX = 0, int KCL = WalkCfg<D>::KC, int NOB = WalkCfg<D>::DB, typename SFrag,
           typename YRows = WalkNoRows>
@@ -304,11 +326,12 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
     for (int i = 0; i < W::DBW; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
-    if (has_state) {
-#pragma unroll
-        for (int i = 0; i < PER; ++i)
-#pragma unroll
-            for (int kc = 0; kc < KCL; ++kc) acc[i] = M::mma(sfrag(db0 + i, kc), xf[kc], acc[i]);
+    if (has_state) {  // (k chunk outer, output block inner: consecutive MFMAs are independent)
+        walk_pipe<PER * KCL, 4, V8>([&](auto j) { return sfrag(db0 + decltype(j)::value % PER, decltype(j)::value / PER); },
+                                    [&](auto j, V8 f) {
+                                        constexpr int I = decltype(j)::value % PER, KC_ = decltype(j)::value / PER;
+                                        acc[I] = M::mma(f, xf[KC_], acc[I]);
+                                    });
     }
     const int s_lo = UPPER ? rb : 0, s_hi = UPPER ? W::NRB - 1 : rb;
 #pragma unroll 1
@@ -316,42 +339,56 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
         f32x16 sc;
 #pragma unroll
         for (int v = 0; v < 16; ++v) sc[v] = 0.f;
-#pragma unroll
-        for (int kc = 0; kc < KCL; ++kc) sc = M::mma(walk_row_frag<T, D>(yt, 32 * s + l32, kc, g), xf[kc], sc);
-        if constexpr (EX == 2) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) sc[v] += *ex;
-        }
-        if constexpr (EX == 3) {
-#pragma unroll
-            for (int a = 0; a < 4; ++a) {
-                const f32x4 y = yrows(s, a);
-#pragma unroll
-                for (int b = 0; b < 4; ++b) sc[4 * a + b] += y[b];
-            }
-        }
-        if (s == rb) {  // the 32 x 32 block on the diagonal: lane = X row l32, register v = Y row jl
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int jl = 8 * (v / 4) + 4 * g + (v % 4);
-                const bool keep = UPPER ? l32 <= jl : l32 >= jl;
-                sc[v] = keep ? sc[v] : 0.f;
-            }
-        }
-        if constexpr (EX == 1) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v) rsum += sc[v];
-        }
+        // fragments 0 .. KCL-1: Y rows for the scores; KCL .. KCL + 2 PER - 1: Z columns for the second
+        // product, requested while the last score MFMAs run
         V8 pf[2];
+        walk_pipe<KCL + 2 * PER, 4, V8>(
+            [&](auto j) {
+                constexpr int J = decltype(j)::value;
+                if constexpr (J < KCL)
+                    return walk_row_frag<T, D>(yt, 32 * s + l32, J, g);
+                else
+                    return walk_col_frag_perm<T, D>(zt, 32 * s + 16 * ((J - KCL) / PER), db0 + (J - KCL) % PER, lane, false);
+            },
+            [&](auto j, V8 f) {
+                constexpr int J = decltype(j)::value;
+                if constexpr (J < KCL) {
+                    sc = M::mma(f, xf[J], sc);
+                } else {
+                    if constexpr (J == KCL) {  // the scores are complete: normaliser's terms, mask, rounding
+                        if constexpr (EX == 2) {
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+                            for (int v = 0; v < 16; ++v) sc[v] += *ex;
+                        }
+                        if constexpr (EX == 3) {
 #pragma unroll
-            for (int e = 0; e < 8; ++e) pf[t][e] = static_cast<T>(sc[8 * t + e]);
+                            for (int a = 0; a < 4; ++a) {
+                                const f32x4 y = yrows(s, a);
 #pragma unroll
-        for (int t = 0; t < 2; ++t)
+                                for (int b = 0; b < 4; ++b) sc[4 * a + b] += y[b];
+                            }
+                        }
+                        if (s == rb) {  // the 32 x 32 block on the diagonal: lane = X row l32, register v = Y row jl
 #pragma unroll
-            for (int i = 0; i < PER; ++i)
-                acc[i] = M::mma(walk_col_frag_perm<T, D>(zt, 32 * s + 16 * t, db0 + i, lane, false), pf[t], acc[i]);
+                            for (int v = 0; v < 16; ++v) {
+                                const int jl = 8 * (v / 4) + 4 * g + (v % 4);
+                                const bool keep = UPPER ? l32 <= jl : l32 >= jl;
+                                sc[v] = keep ? sc[v] : 0.f;
+                            }
+                        }
+                        if constexpr (EX == 1) {
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) rsum += sc[v];
+                        }
+#pragma unroll
+                        for (int t = 0; t < 2; ++t)
+#pragma unroll
+                            for (int e = 0; e < 8; ++e) pf[t][e] = static_cast<T>(sc[8 * t + e]);
+                    }
+                    constexpr int I = (J - KCL) % PER, TT = (J - KCL) / PER;
+                    acc[I] = M::mma(f, pf[TT], acc[I]);
+                }
+            });
     }
     if constexpr (EX == 1) *ex = rsum + __shfl_xor(rsum, 32, 64);  // the two lanes of a row hold half the columns each
 }
@@ -434,18 +471,51 @@ __device__ __forceinline__ void walk_store(__amdgpu_buffer_rsrc_t rs, int stride
 
 // state += Y^T Z over the rows of the tiles, this wave's 32 x 32 blocks (block i: Y columns of block
 // dbk(i), Z columns of block eb): st[i][v] = State[32 dbk(i) + 8(v/4) + 4g + v%4][32 eb + l32]
-template <typename T, int D, typename B = WalkExt<D>>
+// (NEG: state -= Y^T Z -- the sign bits of the Z fragments are flipped.  ACC: the state lives in
+// accumulation registers, see Mma::mma_acc; the wait states an MFMA's result needs before anything
+// but another MFMA reads it are spent at the end, since the compiler does not count them for a
+// statement it cannot look into.)
+template <typename T, int D, typename B = WalkExt<D>, bool NEG = false, bool ACC = false>
 __device__ __forceinline__ void walk_update(const unsigned char *yt, const unsigned char *zt, int wave, int lane,
                                             f32x16 (&st)[WalkCfg<D>::NBW]) {
     using W = WalkCfg<D>;
     using M = Mma<T>;
+    using V8 = typename M::V8;
     if (!B::valid(wave, 0)) return;
+    // per 16 rows: the Z fragment, then the Y fragment of every block -- one group of reads ahead of the MFMAs
+    constexpr int G = 1 + B::SLOTS, KS = W::C / 16;
+    V8 zf = {};
+    walk_pipe<KS * G, G, V8>(
+        [&](auto j) {
+            constexpr int ks = decltype(j)::value / G, r = decltype(j)::value % G;
+            if constexpr (r == 0) {
+                V8 z = walk_col_frag<T, D>(zt, 16 * ks, B::eb(wave), lane);
+                if constexpr (NEG) {
+                    u32x4 raw = __builtin_bit_cast(u32x4, z);
 #pragma unroll
-    for (int ks = 0; ks < W::C / 16; ++ks) {
-        const typename M::V8 zf = walk_col_frag<T, D>(zt, 16 * ks, B::eb(wave), lane);
-#pragma unroll
-        for (int i = 0; i < B::SLOTS; ++i)
-            if (B::valid(wave, i)) st[i] = M::mma(walk_col_frag<T, D>(yt, 16 * ks, B::dbk(wave, i), lane), zf, st[i]);
+                    for (int e = 0; e < 4; ++e) raw[e] ^= 0x80008000u;
+                    z = __builtin_bit_cast(V8, raw);
+                }
+                return z;
+            } else {
+                // (a slot without a block -- only in the last one, with fewer than four blocks in all -- reads block 0)
+                return walk_col_frag<T, D>(yt, 16 * ks, B::valid(wave, r - 1) ? B::dbk(wave, r - 1) : 0, lane);
+            }
+        },
+        [&](auto j, V8 f) {
+            constexpr int r = decltype(j)::value % G;
+            if constexpr (r == 0) {
+                zf = f;
+            } else if (B::valid(wave, r - 1)) {
+                if constexpr (ACC)
+                    M::mma_acc(f, zf, st[r - 1]);
+                else
+                    st[r - 1] = M::mma(f, zf, st[r - 1]);
+            }
+        });
+    if constexpr (ACC) {
+        static_assert(!ACC || B::SLOTS == 4, "written for four blocks per wave");
+        asm volatile("s_nop 15\n\ts_nop 7" : "+a"(st[0]), "+a"(st[1]), "+a"(st[2]), "+a"(st[3]));
     }
 }
 
@@ -488,23 +558,22 @@ __device__ __forceinline__ WalkSlice walk_slice(const WalkParams &p) {
     return s;
 }
 
-// this wave's blocks of the entry state of segment sl.seg (zeros without an init buffer)
+// this wave's blocks of an fp32 state [D][D] in memory (zeros for a null pointer); `transposed`: the
+// buffer holds the transposed matrix ([v index][q/k index])
 template <int D, typename B = WalkExt<D>>
-__device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSlice &sl, int wave, int lane,
-                                               f32x16 (&st)[WalkCfg<D>::NBW]) {
+__device__ __forceinline__ void walk_load_state(const float *init, bool transposed, int wave, int lane,
+                                                f32x16 (&st)[WalkCfg<D>::NBW]) {
     using W = WalkCfg<D>;
     const int l32 = lane & 31, g = lane >> 5;
-    const float *init = nullptr;
-    if (p.init) init = p.init + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D);
 #pragma unroll
     for (int i = 0; i < W::NBW; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v) st[i][v] = 0.f;
     if (!init) return;
     // st[i][v] = State[r = 32 dbk(i) + 8 (v/4) + 4g + v%4][c = 32 eb + l32]: element r D + c of the
-    // buffer, or c D + r when it holds the transposed matrices (then four consecutive floats per v/4)
+    // buffer, or c D + r when it holds the transposed matrix (then four consecutive floats per v/4)
     const int c = 32 * B::eb(wave) + l32;
-    if (p.init_transposed) {
+    if (transposed) {
         typedef float f32x4 __attribute__((ext_vector_type(4)));
 #pragma unroll
         for (int i = 0; i < B::SLOTS; ++i)
@@ -525,6 +594,15 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
                     st[i][v] = init[(32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + c];
             }
     }
+}
+
+// this wave's blocks of the entry state of segment sl.seg (zeros without an init buffer)
+template <int D, typename B = WalkExt<D>>
+__device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSlice &sl, int wave, int lane,
+                                               f32x16 (&st)[WalkCfg<D>::NBW]) {
+    const float *init = nullptr;
+    if (p.init) init = p.init + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D);
+    walk_load_state<D, B>(init, p.init_transposed != 0, wave, lane, st);
 }
 
 // ---- one product with its running state, chunks ascending:
@@ -685,6 +763,16 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
             __syncthreads();  // every wave is done with the tiles and with the old state
         }
         walk_state_to_lds<T, D, B>(tl, wave, lane, st);
+    }
+    if (DOUBLE && p.total_out && sl.c_hi == p.n_chunks) {  // the state after the last chunk, for walk_bwd_rev_kernel
+        float *out = p.total_out + (int64_t)sl.bh * (D * D);
+#pragma unroll
+        for (int i = 0; i < B::SLOTS; ++i)
+            if (B::valid(wave, i)) {
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    out[(32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * B::eb(wave) + l32] = st[i][v];
+            }
     }
 #else
     (void)p;
@@ -930,6 +1018,116 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
         __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS reads of the tiles and of the state are done
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
+        walk_state_to_lds<T, D, B>(tl, wave, lane, st);
+    }
+#else
+    (void)p;
+#endif
+}
+
+// ---- backward at D = 128 in one reverse walk: dV, dK and dQ of a chunk from one set of tiles.
+//   R = sum of Q^T dO over the chunks after this one, as in walk_dkdv_kernel;
+//   X = sum of K^T V over the chunks before it, obtained backwards: X starts as the forward state at
+//   the end of the segment (the next segment's entry state, or the state after the last chunk) and
+//   every chunk's K^T V is subtracted when the walk reaches it.  (In fp32: the difference carries
+//   the rounding of the sums it is taken from, about 1e-7 of the largest state -- far below the
+//   16-bit rounding the state gets before it multiplies dO.)
+// The one 16-bit state in LDS holds R for dV and dK, then X for dQ.  q, k, v, dO are read once and
+// nothing but the results is written, where the walk for dQ followed by walk_dkdv_kernel reads
+// dO, v, k twice.
+template <typename T, int D>
+__global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    using W = WalkCfg<D>;
+    using V8 = typename Mma<T>::V8;
+    using B = WalkExt<D>;
+    using OB = WalkOut<D, W::DB>;
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    unsigned char *tl = smem + 8 * W::TILE;
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rb = W::NCH == 1 ? wave : wave % W::NRB, db0 = OB::db0(wave);
+    const WalkSlice sl = walk_slice(p);
+    if (!sl.valid) return;
+    const int b = sl.bh / p.H, h = sl.bh - b * p.H, N = p.N;
+    const T *Q = static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h;
+    const T *K = static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h;
+    const T *V = static_cast<const T *>(p.v) + b * p.vs_b + h * p.vs_h;
+    const T *G = static_cast<const T *>(p.go) + b * p.gs_b + h * p.gs_h;
+    T *DQ = static_cast<T *>(p.dq) + b * p.dqs_b + h * p.dqs_h;
+    T *DK = static_cast<T *>(p.dk) + b * p.dks_b + h * p.dks_h;
+    T *DV = static_cast<T *>(p.dv) + b * p.dvs_b + h * p.dvs_h;
+    const int qs2 = (int)p.qs_n * 2, ks2 = (int)p.ks_n * 2, vs2 = (int)p.vs_n * 2, gs2 = (int)p.gs_n * 2;
+    const int dqs2 = (int)p.dqs_n * 2, dks2 = (int)p.dks_n * 2, dvs2 = (int)p.dvs_n * 2;
+    const u32x4 rq = make_rsrc(Q, (uint32_t)((N - 1) * qs2 + p.wqk * 2));
+    const u32x4 rk = make_rsrc(K, (uint32_t)((N - 1) * ks2 + p.wqk * 2));
+    const u32x4 rv = make_rsrc(V, (uint32_t)((N - 1) * vs2 + p.wv * 2));
+    const u32x4 rg = make_rsrc(G, (uint32_t)((N - 1) * gs2 + p.wv * 2));
+    const __amdgpu_buffer_rsrc_t rdq = __builtin_amdgcn_make_buffer_rsrc(DQ, 0, (N - 1) * dqs2 + p.wqk * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rdk = __builtin_amdgcn_make_buffer_rsrc(DK, 0, (N - 1) * dks2 + p.wqk * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rdv = __builtin_amdgcn_make_buffer_rsrc(DV, 0, (N - 1) * dvs2 + p.wv * 2, 0x00020000);
+
+    f32x16 st[W::NBW];  // R [q/k index][v index]
+    f32x16 xs[W::NBW];  // X [q/k index][v index]
+    walk_load_init<D, B>(p, sl, wave, lane, st);
+    walk_load_state<D, B>(sl.c_hi < p.n_chunks ? p.xinit + ((int64_t)sl.bh * p.n_seg + sl.seg + 1) * (D * D)
+                                               : p.xtotal + (int64_t)sl.bh * (D * D),
+                          false, wave, lane, xs);
+    walk_state_to_lds<T, D, B>(tl, wave, lane, st);
+
+    auto load_chunk = [&](int c, int buf) {
+        const uint32_t base = lds0 + buf * 4 * W::TILE;
+        const int row0 = c * W::C;
+        walk_load_tile<D>(rq, base, row0, qs2, p.wqk, wave, lane);
+        walk_load_tile<D>(rk, base + W::TILE, row0, ks2, p.wqk, wave, lane);
+        walk_load_tile<D>(rv, base + 2 * W::TILE, row0, vs2, p.wv, wave, lane);
+        walk_load_tile<D>(rg, base + 3 * W::TILE, row0, gs2, p.wv, wave, lane);
+    };
+    auto sync = [&]() {  // this wave's LDS accesses are done; then every wave's
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+    load_chunk(sl.c_hi - 1, 0);
+#pragma unroll 1
+    for (int c = sl.c_hi - 1; c >= sl.c_lo; --c) {
+        const int buf = (sl.c_hi - 1 - c) & 1;
+        unsigned char *tq = smem + buf * 4 * W::TILE, *tk = tq + W::TILE, *tv = tq + 2 * W::TILE, *tg = tq + 3 * W::TILE;
+        const bool more = c > sl.c_lo;
+        if (more) load_chunk(c - 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
+        // this wave's loads of chunk c have landed when at most the loads issued after them are
+        // outstanding (the stores of the previous chunk were issued before those)
+        if (more)
+            wait_vm<4 * W::NI>();
+        else
+            wait_vm<0>();
+        sync();  // the tiles have landed, R is in LDS
+        const int row = c * W::C + 32 * rb + l32;
+        const bool later = c + 1 < p.n_chunks;  // chunks after this one exist: R is not identically zero
+        walk_update<T, D, B, true, true>(tk, tv, wave, lane, xs);  // X: now the sum over the chunks before this one
+        f32x16 acc[W::DBW];
+        // dV = upper(K Q^T) dO + K R: A operand R^T[v index][q/k index] = the LDS copy as it is
+        walk_product<T, D, true>(tk, tq, tg, wave, lane, later, [&](int db, int kc) -> V8 {
+            return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g);
+        }, acc);
+        walk_store<T, D>(rdv, dvs2, p.wv, row, g, db0, acc);
+        // dK = upper(V dO^T) Q + V R^T: A operand R[q/k index][v index] = the LDS copy read transposed
+        walk_product<T, D, true>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
+            return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
+        }, acc);
+        walk_store<T, D>(rdk, dks2, p.wqk, row, g, db0, acc);
+        sync();  // every wave has read R
+        walk_state_to_lds<T, D, B>(tl, wave, lane, xs);
+        sync();  // X is in LDS
+        // dQ = lower(dO V^T) K + dO X^T: A operand X[q/k index][v index], read transposed like R for dK
+        walk_product<T, D, false>(tg, tv, tk, wave, lane, c > 0, [&](int db, int kc) -> V8 {
+            return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
+        }, acc);
+        walk_store<T, D>(rdq, dqs2, p.wqk, row, g, db0, acc);
+        walk_update<T, D, B, false, true>(tq, tg, wave, lane, st);
+        sync();  // every wave has read X and is done with the tiles
         walk_state_to_lds<T, D, B>(tl, wave, lane, st);
     }
 #else
@@ -1281,6 +1479,16 @@ hipError_t launch_walk_dkdv(const WalkParams &p, hipStream_t stream) {
     constexpr auto kern = walk_dkdv_kernel<T, D, false>;
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
     return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+}
+
+template <typename T, int D>
+hipError_t launch_walk_bwd_rev(const WalkParams &p, hipStream_t stream) {
+    const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
+    if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    if (!p.xtotal || (p.n_seg > 1 && !p.xinit)) return hipErrorInvalidValue;
+    constexpr int smem = 8 * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
+    static_assert(smem <= 160 * 1024, "two sets of tiles and the state must fit the LDS of a CU");
+    return launch_walk_kernel<walk_bwd_rev_kernel<T, D>>(grid, smem, p, stream);
 }
 
 }  // namespace fla

@@ -41,9 +41,10 @@ FLA_FOR_EACH_DIM_PAIR(FLA_DECLARE)
 FLA_DECLARE_BATCH(32) FLA_DECLARE_BATCH(64) FLA_DECLARE_BATCH(128) FLA_DECLARE_BATCH(256)
 #undef FLA_DECLARE_BATCH
 // walk kernels (fla_chunk_walk.h), dtype 0 bf16 / 1 f16, padded head dim D = 32, 64 or 128
-// (walk_bwd: 32 and 64; walk_dkdv: 128)
+// (walk_bwd: 32 and 64; walk_dkdv, walk_bwd_rev: 128)
 hipError_t walk_totals(int dtype, int D, const WalkTotalsParams &p, hipStream_t stream);
 hipError_t walk_fwd(int dtype, int D, const WalkParams &p, hipStream_t stream);
+hipError_t walk_bwd_rev(int dtype, int D, const WalkParams &p, hipStream_t stream);
 hipError_t walk_bwd(int dtype, int D, const WalkParams &p, hipStream_t stream);
 hipError_t walk_dkdv(int dtype, int D, const WalkParams &p, hipStream_t stream);
 hipError_t walk_vec_sums(int dtype, int D, const WalkVecParams &p, int64_t BH, hipStream_t stream);

@@ -109,6 +109,13 @@ struct Mma<__bf16> {
     static __device__ __forceinline__ f32x16 mma(V8 a, V8 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
     }
+    // c += a b with c held in accumulation registers throughout (a running sum that only MFMAs and
+    // an occasional read touch leaves the architectural registers to the rest of the kernel).  The
+    // s_nop covers a register copy the compiler may have placed right in front: it does not look
+    // inside the statement for the wait states such a copy needs before an MFMA reads its target.
+    static __device__ __forceinline__ void mma_acc(V8 a, V8 b, f32x16 &c) {
+        asm("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+    }
 };
 
 template <>
@@ -116,6 +123,9 @@ struct Mma<_Float16> {
     using V8 = f16x8;
     static __device__ __forceinline__ f32x16 mma(V8 a, V8 b, f32x16 c) {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ void mma_acc(V8 a, V8 b, f32x16 &c) {
+        asm("s_nop 1\n\tv_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
     }
 };
 

@@ -1,5 +1,6 @@
 // Instantiations of the walk kernels (fla_chunk_walk.h): both storage types, padded head dims 32, 64 and 128
-// (128: no fused backward -- dQ is a forward-direction walk, dK and dV a kernel of their own).
+// (128: backward is one reverse walk when forward handed its states over; otherwise, and with a feature map or
+// the normaliser, dQ is a forward-direction walk and dK, dV a kernel of their own).
 #include "fla_dispatch.h"
 
 namespace fla {
@@ -19,6 +20,10 @@ hipError_t walk_bwd(int dtype, int D, const WalkParams &p, hipStream_t stream) {
 hipError_t walk_dkdv(int dtype, int D, const WalkParams &p, hipStream_t stream) {
     if (D != 128) return hipErrorNotSupported;
     return dtype == 0 ? launch_walk_dkdv<__bf16, 128>(p, stream) : launch_walk_dkdv<_Float16, 128>(p, stream);
+}
+hipError_t walk_bwd_rev(int dtype, int D, const WalkParams &p, hipStream_t stream) {
+    if (D != 128) return hipErrorNotSupported;
+    return dtype == 0 ? launch_walk_bwd_rev<__bf16, 128>(p, stream) : launch_walk_bwd_rev<_Float16, 128>(p, stream);
 }
 hipError_t walk_totals(int dtype, int D, const WalkTotalsParams &p, hipStream_t stream) {
     FLA_WALK_DISPATCH3(launch_walk_totals, p, stream);

@@ -149,9 +149,9 @@ def test_chunked_operator_workspace_is_checked(gpu_device):
     sbytes = lib.fla_linear_attn_chunked_state_bytes(1, 2, 1024, 64, 64)
     # one 64 x 64 state per 128-row chunk and head, and an fp32 vector per chunk (the normalised operator's)
     assert need > 0 and sbytes == 2 * 8 * 64 * 64 * 2 + 2 * 8 * 64 * 4
-    # D = 128: the fp32 entry state of every segment (here single 64-row chunks), which is more than a
-    # 16-bit state per 256-row chunk
-    assert lib.fla_linear_attn_chunked_state_bytes(1, 2, 1024, 128, 128) == 2 * 16 * 128 * 128 * 4 + 2 * 16 * 128 * 4
+    # D = 128: the fp32 entry state of every segment (here single 64-row chunks) and the state after the
+    # last chunk, which is more than a 16-bit state per 256-row chunk
+    assert lib.fla_linear_attn_chunked_state_bytes(1, 2, 1024, 128, 128) == 2 * 17 * 128 * 128 * 4 + 2 * 16 * 128 * 4
     valid = ctypes.c_int32(7)
     rc = lib.fla_linear_attn_chunked_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), 1, 2, 1024, 64, 64,
                                          st(q), st(k), st(v), st(out), 0, None, ctypes.byref(valid), None, 0, stream)
