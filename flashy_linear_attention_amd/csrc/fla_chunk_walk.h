@@ -1119,6 +1119,9 @@ __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p
         }, acc);
         walk_store<T, D>(rdk, dks2, p.wqk, row, g, db0, acc);
         sync();  // every wave has read R
+        // (X stays in its accumulation registers up to here: without this the copies that the rounding
+        // below reads are made right after the update and occupy 64 registers through both products)
+        asm volatile("" : "+a"(xs[0]), "+a"(xs[1]), "+a"(xs[2]), "+a"(xs[3]));
         walk_state_to_lds<T, D, B>(tl, wave, lane, xs);
         sync();  // X is in LDS
         // dQ = lower(dO V^T) K + dO X^T: A operand X[q/k index][v index], read transposed like R for dK
