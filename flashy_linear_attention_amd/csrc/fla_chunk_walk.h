@@ -326,69 +326,98 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
     for (int i = 0; i < W::DBW; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
-    if (has_state) {  // (k chunk outer, output block inner: consecutive MFMAs are independent)
-        walk_pipe<PER * KCL, 4, V8>([&](auto j) { return sfrag(db0 + decltype(j)::value % PER, decltype(j)::value / PER); },
-                                    [&](auto j, V8 f) {
-                                        constexpr int I = decltype(j)::value % PER, KC_ = decltype(j)::value / PER;
-                                        acc[I] = M::mma(f, xf[KC_], acc[I]);
-                                    });
-    }
-    const int s_lo = UPPER ? rb : 0, s_hi = UPPER ? W::NRB - 1 : rb;
-#pragma unroll 1
-    for (int s = s_lo; s <= s_hi; ++s) {
+    // One 32-row block s of Y and Z: scores, mask and rounding, second product.  ST: the state product's
+    // MFMAs are issued in between -- PER / 2 of them after every score MFMA (they share its X fragment
+    // and fill the gaps of the dependent chain), the rest after the last one, where the rounding of the
+    // scores runs beneath them.  Operand fragments are read four ahead, in the order of their use.
+    auto block = [&](int s, auto with_state) {
+        constexpr bool ST = decltype(with_state)::value;
+        constexpr int H = ST ? PER / 2 : 0, GA = 1 + H, GB = PER - H;
+        constexpr int NA = KCL * GA, NB = ST ? GB * KCL : 0, NC = 2 * PER;
+        constexpr int CONV = NB > 2 ? NA + 2 : NA + NB;  // the scores are finished in front of this operation
         f32x16 sc;
 #pragma unroll
         for (int v = 0; v < 16; ++v) sc[v] = 0.f;
-        // fragments 0 .. KCL-1: Y rows for the scores; KCL .. KCL + 2 PER - 1: Z columns for the second
-        // product, requested while the last score MFMAs run
         V8 pf[2];
-        walk_pipe<KCL + 2 * PER, 4, V8>(
+        walk_pipe<NA + NB + NC, 4, V8>(
             [&](auto j) {
                 constexpr int J = decltype(j)::value;
-                if constexpr (J < KCL)
-                    return walk_row_frag<T, D>(yt, 32 * s + l32, J, g);
-                else
-                    return walk_col_frag_perm<T, D>(zt, 32 * s + 16 * ((J - KCL) / PER), db0 + (J - KCL) % PER, lane, false);
+                if constexpr (J < NA) {
+                    if constexpr (J % GA == 0)
+                        return walk_row_frag<T, D>(yt, 32 * s + l32, J / GA, g);
+                    else
+                        return sfrag(db0 + J % GA - 1, J / GA);
+                } else if constexpr (J < NA + NB) {
+                    return sfrag(db0 + H + (J - NA) % GB, (J - NA) / GB);
+                } else {
+                    return walk_col_frag_perm<T, D>(zt, 32 * s + 16 * ((J - NA - NB) / PER), db0 + (J - NA - NB) % PER, lane,
+                                                    false);
+                }
             },
             [&](auto j, V8 f) {
                 constexpr int J = decltype(j)::value;
-                if constexpr (J < KCL) {
-                    sc = M::mma(f, xf[J], sc);
-                } else {
-                    if constexpr (J == KCL) {  // the scores are complete: normaliser's terms, mask, rounding
-                        if constexpr (EX == 2) {
+                if constexpr (J == CONV) {  // normaliser's terms, mask, rounding
+                    if constexpr (EX == 2) {
 #pragma unroll
-                            for (int v = 0; v < 16; ++v) sc[v] += *ex;
-                        }
-                        if constexpr (EX == 3) {
-#pragma unroll
-                            for (int a = 0; a < 4; ++a) {
-                                const f32x4 y = yrows(s, a);
-#pragma unroll
-                                for (int b = 0; b < 4; ++b) sc[4 * a + b] += y[b];
-                            }
-                        }
-                        if (s == rb) {  // the 32 x 32 block on the diagonal: lane = X row l32, register v = Y row jl
-#pragma unroll
-                            for (int v = 0; v < 16; ++v) {
-                                const int jl = 8 * (v / 4) + 4 * g + (v % 4);
-                                const bool keep = UPPER ? l32 <= jl : l32 >= jl;
-                                sc[v] = keep ? sc[v] : 0.f;
-                            }
-                        }
-                        if constexpr (EX == 1) {
-#pragma unroll
-                            for (int v = 0; v < 16; ++v) rsum += sc[v];
-                        }
-#pragma unroll
-                        for (int t = 0; t < 2; ++t)
-#pragma unroll
-                            for (int e = 0; e < 8; ++e) pf[t][e] = static_cast<T>(sc[8 * t + e]);
+                        for (int v = 0; v < 16; ++v) sc[v] += *ex;
                     }
-                    constexpr int I = (J - KCL) % PER, TT = (J - KCL) / PER;
-                    acc[I] = M::mma(f, pf[TT], acc[I]);
+                    if constexpr (EX == 3) {
+#pragma unroll
+                        for (int a = 0; a < 4; ++a) {
+                            const f32x4 y = yrows(s, a);
+#pragma unroll
+                            for (int b = 0; b < 4; ++b) sc[4 * a + b] += y[b];
+                        }
+                    }
+                    if (s == rb) {  // the 32 x 32 block on the diagonal: lane = X row l32, register v = Y row jl
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int jl = 8 * (v / 4) + 4 * g + (v % 4);
+                            const bool keep = UPPER ? l32 <= jl : l32 >= jl;
+                            sc[v] = keep ? sc[v] : 0.f;
+                        }
+                    }
+                    if constexpr (EX == 1) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) rsum += sc[v];
+                    }
+#pragma unroll
+                    for (int t = 0; t < 2; ++t)
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) pf[t][e] = static_cast<T>(sc[8 * t + e]);
+                }
+                if constexpr (J < NA) {
+                    if constexpr (J % GA == 0)
+                        sc = M::mma(f, xf[J / GA], sc);
+                    else
+                        acc[J % GA - 1] = M::mma(f, xf[J / GA], acc[J % GA - 1]);
+                } else if constexpr (J < NA + NB) {
+                    acc[H + (J - NA) % GB] = M::mma(f, xf[(J - NA) / GB], acc[H + (J - NA) % GB]);
+                } else {
+                    acc[(J - NA - NB) % PER] = M::mma(f, pf[(J - NA - NB) / PER], acc[(J - NA - NB) % PER]);
                 }
             });
+    };
+    const int s_lo = UPPER ? rb : 0, s_hi = UPPER ? W::NRB - 1 : rb;
+    if constexpr (D == 128) {
+        if (has_state)
+            block(s_lo, std::true_type{});
+        else
+            block(s_lo, std::false_type{});
+#pragma unroll 1
+        for (int s = s_lo + 1; s <= s_hi; ++s) block(s, std::false_type{});
+    } else {
+        // (two workgroups per CU cover each other's gaps, and the fused backward has no registers to
+        // spare for the longer pipeline: the state product on its own, k chunk outer, output block inner)
+        if (has_state) {
+            walk_pipe<PER * KCL, 4, V8>([&](auto j) { return sfrag(db0 + decltype(j)::value % PER, decltype(j)::value / PER); },
+                                        [&](auto j, V8 f) {
+                                            constexpr int I = decltype(j)::value % PER, KC_ = decltype(j)::value / PER;
+                                            acc[I] = M::mma(f, xf[KC_], acc[I]);
+                                        });
+        }
+#pragma unroll 1
+        for (int s = s_lo; s <= s_hi; ++s) block(s, std::false_type{});
     }
     if constexpr (EX == 1) *ex = rsum + __shfl_xor(rsum, 32, 64);  // the two lanes of a row hold half the columns each
 }
