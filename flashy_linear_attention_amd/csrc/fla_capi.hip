@@ -501,7 +501,7 @@ int64_t state_core_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t d
     if (w.ok && !w.split) return w.saved_bytes;  // one state per 128-row chunk (also room for the 256-row chunks' states)
     if (!states_shareable(dqk, dv, N)) {
         const WidePlan wide = wide_plan(B, H, N, dqk, dv);
-        return wide.ok ? 2 * wide.wp.entry_bytes : w.ok ? w.saved_bytes : 0;
+        return wide.ok ? 2 * wide.wp.saved_bytes : w.ok ? w.saved_bytes : 0;
     }
     const int64_t rows = chunk_rows(dqk, dv);
     const int64_t per_chunk = B * H * ((N + rows - 1) / rows) * padded(dqk) * padded(dv) * 2;
@@ -565,11 +565,13 @@ int wide_forward(const WidePlan &wide, const View &q, const View &k, const View 
         const int64_t wqk = h == 0 ? 128 : dqk - 128;
         const float *entry = nullptr;
         if (wp.n_seg > 1) {
-            float *keep = state_out ? reinterpret_cast<float *>(static_cast<char *>(state_out) + h * wp.entry_bytes) : nullptr;
+            float *keep = state_out ? reinterpret_cast<float *>(static_cast<char *>(state_out) + h * wp.saved_bytes) : nullptr;
             void *work = keep && wp.m == 1 ? static_cast<void *>(keep) : static_cast<void *>(ws + wide.temp_bytes);
             if (int rc = walk_entry_states(wp, kh, v, B, H, N, wqk, dv, dtype, 0, work, keep, &entry, s)) return rc;
         }
-        const fla::WalkParams w = lower_walk_params(wp, qh, kh, v, h == 0 ? o : temp, B, H, N, wqk, dv, entry);
+        fla::WalkParams w = lower_walk_params(wp, qh, kh, v, h == 0 ? o : temp, B, H, N, wqk, dv, entry);
+        if (state_out)  // (behind this half's entry states: the state after the last chunk)
+            w.total_out = reinterpret_cast<float *>(static_cast<char *>(state_out) + h * wp.saved_bytes + wp.entry_bytes);
         if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
     }
     return launch_feature_pass(3, 0, temp, o, B, H, N, dv, dtype, s);
@@ -588,19 +590,39 @@ int wide_backward(const WidePlan &wide, const View &go, const View &q, const Vie
         const float *fwd_entry = nullptr, *entry = nullptr;
         if (wp.n_seg > 1) {
             if (state_in)
-                fwd_entry = reinterpret_cast<const float *>(static_cast<const char *>(state_in) + h * wp.entry_bytes);
+                fwd_entry = reinterpret_cast<const float *>(static_cast<const char *>(state_in) + h * wp.saved_bytes);
             else if (int rc = walk_entry_states(wp, kh, v, B, H, N, wqk, dv, dtype, 0, ws + wide.temp_bytes + wp.work_bytes,
                                                 nullptr, &fwd_entry, s))
                 return rc;
             if (int rc = walk_entry_states(wp, qh, go, B, H, N, wqk, dv, dtype, 1, ws + wide.temp_bytes, nullptr, &entry, s))
                 return rc;
         }
+        const View &dvh = h == 0 ? dvv : temp;
+        if (state_in) {  // forward's states at hand: dQ_h, dK_h and this half's part of dV in one reverse walk
+            fla::WalkParams r{};
+            r.q = qh.ptr, r.k = kh.ptr, r.v = v.ptr, r.go = go.ptr;
+            r.dq = const_cast<void *>(dqh.ptr), r.dk = const_cast<void *>(dkh.ptr), r.dv = const_cast<void *>(dvh.ptr);
+            r.qs_b = qh.strides[0], r.qs_h = qh.strides[1], r.qs_n = qh.strides[2];
+            r.ks_b = kh.strides[0], r.ks_h = kh.strides[1], r.ks_n = kh.strides[2];
+            r.vs_b = v.strides[0], r.vs_h = v.strides[1], r.vs_n = v.strides[2];
+            r.gs_b = go.strides[0], r.gs_h = go.strides[1], r.gs_n = go.strides[2];
+            r.dqs_b = dqh.strides[0], r.dqs_h = dqh.strides[1], r.dqs_n = dqh.strides[2];
+            r.dks_b = dkh.strides[0], r.dks_h = dkh.strides[1], r.dks_n = dkh.strides[2];
+            r.dvs_b = dvh.strides[0], r.dvs_h = dvh.strides[1], r.dvs_n = dvh.strides[2];
+            r.H = (int32_t)H, r.N = (int32_t)N, r.BH = (int32_t)(B * H), r.wqk = (int32_t)wqk, r.wv = (int32_t)dv;
+            r.n_chunks = (int32_t)wp.n_chunks, r.seg_chunks = (int32_t)wp.seg_chunks, r.n_seg = (int32_t)wp.n_seg;
+            r.init = entry;
+            const char *half = static_cast<const char *>(state_in) + h * wp.saved_bytes;
+            r.xinit = reinterpret_cast<const float *>(half);
+            r.xtotal = reinterpret_cast<const float *>(half + wp.entry_bytes);
+            if (fla::walk_bwd_rev(dtype, wp.D, r, s) != hipSuccess) return FLA_ERR_LAUNCH;
+            continue;
+        }
         // dQ_h = lower(dO V^T) K_h + dO S_h^T: the forward walk over (dO, V, K_h)
         fla::WalkParams w = lower_walk_params(wp, go, v, kh, dqh, B, H, N, dv, wqk, fwd_entry);
         w.init_transposed = 1;
         if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
         // dV (this half's part) and dK_h: the reverse walk
-        const View &dvh = h == 0 ? dvv : temp;
         fla::WalkParams r{};
         r.q = qh.ptr, r.k = kh.ptr, r.v = v.ptr, r.go = go.ptr;
         r.dk = const_cast<void *>(dkh.ptr), r.dv = const_cast<void *>(dvh.ptr);

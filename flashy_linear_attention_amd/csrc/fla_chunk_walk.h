@@ -543,8 +543,11 @@ __device__ __forceinline__ void walk_update(const unsigned char *yt, const unsig
             }
         });
     if constexpr (ACC) {
-        static_assert(!ACC || B::SLOTS == 4, "written for four blocks per wave");
-        asm volatile("s_nop 15\n\ts_nop 7" : "+a"(st[0]), "+a"(st[1]), "+a"(st[2]), "+a"(st[3]));
+        static_assert(!ACC || B::SLOTS == 4 || B::SLOTS == 2, "written for two or four blocks per wave");
+        if constexpr (B::SLOTS == 4)
+            asm volatile("s_nop 15\n\ts_nop 7" : "+a"(st[0]), "+a"(st[1]), "+a"(st[2]), "+a"(st[3]));
+        else
+            asm volatile("s_nop 15\n\ts_nop 7" : "+a"(st[0]), "+a"(st[1]));
     }
 }
 
@@ -802,6 +805,11 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
                 for (int v = 0; v < 16; ++v)
                     out[(32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * B::eb(wave) + l32] = st[i][v];
             }
+        // (built for a narrow q / k side: walk_bwd_rev_kernel has no such variant and reads every block)
+        if constexpr (NQ < W::DB) {
+            for (int e = tid; e < D * D; e += 256)
+                if (e / D >= 32 * NQ || e % D >= 32 * NV) out[e] = 0.f;
+        }
     }
 #else
     (void)p;
@@ -1064,19 +1072,20 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
 // The one 16-bit state in LDS holds R for dV and dK, then X for dQ.  q, k, v, dO are read once and
 // nothing but the results is written, where the walk for dQ followed by walk_dkdv_kernel reads
 // dO, v, k twice.
-template <typename T, int D>
+template <typename T, int D, int NQ = D / 32, int NV = D / 32>
 __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
     using V8 = typename Mma<T>::V8;
-    using B = WalkExt<D>;
-    using OB = WalkOut<D, W::DB>;
+    using B = WalkExt<D, NQ, NV>;   // R, X [q/k index][v index]
+    using OV = WalkOut<D, NV>;      // dV is as wide as v,
+    using OQ = WalkOut<D, NQ>;      // dK and dQ as q and k
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     unsigned char *tl = smem + 8 * W::TILE;
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int rb = W::NCH == 1 ? wave : wave % W::NRB, db0 = OB::db0(wave);
+    const int rb = W::NCH == 1 ? wave : wave % W::NRB;
     const WalkSlice sl = walk_slice(p);
     if (!sl.valid) return;
     const int b = sl.bh / p.H, h = sl.bh - b * p.H, N = p.N;
@@ -1138,26 +1147,29 @@ __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p
         walk_update<T, D, B, true, true>(tk, tv, wave, lane, xs);  // X: now the sum over the chunks before this one
         f32x16 acc[W::DBW];
         // dV = upper(K Q^T) dO + K R: A operand R^T[v index][q/k index] = the LDS copy as it is
-        walk_product<T, D, true>(tk, tq, tg, wave, lane, later, [&](int db, int kc) -> V8 {
+        walk_product<T, D, true, 0, B::KQ, NV>(tk, tq, tg, wave, lane, later, [&](int db, int kc) -> V8 {
             return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g);
         }, acc);
-        walk_store<T, D>(rdv, dvs2, p.wv, row, g, db0, acc);
+        walk_store<T, D, OV::PER>(rdv, dvs2, p.wv, row, g, OV::db0(wave), acc);
         // dK = upper(V dO^T) Q + V R^T: A operand R[q/k index][v index] = the LDS copy read transposed
-        walk_product<T, D, true>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
+        walk_product<T, D, true, 0, B::KV, NQ>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
             return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
         }, acc);
-        walk_store<T, D>(rdk, dks2, p.wqk, row, g, db0, acc);
+        walk_store<T, D, OQ::PER>(rdk, dks2, p.wqk, row, g, OQ::db0(wave), acc);
         sync();  // every wave has read R
         // (X stays in its accumulation registers up to here: without this the copies that the rounding
         // below reads are made right after the update and occupy 64 registers through both products)
-        asm volatile("" : "+a"(xs[0]), "+a"(xs[1]), "+a"(xs[2]), "+a"(xs[3]));
+        if constexpr (B::SLOTS == 4)
+            asm volatile("" : "+a"(xs[0]), "+a"(xs[1]), "+a"(xs[2]), "+a"(xs[3]));
+        else
+            asm volatile("" : "+a"(xs[0]), "+a"(xs[1]));
         walk_state_to_lds<T, D, B>(tl, wave, lane, xs);
         sync();  // X is in LDS
         // dQ = lower(dO V^T) K + dO X^T: A operand X[q/k index][v index], read transposed like R for dK
-        walk_product<T, D, false>(tg, tv, tk, wave, lane, c > 0, [&](int db, int kc) -> V8 {
+        walk_product<T, D, false, 0, B::KV, NQ>(tg, tv, tk, wave, lane, c > 0, [&](int db, int kc) -> V8 {
             return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
         }, acc);
-        walk_store<T, D>(rdq, dqs2, p.wqk, row, g, db0, acc);
+        walk_store<T, D, OQ::PER>(rdq, dqs2, p.wqk, row, g, OQ::db0(wave), acc);
         walk_update<T, D, B, false, true>(tq, tg, wave, lane, st);
         sync();  // every wave has read X and is done with the tiles
         walk_state_to_lds<T, D, B>(tl, wave, lane, st);
@@ -1520,6 +1532,9 @@ hipError_t launch_walk_bwd_rev(const WalkParams &p, hipStream_t stream) {
     if (!p.xtotal || (p.n_seg > 1 && !p.xinit)) return hipErrorInvalidValue;
     constexpr int smem = 8 * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
     static_assert(smem <= 160 * 1024, "two sets of tiles and the state must fit the LDS of a CU");
+    if constexpr (D == 128) {  // a half of a wide q / k against a narrow v: without the blocks of padding
+        if (p.wqk > 64 && p.wv <= 64) return launch_walk_kernel<walk_bwd_rev_kernel<T, D, 4, 2>>(grid, smem, p, stream);
+    }
     return launch_walk_kernel<walk_bwd_rev_kernel<T, D>>(grid, smem, p, stream);
 }
 

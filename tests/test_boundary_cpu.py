@@ -215,8 +215,9 @@ def test_chunkwise_state_and_workspace_sizes():
     # state after the last chunk); ten 256-row chunks are less
     assert sb(2, 8, 2450, 128, 128) == 16 * 21 * 128 * 128 * 4 + 16 * 39 * 128 * 4
     assert sb(1, 1, 300, 32, 32) == 3 * 32 * 32 * 2 + 3 * 32 * 4
-    # D_qk = 256, D_v = 64: the fp32 entry states of both 128-column halves, 4 walk segments per (b, h)
-    assert sb(4, 16, 4096, 256, 64) == 2 * 64 * 4 * 128 * 128 * 4
+    # D_qk = 256, D_v = 64: the fp32 entry states of both 128-column halves, 4 walk segments per (b, h), and their
+    # states after the last chunk
+    assert sb(4, 16, 4096, 256, 64) == 2 * 64 * 5 * 128 * 128 * 4
     # nothing to hand over: a value head dim wider than the query / key one, a single chunk
     assert sb(4, 16, 4096, 64, 256) == 0 and sb(1, 2, 256, 128, 128) == 0 and sb(1, 2, 128, 64, 64) == 0
     ws = lib.fla_linear_attn_chunked_workspace_bytes

@@ -196,8 +196,8 @@ def test_chunked_on_strided_operands(dims, gpu_device):
 
 
 def test_chunked_small_v_state_hand_over(gpu_device):
-    """D_qk = 256, D_v = 64: forward hands both halves' entry states to backward; backward without
-    them recomputes; both match the oracle."""
+    """D_qk = 256, D_v = 64: forward hands both halves' states to backward; backward without them
+    recomputes the entry states and takes the two-walk path; both match the oracle."""
     from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
 
     q, k, v, dy = (t.to(gpu_device) for t in reference_style_inputs(2, 8, 4200, 256, 64, torch.bfloat16, seed=41))
@@ -207,6 +207,7 @@ def test_chunked_small_v_state_hand_over(gpu_device):
     want = naive.causal_dot_product_grads(q.float().cpu(), k.float().cpu(), v.float().cpu(), dy.float().cpu())
     with_state = linear_attention_chunked_bwd(dy, q, k, v, state)
     without = linear_attention_chunked_bwd(dy, q, k, v, None)
+    # (with the states: one reverse walk per half; without: dQ's forward-direction walk and the dK / dV walk)
     for name, a, b, w in zip(("dQ", "dK", "dV"), with_state, without, want):
-        assert torch.equal(a, b), f"{name}: recomputed entry states give different gradients"
         assert_close(name, a, w)
+        assert_close(name + " (no saved state)", b, w)
