@@ -558,8 +558,6 @@ int wide_forward(const WidePlan &wide, const View &q, const View &k, const View 
                  int64_t N, int64_t dqk, int64_t dv, int dtype, void *state_out, void *workspace, hipStream_t s) {
     const WalkPlan &wp = wide.wp;
     char *ws = static_cast<char *>(workspace);
-    const int64_t temp_strides[4] = {H * N * dv, N * dv, dv, 1};
-    const View temp{ws, temp_strides};
     for (int h = 0; h < 2; ++h) {
         const View qh = column_half(q, h), kh = column_half(k, h);
         const int64_t wqk = h == 0 ? 128 : dqk - 128;
@@ -569,12 +567,14 @@ int wide_forward(const WidePlan &wide, const View &q, const View &k, const View 
             void *work = keep && wp.m == 1 ? static_cast<void *>(keep) : static_cast<void *>(ws + wide.temp_bytes);
             if (int rc = walk_entry_states(wp, kh, v, B, H, N, wqk, dv, dtype, 0, work, keep, &entry, s)) return rc;
         }
-        fla::WalkParams w = lower_walk_params(wp, qh, kh, v, h == 0 ? o : temp, B, H, N, wqk, dv, entry);
+        // (the second half's walk adds its result to the first one's)
+        fla::WalkParams w = lower_walk_params(wp, qh, kh, v, o, B, H, N, wqk, dv, entry);
+        w.accumulate = h;
         if (state_out)  // (behind this half's entry states: the state after the last chunk)
             w.total_out = reinterpret_cast<float *>(static_cast<char *>(state_out) + h * wp.saved_bytes + wp.entry_bytes);
         if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
     }
-    return launch_feature_pass(3, 0, temp, o, B, H, N, dv, dtype, s);
+    return FLA_OK;
 }
 
 int wide_backward(const WidePlan &wide, const View &go, const View &q, const View &k, const View &v, const View &dq,
@@ -601,14 +601,15 @@ int wide_backward(const WidePlan &wide, const View &go, const View &q, const Vie
         if (state_in) {  // forward's states at hand: dQ_h, dK_h and this half's part of dV in one reverse walk
             fla::WalkParams r{};
             r.q = qh.ptr, r.k = kh.ptr, r.v = v.ptr, r.go = go.ptr;
-            r.dq = const_cast<void *>(dqh.ptr), r.dk = const_cast<void *>(dkh.ptr), r.dv = const_cast<void *>(dvh.ptr);
+            r.dq = const_cast<void *>(dqh.ptr), r.dk = const_cast<void *>(dkh.ptr), r.dv = const_cast<void *>(dvv.ptr);
+            r.accumulate = h;  // (the second half's walk adds its part of dV to the first one's)
             r.qs_b = qh.strides[0], r.qs_h = qh.strides[1], r.qs_n = qh.strides[2];
             r.ks_b = kh.strides[0], r.ks_h = kh.strides[1], r.ks_n = kh.strides[2];
             r.vs_b = v.strides[0], r.vs_h = v.strides[1], r.vs_n = v.strides[2];
             r.gs_b = go.strides[0], r.gs_h = go.strides[1], r.gs_n = go.strides[2];
             r.dqs_b = dqh.strides[0], r.dqs_h = dqh.strides[1], r.dqs_n = dqh.strides[2];
             r.dks_b = dkh.strides[0], r.dks_h = dkh.strides[1], r.dks_n = dkh.strides[2];
-            r.dvs_b = dvh.strides[0], r.dvs_h = dvh.strides[1], r.dvs_n = dvh.strides[2];
+            r.dvs_b = dvv.strides[0], r.dvs_h = dvv.strides[1], r.dvs_n = dvv.strides[2];
             r.H = (int32_t)H, r.N = (int32_t)N, r.BH = (int32_t)(B * H), r.wqk = (int32_t)wqk, r.wv = (int32_t)dv;
             r.n_chunks = (int32_t)wp.n_chunks, r.seg_chunks = (int32_t)wp.seg_chunks, r.n_seg = (int32_t)wp.n_seg;
             r.init = entry;
@@ -637,7 +638,7 @@ int wide_backward(const WidePlan &wide, const View &go, const View &q, const Vie
         r.init = entry;
         if (fla::walk_dkdv(dtype, wp.D, r, s) != hipSuccess) return FLA_ERR_LAUNCH;
     }
-    return launch_feature_pass(3, 0, temp, dvv, B, H, N, dv, dtype, s);
+    return state_in ? FLA_OK : launch_feature_pass(3, 0, temp, dvv, B, H, N, dv, dtype, s);
 }
 
 // fmap != 0 (feature_forward below): q and k hold the arguments xq, xk of the feature map phi, and

@@ -102,6 +102,9 @@ struct WalkParams {
     // states (xinit, the layout of `init`, not transposed; may be null with a single segment).
     float *total_out;
     const float *xinit, *xtotal;
+    // D = 128, plain: the result (forward: o; walk_bwd_rev_kernel: dv) is added to what its place in
+    // memory holds already -- the second of two walks whose results sum up (halves of a wide q / k)
+    int32_t accumulate;
 };
 
 template <int D>
@@ -498,6 +501,37 @@ __device__ __forceinline__ void walk_store(__amdgpu_buffer_rsrc_t rs, int stride
     walk_store_packed<D, PER>(rs, stride2, width, row, g, db0, pk);
 }
 
+// What a result's place in memory holds before the walk adds to it: this lane's 16-byte pieces of the
+// row it will store (the pieces of walk_store_packed).  Ordinary loads, requested once a chunk's tiles
+// have been awaited and used at the end of the chunk: the wait the compiler puts in front of the use
+// also covers the tile loads of the next chunk, issued before the request -- by then they have had
+// the whole chunk's time to land.
+template <typename T, int D, int PER>
+struct WalkPrev {
+    u32x4 val[PER][2];
+    __device__ __forceinline__ void request(__amdgpu_buffer_rsrc_t rs, int stride2, int width, int row, int g, int db0) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+#pragma unroll
+            for (int hq = 0; hq < 2; ++hq) {
+                const int col = 32 * (db0 + i) + 16 * g + 8 * hq;
+                const uint32_t off = (uint32_t)(row * stride2 + col * 2) + (col < width ? 0u : kOobOffset);
+                val[i][hq] = __builtin_amdgcn_raw_buffer_load_b128(rs, off, 0, 0);
+            }
+    }
+    __device__ __forceinline__ void add_to(f32x16 (&acc)[WalkCfg<D>::DBW]) const {
+        typedef T v8 __attribute__((ext_vector_type(8)));
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+#pragma unroll
+            for (int hq = 0; hq < 2; ++hq) {
+                const v8 y = __builtin_bit_cast(v8, val[i][hq]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[i][8 * hq + e] += static_cast<float>(y[e]);
+            }
+    }
+};
+
 // state += Y^T Z over the rows of the tiles, this wave's 32 x 32 blocks (block i: Y columns of block
 // dbk(i), Z columns of block eb): st[i][v] = State[32 dbk(i) + 8(v/4) + 4g + v%4][32 eb + l32]
 // (NEG: state -= Y^T Z -- the sign bits of the Z fragments are flipped.  ACC: the state lives in
@@ -649,7 +683,7 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
 // NORM: the instantiations that take the normaliser's terms: 1 forward (WalkParams::denom), 2 dQ (dn).
 // FM: the instantiations that know of feature maps (WalkParams::fmap, slope_y); the others ignore both.
 // NQ, NV: blocks of the state [q/k index][v index] that hold anything (WalkExt).
-template <typename T, int D, bool DOUBLE, int NORM, bool FM, int NQ = D / 32, int NV = D / 32>
+template <typename T, int D, bool DOUBLE, int NORM, bool FM, int NQ = D / 32, int NV = D / 32, bool ACCUM = false>
 __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
@@ -657,6 +691,7 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
     using B = WalkExt<D, NQ, NV>;
     using OB = WalkOut<D, NV>;  // the result is as wide as v
     static_assert(NORM == 0 || (NQ == W::DB && NV == W::DB), "the normaliser's variants are built for full widths");
+    static_assert(!ACCUM || (DOUBLE && NORM == 0 && !FM), "adding to the result: the plain D = 128 walk only");
     constexpr int SETS = DOUBLE ? 2 : 1;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
@@ -696,6 +731,8 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
         }
     };
     constexpr int n_extra = NORM == 0 ? 0 : NORM == 1 ? 1 : 1 + W::NID;  // loads per chunk and wave beyond the tiles
+    // ACCUM: the result is added to what o holds (in fp32, before the one rounding)
+    WalkPrev<T, D, OB::PER> prev;
     if constexpr (DOUBLE) load_chunk(sl.c_lo, 0);
 #pragma unroll 1
     for (int c = sl.c_lo; c < sl.c_hi; ++c) {
@@ -746,6 +783,7 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
                 __syncthreads();
             }
         }
+        if constexpr (ACCUM) prev.request(ro, os2, p.wv, row, g, db0);
         f32x16 acc[W::DBW];
         const float *vz = reinterpret_cast<const float *>(xv + buf * W::VEC);
         const float *vd = reinterpret_cast<const float *>(xv + buf * W::VEC + 2048);
@@ -773,6 +811,7 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
                 for (int v = 0; v < 16; ++v)
                     acc[i][v] *= feature_slope_from_value(fmap, static_cast<float>(ys[i][v / 8][v % 8]));
         }
+        if constexpr (ACCUM) prev.add_to(acc);
         walk_store<T, D, OB::PER>(ro, os2, p.wv, row, g, db0, acc);
         if (!DOUBLE && p.saved) {  // the state at the entry of this chunk, [q/k index][v index], for backward's dQ
             T *sv = static_cast<T *>(p.saved) + ((int64_t)sl.bh * p.n_chunks + c) * (D * D);
@@ -1072,7 +1111,7 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
 // The one 16-bit state in LDS holds R for dV and dK, then X for dQ.  q, k, v, dO are read once and
 // nothing but the results is written, where the walk for dQ followed by walk_dkdv_kernel reads
 // dO, v, k twice.
-template <typename T, int D, int NQ = D / 32, int NV = D / 32>
+template <typename T, int D, int NQ = D / 32, int NV = D / 32, bool ACCUM = false>
 __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
@@ -1128,6 +1167,8 @@ __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
     };
+    // ACCUM: dV is added to what dv holds (in fp32, before the one rounding)
+    WalkPrev<T, D, OV::PER> prev;
     load_chunk(sl.c_hi - 1, 0);
 #pragma unroll 1
     for (int c = sl.c_hi - 1; c >= sl.c_lo; --c) {
@@ -1144,13 +1185,20 @@ __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p
         sync();  // the tiles have landed, R is in LDS
         const int row = c * W::C + 32 * rb + l32;
         const bool later = c + 1 < p.n_chunks;  // chunks after this one exist: R is not identically zero
+        if constexpr (ACCUM) prev.request(rdv, dvs2, p.wv, row, g, OV::db0(wave));
         walk_update<T, D, B, true, true>(tk, tv, wave, lane, xs);  // X: now the sum over the chunks before this one
         f32x16 acc[W::DBW];
         // dV = upper(K Q^T) dO + K R: A operand R^T[v index][q/k index] = the LDS copy as it is
         walk_product<T, D, true, 0, B::KQ, NV>(tk, tq, tg, wave, lane, later, [&](int db, int kc) -> V8 {
             return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g);
         }, acc);
-        walk_store<T, D, OV::PER>(rdv, dvs2, p.wv, row, g, OV::db0(wave), acc);
+        f32x16 held[W::DBW];  // ACCUM: dV waits for the end of the chunk (see WalkPrev)
+        if constexpr (ACCUM) {
+#pragma unroll
+            for (int i = 0; i < OV::PER; ++i) held[i] = acc[i];
+        } else {
+            walk_store<T, D, OV::PER>(rdv, dvs2, p.wv, row, g, OV::db0(wave), acc);
+        }
         // dK = upper(V dO^T) Q + V R^T: A operand R[q/k index][v index] = the LDS copy read transposed
         walk_product<T, D, true, 0, B::KV, NQ>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
             return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
@@ -1170,6 +1218,10 @@ __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p
             return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
         }, acc);
         walk_store<T, D, OQ::PER>(rdq, dqs2, p.wqk, row, g, OQ::db0(wave), acc);
+        if constexpr (ACCUM) {
+            prev.add_to(held);
+            walk_store<T, D, OV::PER>(rdv, dvs2, p.wv, row, g, OV::db0(wave), held);
+        }
         walk_update<T, D, B, false, true>(tq, tg, wave, lane, st);
         sync();  // every wave has read X and is done with the tiles
         walk_state_to_lds<T, D, B>(tl, wave, lane, st);
@@ -1464,7 +1516,7 @@ hipError_t launch_walk_fwd(const WalkParams &p, hipStream_t stream) {
     constexpr int smem = (kDouble ? 6 : 3) * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
     const bool fm = p.fmap || p.slope_y;
     if (p.denom || p.dn) {  // the normaliser's terms: its vectors live behind the state
-        if (!p.zc) return hipErrorInvalidValue;
+        if (!p.zc || p.accumulate) return hipErrorInvalidValue;
         constexpr int smem_n = smem + (kDouble ? 2 : 1) * WalkCfg<D>::VEC;
         if (p.denom)
             return fm ? launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 1, true>>(grid, smem_n, p, stream)
@@ -1472,15 +1524,19 @@ hipError_t launch_walk_fwd(const WalkParams &p, hipStream_t stream) {
         return fm ? launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 2, true>>(grid, smem_n, p, stream)
                   : launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 2, false>>(grid, smem_n, p, stream);
     }
-    if (fm) return launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, true>>(grid, smem, p, stream);
+    if (fm) return p.accumulate ? hipErrorNotSupported : launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, true>>(grid, smem, p, stream);
     if constexpr (D == 128) {
         // operands of at most 64 true columns on one side (the halves of a wide q / k against a narrow v):
         // the kernels that leave out the blocks of padding
         if (p.wqk > 64 && p.wv <= 64)
-            return launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, false, 4, 2>>(grid, smem, p, stream);
+            return p.accumulate ? launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, false, 4, 2, true>>(grid, smem, p, stream)
+                                : launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, false, 4, 2>>(grid, smem, p, stream);
         if (p.wqk <= 64 && p.wv > 64)
-            return launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, false, 2, 4>>(grid, smem, p, stream);
+            return p.accumulate ? launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, false, 2, 4, true>>(grid, smem, p, stream)
+                                : launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, false, 2, 4>>(grid, smem, p, stream);
+        if (p.accumulate) return launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, false, 4, 4, true>>(grid, smem, p, stream);
     }
+    if (p.accumulate) return hipErrorNotSupported;
     return launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, false>>(grid, smem, p, stream);
 }
 
@@ -1533,8 +1589,11 @@ hipError_t launch_walk_bwd_rev(const WalkParams &p, hipStream_t stream) {
     constexpr int smem = 8 * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
     static_assert(smem <= 160 * 1024, "two sets of tiles and the state must fit the LDS of a CU");
     if constexpr (D == 128) {  // a half of a wide q / k against a narrow v: without the blocks of padding
-        if (p.wqk > 64 && p.wv <= 64) return launch_walk_kernel<walk_bwd_rev_kernel<T, D, 4, 2>>(grid, smem, p, stream);
+        if (p.wqk > 64 && p.wv <= 64)
+            return p.accumulate ? launch_walk_kernel<walk_bwd_rev_kernel<T, D, 4, 2, true>>(grid, smem, p, stream)
+                                : launch_walk_kernel<walk_bwd_rev_kernel<T, D, 4, 2>>(grid, smem, p, stream);
     }
+    if (p.accumulate) return launch_walk_kernel<walk_bwd_rev_kernel<T, D, D / 32, D / 32, true>>(grid, smem, p, stream);
     return launch_walk_kernel<walk_bwd_rev_kernel<T, D>>(grid, smem, p, stream);
 }
 
