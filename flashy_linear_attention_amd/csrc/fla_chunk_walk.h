@@ -968,9 +968,9 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
 // one is multiplied.  (dQ is a walk_fwd_kernel launch over dO, V, K.)
 // NORM: dK with the normaliser's terms (scores + dn_i, i the dO row; result + rc).  Tiles and state
 // fill the LDS at D = 128, so the chunk's dn and this wave's columns of rc travel in registers: a
-// lane loads one value of each, a chunk ahead and after the tiles' loads, and the values are
-// handed round within the wave (ds_bpermute: 64 per chunk, about 30 clocks each -- 28 us of a 207 us
-// launch at B H = 128, N = 4096) when the chunk's turn comes.
+// lane loads one value of each, a chunk ahead, and the values are handed round within the wave
+// (ds_bpermute: 64 per chunk, about 30 clocks each -- 28 us of a 207 us launch at B H = 128,
+// N = 4096) when the chunk's turn comes.
 template <typename T, int D, bool NORM, int NQ = D / 32, int NV = D / 32>
 __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -1017,21 +1017,21 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
         walk_load_tile<D>(rg, base + 3 * W::TILE, row0, gs2, p.wv, wave, lane);
     };
     static_assert(!NORM || W::C == 64, "one dn value per lane covers a chunk of 64 rows");
-    // The two loads go out as inline assembly, like the tiles': a load the compiler knows of would be
-    // awaited with vmcnt(0) at its first use (loads and stores may complete out of order among each
-    // other, so it cannot count past the stores issued in between), and the previous chunk's stores
-    // with it.  Here the values are needed after the wait for the tiles, which covers every older load.
+    // Ordinary loads, requested a chunk ahead (once the tiles of the chunk before have been awaited) and
+    // read at the top of their chunk, BEFORE the next tile loads go out: the wait the compiler puts
+    // in front of the first use is one for every outstanding load and store (it cannot count past
+    // stores), and at that point nothing is in flight that the walk would not wait for anyway but the
+    // previous chunk's stores, issued two products earlier.
     float nxt_dn = 0.f, nxt_rc = 0.f;
-    u32x4 rs_dn = {0u, 0u, 0u, 0u}, rs_rc = {0u, 0u, 0u, 0u};
-    if constexpr (NORM) {
-        rs_dn = walk_uniform_rsrc(p.dn + (int64_t)sl.bh * N, (uint32_t)N * 4);  // (rows past the end read as zero)
-        rs_rc = walk_uniform_rsrc(p.rc + (int64_t)sl.bh * p.n_chunks * D, (uint32_t)p.n_chunks * D * 4);
-    }
+    // (rows past the end read as zero; without the normaliser the two descriptors are never used)
+    const __amdgpu_buffer_rsrc_t rs_dn =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(NORM ? p.dn + (int64_t)sl.bh * N : nullptr), 0, NORM ? N * 4 : 0, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rs_rc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float *>(NORM ? p.rc + (int64_t)sl.bh * p.n_chunks * D : nullptr), 0, NORM ? p.n_chunks * D * 4 : 0, 0x00020000);
     auto load_vecs = [&](int c) {  // lane l: dn of row l of chunk c, rc of column 32 db0 + l
         if constexpr (NORM) {
-            const uint32_t off_dn = (uint32_t)(c * W::C + lane) * 4, off_rc = (uint32_t)(c * D + 32 * db0 + lane) * 4;
-            asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "+v"(nxt_dn) : "v"(off_dn), "s"(rs_dn) : "memory");
-            asm volatile("buffer_load_dword %0, %1, %2, 0 offen" : "+v"(nxt_rc) : "v"(off_rc), "s"(rs_rc) : "memory");
+            nxt_dn = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_dn, (c * W::C + lane) * 4, 0, 0));
+            nxt_rc = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rs_rc, (c * D + 32 * db0 + lane) * 4, 0, 0));
         }
     };
     load_chunk(sl.c_hi - 1, 0);
@@ -1041,19 +1041,11 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
         const int buf = (sl.c_hi - 1 - c) & 1;
         unsigned char *tq = smem + buf * 4 * W::TILE, *tk = tq + W::TILE, *tv = tq + 2 * W::TILE, *tg = tq + 3 * W::TILE;
         const bool more = c > sl.c_lo;
-        if (more) load_chunk(c - 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
-        // this wave's loads of chunk c have landed when at most the loads issued after them are
-        // outstanding (the stores of the previous chunk were issued before those)
-        if (more)
-            wait_vm<4 * W::NI>();
-        else
-            wait_vm<0>();
         // this chunk's vectors, from the lanes that loaded them: dnv[a][b] = dn of tile row 8 a + 4 g + b,
-        // rcv[i][v] = rc of column 32 (db0 + i) + 16 g + v; then the next chunk's loads
+        // rcv[i][v] = rc of column 32 (db0 + i) + 16 g + v
         f32x4 dnv[8];
         f32x16 rcv[W::DBW];
         if constexpr (NORM) {
-            asm volatile("" : "+v"(nxt_dn), "+v"(nxt_rc));  // (the values as they are after the wait)
 #pragma unroll
             for (int a8 = 0; a8 < 8; ++a8)
 #pragma unroll
@@ -1062,7 +1054,16 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
             for (int i = 0; i < W::DBW; ++i)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) rcv[i][v] = __shfl(nxt_rc, 32 * i + 16 * g + v, 64);
-            asm volatile("" ::"v"(dnv[7]), "v"(rcv[W::DBW - 1]));  // (handed round before the registers are loaded again)
+            asm volatile("" ::"v"(dnv[7]), "v"(rcv[W::DBW - 1]) : "memory");  // (handed round before the tile loads below)
+        }
+        if (more) load_chunk(c - 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
+        // this wave's loads of chunk c have landed when at most the loads issued after them are
+        // outstanding (the stores of the previous chunk were issued before those)
+        if (more)
+            wait_vm<4 * W::NI>();
+        else
+            wait_vm<0>();
+        if constexpr (NORM) {
             if (more) load_vecs(c - 1);
         }
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): this wave's part of the state is in LDS
