@@ -796,8 +796,8 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         if (state_in && reinterpret_cast<uintptr_t>(state_in) % 16 != 0) return FLA_ERR_WORKSPACE;
         hipStream_t s = static_cast<hipStream_t>(stream);
         const float *entry = nullptr;
-        // with forward's states at hand (and neither a feature map nor the normaliser): one reverse walk
-        const bool one_walk = state_in && !fmap && !nx;
+        // with forward's states at hand (and without the normaliser): one reverse walk
+        const bool one_walk = state_in && !nx;
         if (wp.n_seg > 1) {
             if (!state_in) {
                 const float *fwd_entry = nullptr;
@@ -829,7 +829,7 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
             r.dvs_b = dvv.strides[0], r.dvs_h = dvv.strides[1], r.dvs_n = dvv.strides[2];
             r.H = (int32_t)H, r.N = (int32_t)N, r.BH = (int32_t)(B * H), r.wqk = (int32_t)dqk, r.wv = (int32_t)dv;
             r.n_chunks = (int32_t)wp.n_chunks, r.seg_chunks = (int32_t)wp.seg_chunks, r.n_seg = (int32_t)wp.n_seg;
-            r.init = entry;
+            r.init = entry, r.fmap = fmap;  // (dQ, dK: the slopes from phi(xq), phi(xk) in the Q and K tiles)
             r.xinit = static_cast<const float *>(state_in);
             r.xtotal = reinterpret_cast<const float *>(static_cast<const char *>(state_in) + wp.entry_bytes);
             return fla::walk_bwd_rev(dtype, wp.D, r, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;

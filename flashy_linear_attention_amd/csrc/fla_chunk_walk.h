@@ -1112,7 +1112,7 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
 // The one 16-bit state in LDS holds R for dV and dK, then X for dQ.  q, k, v, dO are read once and
 // nothing but the results is written, where the walk for dQ followed by walk_dkdv_kernel reads
 // dO, v, k twice.
-template <typename T, int D, int NQ = D / 32, int NV = D / 32, bool ACCUM = false>
+template <typename T, int D, int NQ = D / 32, int NV = D / 32, bool ACCUM = false, bool FM = false>
 __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
@@ -1128,6 +1128,8 @@ __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p
     const int rb = W::NCH == 1 ? wave : wave % W::NRB;
     const WalkSlice sl = walk_slice(p);
     if (!sl.valid) return;
+    // FM: q and k hold y = phi(x); dQ and dK leave multiplied by the slope of phi, computed from the tiles
+    const int fmap = FM ? p.fmap : 0;
     const int b = sl.bh / p.H, h = sl.bh - b * p.H, N = p.N;
     const T *Q = static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h;
     const T *K = static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h;
@@ -1204,7 +1206,7 @@ __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p
         walk_product<T, D, true, 0, B::KV, NQ>(tv, tg, tq, wave, lane, later, [&](int db, int kc) -> V8 {
             return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
         }, acc);
-        walk_store<T, D, OQ::PER>(rdk, dks2, p.wqk, row, g, OQ::db0(wave), acc);
+        walk_store<T, D, OQ::PER>(rdk, dks2, p.wqk, row, g, OQ::db0(wave), acc, fmap, tk, 32 * rb + l32);
         sync();  // every wave has read R
         // (X stays in its accumulation registers up to here: without this the copies that the rounding
         // below reads are made right after the update and occupy 64 registers through both products)
@@ -1218,7 +1220,7 @@ __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p
         walk_product<T, D, false, 0, B::KV, NQ>(tg, tv, tk, wave, lane, c > 0, [&](int db, int kc) -> V8 {
             return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
         }, acc);
-        walk_store<T, D, OQ::PER>(rdq, dqs2, p.wqk, row, g, OQ::db0(wave), acc);
+        walk_store<T, D, OQ::PER>(rdq, dqs2, p.wqk, row, g, OQ::db0(wave), acc, fmap, tq, 32 * rb + l32);
         if constexpr (ACCUM) {
             prev.add_to(held);
             walk_store<T, D, OV::PER>(rdv, dvs2, p.wv, row, g, OV::db0(wave), held);
@@ -1590,9 +1592,13 @@ hipError_t launch_walk_bwd_rev(const WalkParams &p, hipStream_t stream) {
     constexpr int smem = 8 * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
     static_assert(smem <= 160 * 1024, "two sets of tiles and the state must fit the LDS of a CU");
     if constexpr (D == 128) {  // a half of a wide q / k against a narrow v: without the blocks of padding
-        if (p.wqk > 64 && p.wv <= 64)
+        if (!p.fmap && p.wqk > 64 && p.wv <= 64)
             return p.accumulate ? launch_walk_kernel<walk_bwd_rev_kernel<T, D, 4, 2, true>>(grid, smem, p, stream)
                                 : launch_walk_kernel<walk_bwd_rev_kernel<T, D, 4, 2>>(grid, smem, p, stream);
+    }
+    if (p.fmap) {
+        if (p.accumulate) return hipErrorNotSupported;
+        return launch_walk_kernel<walk_bwd_rev_kernel<T, D, D / 32, D / 32, false, true>>(grid, smem, p, stream);
     }
     if (p.accumulate) return launch_walk_kernel<walk_bwd_rev_kernel<T, D, D / 32, D / 32, true>>(grid, smem, p, stream);
     return launch_walk_kernel<walk_bwd_rev_kernel<T, D>>(grid, smem, p, stream);
