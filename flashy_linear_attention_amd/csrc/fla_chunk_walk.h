@@ -432,16 +432,18 @@ template <typename T, int D>
 __device__ __forceinline__ void walk_map_tile(unsigned char *tile, int fmap, int row0, int N, int width, T *out,
                                               int64_t out_stride, int tid) {
     using W = WalkCfg<D>;
+    feature_dispatch(fmap, [&](auto map) {
 #pragma unroll
-    for (int v = 0; v < W::C * W::CR / 256; ++v) {
-        const int u = tid + 256 * v, r = u / W::CR, pos = u % W::CR, c = pos ^ swizzle_y<W::CR>(r);
-        if (row0 + r < N && c * 8 < width) {
-            u32x4 *ptr = reinterpret_cast<u32x4 *>(tile + r * W::RB + (pos << 4));
-            const u32x4 m = feature_map8<T>(fmap, *ptr);
-            *ptr = m;
-            *reinterpret_cast<u32x4 *>(out + (int64_t)(row0 + r) * out_stride + c * 8) = m;
+        for (int v = 0; v < W::C * W::CR / 256; ++v) {
+            const int u = tid + 256 * v, r = u / W::CR, pos = u % W::CR, c = pos ^ swizzle_y<W::CR>(r);
+            if (row0 + r < N && c * 8 < width) {
+                u32x4 *ptr = reinterpret_cast<u32x4 *>(tile + r * W::RB + (pos << 4));
+                const u32x4 m = feature_map8_c<T, decltype(map)::value>(*ptr);
+                *ptr = m;
+                *reinterpret_cast<u32x4 *>(out + (int64_t)(row0 + r) * out_stride + c * 8) = m;
+            }
         }
-    }
+    });
 }
 
 // acc[i][v] = Out[row][32 (db0 + i) + 16 g + v] rounded to the storage type: pk[i][hq] = columns
@@ -454,23 +456,27 @@ __device__ __forceinline__ void walk_pack(const f32x16 (&acc)[WalkCfg<D>::DBW], 
                                           const unsigned char *ytile = nullptr, int trow = 0) {
     using W = WalkCfg<D>;
     using V8 = typename Mma<T>::V8;
+    float sl[PER][2][8];  // the slopes (one branch on the map around all of them)
+    if (fmap) {
+        feature_dispatch(fmap, [&](auto map) {
+#pragma unroll
+            for (int i = 0; i < PER; ++i)
+#pragma unroll
+                for (int hq = 0; hq < 2; ++hq) {
+                    const int ch = (4 * (db0 + i) + 2 * g + hq) ^ swizzle_y<W::CR>(trow);
+                    const V8 y = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4 *>(ytile + trow * W::RB + (ch << 4)));
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) sl[i][hq][e] = feature_slope_c<decltype(map)::value>(static_cast<float>(y[e]));
+                }
+        });
+    }
 #pragma unroll
     for (int i = 0; i < PER; ++i) {
-        const int db = db0 + i;
 #pragma unroll
         for (int hq = 0; hq < 2; ++hq) {
-            float f[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) f[e] = acc[i][8 * hq + e];
-            if (fmap) {
-                const int ch = (4 * db + 2 * g + hq) ^ swizzle_y<W::CR>(trow);
-                const V8 y = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4 *>(ytile + trow * W::RB + (ch << 4)));
-#pragma unroll
-                for (int e = 0; e < 8; ++e) f[e] *= feature_slope_from_value(fmap, static_cast<float>(y[e]));
-            }
             V8 o8;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) o8[e] = static_cast<T>(f[e]);
+            for (int e = 0; e < 8; ++e) o8[e] = static_cast<T>(fmap ? acc[i][8 * hq + e] * sl[i][hq][e] : acc[i][8 * hq + e]);
             pk[i][hq] = __builtin_bit_cast(u32x4, o8);
         }
     }
@@ -805,11 +811,13 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
             walk_product<T, D, false, 0, B::KQ, NV>(tq, tk, tv, wave, lane, c > 0, sfrag, acc);
         }
         if (slope_y) {
+            feature_dispatch(fmap, [&](auto map) {
 #pragma unroll
-            for (int i = 0; i < W::DBW; ++i)
+                for (int i = 0; i < W::DBW; ++i)
 #pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    acc[i][v] *= feature_slope_from_value(fmap, static_cast<float>(ys[i][v / 8][v % 8]));
+                    for (int v = 0; v < 16; ++v)
+                        acc[i][v] *= feature_slope_c<decltype(map)::value>(static_cast<float>(ys[i][v / 8][v % 8]));
+            });
         }
         if constexpr (ACCUM) prev.add_to(acc);
         walk_store<T, D, OB::PER>(ro, os2, p.wv, row, g, db0, acc);
