@@ -29,13 +29,28 @@
 //   D = 128: tiles and state must share the 160 KiB of LDS: 64-row chunks, one workgroup per CU
 //            with two sets of tiles (the next chunk's loads are in flight while this one is
 //            multiplied).  A saved per-chunk state would cost as much traffic as an operand, so
-//            forward hands over its segments' fp32 entry states only and backward is split: dQ is
-//            the forward walk over (dO, V, K), whose states V^T K start from the transposed entry
-//            states, and walk_dkdv_kernel is the reverse walk for dV and dK.
+//            forward hands over its segments' fp32 entry states and the state after the last chunk,
+//            and backward is ONE reverse walk all the same (walk_bwd_rev_kernel): dQ's state, the
+//            sum of K^T V over the chunks BEFORE, is obtained going backwards, by subtracting
+//            every chunk's K^T V from the forward state at the segment's end.  Without forward's
+//            states, and with the normaliser, backward is split instead: dQ is the forward walk over
+//            (dO, V, K), whose states V^T K start from the transposed entry states, and
+//            walk_dkdv_kernel is the reverse walk for dV and dK.
 //
 // Options of the walks: an element-wise feature map applied to q, k as they are loaded, with its
 // slope multiplied into dQ, dK (WalkParams::fmap); the normaliser of linear attention and its
-// gradient terms as rank-one additions to the products (WalkParams::denom ...).
+// gradient terms as rank-one additions to the products (WalkParams::denom ...); at D = 128,
+// operands of at most 64 true columns on one side without the MFMAs on their padding (WalkExt), and
+// a result added to what its place in memory holds (WalkParams::accumulate) -- both for a wide
+// q / k evaluated as two 128-column halves.
+//
+// Scheduling.  With one wave per SIMD nothing hides the latency of an LDS read but the wave's own
+// instruction order, and the compiler, short of registers, moves every operand read down to the
+// MFMA that uses it.  The products therefore name their order themselves (walk_pipe: fragment
+// j + 4 is read before fragment j is used, kept in place by scheduling barriers), the state
+// product's MFMAs go between the score MFMAs of the first block (D = 128), running sums that only
+// MFMAs touch live in accumulation registers (Mma::mma_acc), and code for feature maps is compiled
+// only into the instantiations that use it.
 //
 // Layout.  An operand tile is C rows x D 16-bit values, row-major, the 16-byte chunk index of
 // a row XORed with swizzle_y (fla_tri_fast.h) -- one layout for the 16-byte row reads (MFMA
