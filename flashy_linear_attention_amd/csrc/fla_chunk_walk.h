@@ -1230,6 +1230,12 @@ __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p
             return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true);
         }, acc);
         walk_store<T, D, OQ::PER>(rdk, dks2, p.wqk, row, g, OQ::db0(wave), acc, fmap, tk, 32 * rb + l32);
+        // R += Q^T dO touches registers and tiles only, so it can sit on either side of the barriers: the waves of
+        // the last row block, with one score block in dV and dK against two, take it here, the others after dQ,
+        // where they have one score block against two
+        // (full widths only: with a narrow v side the balance is the other way round, measured)
+        constexpr bool kSplitUpdate = W::NRB == 2 && NQ == W::DB && NV == W::DB;
+        if (kSplitUpdate && rb == 1) walk_update<T, D, B, false, true>(tq, tg, wave, lane, st);
         sync();  // every wave has read R
         // (X stays in its accumulation registers up to here: without this the copies that the rounding
         // below reads are made right after the update and occupy 64 registers through both products)
@@ -1248,7 +1254,7 @@ __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p
             prev.add_to(held);
             walk_store<T, D, OV::PER>(rdv, dvs2, p.wv, row, g, OV::db0(wave), held);
         }
-        walk_update<T, D, B, false, true>(tq, tg, wave, lane, st);
+        if (!(kSplitUpdate && rb == 1)) walk_update<T, D, B, false, true>(tq, tg, wave, lane, st);
         sync();  // every wave has read X and is done with the tiles
         walk_state_to_lds<T, D, B>(tl, wave, lane, st);
     }
