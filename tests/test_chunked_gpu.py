@@ -1,6 +1,8 @@
 """Chunk-wise evaluation (fla_tri_xyt_z_chunked) against the CPU oracle and against the
 quadratic kernels (``-m gpu``)."""
 
+import math
+
 import pytest
 import torch
 
@@ -133,6 +135,31 @@ def test_chunked_backward_with_and_without_the_forward_state(gpu_device):
     q2, k2, v2, _ = (t.to(gpu_device) for t in reference_style_inputs(1, 2, 1024, 64, 256, torch.bfloat16, seed=32))
     assert linear_attention_chunked_fwd(q2, k2, v2, want_state=True)[1] is None
     assert linear_attention_chunked_fwd(q[:, :, :256], k[:, :, :256], v[:, :, :256], want_state=True)[1] is None
+
+
+@pytest.mark.parametrize("dims", [(128, 128), (256, 64)])
+def test_chunked_backward_when_late_rows_dwarf_early_ones(dims, gpu_device):
+    """At padded head dims above 64 the backward walk forms dQ's state -- the sum of K^T V over the chunks
+    BEFORE -- by subtracting chunks from the forward state at the end of a segment, in fp32.  Its error
+    is a rounding of the LARGEST state, so rows whose own state is much smaller are where it would
+    show: k and v grow by a factor of 64 over the sequence (4096 in their products), and the first
+    quarter of the rows of every gradient is held to the usual tolerance on its own."""
+    from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
+
+    dqk, dv = dims
+    n = 2048
+    q, k, v, dy = reference_style_inputs(1, 4, n, dqk, dv, torch.bfloat16, seed=77)
+    ramp = torch.logspace(0, math.log10(64.0), n).view(1, 1, n, 1)
+    k = (k.float() * ramp).to(torch.bfloat16)
+    v = (v.float() * ramp).to(torch.bfloat16)
+    want = naive.causal_dot_product_grads(q.float(), k.float(), v.float(), dy.float())
+    q, k, v, dy = (t.to(gpu_device) for t in (q, k, v, dy))
+    out, state = linear_attention_chunked_fwd(q, k, v, want_state=True)
+    assert state is not None
+    got = linear_attention_chunked_bwd(dy, q, k, v, state)
+    for name, g, w in zip(("dQ", "dK", "dV"), got, want):
+        assert_close(name, g, w)
+        assert_close(name + ", first quarter of the rows", g[:, :, : n // 4], w[:, :, : n // 4])
 
 
 def test_chunked_operator_workspace_is_checked(gpu_device):
