@@ -38,6 +38,8 @@ CASES = [
     (2, 4, 1300, 256, 64),
     (1, 2, 1024, 200, 128),
     (2, 8, 2450, 136, 24),
+    # (a second half of at most 64 columns against a v wider than 64: the forward walk built for a narrow q / k side)
+    (1, 3, 1100, 160, 96),
 ]
 
 
