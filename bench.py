@@ -90,6 +90,10 @@ def _parse():
                     help="instead of one workload: forward + backward of the quadratic kernels over a grid of "
                          "(B*H, N, D_qk, D_v) off the benchmark shapes, one JSON line with a `sweep` list (what the "
                          "fixed launch rules give where nobody tuned them)")
+    ap.add_argument("--crossover", action="store_true",
+                    help="instead of the benchmark: time the quadratic and the chunk-wise forward + backward over a grid "
+                         "of shapes and print one JSON line with a `crossover` list (what the library's selection table, "
+                         "fla_linear_attn_prefers_chunked, is read off)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one plain device copy of 256 MiB (a known-size reference for scaling "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -263,6 +267,59 @@ def _other_workload(torch, name, algo, dev, steps):
     del o
     torch.cuda.empty_cache()
     return rec
+
+
+def _crossover(torch, dev, steps) -> int:
+    """Quadratic against chunk-wise forward + backward (bf16, B = 1, through the Python wrappers, the
+    chunk-wise pair with forward's state handed over) over a grid of shapes, next to what the library's
+    selection table answers for each.  Medians of per-iteration event pairs."""
+    from flashy_linear_attention_amd import _lib
+    from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
+    from flashy_linear_attention_amd.kernels import (
+        linear_flash_wrapper_bwd,
+        linear_flash_wrapper_bwd_smallv_hd,
+        linear_flash_wrapper_fwd,
+        linear_flash_wrapper_fwd_smallv_hd,
+    )
+
+    pick = _lib.load().fla_linear_attn_prefers_chunked
+    gen = torch.Generator(device=dev).manual_seed(0)
+    out = []
+    for d_qk, d_v in ((32, 32), (64, 64), (128, 128), (256, 64), (192, 128), (256, 256)):
+        for bh in (16, 64, 128, 256, 512):
+            for n in (256, 512, 1024, 2048, 4096, 8192):
+                if bh * n * max(d_qk, d_v) > 2 ** 28 or (d_qk != d_v and bh > 256):
+                    continue
+                q = (torch.rand(1, bh, n, d_qk, device=dev, generator=gen) + 0.5).bfloat16()
+                k = (torch.rand(1, bh, n, d_qk, device=dev, generator=gen) + 0.5).bfloat16()
+                v = torch.randn(1, bh, n, d_v, device=dev, generator=gen).bfloat16()
+                do = torch.randn(1, bh, n, d_v, device=dev, generator=gen).bfloat16()
+                small = d_qk != d_v
+
+                def quadratic():
+                    if small:
+                        linear_flash_wrapper_fwd_smallv_hd(q, k, v)
+                        linear_flash_wrapper_bwd_smallv_hd(do, q, k, v)
+                    else:
+                        linear_flash_wrapper_fwd(q, k, v)
+                        linear_flash_wrapper_bwd(do, q, k, v)
+
+                def chunked():
+                    _, st = linear_attention_chunked_fwd(q, k, v, want_state=True)
+                    linear_attention_chunked_bwd(do, q, k, v, st)
+
+                _settle(torch, chunked, 0.05)
+                us_q, us_c = 1e3 * _median_ms(torch, quadratic, steps), 1e3 * _median_ms(torch, chunked, steps)
+                out.append({"BH": bh, "N": n, "D_qk": d_qk, "D_v": d_v, "quadratic_us": round(us_q, 1),
+                            "chunked_us": round(us_c, 1), "table_says_chunked": int(pick(1, bh, n, d_qk, d_v)),
+                            "chunked_is_faster": int(us_c < us_q)})
+                del q, k, v, do
+    wrong = [r for r in out if r["table_says_chunked"] != r["chunked_is_faster"]]
+    worst = max((max(r["quadratic_us"], r["chunked_us"]) / min(r["quadratic_us"], r["chunked_us"]) for r in wrong), default=1.0)
+    print(json.dumps({"metric": "quadratic against chunk-wise forward + backward over a grid of shapes, bf16, 1 MI355X",
+                      "unit": "us", "steps": steps, "cells": len(out), "cells_where_the_table_picks_the_slower": len(wrong),
+                      "worst_loss_factor": round(worst, 2), "crossover": out}))
+    return 0
 
 
 def _sweep(torch, dev, steps) -> int:
@@ -536,6 +593,8 @@ def main() -> int:
     dev = torch.device("cuda:0")
     if args.sweep:
         return _sweep(torch, dev, min(args.steps, 30))
+    if args.crossover:
+        return _crossover(torch, dev, min(args.steps, 30))
     if args.algo == "poly":
         return _bench_poly(torch, args, w, dev)
     if args.algo == "feature":

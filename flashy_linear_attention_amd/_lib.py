@@ -12,7 +12,7 @@ import threading
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libfla_gfx950.so")
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 FLA_DTYPE_BF16 = 0
 FLA_DTYPE_F16 = 1
@@ -35,6 +35,7 @@ SIGNATURES = {
                               ctypes.c_int),
     "fla_linear_attn_chunked_state_bytes": ([_i64] * 5, ctypes.c_int64),
     "fla_linear_attn_chunked_workspace_bytes": ([_i64] * 5, ctypes.c_int64),
+    "fla_linear_attn_prefers_chunked": ([_i64] * 5, ctypes.c_int),
     "fla_linear_attn_chunked_fwd": ([_ptr] * 4 + [_i64] * 5 + [_strides] * 4
                                     + [ctypes.c_int, _ptr, ctypes.POINTER(ctypes.c_int32), _ptr, _i64, _ptr], ctypes.c_int),
     "fla_feature_attn_fwd": ([_ptr] * 6 + [_i64] * 5 + [_strides] * 6

@@ -35,7 +35,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 2
+#define FLA_ABI_VERSION 3
 
 enum fla_dtype { FLA_DTYPE_BF16 = 0, FLA_DTYPE_F16 = 1 };
 
@@ -160,6 +160,10 @@ int fla_tri_xyt_z_chunked(const void *x, const void *y, const void *z, void *out
  * `workspace`: fla_linear_attn_chunked_workspace_bytes() bytes of scratch, 16-byte aligned.
  * No counterpart in the reference (quadratic kernels only, linear_attn_kernels.py:63, 166-171). */
 int64_t fla_linear_attn_chunked_state_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v);
+/* 1 when fla_linear_attn_chunked_fwd + bwd are the faster pair for this shape on MI355X, 0 when the
+ * quadratic fla_linear_attn(_smallv)_fwd + bwd are: a table of measured thresholds (host arithmetic,
+ * no device call) in place of the autotuning the reference lists as a to-do (README.md:68). */
+int fla_linear_attn_prefers_chunked(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v);
 int64_t fla_linear_attn_chunked_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v);
 int fla_linear_attn_chunked_fwd(const void *q, const void *k, const void *v, void *o,
                                 int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,

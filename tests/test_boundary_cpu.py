@@ -225,3 +225,20 @@ def test_chunkwise_state_and_workspace_sizes():
         assert ws(*shape) >= 4 * (sb(*shape) - shape[0] * shape[1] * 4)  # room for the 256-row path's four buffers
         assert lib.fla_normalised_workspace_bytes(*shape, 1) > ws(*shape)
     assert ws(4, 16, 4096, 256, 64) > 0 and ws(4, 16, 4096, 64, 256) > 0 and ws(1, 2, 256, 128, 128) == 0
+
+
+def test_algorithm_table():
+    """fla_linear_attn_prefers_chunked is host arithmetic on measured thresholds: the benchmark workloads
+    with long sequences go chunk-wise, short or single-chunk problems stay with the quadratic kernels,
+    and the answer grows monotonically with the sequence length."""
+    pick = _lib.load().fla_linear_attn_prefers_chunked
+    assert pick(4, 32, 4096, 128, 128) == 1 and pick(1, 16, 32768, 64, 64) == 1 and pick(4, 16, 4096, 256, 64) == 1
+    assert pick(1, 2, 256, 64, 64) == 0 and pick(1, 16, 1024, 64, 64) == 0 and pick(1, 128, 512, 128, 128) == 0
+    assert pick(1, 128, 1024, 128, 128) == 1 and pick(1, 512, 512, 64, 64) == 1
+    assert pick(1, 64, 512, 256, 64) == 0 and pick(1, 64, 2048, 256, 64) == 1
+    assert pick(1, 16, 2048, 256, 256) == 0 and pick(1, 16, 4096, 256, 256) == 1
+    assert pick(0, 4, 4096, 64, 64) == 0 and pick(1, 4, 4096, 300, 64) == 0
+    for shape in [(1, 16, 64, 64), (2, 8, 128, 128), (1, 64, 256, 64), (1, 4, 192, 128), (1, 8, 256, 256)]:
+        b, h, dqk, dv = shape
+        answers = [pick(b, h, n, dqk, dv) for n in (256, 512, 1024, 2048, 4096, 8192, 16384, 32768)]
+        assert answers == sorted(answers) and answers[-1] == 1

@@ -240,3 +240,23 @@ def test_chunked_small_v_state_hand_over(gpu_device):
     for name, a, b, w in zip(("dQ", "dK", "dV"), with_state, without, want):
         assert_close(name, a, w)
         assert_close(name + " (no saved state)", b, w)
+
+
+@pytest.mark.parametrize("dims", [(1, 2, 256, 64, 64, 0), (1, 16, 4096, 64, 64, 1), (1, 2, 1000, 128, 128, 0),
+                                  (1, 32, 2048, 256, 64, 1), (1, 2, 512, 256, 64, 0)], ids=lambda d: "x".join(map(str, d)))
+def test_auto_operator_picks_an_evaluation_and_matches_the_oracle(dims, gpu_device):
+    """LinearAttentionAuto: quadratic kernels for the short shapes, chunk-wise for the long ones and
+    for what the quadratic wrappers refuse (N not a multiple of 64); same function either way."""
+    from flashy_linear_attention_amd import LinearAttentionAuto
+    from flashy_linear_attention_amd.auto import prefers_chunked
+
+    b, h, n, dqk, dv, chunked = dims
+    q, k, v, dy = (t.to(gpu_device) for t in reference_style_inputs(b, h, n, dqk, dv, torch.bfloat16, seed=91))
+    assert prefers_chunked(q, v) == bool(chunked)
+    q.requires_grad_(True), k.requires_grad_(True), v.requires_grad_(True)
+    out = LinearAttentionAuto.apply(q, k, v)
+    got = torch.autograd.grad(out, (q, k, v), dy)
+    qc, kc, vc = (t.detach().float().cpu() for t in (q, k, v))
+    assert_close("O", out.detach(), naive.causal_dot_product(qc, kc, vc))
+    for name, g, w in zip(("dQ", "dK", "dV"), got, naive.causal_dot_product_grads(qc, kc, vc, dy.float().cpu())):
+        assert_close(name, g, w)
