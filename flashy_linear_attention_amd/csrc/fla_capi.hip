@@ -477,12 +477,14 @@ bool states_shareable(int64_t dqk, int64_t dv, int64_t N) {
 //     O  = tril(Q_0 K_0^T) V + tril(Q_1 K_1^T) V        dV = the same sum of the halves' dV
 //     dQ_h = tril(dO V^T) K_h                           dK_h = triu(V dO^T) Q_h
 // so each half runs the D = 128 walk kernels on column views of q, k, dq, dk (v and dO are padded
-// with zeros in LDS, never in memory); the second half's O and dV go to a scratch tensor and one
-// element-wise pass adds them.  Forward hands over both halves' entry states.
+// with zeros in LDS, never in memory); the second half's walk adds its O (its part of dV) to what the
+// first one wrote.  Forward hands over both halves' entry and final states, and backward of a half
+// is then one reverse walk; without them it is the forward-direction walk for dQ_h and the dK / dV
+// walk, whose second dV goes to a scratch tensor that one element-wise pass adds.
 struct WidePlan {
     bool ok;
     WalkPlan wp;         // the plan of a 128 / 128 problem of the same B, H, N
-    int64_t temp_bytes;  // the second half's O (forward) or dV (backward), contiguous (B, H, N, D_v)
+    int64_t temp_bytes;  // the second half's dV in backward without forward's states, contiguous (B, H, N, D_v)
 };
 
 WidePlan wide_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
@@ -515,7 +517,7 @@ int64_t shared_state_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t
     return core ? core + walk_vec_bytes(B, H, N, dqk, dv) : 0;
 }
 
-// workspace of the two-halves evaluation: the scratch tensor, then totals and entry states of one
+// workspace of the two-halves evaluation: the scratch tensor for dV, then totals and entry states of one
 // half at a time (two sets in backward: Q^T dO, and K^T V when forward's entry states are not given)
 int64_t wide_workspace_bytes(const WidePlan &w) { return w.temp_bytes + 2 * w.wp.work_bytes; }
 

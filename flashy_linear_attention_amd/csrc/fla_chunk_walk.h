@@ -704,6 +704,7 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
 // NORM: the instantiations that take the normaliser's terms: 1 forward (WalkParams::denom), 2 dQ (dn).
 // FM: the instantiations that know of feature maps (WalkParams::fmap, slope_y); the others ignore both.
 // NQ, NV: blocks of the state [q/k index][v index] that hold anything (WalkExt).
+// ACCUM: the result is added to what o holds already (WalkParams::accumulate, WalkPrev).
 template <typename T, int D, bool DOUBLE, int NORM, bool FM, int NQ = D / 32, int NV = D / 32, bool ACCUM = false>
 __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
