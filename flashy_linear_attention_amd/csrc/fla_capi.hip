@@ -434,7 +434,8 @@ int walk_entry_states(const WalkPlan &w, const View &y, const View &z, int64_t B
     tp.seg_hi = (int32_t)(!reverse && !map_y ? n_fine - w.m : n_fine);
     if (fla::walk_totals(dtype, w.D, tp, s) != hipSuccess) return FLA_ERR_LAUNCH;
     *where = entry;
-    return fla::walk_scan(totals, entry, B * H, (int)w.n_seg, (int)w.m, w.D * w.D, reverse, s) == hipSuccess
+    return fla::walk_scan(totals, entry, B * H, (int)w.n_seg, (int)w.m, w.D, fla::walk_totals_cols(w.D, (int)dy, (int)dz),
+                          reverse, s) == hipSuccess
                ? FLA_OK
                : FLA_ERR_LAUNCH;
 }

@@ -1360,14 +1360,18 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
 // thread reads an element before it writes it).  One thread per pair of elements; the loads of up
 // to sixteen segments are issued together (a chain of dependent loads would cost a memory latency
 // each).
+// `cols`: only the first `cols` columns of every row of the D-wide states are summed (the totals
+// kernel built for a narrow v side writes no others, and no walk of that extent reads them).
 // (a template only so that the header can be included by several translation units)
 template <int kUnused = 0>
 __global__ __launch_bounds__(256) void walk_scan_kernel(const float *totals, float *entry, int n_seg, int m, int E,
-                                                        int64_t total2, int reverse) {
+                                                        int64_t total2, int reverse, int D, int cols) {
     typedef float f32x2 __attribute__((ext_vector_type(2)));
     const int64_t i2 = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i2 >= total2) return;
-    const int64_t bh = (i2 * 2) / E, e = i2 * 2 - bh * E;
+    const int half = cols / 2;
+    const int64_t per_bh = (int64_t)(E / D) * half, bh = i2 / per_bh, r = i2 - bh * per_bh;
+    const int64_t e = (r / half) * D + 2 * (r % half);
     const int n_fine = n_seg * m;
     const float *pt = totals + bh * n_fine * E + e;
     float *pe = entry + bh * n_seg * E + e;
@@ -1510,13 +1514,17 @@ hipError_t launch_walk_vec_sums(const WalkVecParams &p, int64_t BH, hipStream_t 
     return launch_kernel(walk_vec_sums_kernel<T, D>, dim3((unsigned)p.n_chunks, (unsigned)BH), dim3(256), 0, stream, p);
 }
 
+// columns of the D x D totals that walk_totals_kernel writes for operands of true widths dy, dz (the
+// variant without the padding blocks of a narrow z leaves the others unwritten)
+inline int walk_totals_cols(int D, int dy, int dz) { return D == 128 && dy > 64 && dz <= 64 ? 64 : D; }
+
 template <typename T, int D>
 hipError_t launch_walk_totals(const WalkTotalsParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     constexpr int smem = 4 * WalkCfg<D>::TILE;
     if constexpr (D == 128) {
-        if (p.dy > 64 && p.dz <= 64) {  // z of at most 64 true columns: the state's other v blocks hold zeros
+        if (walk_totals_cols(D, p.dy, p.dz) == 64) {  // z of at most 64 true columns: the state's other v blocks hold zeros
             constexpr auto kern = walk_totals_kernel<T, D, 4, 2>;
             if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
             return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
@@ -1527,12 +1535,13 @@ hipError_t launch_walk_totals(const WalkTotalsParams &p, hipStream_t stream) {
     return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
 }
 
-inline hipError_t launch_walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, int m, int E, int reverse,
-                                   hipStream_t stream) {
-    const int64_t total2 = BH * E / 2;
-    if (m < 1 || (m > 1 && entry == totals)) return hipErrorInvalidValue;
+inline hipError_t launch_walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, int m, int D, int cols,
+                                   int reverse, hipStream_t stream) {
+    const int E = D * D;
+    const int64_t total2 = BH * D * (cols / 2);
+    if (m < 1 || (m > 1 && entry == totals) || cols < 2 || cols > D || cols % 2) return hipErrorInvalidValue;
     return launch_kernel(walk_scan_kernel<0>, dim3((unsigned)((total2 + 255) / 256)), dim3(256), 0, stream, totals, entry,
-                         n_seg, m, E, total2, reverse);
+                         n_seg, m, E, total2, reverse, D, cols);
 }
 
 template <auto kern>
