@@ -381,8 +381,9 @@ struct WalkPlan {
     int64_t fine_bytes;                   // fp32 totals of the finer segments
     int64_t entry_bytes;                  // fp32 entry states of the walk segments (in place over the totals when m == 1)
     int64_t work_bytes;                   // workspace of one direction: totals, and entry states when m > 1
-    int64_t saved_bytes;                  // what forward hands to backward: per-chunk 16-bit states / split: the entry
-                                          // states and, behind them, the state after the last chunk of every (b, h)
+    int64_t saved_bytes;                  // what forward hands to backward: the entry states and, behind them, the state
+                                          // after the last chunk of every (b, h); with the normaliser at padded head dims
+                                          // up to 64, the 16-bit state of every chunk (room for the larger of the two)
 };
 
 WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
@@ -405,7 +406,9 @@ WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     w.entry_bytes = B * H * w.n_seg * w.D * w.D * 4;
     w.fine_bytes = w.entry_bytes * w.m;
     w.work_bytes = w.fine_bytes + (w.m > 1 ? w.entry_bytes : 0);  // (a single segment needs them only with a feature map)
-    w.saved_bytes = w.split ? w.entry_bytes + B * H * w.D * w.D * 4 : B * H * w.n_chunks * w.D * w.D * 2;
+    // (padded head dims up to 64: the per-chunk states of the normalised operator are the larger of the two)
+    const int64_t states = w.entry_bytes + B * H * w.D * w.D * 4, per_chunk = B * H * w.n_chunks * w.D * w.D * 2;
+    w.saved_bytes = w.split || states > per_chunk ? states : per_chunk;
     return w;
 }
 
@@ -678,9 +681,10 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         // the segments' entry states; with a feature map the same kernel maps xk as it loads it and
         // writes phi(xk), which the walk then reads (so it runs for a single segment as well)
         const bool need_totals = wp.n_seg > 1 || fmap;
-        // split: the entry states are what backward gets, so the scan writes them to state_out
-        // (m == 1: the totals themselves are computed there, and no workspace is used)
-        const bool in_state = wp.split && state_out;
+        // the entry states (and the state after the last chunk) are what backward gets, so the scan writes
+        // them to state_out (m == 1: the totals themselves are computed there, and no workspace is used);
+        // the normalised operator at padded head dims up to 64 hands over the 16-bit state of every chunk instead
+        const bool in_state = state_out && (wp.split || !nx);
         if (need_totals && !(in_state && wp.m == 1) &&
             (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 ||
              workspace_bytes < (in_state ? wp.fine_bytes : wp.work_bytes)))
@@ -706,7 +710,7 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         w.os_b = o.strides[0], w.os_h = o.strides[1], w.os_n = o.strides[2];
         w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dqk, w.wv = (int32_t)dv;
         w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
-        w.init = wp.n_seg > 1 ? entry : nullptr, w.saved = wp.split ? nullptr : state_out;
+        w.init = wp.n_seg > 1 ? entry : nullptr, w.saved = in_state ? nullptr : state_out;
         if (in_state) w.total_out = reinterpret_cast<float *>(static_cast<char *>(state_out) + wp.entry_bytes);
         if (nx) {  // the normaliser inside the walk: zc = running sum of k at the entry of every chunk
             // (kept behind the state, when there is one, for backward)
@@ -891,7 +895,13 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         w.dvs_b = dvv.strides[0], w.dvs_h = dvv.strides[1], w.dvs_n = dvv.strides[2];
         w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dqk, w.wv = (int32_t)dv;
         w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
-        w.init = entry, w.saved = const_cast<void *>(state_in);
+        w.init = entry;
+        if (nx) {
+            w.saved = const_cast<void *>(state_in);
+        } else {  // forward's entry states and, behind them, its state after the last chunk
+            w.xinit = static_cast<const float *>(state_in);
+            w.xtotal = reinterpret_cast<const float *>(static_cast<const char *>(state_in) + wp.entry_bytes);
+        }
         if (nx) {
             const int64_t vb = walk_vec_bytes(B, H, N, dqk, dv);
             float *zc = static_cast<float *>(nx->vec), *rcv = reinterpret_cast<float *>(static_cast<char *>(nx->vec) + vb);

@@ -859,7 +859,7 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
         }
         walk_state_to_lds<T, D, B>(tl, wave, lane, st);
     }
-    if (DOUBLE && p.total_out && sl.c_hi == p.n_chunks) {  // the state after the last chunk, for walk_bwd_rev_kernel
+    if (p.total_out && sl.c_hi == p.n_chunks) {  // the state after the last chunk, for the backward walks
         float *out = p.total_out + (int64_t)sl.bh * (D * D);
 #pragma unroll
         for (int i = 0; i < B::SLOTS; ++i)
@@ -879,7 +879,13 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
 #endif
 }
 
-// ---- backward: dQ, dV, dK of a chunk from one set of tiles; R += Q_c^T dO_c, chunks descending
+// ---- backward: dQ, dV, dK of a chunk from one set of tiles; R += Q_c^T dO_c, chunks descending.
+// dQ's state, the sum of K^T V over the chunks before:
+//   NORM (the normaliser's terms): the 16-bit state forward saved at the entry of every chunk
+//   (WalkParams::saved), fragments straight from memory;
+//   otherwise obtained backwards as in walk_bwd_rev_kernel: X starts as the forward state at the
+//   segment's end (xinit / xtotal) and every chunk's K^T V is subtracted when the walk reaches it;
+//   X has a 16-bit copy of its own in LDS beside R's.  Forward then saves no per-chunk states.
 template <typename T, int D, bool NORM>
 __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -890,6 +896,7 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     unsigned char *tq = smem, *tk = smem + W::TILE, *tv = smem + 2 * W::TILE, *tg = smem + 3 * W::TILE,
                   *tl = smem + 4 * W::TILE;
+    unsigned char *tx = tl + W::STATE;  // (!NORM) X's copy; (NORM) the chunk's vectors
     const float *vz = reinterpret_cast<const float *>(tl + W::STATE), *vr = vz + 256, *vd = vz + 512;
     const uint32_t xbase = lds0 + 4 * W::TILE + W::STATE;
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
@@ -917,6 +924,11 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
     f32x16 st[W::NBW];  // R[q/k index][v index]
     walk_load_init<D>(p, sl, wave, lane, st);
     walk_state_to_lds<T, D>(tl, wave, lane, st);
+    f32x16 xs[W::NBW];  // X[q/k index][v index]
+    if constexpr (!NORM)
+        walk_load_state<D>(sl.c_hi < p.n_chunks ? p.xinit + ((int64_t)sl.bh * p.n_seg + sl.seg + 1) * (D * D)
+                                                : p.xtotal + (int64_t)sl.bh * (D * D),
+                           false, wave, lane, xs);
 
 #pragma unroll 1
     for (int c = sl.c_hi - 1; c >= sl.c_lo; --c) {
@@ -930,34 +942,37 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
             walk_load_vec<D>(p.rc + ((int64_t)sl.bh * p.n_chunks + c) * D, xbase + 1024, lane);
             walk_load_rows<D>(p.dn + (int64_t)sl.bh * N, row0, N, xbase + 2048, lane);
         }
-        // dQ's state, S_c[q/k index][v index] as saved by forward: A-operand fragments straight from
+        // NORM: dQ's state, S_c[q/k index][v index] as saved by forward: A-operand fragments straight from
         // memory (row = output column of dQ, eight consecutive v indices)
-        const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
-            static_cast<T *>(p.saved) + ((int64_t)sl.bh * p.n_chunks + c) * (D * D), 0, D * D * 2, 0x00020000);
-        V8 sfq[W::DB][W::KC];
-        if (c > 0) {
+        V8 sfq[NORM ? W::DB : 1][NORM ? W::KC : 1];
+        if constexpr (NORM) {
+            const __amdgpu_buffer_rsrc_t rs = __builtin_amdgcn_make_buffer_rsrc(
+                static_cast<T *>(p.saved) + ((int64_t)sl.bh * p.n_chunks + c) * (D * D), 0, D * D * 2, 0x00020000);
+            if (c > 0) {
 #pragma unroll
-            for (int db = 0; db < W::DB; ++db)
+                for (int db = 0; db < W::DB; ++db)
 #pragma unroll
-                for (int kc = 0; kc < W::KC; ++kc)
-                    sfq[db][kc] = __builtin_bit_cast(V8, __builtin_amdgcn_raw_buffer_load_b128(
-                                                             rs, (uint32_t)(((32 * db + walk_e_lane(l32)) * D + 16 * kc + 8 * g) * 2), 0, 0));
+                    for (int kc = 0; kc < W::KC; ++kc)
+                        sfq[db][kc] = __builtin_bit_cast(V8, __builtin_amdgcn_raw_buffer_load_b128(
+                                                                 rs, (uint32_t)(((32 * db + walk_e_lane(l32)) * D + 16 * kc + 8 * g) * 2), 0, 0));
+            }
         }
         wait_vm<0>();
         __syncthreads();
         const int row = row0 + 32 * wave + l32;
         const bool later = c + 1 < p.n_chunks;  // chunks after this one exist: R is not identically zero
         f32x16 acc[W::DBW];
-        // dQ = lower(dO V^T) K + dO S_c^T  (normaliser: scores + dn_i, result + dn_i zc)
         if constexpr (NORM) {
+            // dQ = lower(dO V^T) K + dO S_c^T  (normaliser: scores + dn_i, result + dn_i zc)
             float ax = vd[32 * wave + l32];
             walk_product<T, D, false, 2>(tg, tv, tk, wave, lane, c > 0, [&](int db, int kc) -> V8 { return sfq[db][kc]; },
                                          acc, &ax);
             walk_add_vec<D>(acc, ax, vz, 0, g);
+            walk_store<T, D>(rdq, dqs2, p.wqk, row, g, 0, acc, p.fmap, tq, 32 * wave + l32);
         } else {
-            walk_product<T, D, false>(tg, tv, tk, wave, lane, c > 0, [&](int db, int kc) -> V8 { return sfq[db][kc]; }, acc);
+            walk_update<T, D, WalkExt<D>, true>(tk, tv, wave, lane, xs);  // X: now the sum over the chunks before this one
+            walk_state_to_lds<T, D>(tx, wave, lane, xs);
         }
-        walk_store<T, D>(rdq, dqs2, p.wqk, row, g, 0, acc, p.fmap, tq, 32 * wave + l32);
         // dV = upper(K Q^T) dO + K R: A operand R^T[v index][q/k index] = the LDS copy as it is
         walk_product<T, D, true>(tk, tq, tg, wave, lane, later, [&](int db, int kc) -> V8 {
             return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g);
@@ -978,6 +993,14 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
             }, acc);
         }
         walk_store<T, D>(rdk, dks2, p.wqk, row, g, 0, acc, p.fmap, tk, 32 * wave + l32);
+        if constexpr (!NORM) {
+            __syncthreads();  // every wave's part of X is in LDS
+            // dQ = lower(dO V^T) K + dO X^T: A operand X[q/k index][v index], its LDS copy read transposed
+            walk_product<T, D, false>(tg, tv, tk, wave, lane, c > 0, [&](int db, int kc) -> V8 {
+                return walk_col_frag_perm<T, D>(tx, 16 * kc, db, lane, true);
+            }, acc);
+            walk_store<T, D>(rdq, dqs2, p.wqk, row, g, 0, acc, p.fmap, tq, 32 * wave + l32);
+        }
         walk_update<T, D>(tq, tg, wave, lane, st);
         __syncthreads();
         walk_state_to_lds<T, D>(tl, wave, lane, st);
@@ -1594,9 +1617,11 @@ hipError_t launch_walk_bwd(const WalkParams &p, hipStream_t stream) {
         if (hipError_t e = ensure_dynamic_lds<kern>(smem_n)) return e;
         return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem_n, stream, p);
     }
+    if (!p.xtotal || (p.n_seg > 1 && !p.xinit)) return hipErrorInvalidValue;
     constexpr auto kern = walk_bwd_kernel<T, D, false>;
-    if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-    return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+    constexpr int smem_x = smem + WalkCfg<D>::STATE;  // X's copy beside R's
+    if (hipError_t e = ensure_dynamic_lds<kern>(smem_x)) return e;
+    return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem_x, stream, p);
 }
 
 template <typename T, int D>

@@ -202,9 +202,9 @@ def test_synthetic_workloads_have_the_stated_shapes_and_features():
 
 def test_chunkwise_state_and_workspace_sizes():
     """The size queries are host arithmetic on the chunk-wise plan (no GPU): values derived by hand.
-    State = what forward hands to backward (D <= 64: a 16-bit D x D state per 128-row chunk; D = 128:
-    the fp32 entry state of every walk segment plus the final state, or the 16-bit states of the
-    256-row chunks if those are larger) plus an fp32 vector of D per chunk for the normalised operator."""
+    State = what forward hands to backward: the fp32 entry state of every walk segment plus the final
+    state, or, if larger, the 16-bit states of the chunks (D <= 64: per 128-row chunk, what the
+    normalised operator hands over; D = 128: of the 256-row chunks) plus an fp32 vector of D per chunk for the normalised operator."""
     lib = _lib.load()
     sb = lib.fla_linear_attn_chunked_state_bytes
     # B H = 128, N = 4096, D = 128: 16 chunks of 256 rows x 32 KiB > 2 segments x 64 KiB; 64 chunks of 64 rows
@@ -214,7 +214,8 @@ def test_chunkwise_state_and_workspace_sizes():
     # ragged: N = 2450 at D = 128 is 39 chunks of 64 rows in 20 walk segments of 2 (their entry states, and the
     # state after the last chunk); ten 256-row chunks are less
     assert sb(2, 8, 2450, 128, 128) == 16 * 21 * 128 * 128 * 4 + 16 * 39 * 128 * 4
-    assert sb(1, 1, 300, 32, 32) == 3 * 32 * 32 * 2 + 3 * 32 * 4
+    # three single-chunk segments at D = 32: their fp32 entry states and the final state outweigh three 16-bit states
+    assert sb(1, 1, 300, 32, 32) == 4 * 32 * 32 * 4 + 3 * 32 * 4
     # D_qk = 256, D_v = 64: the fp32 entry states of both 128-column halves, 4 walk segments per (b, h), and their
     # states after the last chunk
     assert sb(4, 16, 4096, 256, 64) == 2 * 64 * 5 * 128 * 128 * 4

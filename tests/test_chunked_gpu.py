@@ -139,10 +139,10 @@ def test_chunked_backward_with_and_without_the_forward_state(gpu_device):
     assert linear_attention_chunked_fwd(q[:, :, :256], k[:, :, :256], v[:, :, :256], want_state=True)[1] is None
 
 
-@pytest.mark.parametrize("dims", [(128, 128), (256, 64)])
+@pytest.mark.parametrize("dims", [(64, 64), (128, 128), (256, 64)])
 def test_chunked_backward_when_late_rows_dwarf_early_ones(dims, gpu_device):
-    """At padded head dims above 64 the backward walk forms dQ's state -- the sum of K^T V over the chunks
-    BEFORE -- by subtracting chunks from the forward state at the end of a segment, in fp32.  Its error
+    """The backward walk forms dQ's state -- the sum of K^T V over the chunks BEFORE -- by subtracting
+    chunks from the forward state at the end of a segment, in fp32.  Its error
     is a rounding of the LARGEST state, so rows whose own state is much smaller are where it would
     show: k and v grow by a factor of 64 over the sequence (4096 in their products), and the first
     quarter of the rows of every gradient is held to the usual tolerance on its own."""
@@ -176,8 +176,9 @@ def test_chunked_operator_workspace_is_checked(gpu_device):
     stream = torch.cuda.current_stream().cuda_stream
     need = lib.fla_linear_attn_chunked_workspace_bytes(1, 2, 1024, 64, 64)
     sbytes = lib.fla_linear_attn_chunked_state_bytes(1, 2, 1024, 64, 64)
-    # one 64 x 64 state per 128-row chunk and head, and an fp32 vector per chunk (the normalised operator's)
-    assert need > 0 and sbytes == 2 * 8 * 64 * 64 * 2 + 2 * 8 * 64 * 4
+    # the fp32 entry state of each of the eight single-chunk segments and the final state, per head (more than
+    # the normalised operator's 16-bit state per 128-row chunk), and an fp32 vector per chunk
+    assert need > 0 and sbytes == 2 * 9 * 64 * 64 * 4 + 2 * 8 * 64 * 4
     # D = 128: the fp32 entry state of every segment (here single 64-row chunks) and the state after the
     # last chunk, which is more than a 16-bit state per 256-row chunk
     assert lib.fla_linear_attn_chunked_state_bytes(1, 2, 1024, 128, 128) == 2 * 17 * 128 * 128 * 4 + 2 * 16 * 128 * 4
