@@ -23,16 +23,18 @@
 // each walking workgroup starts from its segment's entry state.  No fp32 per-chunk state ever
 // goes to memory.
 //
-//   D <= 64: 128-row chunks, two workgroups per CU.  Forward saves the 16-bit state at the entry
-//            of every chunk (S_c), and ONE backward kernel (walk_bwd_kernel) computes dQ, dV and
-//            dK of a chunk from one set of tiles.
+//   D <= 64: 128-row chunks, two workgroups per CU.  ONE backward kernel (walk_bwd_kernel)
+//            computes dQ, dV and dK of a chunk from one set of tiles; dQ's state -- the sum of
+//            K^T V over the chunks BEFORE -- is obtained going backwards, by subtracting every
+//            chunk's K^T V from the forward state at the segment's end, so forward hands over
+//            only its segments' fp32 entry states and the state after the last chunk.  (With
+//            the normaliser, whose vectors take the LDS a second state copy would need, forward
+//            saves the 16-bit state at the entry of every chunk instead.)
 //   D = 128: tiles and state must share the 160 KiB of LDS: 64-row chunks, one workgroup per CU
 //            with two sets of tiles (the next chunk's loads are in flight while this one is
 //            multiplied).  A saved per-chunk state would cost as much traffic as an operand, so
-//            forward hands over its segments' fp32 entry states and the state after the last chunk,
-//            and backward is ONE reverse walk all the same (walk_bwd_rev_kernel): dQ's state, the
-//            sum of K^T V over the chunks BEFORE, is obtained going backwards, by subtracting
-//            every chunk's K^T V from the forward state at the segment's end.  Without forward's
+//            forward hands over the same fp32 states, and backward is ONE reverse walk as well
+//            (walk_bwd_rev_kernel), with dQ's state by the same subtraction.  Without forward's
 //            states, and with the normaliser, backward is split instead: dQ is the forward walk over
 //            (dO, V, K), whose states V^T K start from the transposed entry states, and
 //            walk_dkdv_kernel is the reverse walk for dV and dK.

@@ -151,12 +151,14 @@ int fla_tri_xyt_z_chunked(const void *x, const void *y, const void *z, void *out
  * every other case evaluates each product with fla_tri_xyt_z_chunked's method, same results.
  *
  * forward:  `state_out` (optional, fla_linear_attn_chunked_state_bytes() bytes, 16-byte aligned)
- *           receives what a later backward call can reuse of the running state (padded head dims
- *           up to 64: the rounded state at the entry of every chunk; wider: the fp32 state at the
- *           entry of every segment of the walk and after the last chunk); *state_valid (host
+ *           receives what a later backward call can reuse of the running state (the fp32 state at
+ *           the entry of every segment of the walk and after the last chunk; the normalised
+ *           operator at padded head dims up to 64: the rounded state at the entry of every
+ *           chunk); *state_valid (host
  *           memory, optional) is set to 1 when it was written, else 0.
  * backward: `state_in` is that buffer, written by the forward call on the same q, k, v, or NULL
- *           (the state is then recomputed; wider head dims take two walks instead of one).
+ *           (the state is then recomputed by another evaluation: two walks instead of one at
+ *           padded head dims above 64, chunk states in memory below).
  * `workspace`: fla_linear_attn_chunked_workspace_bytes() bytes of scratch, 16-byte aligned.
  * No counterpart in the reference (quadratic kernels only, linear_attn_kernels.py:63, 166-171). */
 int64_t fla_linear_attn_chunked_state_bytes(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v);
