@@ -36,9 +36,12 @@ class LinearAttentionAuto(Function):
     @torch.amp.custom_fwd(device_type="cuda", cast_inputs=torch.bfloat16)
     def forward(ctx: Any, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
         assert q.dim() == 4 and q.shape == k.shape and v.shape[:3] == q.shape[:3], "q, k: (B,H,N,D_qk); v: (B,H,N,D_v)"
-        # (the quadratic wrappers keep the reference's limits: N a multiple of 64, D_v <= D_qk)
-        ctx.chunked = prefers_chunked(q, v) or q.shape[2] % 64 != 0 or v.shape[-1] > q.shape[-1]
-        ctx.equal = q.shape[-1] == v.shape[-1]
+        # (the quadratic wrappers keep the reference's limits: N a multiple of 64 and, with unequal head dims,
+        # D_v a power of two not above D_qk -- what they refuse goes to the chunk-wise kernels)
+        dqk, dv = q.shape[-1], v.shape[-1]
+        ctx.equal = dqk == dv
+        refused = q.shape[2] % 64 != 0 or (not ctx.equal and (dv > dqk or dv & (dv - 1)))
+        ctx.chunked = prefers_chunked(q, v) or refused
         state = None
         if ctx.chunked:
             if any(ctx.needs_input_grad[:3]):

@@ -244,10 +244,12 @@ def test_chunked_small_v_state_hand_over(gpu_device):
 
 
 @pytest.mark.parametrize("dims", [(1, 2, 256, 64, 64, 0), (1, 16, 4096, 64, 64, 1), (1, 2, 1000, 128, 128, 0),
-                                  (1, 32, 2048, 256, 64, 1), (1, 2, 512, 256, 64, 0)], ids=lambda d: "x".join(map(str, d)))
+                                  (1, 32, 2048, 256, 64, 1), (1, 2, 512, 256, 64, 0), (1, 2, 384, 160, 96, 0)],
+                         ids=lambda d: "x".join(map(str, d)))
 def test_auto_operator_picks_an_evaluation_and_matches_the_oracle(dims, gpu_device):
     """LinearAttentionAuto: quadratic kernels for the short shapes, chunk-wise for the long ones and
-    for what the quadratic wrappers refuse (N not a multiple of 64); same function either way."""
+    for what the quadratic wrappers refuse (N not a multiple of 64, a value head dim that is no power
+    of two); same function either way."""
     from flashy_linear_attention_amd import LinearAttentionAuto
     from flashy_linear_attention_amd.auto import prefers_chunked
 
