@@ -370,17 +370,14 @@ int run_tri_chunked(const View &x, const View &y, const View &z, const View &out
 //   D = 128 (`split`): one workgroup per CU with two sets of tiles.  A per-chunk state would cost as
 //            much traffic as an operand, so forward hands over its segments' fp32 entry states
 //            only; backward is a forward-direction walk for dQ (from those entry states,
-//            transposed) and a reverse walk for dK and dV.  The totals kernel keeps two workgroups
-//            per CU busy on a part of the sequence only (the last segment's total is never
-//            needed), so it works on `m` finer segments per walk segment.
+//            transposed) and a reverse walk for dK and dV.  The totals kernel visits a part of the
+//            sequence only (the last segment's total is never needed).
 struct WalkPlan {
     bool ok, split;
     int D, rows;
     int64_t n_chunks, seg_chunks, n_seg;  // the walks' segments
-    int64_t m;                            // totals: finer segments per walk segment (seg_chunks / m chunks each)
-    int64_t fine_bytes;                   // fp32 totals of the finer segments
-    int64_t entry_bytes;                  // fp32 entry states of the walk segments (in place over the totals when m == 1)
-    int64_t work_bytes;                   // workspace of one direction: totals, and entry states when m > 1
+    int64_t entry_bytes;                  // fp32 entry states of the walk segments (formed in place over their totals)
+    int64_t work_bytes;                   // workspace of one direction: the same
     int64_t saved_bytes;                  // what forward hands to backward: the entry states and, behind them, the state
                                           // after the last chunk of every (b, h); with the normaliser at padded head dims
                                           // up to 64, the 16-bit state of every chunk (room for the larger of the two)
@@ -399,22 +396,22 @@ WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     // 256 / 512 / 1024 / 2048 workgroups give 0.265 / 0.231 / 0.243 / 0.268 ms per forward + backward)
     const int64_t target = w.split ? 256 : 512, total = B * H * w.n_chunks;
     w.seg_chunks = total / target > 1 ? total / target : 1;
-    w.m = !w.split ? 1 : w.seg_chunks >= 4 ? 4 : w.seg_chunks >= 2 ? 2 : 1;
-    w.seg_chunks = (w.seg_chunks + w.m - 1) / w.m * w.m;
-    if (w.seg_chunks >= w.n_chunks) w.seg_chunks = w.n_chunks, w.m = 1;  // a single segment: no totals
+    // (totals over finer segments than the walk's, 2 or 4 per walk segment, would put more workgroups on the
+    // totals kernel; measured at D = 128 over B H = 8 ... 256, N = 1024 ... 32768, one total per walk segment
+    // is the fastest everywhere, by 3 to 27 % of a forward + backward step)
+    if (w.seg_chunks >= w.n_chunks) w.seg_chunks = w.n_chunks;  // a single segment: no totals
     w.n_seg = (w.n_chunks + w.seg_chunks - 1) / w.seg_chunks;
     w.entry_bytes = B * H * w.n_seg * w.D * w.D * 4;
-    w.fine_bytes = w.entry_bytes * w.m;
-    w.work_bytes = w.fine_bytes + (w.m > 1 ? w.entry_bytes : 0);  // (a single segment needs them only with a feature map)
+    w.work_bytes = w.entry_bytes;  // (a single segment needs them only with a feature map)
     // (padded head dims up to 64: the per-chunk states of the normalised operator are the larger of the two)
     const int64_t states = w.entry_bytes + B * H * w.D * w.D * 4, per_chunk = B * H * w.n_chunks * w.D * w.D * 2;
     w.saved_bytes = w.split || states > per_chunk ? states : per_chunk;
     return w;
 }
 
-// totals of Y^T Z over the finer segments into `work`, then the walk segments' entry states: their
-// sums over the segments before (reverse == 0) or after (reverse != 0), written to `entry` (null:
-// behind the totals in `work`, or over them when m == 1).  Returns where the entry states are.
+// totals of Y^T Z over the walk's segments into `work`, then the segments' entry states: their sums
+// over the segments before (reverse == 0) or after (reverse != 0), written to `entry` (null: over
+// the totals in `work`).  Returns where the entry states are.
 int walk_entry_states(const WalkPlan &w, const View &y, const View &z, int64_t B, int64_t H, int64_t N, int64_t dy,
                       int64_t dz, int dtype, int reverse, void *work, float *entry, const float **where, hipStream_t s,
                       int map_y = 0, const View *ymap_out = nullptr) {
@@ -424,21 +421,25 @@ int walk_entry_states(const WalkPlan &w, const View &y, const View &z, int64_t B
         tp.yo_b = ymap_out->strides[0], tp.yo_h = ymap_out->strides[1], tp.yo_n = ymap_out->strides[2];
     }
     float *totals = static_cast<float *>(work);
-    if (!entry) entry = w.m == 1 ? totals : reinterpret_cast<float *>(static_cast<char *>(work) + w.fine_bytes);
-    tp.y = y.ptr, tp.z = z.ptr, tp.totals = totals;
+    if (!entry) entry = totals;
+    // (two segments: the one total needed is the other segment's entry state; the totals kernel writes it as the
+    // walks read it, two partial sums, and no scan follows)
+    const bool direct = w.n_seg == 2;
+    tp.y = y.ptr, tp.z = z.ptr, tp.totals = direct ? entry : totals, tp.direct = direct;
     tp.ys_b = y.strides[0], tp.ys_h = y.strides[1], tp.ys_n = y.strides[2];
     tp.zs_b = z.strides[0], tp.zs_h = z.strides[1], tp.zs_n = z.strides[2];
     tp.H = (int32_t)H, tp.N = (int32_t)N, tp.BH = (int32_t)(B * H), tp.dy = (int32_t)dy, tp.dz = (int32_t)dz;
-    const int64_t n_fine = w.n_seg * w.m;
-    tp.n_chunks = (int32_t)w.n_chunks, tp.seg_chunks = (int32_t)(w.seg_chunks / w.m), tp.n_seg = (int32_t)n_fine;
+    tp.n_chunks = (int32_t)w.n_chunks, tp.seg_chunks = (int32_t)w.seg_chunks, tp.n_seg = (int32_t)w.n_seg;
     // the total of the walk's last segment (first, walking in reverse) is under no sum; a feature map
     // is applied by this kernel, which then has to visit every row
-    tp.seg_lo = reverse && !map_y ? (int32_t)w.m : 0;
-    tp.seg_hi = (int32_t)(!reverse && !map_y ? n_fine - w.m : n_fine);
+    tp.seg_lo = reverse && !map_y ? 1 : 0;
+    tp.seg_hi = (int32_t)(!reverse && !map_y ? w.n_seg - 1 : w.n_seg);
+    if (direct) tp.seg_lo = reverse ? 1 : 0, tp.seg_hi = tp.seg_lo + 1;  // (the needed one)
     if (fla::walk_totals(dtype, w.D, tp, s) != hipSuccess) return FLA_ERR_LAUNCH;
     *where = entry;
-    return fla::walk_scan(totals, entry, B * H, (int)w.n_seg, (int)w.m, w.D, fla::walk_totals_cols(w.D, (int)dy, (int)dz),
-                          reverse, s) == hipSuccess
+    if (direct) return FLA_OK;
+    return fla::walk_scan(totals, entry, B * H, (int)w.n_seg, w.D, fla::walk_totals_cols(w.D, (int)dy, (int)dz), reverse,
+                          s) == hipSuccess
                ? FLA_OK
                : FLA_ERR_LAUNCH;
 }
@@ -570,7 +571,7 @@ int wide_forward(const WidePlan &wide, const View &q, const View &k, const View 
         const float *entry = nullptr;
         if (wp.n_seg > 1) {
             float *keep = state_out ? reinterpret_cast<float *>(static_cast<char *>(state_out) + h * wp.saved_bytes) : nullptr;
-            void *work = keep && wp.m == 1 ? static_cast<void *>(keep) : static_cast<void *>(ws + wide.temp_bytes);
+            void *work = keep ? static_cast<void *>(keep) : static_cast<void *>(ws + wide.temp_bytes);
             if (int rc = walk_entry_states(wp, kh, v, B, H, N, wqk, dv, dtype, 0, work, keep, &entry, s)) return rc;
         }
         // (the second half's walk adds its result to the first one's)
@@ -682,18 +683,17 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         // writes phi(xk), which the walk then reads (so it runs for a single segment as well)
         const bool need_totals = wp.n_seg > 1 || fmap;
         // the entry states (and the state after the last chunk) are what backward gets, so the scan writes
-        // them to state_out (m == 1: the totals themselves are computed there, and no workspace is used);
+        // them to state_out (the totals themselves are computed there, and no workspace is used);
         // the normalised operator at padded head dims up to 64 hands over the 16-bit state of every chunk instead
         const bool in_state = state_out && (wp.split || !nx);
-        if (need_totals && !(in_state && wp.m == 1) &&
-            (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 ||
-             workspace_bytes < (in_state ? wp.fine_bytes : wp.work_bytes)))
+        if (need_totals && !in_state &&
+            (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.work_bytes))
             return FLA_ERR_WORKSPACE;
         if (state_out && reinterpret_cast<uintptr_t>(state_out) % 16 != 0) return FLA_ERR_WORKSPACE;
         hipStream_t s = static_cast<hipStream_t>(stream);
         const float *entry = nullptr;
         if (need_totals)
-            if (int rc = walk_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, in_state && wp.m == 1 ? state_out : workspace,
+            if (int rc = walk_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, in_state ? state_out : workspace,
                                            in_state ? static_cast<float *>(state_out) : nullptr, &entry, s, fmap,
                                            fmap ? &mapped[1] : nullptr))
                 return rc;

@@ -55,8 +55,8 @@
 // only into the instantiations that use it.
 //
 // Layout.  An operand tile is C rows x D 16-bit values, row-major, the 16-byte chunk index of
-// a row XORed with swizzle_y (fla_tri_fast.h) -- one layout for the 16-byte row reads (MFMA
-// operands with k along the row) and for the transposing column reads (k down the rows).  A wave
+// a row XORed with walk_swizzle(row) -- one layout, free of bank conflicts for the 16-byte row
+// reads (MFMA operands with k along the row) and for the transposing column reads (k down the rows).  A wave
 // owns one 32-row block of the chunk as the "X rows" of every product (and, at D = 128, one half
 // of the output columns; the two waves of a row block then form the same scores); the MFMA
 // operand chaining is that of the other kernels: S^T = Y X^T leaves a lane holding one X row
@@ -176,7 +176,30 @@ struct WalkOut {
     __device__ static __forceinline__ int db0(int wave) { return W::NCH == 1 ? 0 : (wave / W::NRB) * PER; }
 };
 
-// ---- LDS tile access (tile: row-major [rows][D], chunk index XOR swizzle_y(row))
+// ---- LDS tile access (tile: row-major [rows][D], chunk index XOR walk_swizzle(row))
+
+// XOR applied to the 16-byte chunk index of tile row `row`.  Every tile is read both ways:
+//   * along its rows (walk_row_frag): 16 lanes read the same chunk index of 16 consecutive rows,
+//     which must land in the 16 different 16-byte slots of the 256 bytes that 64 banks span;
+//   * down its columns (walk_col_frag*, transposing 8-byte reads): 32 lanes read 64 consecutive
+//     bytes of each of 4 consecutive rows, which must land in 4 different 64-byte quarters.
+// With 256-byte rows (D = 128) the row's low four bits go into the chunk index with its low two
+// bits on top -- the bits that pick the 64-byte quarter -- and with 128-byte rows (D = 64, where
+// the row's lowest bit already picks a half) bits 1 .. 3, bit 1 on top.  (Folding the bits in
+// unpermuted serves the row reads just as well, but the 4 rows of a column read then meet in the
+// same quarter: a 4-way bank conflict at D = 128, 2-way at D = 64.)
+template <int CR>
+__device__ __forceinline__ int walk_swizzle(int row) {
+    if constexpr (CR == 4) {
+        return (row >> 2) & 3;  // (64-byte rows: the 4 rows of a column read are the 4 quarters)
+    } else if constexpr (CR == 8) {
+        const int t = (row >> 1) & 7;
+        return ((t & 1) << 2) | (t >> 1);
+    } else {
+        const int t = row & 15;
+        return ((t & 3) << 2) | (t >> 2);
+    }
+}
 
 // whole 128-row tile HBM -> LDS; rows >= N and chunks beyond the true width arrive as zeros
 template <int D>
@@ -184,7 +207,7 @@ __device__ __forceinline__ void walk_load_tile(u32x4 rsrc, uint32_t lds_tile, in
                                                int lane) {
     using W = WalkCfg<D>;
     const int r = wave * W::RPI + lane / W::CR;
-    const int c = (lane % W::CR) ^ swizzle_y<W::CR>(r);
+    const int c = (lane % W::CR) ^ walk_swizzle<W::CR>(r);
     const uint32_t voff = (uint32_t)(r * stride2 + c * 16) + (c * 8 < width ? 0u : kOobOffset);
     const uint32_t base = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_tile + wave * 1024));
     u32x4 rs = {(uint32_t)__builtin_amdgcn_readfirstlane((int)rsrc[0]), (uint32_t)__builtin_amdgcn_readfirstlane((int)rsrc[1]),
@@ -200,7 +223,7 @@ __device__ __forceinline__ void walk_load_tile(u32x4 rsrc, uint32_t lds_tile, in
 template <typename T, int D>
 __device__ __forceinline__ typename Mma<T>::V8 walk_row_frag(const unsigned char *tile, int row, int kc, int g) {
     using W = WalkCfg<D>;
-    const int ch = (2 * kc + g) ^ swizzle_y<W::CR>(row);
+    const int ch = (2 * kc + g) ^ walk_swizzle<W::CR>(row);
     return __builtin_bit_cast(typename Mma<T>::V8, *reinterpret_cast<const u32x4 *>(tile + row * W::RB + (ch << 4)));
 }
 
@@ -220,8 +243,8 @@ __device__ __forceinline__ typename Mma<T>::V8 walk_col_frag_perm(const unsigned
     const int lam = lane & 15, g = lane >> 5, beta = (lane >> 4) & 1, zc = lam & 3;
     const int row_lo = R0 + (consecutive ? 8 * g : 4 * g) + (lam >> 2), row_hi = row_lo + (consecutive ? 4 : 8);
     const int ch = 4 * cb + 2 * (zc & 1) + beta, byte = 8 * (zc >> 1);
-    const s16x4 lo = walk_tr_read(tile + row_lo * W::RB + ((ch ^ swizzle_y<W::CR>(row_lo)) << 4) + byte);
-    const s16x4 hi = walk_tr_read(tile + row_hi * W::RB + ((ch ^ swizzle_y<W::CR>(row_hi)) << 4) + byte);
+    const s16x4 lo = walk_tr_read(tile + row_lo * W::RB + ((ch ^ walk_swizzle<W::CR>(row_lo)) << 4) + byte);
+    const s16x4 hi = walk_tr_read(tile + row_hi * W::RB + ((ch ^ walk_swizzle<W::CR>(row_hi)) << 4) + byte);
     return __builtin_bit_cast(typename Mma<T>::V8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 }
 
@@ -233,8 +256,8 @@ __device__ __forceinline__ typename Mma<T>::V8 walk_col_frag(const unsigned char
     const int lam = lane & 15, g = lane >> 5, beta = (lane >> 4) & 1;
     const int row_lo = R0 + 4 * g + (lam >> 2), row_hi = row_lo + 8;
     const int ch = 4 * cb + 2 * beta + ((lam & 3) >> 1), sub = 8 * (lam & 1);
-    const s16x4 lo = walk_tr_read(tile + row_lo * W::RB + ((ch ^ swizzle_y<W::CR>(row_lo)) << 4) + sub);
-    const s16x4 hi = walk_tr_read(tile + row_hi * W::RB + ((ch ^ swizzle_y<W::CR>(row_hi)) << 4) + sub);
+    const s16x4 lo = walk_tr_read(tile + row_lo * W::RB + ((ch ^ walk_swizzle<W::CR>(row_lo)) << 4) + sub);
+    const s16x4 hi = walk_tr_read(tile + row_hi * W::RB + ((ch ^ walk_swizzle<W::CR>(row_hi)) << 4) + sub);
     return __builtin_bit_cast(typename Mma<T>::V8, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
 }
 
@@ -452,7 +475,7 @@ __device__ __forceinline__ void walk_map_tile(unsigned char *tile, int fmap, int
     feature_dispatch(fmap, [&](auto map) {
 #pragma unroll
         for (int v = 0; v < W::C * W::CR / 256; ++v) {
-            const int u = tid + 256 * v, r = u / W::CR, pos = u % W::CR, c = pos ^ swizzle_y<W::CR>(r);
+            const int u = tid + 256 * v, r = u / W::CR, pos = u % W::CR, c = pos ^ walk_swizzle<W::CR>(r);
             if (row0 + r < N && c * 8 < width) {
                 u32x4 *ptr = reinterpret_cast<u32x4 *>(tile + r * W::RB + (pos << 4));
                 const u32x4 m = feature_map8_c<T, decltype(map)::value>(*ptr);
@@ -480,7 +503,7 @@ __device__ __forceinline__ void walk_pack(const f32x16 (&acc)[WalkCfg<D>::DBW], 
             for (int i = 0; i < PER; ++i)
 #pragma unroll
                 for (int hq = 0; hq < 2; ++hq) {
-                    const int ch = (4 * (db0 + i) + 2 * g + hq) ^ swizzle_y<W::CR>(trow);
+                    const int ch = (4 * (db0 + i) + 2 * g + hq) ^ walk_swizzle<W::CR>(trow);
                     const V8 y = __builtin_bit_cast(V8, *reinterpret_cast<const u32x4 *>(ytile + trow * W::RB + (ch << 4)));
 #pragma unroll
                     for (int e = 0; e < 8; ++e) sl[i][hq][e] = feature_slope_c<decltype(map)::value>(static_cast<float>(y[e]));
@@ -625,7 +648,7 @@ __device__ __forceinline__ void walk_state_to_lds(unsigned char *tl, int wave, i
             t4 w;
 #pragma unroll
             for (int b = 0; b < 4; ++b) w[b] = static_cast<T>(st[i][4 * a + b]);
-            *reinterpret_cast<t4 *>(tl + row * W::RB + (((4 * dbk + a) ^ swizzle_y<W::CR>(row)) << 4) + 8 * g) = w;
+            *reinterpret_cast<t4 *>(tl + row * W::RB + (((4 * dbk + a) ^ walk_swizzle<W::CR>(row)) << 4) + 8 * g) = w;
         }
     }
 }
@@ -647,18 +670,12 @@ __device__ __forceinline__ WalkSlice walk_slice(const WalkParams &p) {
     return s;
 }
 
-// this wave's blocks of an fp32 state [D][D] in memory (zeros for a null pointer); `transposed`: the
-// buffer holds the transposed matrix ([v index][q/k index])
-template <int D, typename B = WalkExt<D>>
-__device__ __forceinline__ void walk_load_state(const float *init, bool transposed, int wave, int lane,
+// this wave's blocks of an fp32 state [D][D] in memory, assigned to st or (ADD) added to it;
+// `transposed`: the buffer holds the transposed matrix ([v index][q/k index])
+template <int D, typename B, bool ADD>
+__device__ __forceinline__ void walk_read_state(const float *init, bool transposed, int wave, int lane,
                                                 f32x16 (&st)[WalkCfg<D>::NBW]) {
-    using W = WalkCfg<D>;
     const int l32 = lane & 31, g = lane >> 5;
-#pragma unroll
-    for (int i = 0; i < W::NBW; ++i)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) st[i][v] = 0.f;
-    if (!init) return;
     // st[i][v] = State[r = 32 dbk(i) + 8 (v/4) + 4g + v%4][c = 32 eb + l32]: element r D + c of the
     // buffer, or c D + r when it holds the transposed matrix (then four consecutive floats per v/4)
     const int c = 32 * B::eb(wave) + l32;
@@ -671,7 +688,7 @@ __device__ __forceinline__ void walk_load_state(const float *init, bool transpos
                 for (int a = 0; a < 4; ++a) {
                     const f32x4 t = *reinterpret_cast<const f32x4 *>(init + c * D + 32 * B::dbk(wave, i) + 8 * a + 4 * g);
 #pragma unroll
-                    for (int b = 0; b < 4; ++b) st[i][4 * a + b] = t[b];
+                    for (int b = 0; b < 4; ++b) st[i][4 * a + b] = ADD ? st[i][4 * a + b] + t[b] : t[b];
                 }
             }
     } else {
@@ -679,19 +696,62 @@ __device__ __forceinline__ void walk_load_state(const float *init, bool transpos
         for (int i = 0; i < B::SLOTS; ++i)
             if (B::valid(wave, i)) {
 #pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    st[i][v] = init[(32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + c];
+                for (int v = 0; v < 16; ++v) {
+                    const float t = init[(32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + c];
+                    st[i][v] = ADD ? st[i][v] + t : t;
+                }
             }
     }
 }
 
-// this wave's blocks of the entry state of segment sl.seg (zeros without an init buffer)
+// ... zeros for a null pointer; with `init2` the state is the sum of the two buffers
+template <int D, typename B = WalkExt<D>>
+__device__ __forceinline__ void walk_load_state(const float *init, bool transposed, int wave, int lane,
+                                                f32x16 (&st)[WalkCfg<D>::NBW], const float *init2 = nullptr) {
+    using W = WalkCfg<D>;
+#pragma unroll
+    for (int i = 0; i < W::NBW; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) st[i][v] = 0.f;
+    if (!init) return;
+    walk_read_state<D, B, false>(init, transposed, wave, lane, st);
+    if (init2) walk_read_state<D, B, true>(init2, transposed, wave, lane, st);
+}
+
+// Entry states in memory: one fp32 [D][D] per segment, [bh][seg] -- except with two segments per
+// (b, h), where the first segment in walking order starts from zero and the other one from the one
+// total the totals kernel forms; its two workgroups of a (b, h) then add up half of that segment
+// each, and the two slots hold their partial sums.
+//
+// this wave's blocks of the entry state of segment sl.seg (zeros without an init buffer) of a walk
+// in ascending (`reverse` false) or descending order of the chunks
 template <int D, typename B = WalkExt<D>>
 __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSlice &sl, int wave, int lane,
-                                               f32x16 (&st)[WalkCfg<D>::NBW]) {
-    const float *init = nullptr;
-    if (p.init) init = p.init + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D);
-    walk_load_state<D, B>(init, p.init_transposed != 0, wave, lane, st);
+                                               f32x16 (&st)[WalkCfg<D>::NBW], bool reverse) {
+    const float *init = nullptr, *init2 = nullptr;
+    if (p.init) {
+        if (p.n_seg == 2) {
+            if (sl.seg != (reverse ? 1 : 0)) init = p.init + (int64_t)sl.bh * 2 * (D * D), init2 = init + D * D;
+        } else {
+            init = p.init + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D);
+        }
+    }
+    walk_load_state<D, B>(init, p.init_transposed != 0, wave, lane, st, init2);
+}
+
+// the forward state at the end of segment sl.seg from what forward handed over: the entry state of
+// the next segment (xinit, in the layout above) or, for the last one, the final state (xtotal)
+template <int D, typename B = WalkExt<D>>
+__device__ __forceinline__ void walk_load_end_state(const WalkParams &p, const WalkSlice &sl, int wave, int lane,
+                                                    f32x16 (&xs)[WalkCfg<D>::NBW]) {
+    const float *x = p.xtotal + (int64_t)sl.bh * (D * D), *x2 = nullptr;
+    if (sl.c_hi < p.n_chunks) {
+        if (p.n_seg == 2)
+            x = p.xinit + (int64_t)sl.bh * 2 * (D * D), x2 = x + D * D;
+        else
+            x = p.xinit + ((int64_t)sl.bh * p.n_seg + sl.seg + 1) * (D * D);
+    }
+    walk_load_state<D, B>(x, false, wave, lane, xs, x2);
 }
 
 // ---- one product with its running state, chunks ascending:
@@ -740,7 +800,7 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(O, 0, (N - 1) * os2 + p.wv * 2, 0x00020000);
 
     f32x16 st[W::NBW];
-    walk_load_init<D, B>(p, sl, wave, lane, st);
+    walk_load_init<D, B>(p, sl, wave, lane, st, false);
     walk_state_to_lds<T, D, B>(tl, wave, lane, st);
 
     auto load_chunk = [&](int c, int buf) {
@@ -924,13 +984,11 @@ __global__ __launch_bounds__(256, 2) void walk_bwd_kernel(const WalkParams p) {
     const __amdgpu_buffer_rsrc_t rdv = __builtin_amdgcn_make_buffer_rsrc(DV, 0, (N - 1) * dvs2 + p.wv * 2, 0x00020000);
 
     f32x16 st[W::NBW];  // R[q/k index][v index]
-    walk_load_init<D>(p, sl, wave, lane, st);
+    walk_load_init<D>(p, sl, wave, lane, st, true);
     walk_state_to_lds<T, D>(tl, wave, lane, st);
     f32x16 xs[W::NBW];  // X[q/k index][v index]
     if constexpr (!NORM)
-        walk_load_state<D>(sl.c_hi < p.n_chunks ? p.xinit + ((int64_t)sl.bh * p.n_seg + sl.seg + 1) * (D * D)
-                                                : p.xtotal + (int64_t)sl.bh * (D * D),
-                           false, wave, lane, xs);
+        walk_load_end_state<D>(p, sl, wave, lane, xs);
 
 #pragma unroll 1
     for (int c = sl.c_hi - 1; c >= sl.c_lo; --c) {
@@ -1054,7 +1112,7 @@ __global__ __launch_bounds__(256, 1) void walk_dkdv_kernel(const WalkParams p) {
     const __amdgpu_buffer_rsrc_t rdv = __builtin_amdgcn_make_buffer_rsrc(DV, 0, (N - 1) * dvs2 + p.wv * 2, 0x00020000);
 
     f32x16 st[W::NBW];  // R[q/k index][v index]
-    walk_load_init<D, B>(p, sl, wave, lane, st);
+    walk_load_init<D, B>(p, sl, wave, lane, st, true);
     walk_state_to_lds<T, D, B>(tl, wave, lane, st);
 
     auto load_chunk = [&](int c, int buf) {
@@ -1199,10 +1257,8 @@ __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p
 
     f32x16 st[W::NBW];  // R [q/k index][v index]
     f32x16 xs[W::NBW];  // X [q/k index][v index]
-    walk_load_init<D, B>(p, sl, wave, lane, st);
-    walk_load_state<D, B>(sl.c_hi < p.n_chunks ? p.xinit + ((int64_t)sl.bh * p.n_seg + sl.seg + 1) * (D * D)
-                                               : p.xtotal + (int64_t)sl.bh * (D * D),
-                          false, wave, lane, xs);
+    walk_load_init<D, B>(p, sl, wave, lane, st, true);
+    walk_load_end_state<D, B>(p, sl, wave, lane, xs);
     walk_state_to_lds<T, D, B>(tl, wave, lane, st);
 
     auto load_chunk = [&](int c, int buf) {
@@ -1297,12 +1353,18 @@ struct WalkTotalsParams {
     int32_t n_chunks, seg_chunks, n_seg;
     int32_t seg_lo, seg_hi;  // only segments seg_lo .. seg_hi - 1 are needed (the others' totals stay unwritten)
     float *totals;
+    // two segments: only the total of segment seg_lo is needed, as the other segment's entry state.
+    // The kernel writes it in the layout the walks read (see walk_load_init) -- `totals` is where
+    // the entry states go -- and no scan follows.
+    int32_t direct;
     // feature map on load: Y holds the argument of the map; every Y tile is mapped in LDS as it lands
     // and the mapped rows are written to ymap_out (Y's shape, element strides yo_*).  0: none.
     int32_t map_y;
     void *ymap_out;
     int64_t yo_b, yo_h, yo_n;
 };
+
+constexpr int walk_totals_sets(int D) { return D == 128 ? 4 : 2; }  // sets of (Y, Z) tiles in LDS
 
 template <typename T, int D, int NQ = D / 32, int NV = D / 32>
 __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsParams p) {
@@ -1313,15 +1375,36 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wg = blockIdx.x, xcd = wg & 7, slot = wg >> 3;
-    const int hl = slot / p.n_seg, seg = slot - hl * p.n_seg, bh = hl * 8 + xcd;
-    const int c_lo = seg * p.seg_chunks;
-    const int c_hi = c_lo + p.seg_chunks < p.n_chunks ? c_lo + p.seg_chunks : p.n_chunks;
-    if (bh >= p.BH || seg < p.seg_lo || seg >= p.seg_hi) return;
-    if (c_lo >= p.n_chunks) {  // a segment beyond the end of the sequence: its total is zero
-        float *out = p.totals + ((int64_t)bh * p.n_seg + seg) * (D * D);
+    const int hl = slot / p.n_seg, bh = hl * 8 + xcd;
+    int seg = slot - hl * p.n_seg;
+    if (bh >= p.BH) return;
+    float *out;
+    int c_lo, c_hi;
+    if (p.direct) {
+        // both workgroups of a (b, h) at work: half of the needed segment's chunks each (with a feature map
+        // every row has to be visited: the needed segment's workgroup forms its total alone, the other one
+        // maps its own segment's rows and hands in zeros)
+        const int needed = p.seg_lo, part = seg != needed;
+        out = p.totals + ((int64_t)bh * 2 + part) * (D * D);
+        c_lo = seg * p.seg_chunks;
+        c_hi = c_lo + p.seg_chunks < p.n_chunks ? c_lo + p.seg_chunks : p.n_chunks;
+        if (!p.map_y) {
+            const int n_lo = needed * p.seg_chunks;
+            const int n_hi = n_lo + p.seg_chunks < p.n_chunks ? n_lo + p.seg_chunks : p.n_chunks;
+            const int mid = n_lo + (n_hi - n_lo + 1) / 2;
+            c_lo = part ? mid : n_lo, c_hi = part ? n_hi : mid;
+        }
+    } else {
+        if (seg < p.seg_lo || seg >= p.seg_hi) return;
+        out = p.totals + ((int64_t)bh * p.n_seg + seg) * (D * D);
+        c_lo = seg * p.seg_chunks;
+        c_hi = c_lo + p.seg_chunks < p.n_chunks ? c_lo + p.seg_chunks : p.n_chunks;
+    }
+    if (c_lo >= c_hi) {  // nothing to add up (a segment beyond the end of the sequence, the second half of one chunk)
         for (int i = tid; i < D * D; i += 256) out[i] = 0.f;
         return;
     }
+    const bool discard = p.direct && p.map_y && seg != p.seg_lo;  // (visited for the map only)
     const int b = bh / p.H, h = bh - b * p.H, N = p.N;
     const T *Y = static_cast<const T *>(p.y) + b * p.ys_b + h * p.ys_h;
     const T *Z = static_cast<const T *>(p.z) + b * p.zs_b + h * p.zs_h;
@@ -1334,62 +1417,94 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
     for (int i = 0; i < W::NBW; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v) st[i][v] = 0.f;
-    // two sets of tiles: the loads of chunk c + 1 are in flight while chunk c is multiplied
-    auto load_chunk = [&](int c, int buf) {
-        walk_load_tile<D>(ry, lds0 + buf * 2 * W::TILE, c * W::C, ys2, p.dy, wave, lane);
-        walk_load_tile<D>(rz, lds0 + buf * 2 * W::TILE + W::TILE, c * W::C, zs2, p.dz, wave, lane);
+    // SETS sets of tiles.  Two (two workgroups per CU): the loads of chunk c + 1 are in flight while
+    // chunk c is multiplied.  Four (D = 128, where the grid has at most one workgroup per CU and a
+    // workgroup's own chain load -> barrier -> product bounds its rate): three chunks in flight.
+    constexpr int SETS = walk_totals_sets(D);
+    auto load_chunk = [&](int c, int set) {
+        walk_load_tile<D>(ry, lds0 + set * 2 * W::TILE, c * W::C, ys2, p.dy, wave, lane);
+        walk_load_tile<D>(rz, lds0 + set * 2 * W::TILE + W::TILE, c * W::C, zs2, p.dz, wave, lane);
     };
-    load_chunk(c_lo, 0);
-#pragma unroll 1
-    for (int c = c_lo; c < c_hi; ++c) {
-        const int buf = (c - c_lo) & 1;
-        unsigned char *ty = smem + buf * 2 * W::TILE, *tz = ty + W::TILE;
-        const bool more = c + 1 < c_hi;
-        if (more) load_chunk(c + 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
-        // this wave's loads of chunk c have landed: only those of chunk c + 1 may still be in flight
-        // (the mapped rows' stores of a feature map share the counter: then everything is awaited)
-        if (more && !p.map_y)
-            wait_vm<2 * W::NI>();
-        else
-            wait_vm<0>();
+    auto map_tile = [&](unsigned char *ty, int c) {
+        walk_map_tile<T, D>(ty, p.map_y, c * W::C, N, p.dy, static_cast<T *>(p.ymap_out) + b * p.yo_b + h * p.yo_h,
+                            p.yo_n, tid);
+        __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the rewritten tile is in LDS
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (p.map_y) {
-            walk_map_tile<T, D>(ty, p.map_y, c * W::C, N, p.dy, static_cast<T *>(p.ymap_out) + b * p.yo_b + h * p.yo_h,
-                                p.yo_n, tid);
-            __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the rewritten tile is in LDS
+    };
+    if constexpr (SETS == 2) {
+        load_chunk(c_lo, 0);
+#pragma unroll 1
+        for (int c = c_lo; c < c_hi; ++c) {
+            const int buf = (c - c_lo) & 1;
+            unsigned char *ty = smem + buf * 2 * W::TILE, *tz = ty + W::TILE;
+            const bool more = c + 1 < c_hi;
+            if (more) load_chunk(c + 1, buf ^ 1);  // (every wave has left the barrier that ended the reads of that set)
+            // this wave's loads of chunk c have landed: only those of chunk c + 1 may still be in flight
+            // (the mapped rows' stores of a feature map share the counter: then everything is awaited)
+            if (more && !p.map_y)
+                wait_vm<2 * W::NI>();
+            else
+                wait_vm<0>();
             __builtin_amdgcn_s_barrier();
             asm volatile("" ::: "memory");
+            if (p.map_y) map_tile(ty, c);
+            walk_update<T, D, B>(ty, tz, wave, lane, st);
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS reads of the set are done
+            __builtin_amdgcn_s_barrier();
         }
-        walk_update<T, D, B>(ty, tz, wave, lane, st);
-        asm volatile("" ::: "memory");
-        __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS reads of the set are done
-        __builtin_amdgcn_s_barrier();
+    } else {
+        static_assert(SETS == 4, "the waits below count two chunks behind the awaited one");
+#pragma unroll
+        for (int i = 0; i < SETS - 1; ++i)
+            if (c_lo + i < c_hi) load_chunk(c_lo + i, i);
+        int set = 0;
+#pragma unroll 1
+        for (int c = c_lo; c < c_hi; ++c) {
+            unsigned char *ty = smem + set * 2 * W::TILE, *tz = ty + W::TILE;
+            // this wave's loads of chunk c have landed: those of up to two later chunks may still be in
+            // flight (the mapped rows' stores of a feature map share the counter: then everything is awaited)
+            const int behind = c_hi - 1 - c;
+            if (p.map_y || behind == 0)
+                wait_vm<0>();
+            else if (behind == 1)
+                wait_vm<2 * W::NI>();
+            else
+                wait_vm<4 * W::NI>();
+            __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS reads of the chunk before are done
+            __builtin_amdgcn_s_barrier();        // ... and so are every wave's: its set can be loaded over
+            asm volatile("" ::: "memory");
+            if (c + SETS - 1 < c_hi) load_chunk(c + SETS - 1, (set + SETS - 1) % SETS);
+            if (p.map_y) map_tile(ty, c);
+            walk_update<T, D, B>(ty, tz, wave, lane, st);
+            asm volatile("" ::: "memory");
+            set = (set + 1) % SETS;
+        }
     }
-    float *out = p.totals + ((int64_t)bh * p.n_seg + seg) * (D * D);
 #pragma unroll
     for (int i = 0; i < B::SLOTS; ++i)
         if (B::valid(wave, i)) {
 #pragma unroll
             for (int v = 0; v < 16; ++v)
-                out[(32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * B::eb(wave) + l32] = st[i][v];
+                out[(32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * B::eb(wave) + l32] =
+                    discard ? 0.f : st[i][v];
         }
 #else
     (void)p;
 #endif
 }
 
-// Entry states of the walk's segments from the totals of finer segments, `m` of them per walk
-// segment: entry[bh][s][e] = sum of totals[bh][f][e] over f < s m (reverse == 0) or f >= (s + 1) m
-// (reverse != 0).  Only the totals under those sums are read.  entry may be totals when m == 1 (a
-// thread reads an element before it writes it).  One thread per pair of elements; the loads of up
-// to sixteen segments are issued together (a chain of dependent loads would cost a memory latency
-// each).
+// Entry states of the walk's segments from the segments' totals: entry[bh][s][e] = sum of
+// totals[bh][f][e] over f < s (reverse == 0) or f > s (reverse != 0).  Only the totals under those
+// sums are read.  entry may be totals (a thread reads an element before it writes it).  One thread
+// per pair of elements; the loads of up to sixteen segments are issued together (a chain of
+// dependent loads would cost a memory latency each).
 // `cols`: only the first `cols` columns of every row of the D-wide states are summed (the totals
 // kernel built for a narrow v side writes no others, and no walk of that extent reads them).
 // (a template only so that the header can be included by several translation units)
 template <int kUnused = 0>
-__global__ __launch_bounds__(256) void walk_scan_kernel(const float *totals, float *entry, int n_seg, int m, int E,
+__global__ __launch_bounds__(256) void walk_scan_kernel(const float *totals, float *entry, int n_seg, int E,
                                                         int64_t total2, int reverse, int D, int cols) {
     typedef float f32x2 __attribute__((ext_vector_type(2)));
     const int64_t i2 = (int64_t)blockIdx.x * 256 + threadIdx.x;
@@ -1397,48 +1512,30 @@ __global__ __launch_bounds__(256) void walk_scan_kernel(const float *totals, flo
     const int half = cols / 2;
     const int64_t per_bh = (int64_t)(E / D) * half, bh = i2 / per_bh, r = i2 - bh * per_bh;
     const int64_t e = (r / half) * D + 2 * (r % half);
-    const int n_fine = n_seg * m;
-    const float *pt = totals + bh * n_fine * E + e;
+    const float *pt = totals + bh * n_seg * E + e;
     float *pe = entry + bh * n_seg * E + e;
     const int64_t step = reverse ? -(int64_t)E : (int64_t)E;
-    if (reverse) pt += (int64_t)(n_fine - 1) * E, pe += (int64_t)(n_seg - 1) * E;
+    if (reverse) pt += (int64_t)(n_seg - 1) * E, pe += (int64_t)(n_seg - 1) * E;
     f32x2 run = {0.f, 0.f};
-    if (m == 1) {
-        int s = 0;
-        auto batch = [&](auto nn) {
-            constexpr int NB = decltype(nn)::value;
-            for (; s + NB <= n_seg - 1; s += NB) {
-                f32x2 t[NB];
+    int s = 0;
+    auto batch = [&](auto nn) {
+        constexpr int NB = decltype(nn)::value;
+        for (; s + NB <= n_seg - 1; s += NB) {
+            f32x2 t[NB];
 #pragma unroll
-                for (int u = 0; u < NB; ++u) t[u] = *reinterpret_cast<const f32x2 *>(pt + u * step);
+            for (int u = 0; u < NB; ++u) t[u] = *reinterpret_cast<const f32x2 *>(pt + u * step);
 #pragma unroll
-                for (int u = 0; u < NB; ++u) {
-                    *reinterpret_cast<f32x2 *>(pe + u * step) = run;
-                    run += t[u];
-                }
-                pt += NB * step, pe += NB * step;
+            for (int u = 0; u < NB; ++u) {
+                *reinterpret_cast<f32x2 *>(pe + u * step) = run;
+                run += t[u];
             }
-        };
-        batch(std::integral_constant<int, 16>{});
-        batch(std::integral_constant<int, 4>{});
-        batch(std::integral_constant<int, 1>{});
-        *reinterpret_cast<f32x2 *>(pe) = run;  // the last segment in walking order: its own total is not needed
-        return;
-    }
-    for (int s = 0; s < n_seg; ++s) {
-        *reinterpret_cast<f32x2 *>(pe) = run;
-        pe += step;
-        if (s == n_seg - 1) break;
-        for (int u0 = 0; u0 < m; u0 += 4) {
-            f32x2 t[4];
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-                t[u] = u0 + u < m ? *reinterpret_cast<const f32x2 *>(pt + (u0 + u) * step) : f32x2{0.f, 0.f};
-#pragma unroll
-            for (int u = 0; u < 4; ++u) run += t[u];
+            pt += NB * step, pe += NB * step;
         }
-        pt += m * step;
-    }
+    };
+    batch(std::integral_constant<int, 16>{});
+    batch(std::integral_constant<int, 4>{});
+    batch(std::integral_constant<int, 1>{});
+    *reinterpret_cast<f32x2 *>(pe) = run;  // the last segment in walking order: its own total is not needed
 }
 
 // ---- per-chunk column sums for the normaliser's running vectors: out[bh][c][col] = sum over the
@@ -1547,7 +1644,8 @@ template <typename T, int D>
 hipError_t launch_walk_totals(const WalkTotalsParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-    constexpr int smem = 4 * WalkCfg<D>::TILE;
+    constexpr int smem = walk_totals_sets(D) * 2 * WalkCfg<D>::TILE;
+    if (p.direct && (p.n_seg != 2 || p.seg_lo < 0 || p.seg_lo > 1)) return hipErrorInvalidValue;
     if constexpr (D == 128) {
         if (walk_totals_cols(D, p.dy, p.dz) == 64) {  // z of at most 64 true columns: the state's other v blocks hold zeros
             constexpr auto kern = walk_totals_kernel<T, D, 4, 2>;
@@ -1560,13 +1658,13 @@ hipError_t launch_walk_totals(const WalkTotalsParams &p, hipStream_t stream) {
     return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
 }
 
-inline hipError_t launch_walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, int m, int D, int cols,
+inline hipError_t launch_walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, int D, int cols,
                                    int reverse, hipStream_t stream) {
     const int E = D * D;
     const int64_t total2 = BH * D * (cols / 2);
-    if (m < 1 || (m > 1 && entry == totals) || cols < 2 || cols > D || cols % 2) return hipErrorInvalidValue;
+    if (n_seg < 1 || cols < 2 || cols > D || cols % 2) return hipErrorInvalidValue;
     return launch_kernel(walk_scan_kernel<0>, dim3((unsigned)((total2 + 255) / 256)), dim3(256), 0, stream, totals, entry,
-                         n_seg, m, E, total2, reverse, D, cols);
+                         n_seg, E, total2, reverse, D, cols);
 }
 
 template <auto kern>

@@ -49,6 +49,6 @@ hipError_t walk_bwd(int dtype, int D, const WalkParams &p, hipStream_t stream);
 hipError_t walk_dkdv(int dtype, int D, const WalkParams &p, hipStream_t stream);
 hipError_t walk_vec_sums(int dtype, int D, const WalkVecParams &p, int64_t BH, hipStream_t stream);
 hipError_t walk_vec_scan(float *v, int64_t BH, int n_chunks, int D, int reverse, hipStream_t stream);
-hipError_t walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, int m, int D, int cols, int reverse,
+hipError_t walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, int D, int cols, int reverse,
                      hipStream_t stream);
 }  // namespace fla

@@ -37,9 +37,9 @@ hipError_t walk_vec_sums(int dtype, int D, const WalkVecParams &p, int64_t BH, h
 hipError_t walk_vec_scan(float *v, int64_t BH, int n_chunks, int D, int reverse, hipStream_t stream) {
     return launch_walk_vec_scan(v, BH, n_chunks, D, reverse, stream);
 }
-hipError_t walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, int m, int D, int cols, int reverse,
+hipError_t walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, int D, int cols, int reverse,
                      hipStream_t stream) {
-    return launch_walk_scan(totals, entry, BH, n_seg, m, D, cols, reverse, stream);
+    return launch_walk_scan(totals, entry, BH, n_seg, D, cols, reverse, stream);
 }
 
 }  // namespace fla

@@ -34,6 +34,9 @@ CASES = [
     (1, 2, 768, 256, 64),
     (1, 1, 640, 64, 128),
     (1, 1, 200, 256, 64),
+    # two segments per (b, h): the totals kernel hands the walks their entry states itself
+    (2, 80, 330, 128, 128),
+    (4, 80, 640, 64, 64),
 ]
 
 
@@ -128,6 +131,8 @@ NORMALISED_CASES = [
     (1, 2, 1000, 64, 64),
     (1, 2, 768, 256, 64),
     (1, 1, 200, 96, 32),
+    (2, 80, 330, 128, 128),
+    (4, 80, 640, 64, 64),
 ]
 
 

@@ -38,6 +38,9 @@ CASES = [
     (1, 1, 192, 91, 64),
     (1, 1, 64, 256, 256),
     (1, 2, 1000, 64, 64),
+    # two segments per (b, h): the totals kernel hands the walks their entry states itself
+    (2, 80, 330, 128, 128),
+    (4, 80, 640, 64, 64),
 ]
 
 
