@@ -152,7 +152,8 @@ int fla_tri_xyt_z_chunked(const void *x, const void *y, const void *z, void *out
  *
  * forward:  `state_out` (optional, fla_linear_attn_chunked_state_bytes() bytes, 16-byte aligned)
  *           receives what a later backward call can reuse of the running state (the fp32 state at
- *           the entry of every segment of the walk and after the last chunk; the normalised
+ *           the entry of every segment of the walk -- with two segments per (b, h), two partial
+ *           sums whose sum is the second segment's -- and after the last chunk; the normalised
  *           operator at padded head dims up to 64: the rounded state at the entry of every
  *           chunk); *state_valid (host
  *           memory, optional) is set to 1 when it was written, else 0.

@@ -47,6 +47,11 @@ CASES = [
     (1, 160, 330, 128, 72),
     (2, 80, 330, 256, 64),
     (4, 80, 640, 64, 64),
+    # three and four segments per (b, h)
+    (1, 100, 330, 128, 128),
+    (1, 72, 512, 128, 128),
+    (1, 72, 512, 256, 64),
+    (3, 64, 1024, 64, 64),
 ]
 
 

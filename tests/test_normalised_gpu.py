@@ -41,6 +41,8 @@ CASES = [
     # two segments per (b, h): the totals kernel hands the walks their entry states itself
     (2, 80, 330, 128, 128),
     (4, 80, 640, 64, 64),
+    (1, 100, 330, 128, 128),  # (three segments per (b, h))
+    (3, 64, 1024, 64, 64),
 ]
 
 
