@@ -392,14 +392,19 @@ WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     w.ok = N > (w.split ? 256 : w.rows);  // (D = 128: up to 256 rows one diagonal block of the quadratic kernel does it)
     if (!w.ok) return w;
     w.n_chunks = (N + w.rows - 1) / w.rows;
-    // as many workgroups as are resident at once (measured at B H = 16, N = 32768, D = 64, two per CU:
-    // 256 / 512 / 1024 / 2048 workgroups give 0.265 / 0.231 / 0.243 / 0.268 ms per forward + backward)
-    const int64_t target = w.split ? 256 : 512, total = B * H * w.n_chunks;
-    w.seg_chunks = total / target > 1 ? total / target : 1;
+    // Segments per (b, h): the largest number that keeps B H n_seg within the workgroups that run at once (one per
+    // CU at D = 128, two below; measured at B H = 16, N = 32768, D = 64: 256 / 512 / 1024 / 2048 workgroups give
+    // 0.265 / 0.231 / 0.243 / 0.268 ms per forward + backward).  Workgroups beyond those wait for a free CU and run
+    // as a second round: B H = 192, N = 4096, D = 128 takes 0.87 ms with two unequal segments in 384 workgroups
+    // and 0.53 ms with one segment each; plans of several rounds of shorter segments, chosen by a cost model of
+    // rounds x segment length, measured 5 to 35 % slower than this rule over B H = 65 ... 300.
     // (totals over finer segments than the walk's, 2 or 4 per walk segment, would put more workgroups on the
     // totals kernel; measured at D = 128 over B H = 8 ... 256, N = 1024 ... 32768, one total per walk segment
     // is the fastest everywhere, by 3 to 27 % of a forward + backward step)
-    if (w.seg_chunks >= w.n_chunks) w.seg_chunks = w.n_chunks;  // a single segment: no totals
+    const int64_t resident = w.split ? 256 : 512;
+    int64_t segs = resident / (B * H) > 1 ? resident / (B * H) : 1;
+    if (segs > w.n_chunks) segs = w.n_chunks;
+    w.seg_chunks = (w.n_chunks + segs - 1) / segs;
     w.n_seg = (w.n_chunks + w.seg_chunks - 1) / w.seg_chunks;
     w.entry_bytes = B * H * w.n_seg * w.D * w.D * 4;
     w.work_bytes = w.entry_bytes;  // (a single segment needs them only with a feature map)

@@ -211,9 +211,9 @@ def test_chunkwise_state_and_workspace_sizes():
     assert sb(4, 32, 4096, 128, 128) == 128 * 16 * 128 * 128 * 2 + 128 * 64 * 128 * 4
     # B H = 16, N = 32768, D = 64: 256 chunks of 128 rows
     assert sb(1, 16, 32768, 64, 64) == 16 * 256 * 64 * 64 * 2 + 16 * 256 * 64 * 4
-    # ragged: N = 2450 at D = 128 is 39 chunks of 64 rows in 20 walk segments of 2 (their entry states, and the
-    # state after the last chunk); ten 256-row chunks are less
-    assert sb(2, 8, 2450, 128, 128) == 16 * 21 * 128 * 128 * 4 + 16 * 39 * 128 * 4
+    # ragged: N = 2450 at D = 128 is 39 chunks of 64 rows in 13 walk segments of 3 (16 segments per (b, h) would
+    # fill the chip; their entry states, and the state after the last chunk); ten 256-row chunks are less
+    assert sb(2, 8, 2450, 128, 128) == 16 * 14 * 128 * 128 * 4 + 16 * 39 * 128 * 4
     # three single-chunk segments at D = 32: their fp32 entry states and the final state outweigh three 16-bit states
     assert sb(1, 1, 300, 32, 32) == 4 * 32 * 32 * 4 + 3 * 32 * 4
     # D_qk = 256, D_v = 64: the fp32 entry states of both 128-column halves, 4 walk segments per (b, h), and their

@@ -28,8 +28,8 @@ CASES = [
     (1, 1, 512, 128, 256),
     (1, 2, 576, 48, 48),
     (1, 1, 1024, 32, 32),
-    # several chunks per walking workgroup with a ragged last segment: D = 128 with segments of two and
-    # of four chunks, padded widths, and D = 64
+    # several chunks per walking workgroup with a ragged last segment: D = 128 with segments of three and
+    # of five chunks, padded widths, and D = 64
     (2, 8, 2450, 128, 128),
     (2, 8, 4136, 128, 128),
     (1, 4, 1500, 104, 120),
@@ -40,18 +40,22 @@ CASES = [
     (2, 8, 2450, 136, 24),
     # (a second half of at most 64 columns against a v wider than 64: the forward walk built for a narrow q / k side)
     (1, 3, 1100, 160, 96),
-    # two segments per (b, h): the totals kernel writes the entry states itself (D = 128: two workgroups per total,
-    # one per half of the v columns -- with 56 and with 8 true columns in the upper half), ragged second segment
+    # a B H that leaves no room for a second segment per (b, h) among the workgroups that run at once: one segment
     (2, 80, 320, 128, 128),
-    (2, 80, 330, 104, 120),
-    (1, 160, 330, 128, 72),
-    (2, 80, 330, 256, 64),
     (4, 80, 640, 64, 64),
-    # three and four segments per (b, h)
+    # two segments per (b, h): the totals kernel writes the entry states itself, half a segment per workgroup (three
+    # chunks: two and one), and the walks add the two partial sums; padded widths, a wide q / k, D = 64
     (1, 100, 330, 128, 128),
+    (2, 50, 330, 104, 120),
+    (1, 100, 330, 128, 72),
+    (1, 100, 330, 256, 64),
+    (2, 100, 1024, 64, 64),
+    (2, 100, 900, 64, 64),
+    # three and four segments per (b, h)
     (1, 72, 512, 128, 128),
+    (1, 64, 1024, 128, 128),
     (1, 72, 512, 256, 64),
-    (3, 64, 1024, 64, 64),
+    (1, 160, 1500, 64, 64),
 ]
 
 

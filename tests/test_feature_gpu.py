@@ -35,10 +35,10 @@ CASES = [
     (1, 1, 640, 64, 128),
     (1, 1, 200, 256, 64),
     # two segments per (b, h): the totals kernel hands the walks their entry states itself
-    (2, 80, 330, 128, 128),
-    (4, 80, 640, 64, 64),
-    (1, 100, 330, 128, 128),  # (three segments per (b, h))
-    (3, 64, 1024, 64, 64),
+    (1, 100, 330, 128, 128),
+    (2, 100, 1024, 64, 64),
+    (1, 72, 512, 128, 128),  # (three segments per (b, h))
+    (2, 80, 330, 128, 128),  # (no room for a second segment per (b, h): one)
 ]
 
 
@@ -133,10 +133,10 @@ NORMALISED_CASES = [
     (1, 2, 1000, 64, 64),
     (1, 2, 768, 256, 64),
     (1, 1, 200, 96, 32),
-    (2, 80, 330, 128, 128),
-    (4, 80, 640, 64, 64),
-    (1, 100, 330, 128, 128),  # (three segments per (b, h))
-    (3, 64, 1024, 64, 64),
+    (1, 100, 330, 128, 128),
+    (2, 100, 1024, 64, 64),
+    (1, 72, 512, 128, 128),  # (three segments per (b, h))
+    (2, 80, 330, 128, 128),  # (no room for a second segment per (b, h): one)
 ]
 
 
