@@ -1,5 +1,5 @@
 """Seeded sweep of the chunk-wise operators over shapes the fixed grids do not hit: the plan of
-segments per (b, h), chunks per segment and finer total segments depends on B H and N, the kernels
+segments per (b, h) and chunks per segment depends on B H and N, the kernels
 on the padded head dims -- so head counts, lengths (ragged against 64, 128 and the segment length)
 and widths are drawn at random; forward and backward, with the forward state handed over, against
 the oracle's formula evaluated in fp32 on the GPU (``-m gpu``)."""

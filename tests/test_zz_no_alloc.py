@@ -79,12 +79,13 @@ def test_static_scratch_entry_point_rejects_what_does_not_fit(gpu_device):
 
 
 def test_static_scratch_entry_point_at_other_widths(gpu_device):
-    """D = 128 (two sets of tiles, finer total segments) and D_qk = 256 / D_v = 64 (two halves and a
-    scratch tensor for the second half's output), after the calls above have used the array."""
+    """D = 128 (two sets of tiles) and D_qk = 256 / D_v = 64 (two halves, the second adding to the
+    first one's results), after the calls above have used the array."""
     from helpers import reference_style_inputs
 
     lib = _lib.load()
-    for case, dims in enumerate(((1, 4, 2048, 128, 128), (1, 2, 1024, 256, 64), (1, 3, 700, 128, 128))):
+    # (the last one: two segments per (b, h), whose entry states the totals kernel writes itself)
+    for case, dims in enumerate(((1, 4, 2048, 128, 128), (1, 2, 1024, 256, 64), (1, 3, 700, 128, 128), (1, 200, 900, 64, 64))):
         q, k, v, _ = (t.to(gpu_device) for t in reference_style_inputs(*dims, torch.bfloat16, seed=90 + case))
         want, nbytes = _with_workspace(lib, q, k, v)
         assert 0 < nbytes <= STATIC_BYTES
