@@ -133,12 +133,15 @@ def test_chunked_workspace_errors(gpu_device):
     assert rc == -9
 
 
-def test_chunked_backward_with_and_without_the_forward_state(gpu_device):
-    """Backward given what the forward pass saved, and backward without it (which evaluates the 256-row
-    chunks with states of its own), both match the oracle; shapes that cannot share a state report none."""
+@pytest.mark.parametrize("dims", [(2, 3, 1280, 128, 128), (1, 100, 330, 128, 128), (1, 100, 330, 256, 64), (1, 72, 512, 128, 128),
+                                  (2, 100, 900, 64, 64)], ids=lambda d: "x".join(map(str, d)))
+def test_chunked_backward_with_and_without_the_forward_state(dims, gpu_device):
+    """Backward given what the forward pass saved, and backward without it (D = 128: two walks from entry
+    states it forms again; below: the 256-row chunks with states of their own), both match the oracle -- on
+    plans of many, two and three segments per (b, h); shapes that cannot share a state report none."""
     from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
 
-    q, k, v, dy = (t.to(gpu_device) for t in reference_style_inputs(2, 3, 1280, 128, 128, torch.bfloat16, seed=31))
+    q, k, v, dy = (t.to(gpu_device) for t in reference_style_inputs(*dims, torch.bfloat16, seed=31))
     out, state = linear_attention_chunked_fwd(q, k, v, want_state=True)
     assert state is not None
     plain = linear_attention_chunked_fwd(q, k, v)
@@ -149,6 +152,8 @@ def test_chunked_backward_with_and_without_the_forward_state(gpu_device):
     for name, got, other, w in zip(("dQ", "dK", "dV"), with_state, without, want):
         assert_close(name, got, w)
         assert_close(name + " (no saved state)", other, w)
+    if dims != (2, 3, 1280, 128, 128):
+        return
     # a value head dim wider than the query / key one, and a single chunk: no shared state
     q2, k2, v2, _ = (t.to(gpu_device) for t in reference_style_inputs(1, 2, 1024, 64, 256, torch.bfloat16, seed=32))
     assert linear_attention_chunked_fwd(q2, k2, v2, want_state=True)[1] is None
