@@ -79,6 +79,60 @@ def build(jobs: int | None = None, verbose: bool = True) -> str:
     return LIB_PATH
 
 
+TRACE_LIB_PATH = os.path.join(OBJ_DIR, "trace", "libfla_trace.so")
+
+
+def build_trace(jobs: int | None = None) -> str:
+    """The host-only trace build of the same sources (``-DFLA_TRACE_LAUNCHES``): a library with the
+    same C ABI that makes no launch and writes every launch down instead (kernel, grid, LDS, every
+    argument), plus ``fla_trace_take``.  Runs without a GPU; the launch-plan tests load it."""
+    out_dir = os.path.dirname(TRACE_LIB_PATH)
+    os.makedirs(out_dir, exist_ok=True)
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    flags = ["--offload-arch=gfx950", "--offload-host-only", "-O1", "-std=c++17", "-fPIC", "-DFLA_TRACE_LAUNCHES",
+             "-Wno-unused-command-line-argument", "-I" + INCLUDE, "-I" + CSRC]
+
+    def one(args) -> str:
+        src, obj, defs = args
+        _run([_hipcc(), *flags, *defs, "-c", os.path.join(CSRC, src), "-o", os.path.join(out_dir, obj)])
+        return os.path.join(out_dir, obj)
+
+    work = [("fla_inst.hip", f"inst_t{t}_c{dc}_o{do}.o",
+             [f"-DFLA_INST_DTYPE={t}", f"-DFLA_INST_DC={dc}", f"-DFLA_INST_DO={do}"])
+            for t in (0, 1) for dc in DIMS for do in DIMS]
+    work += [("fla_capi.hip", "fla_capi.o", []), ("fla_walk_inst.hip", "fla_walk_inst.o", []),
+             ("fla_trace.cc", "fla_trace.o", ["-x", "c++"])]
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = list(pool.map(one, work))
+    # A host-only object still registers its (absent) device code with the HIP runtime when it is
+    # loaded: it refers to a code-object symbol that the device link would have made, and calls the
+    # runtime's registration hooks.  The trace library brings both itself -- empty code objects and
+    # hooks that do nothing, bound inside the library -- so that loading it touches no HIP runtime.
+    names = set()
+    for obj in objs:
+        out = subprocess.run(["nm", "-u", obj], stdout=subprocess.PIPE, text=True, check=True).stdout
+        names.update(tok for tok in out.split() if tok.startswith("__hip_fatbin_"))
+    stubs = os.path.join(out_dir, "registration_stubs.c")
+    with open(stubs, "w") as f:
+        for name in sorted(names):
+            f.write(f"const char {name}[64] = {{0}};\n")
+        f.write("void **__hipRegisterFatBinary(const void *d) { static void *h; (void)d; return &h; }\n"
+                "void __hipUnregisterFatBinary(void **h) { (void)h; }\n"
+                "void __hipRegisterFunction(void **m, const void *f, char *a, const char *b, unsigned c, void *d,\n"
+                "                           void *e, void *g, void *h, int *i) {}\n"
+                "void __hipRegisterVar(void **m, void *v, char *a, const char *b, int c, unsigned long d, int e,\n"
+                "                      int g) {}\n")
+    stubs_obj = os.path.join(out_dir, "registration_stubs.o")
+    _run(["gcc", "-O1", "-fPIC", "-c", stubs, "-o", stubs_obj])
+    tmp = TRACE_LIB_PATH + ".tmp"
+    _run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-Wl,-Bsymbolic", "-o", tmp, *objs, stubs_obj])
+    os.replace(tmp, TRACE_LIB_PATH)
+    return TRACE_LIB_PATH
+
+
 if __name__ == "__main__":
-    build()
+    if len(sys.argv) > 1 and sys.argv[1] == "trace":
+        print(build_trace())
+    else:
+        build()
     sys.exit(0)

@@ -25,6 +25,10 @@ std::atomic<void *> g_scratch_ptr[kMaxDevices];
 
 // Device address of `scratch` on the current device (looked up on the first call per device).
 int static_scratch(void **out) {
+#if defined(FLA_TRACE_LAUNCHES)
+    *out = reinterpret_cast<void *>((uintptr_t)0x700000000000ull);  // (no device: a made-up, aligned address)
+    return FLA_OK;
+#endif
     int dev = -1;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return FLA_ERR_LAUNCH;
     void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
@@ -268,7 +272,7 @@ int launch_feature_pass(int mode, int fmap, const View &src, const View &dst, in
     hipStream_t s = static_cast<hipStream_t>(stream);
     hipError_t e;
 #define FLA_FEATURE_PASS(T, V)                                                                                      \
-    fla::launch_kernel(feature_pass_kernel<T, V>, dim3((unsigned)grid), dim3(256), 0, s, mode, fmap,                \
+    fla::launch_kernel<feature_pass_kernel<T, V>>(dim3((unsigned)grid), dim3(256), 0, s, mode, fmap,                \
                        static_cast<const T *>(src.ptr), src.strides[0], src.strides[1], src.strides[2],            \
                        static_cast<T *>(const_cast<void *>(dst.ptr)), dst.strides[0], dst.strides[1], dst.strides[2], \
                        (int)H, N, (int)D, total)
@@ -385,6 +389,7 @@ struct WalkPlan {
 
 WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     WalkPlan w{};
+    if (B <= 0 || H <= 0 || N <= 0) return w;  // (an empty problem has no plan; the callers return before any launch)
     if (pad_index(dqk) != pad_index(dv) || padded(dqk) > 128) return w;
     w.D = (int)padded(dqk);
     w.rows = fla::walk_rows(w.D);
@@ -731,7 +736,9 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         return FLA_OK;
     }
     TriParams p = make_params(q, fmap ? mapped[1] : k, v, o, B, H, N, dqk, dv, 0);
-    const bool k_fast = !fmap || fla::fast_path_ok(make_params(q, k, v, o, B, H, N, dqk, dv, 0));  // xk under the state kernel's loads
+    // with a feature map: xk is read by the state kernel's loads, and phi(xq), phi(xk) are written with 16-byte stores
+    const bool k_fast = !fmap || (fla::fast_path_ok(make_params(q, k, v, o, B, H, N, dqk, dv, 0)) &&
+                                  fla::fast_path_ok(make_params(mapped[0], mapped[1], v, o, B, H, N, dqk, dv, 0)));
     if (!states_shareable(dqk, dv, N) || !fla::fast_path_ok(p) || !k_fast) {
         if (fmap) return FLA_OK;  // *mapped_done stays false: the caller maps with a pass of its own
         return run_tri_chunked(q, k, v, o, B, H, N, dqk, dv, 0, dtype, workspace, workspace_bytes, stream);
@@ -750,7 +757,9 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         return rc;
     if (int rc = chunk_main(p, dqk, dv, dtype, state, 0, stream)) return rc;
     if (mapped_done) *mapped_done = true;
-    if (state_out && state_valid) *state_valid = 1;
+    // (where the walk kernels exist, backward reads a handed-over state in THEIR format: the 256-row
+    // chunks' state written here is not offered, and backward computes its own)
+    if (state_out && state_valid && !wp.ok) *state_valid = 1;
     return FLA_OK;
 }
 
@@ -1237,7 +1246,7 @@ template <typename T>
 hipError_t launch_pack(const View &a, int wa, const View &x, int wx, void *out, int64_t B, int64_t H, int64_t N, int split,
                  int rp, int bias_mode, const float *bias, hipStream_t s) {
     const int64_t total = B * H * N * ((split + rp) / 8);
-    return fla::launch_kernel(pack_pair_kernel<T>, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
+    return fla::launch_kernel<pack_pair_kernel<T>>(dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s,
                               static_cast<const T *>(a.ptr), a.strides[0], a.strides[1], a.strides[2], wa,
                               static_cast<const T *>(x.ptr), x.strides[0], x.strides[1], x.strides[2], wx,
                               static_cast<T *>(out), (int)H, N, split, rp, total, bias_mode, bias);
@@ -1505,14 +1514,17 @@ int fla_linear_attn_chunked_fwd_static(const void *q, const void *k, const void 
     if (int rc = check_common(B, H, N, dtype)) return rc;
     if (D_qk < 1 || D_qk > 256) return FLA_ERR_HEAD_DIM;
     if (D_v < 1 || D_v > 256) return FLA_ERR_V_HEAD_DIM;
-    // what this call's kernels use of the workspace: without a state to hand over, the walk path
-    // needs the segments' entry states only
+    // what this call's kernels use of the workspace: without a state to hand over the walk path needs
+    // the segments' entry states only; operands off that path take the 256-row chunks with their states
+    const View vq{q, q_strides}, vk{k, k_strides}, vv{v, v_strides}, vo{o, o_strides};
+    const View all[] = {vq, vk, vv, vo};
+    for (const View &t : all)
+        if (int rc = check_view(t)) return rc;
     const WalkPlan wp = walk_plan(B, H, N, D_qk, D_v);
     int64_t need = chunked_op_workspace_bytes(B, H, N, D_qk, D_v);
-    if (wp.ok) {
-        const int64_t other = chunked_bytes(B, H, N, D_qk, D_v);  // operands off the speed path
-        need = wp.work_bytes > other ? wp.work_bytes : other;
-    }
+    if (wp.ok)
+        need = fla::fast_path_ok(make_params(vq, vk, vv, vo, B, H, N, D_qk, D_v, 0)) ? wp.work_bytes
+                                                                                      : chunked_bytes(B, H, N, D_qk, D_v);
     if (need > (int64_t)FLA_STATIC_SCRATCH_BYTES) return FLA_ERR_WORKSPACE;
     void *ws = nullptr;
     if (int rc = static_scratch(&ws)) return rc;
@@ -1655,3 +1667,5 @@ int fla_linear_attn_normalised_bwd(const void *grad_out, const void *q, const vo
 }
 
 }  // extern "C"
+
+#include "fla_trace_structs.h"  // (the trace build's descriptions of the parameter structs; empty otherwise)

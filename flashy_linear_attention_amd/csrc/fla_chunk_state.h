@@ -275,7 +275,7 @@ hipError_t launch_chunk_state(ChunkStateParams p, hipStream_t stream) {
         constexpr auto kern = chunk_state_kernel<T, DC, DO>;
         constexpr int smem = ChunkStateLds<DC, DO>::kBytes;
         if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-        return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+        return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), smem, stream, p);
     }
 }
 
@@ -285,7 +285,7 @@ hipError_t launch_chunk_scan(const float *w, void *state, int64_t BH, int n_chun
     const int64_t total2 = BH * E / 2;
     const int64_t grid = (total2 + 255) / 256;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
-    return launch_kernel(chunk_scan_kernel<T>, dim3((unsigned)grid), dim3(256), 0, stream, w, static_cast<T *>(state),
+    return launch_kernel<chunk_scan_kernel<T>>(dim3((unsigned)grid), dim3(256), 0, stream, w, static_cast<T *>(state),
                          n_chunks, E, total2, reverse);
 }
 

@@ -1626,14 +1626,14 @@ __global__ __launch_bounds__(256) void walk_vec_scan_kernel(float *v, int n_chun
 
 inline hipError_t launch_walk_vec_scan(float *v, int64_t BH, int n_chunks, int D, int reverse, hipStream_t stream) {
     if (BH > 65535 || D % 16 != 0) return hipErrorInvalidConfiguration;
-    return launch_kernel(walk_vec_scan_kernel<0>, dim3((unsigned)(D / 16), (unsigned)BH), dim3(256), 0, stream, v, n_chunks,
+    return launch_kernel<walk_vec_scan_kernel<0>>(dim3((unsigned)(D / 16), (unsigned)BH), dim3(256), 0, stream, v, n_chunks,
                          D, reverse);
 }
 
 template <typename T, int D>
 hipError_t launch_walk_vec_sums(const WalkVecParams &p, int64_t BH, hipStream_t stream) {
     if (BH > 65535) return hipErrorInvalidConfiguration;
-    return launch_kernel(walk_vec_sums_kernel<T, D>, dim3((unsigned)p.n_chunks, (unsigned)BH), dim3(256), 0, stream, p);
+    return launch_kernel<walk_vec_sums_kernel<T, D>>(dim3((unsigned)p.n_chunks, (unsigned)BH), dim3(256), 0, stream, p);
 }
 
 // columns of the D x D totals that walk_totals_kernel writes for operands of true widths dy, dz (the
@@ -1650,12 +1650,12 @@ hipError_t launch_walk_totals(const WalkTotalsParams &p, hipStream_t stream) {
         if (walk_totals_cols(D, p.dy, p.dz) == 64) {  // z of at most 64 true columns: the state's other v blocks hold zeros
             constexpr auto kern = walk_totals_kernel<T, D, 4, 2>;
             if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-            return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+            return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), smem, stream, p);
         }
     }
     constexpr auto kern = walk_totals_kernel<T, D>;
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-    return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+    return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), smem, stream, p);
 }
 
 inline hipError_t launch_walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, int D, int cols,
@@ -1663,14 +1663,14 @@ inline hipError_t launch_walk_scan(const float *totals, float *entry, int64_t BH
     const int E = D * D;
     const int64_t total2 = BH * D * (cols / 2);
     if (n_seg < 1 || cols < 2 || cols > D || cols % 2) return hipErrorInvalidValue;
-    return launch_kernel(walk_scan_kernel<0>, dim3((unsigned)((total2 + 255) / 256)), dim3(256), 0, stream, totals, entry,
+    return launch_kernel<walk_scan_kernel<0>>(dim3((unsigned)((total2 + 255) / 256)), dim3(256), 0, stream, totals, entry,
                          n_seg, E, total2, reverse, D, cols);
 }
 
 template <auto kern>
 hipError_t launch_walk_kernel(int64_t grid, int smem, const WalkParams &p, hipStream_t stream) {
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-    return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+    return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), smem, stream, p);
 }
 
 template <typename T, int D>
@@ -1715,13 +1715,13 @@ hipError_t launch_walk_bwd(const WalkParams &p, hipStream_t stream) {
         constexpr auto kern = walk_bwd_kernel<T, D, true>;
         constexpr int smem_n = smem + WalkCfg<D>::VEC;
         if (hipError_t e = ensure_dynamic_lds<kern>(smem_n)) return e;
-        return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem_n, stream, p);
+        return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), smem_n, stream, p);
     }
     if (!p.xtotal || (p.n_seg > 1 && !p.xinit)) return hipErrorInvalidValue;
     constexpr auto kern = walk_bwd_kernel<T, D, false>;
     constexpr int smem_x = smem + WalkCfg<D>::STATE;  // X's copy beside R's
     if (hipError_t e = ensure_dynamic_lds<kern>(smem_x)) return e;
-    return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem_x, stream, p);
+    return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), smem_x, stream, p);
 }
 
 template <typename T, int D>
@@ -1734,18 +1734,18 @@ hipError_t launch_walk_dkdv(const WalkParams &p, hipStream_t stream) {
         if (!p.rc) return hipErrorInvalidValue;
         constexpr auto kern = walk_dkdv_kernel<T, D, true>;
         if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-        return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+        return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), smem, stream, p);
     }
     if constexpr (D == 128) {
         if (!p.fmap && p.wqk > 64 && p.wv <= 64) {
             constexpr auto kern = walk_dkdv_kernel<T, D, false, 4, 2>;
             if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-            return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+            return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), smem, stream, p);
         }
     }
     constexpr auto kern = walk_dkdv_kernel<T, D, false>;
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-    return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+    return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), smem, stream, p);
 }
 
 template <typename T, int D>

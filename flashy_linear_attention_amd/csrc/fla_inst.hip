@@ -50,3 +50,5 @@ int FLA_CHUNK_ROWS_NAME(FLA_INST_DC, FLA_INST_DO)() {
 #endif
 
 }  // namespace fla
+
+#include "fla_trace_structs.h"  // (the trace build's descriptions of the parameter structs; empty otherwise)

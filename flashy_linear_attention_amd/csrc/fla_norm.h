@@ -151,7 +151,9 @@ __global__ __launch_bounds__(256) void norm_chunk_sums_kernel(const NormParams p
 }
 
 // ---- chunk sums -> exclusive prefix sums over the chunks (ksum) and exclusive suffix sums
-// (wsum, when given), in place.  One thread per (batch-head, column).
+// (wsum, when given), in place.  One thread per (batch-head, column).  (A template only so that the
+// definition may sit in a header that several translation units include.)
+template <int kUnused = 0>
 __global__ __launch_bounds__(256) void norm_scan_kernel(float *ksum, float *wsum, int BH, int chunks, int DP) {
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (t >= (int64_t)BH * DP) return;
@@ -404,7 +406,7 @@ inline int norm_chunk_rows(int lpr) { return 4 * (64 / lpr) * kNormSegRows; }
 
 inline hipError_t launch_norm_scan(const NormParams &p, int dp, bool with_w, hipStream_t s) {
     const int64_t threads = (int64_t)p.BH * dp;
-    return launch_kernel(norm_scan_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, p.ksum,
+    return launch_kernel<norm_scan_kernel<0>>(dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, p.ksum,
                          with_w ? p.wsum : nullptr, p.BH, p.n_chunks, dp);
 }
 
@@ -415,17 +417,17 @@ hipError_t launch_norm_lpr(int which, const NormParams &p, hipStream_t s) {
     // every launch is checked on its own: nothing further is enqueued after a failed one
     if (which == 0) {
         if (p.n_chunks > 1) {
-            if (hipError_t e = launch_kernel(norm_chunk_sums_kernel<T, LPR, VEC, false>, grid, dim3(256), 0, s, p)) return e;
+            if (hipError_t e = launch_kernel<norm_chunk_sums_kernel<T, LPR, VEC, false>>(grid, dim3(256), 0, s, p)) return e;
             if (hipError_t e = launch_norm_scan(p, LPR * 8, false, s)) return e;
         }
-        return launch_kernel(norm_fwd_kernel<T, LPR, VEC>, grid, dim3(256), 0, s, p);
+        return launch_kernel<norm_fwd_kernel<T, LPR, VEC>>(grid, dim3(256), 0, s, p);
     }
-    if (which == 1) return launch_kernel(norm_bwd_pre_kernel<T, LPR, VEC>, grid, dim3(256), 0, s, p);
+    if (which == 1) return launch_kernel<norm_bwd_pre_kernel<T, LPR, VEC>>(grid, dim3(256), 0, s, p);
     if (p.n_chunks > 1) {
-        if (hipError_t e = launch_kernel(norm_chunk_sums_kernel<T, LPR, VEC, true>, grid, dim3(256), 0, s, p)) return e;
+        if (hipError_t e = launch_kernel<norm_chunk_sums_kernel<T, LPR, VEC, true>>(grid, dim3(256), 0, s, p)) return e;
         if (hipError_t e = launch_norm_scan(p, LPR * 8, true, s)) return e;
     }
-    return launch_kernel(norm_bwd_post_kernel<T, LPR, VEC>, dim3(grid.x, grid.y, p.only_dk ? 1 : 2), dim3(256), 0, s, p);
+    return launch_kernel<norm_bwd_post_kernel<T, LPR, VEC>>(dim3(grid.x, grid.y, p.only_dk ? 1 : 2), dim3(256), 0, s, p);
 }
 
 // lpr from norm_lanes_per_row; vec: every operand of this call qualifies for 16-byte accesses

@@ -1003,10 +1003,14 @@ __global__ __launch_bounds__(256, (FastConfig<DC, DO, true>::kMinWavesPerSimd)) 
 }
 
 // True when the fast kernel can take this problem: every operand 16-byte
-// aligned with widths in whole chunks, and each (b, h) slice addressable with
-// 32-bit byte offsets.
+// aligned with widths in whole chunks, rows that do not overlap, and each
+// (b, h) slice addressable with 32-bit byte offsets.
 inline bool fast_path_ok(const TriParams &p) {
     if (!(p.vec_x && p.vec_y && p.vec_z && p.vec_out)) return false;
+    // Rows beyond N are aimed past the end of a buffer resource that covers rows 0 .. N-1 and arrive
+    // as zeros: with a row stride below the width (a tensor expanded along the sequence has stride
+    // 0) those offsets would fall inside it again.  Such operands take the bounds-checked kernel.
+    if (p.xs_n < p.dc || p.ys_n < p.dc || p.zs_n < p.dout || p.os_n < p.dout) return false;
     const int64_t n = p.N;
     return n * p.xs_n * 2 <= kMaxFastExtent && n * p.ys_n * 2 <= kMaxFastExtent && n * p.zs_n * 2 <= kMaxFastExtent;
 }
@@ -1069,7 +1073,7 @@ hipError_t launch_tri_fast_variant(TriParams p, hipStream_t stream) {
         constexpr auto kern = tri_xyt_z_fast_kernel<T, DC, DO, CHUNKED, FLAGS>;
         constexpr int smem = Cfg::SMEM_BYTES + (Cfg::kStateInLds ? Cfg::STATE_BYTES : 0);
         if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-        return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, p);
+        return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), smem, stream, p);
     }
 }
 
@@ -1087,7 +1091,7 @@ hipError_t launch_tri_fast_batch(TriBatch b, int count, hipStream_t stream) {
         if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
         constexpr auto kern = tri_xyt_z_fast_batch_kernel<T, DC, DO>;
         if (hipError_t e = ensure_dynamic_lds<kern>(Cfg::SMEM_BYTES)) return e;
-        return launch_kernel(kern, dim3((unsigned)grid, (unsigned)count), dim3(256), Cfg::SMEM_BYTES, stream, b);
+        return launch_kernel<kern>(dim3((unsigned)grid, (unsigned)count), dim3(256), Cfg::SMEM_BYTES, stream, b);
     }
 }
 
@@ -1109,7 +1113,7 @@ hipError_t launch_tri_fast_chunked_batch(TriBatch b, int count, hipStream_t stre
         constexpr auto kern = tri_xyt_z_fast_chunked_batch_kernel<T, DC, DO>;
         constexpr int smem = Cfg::SMEM_BYTES + (Cfg::kStateInLds ? Cfg::STATE_BYTES : 0);
         if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-        return launch_kernel(kern, dim3((unsigned)grid), dim3(256), smem, stream, b, count);
+        return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), smem, stream, b, count);
     }
 }
 

@@ -382,7 +382,7 @@ hipError_t launch_tri(TriParams p, hipStream_t stream) {
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     constexpr auto kern = tri_xyt_z_kernel<T, DC, DO>;
     if (hipError_t e = ensure_dynamic_lds<kern>(Cfg::SMEM_BYTES)) return e;
-    return launch_kernel(kern, dim3((unsigned)grid), dim3(256), Cfg::SMEM_BYTES, stream, p);
+    return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), Cfg::SMEM_BYTES, stream, p);
 }
 
 }  // namespace fla

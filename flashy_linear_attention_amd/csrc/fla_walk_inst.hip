@@ -43,3 +43,5 @@ hipError_t walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, i
 }
 
 }  // namespace fla
+
+#include "fla_trace_structs.h"  // (the trace build's descriptions of the parameter structs; empty otherwise)

@@ -257,9 +257,13 @@ int fla_feature_attn_normalised_bwd(const void *grad_out, const void *q, const v
  * counterpart in the reference.  Same arguments and results as fla_linear_attn_chunked_fwd with
  * state_out = NULL; the scratch its kernels need (per-chunk states and their running sums) lives
  * in a static device array of FLA_STATIC_SCRATCH_BYTES that every GPU the library runs on holds
- * until the process ends.  The call allocates and frees nothing.  Problems whose
- * fla_linear_attn_chunked_workspace_bytes() exceeds FLA_STATIC_SCRATCH_BYTES are rejected with
- * FLA_ERR_WORKSPACE before anything is enqueued.  All calls on one GPU share that array (it keeps
+ * until the process ends.  The call allocates and frees nothing.  A problem whose kernels need more
+ * scratch than FLA_STATIC_SCRATCH_BYTES is rejected with FLA_ERR_WORKSPACE before anything is
+ * enqueued.  What they need depends on the path the operands take: equal padded head dims up to 128
+ * with 16-byte aligned rows use the segments' fp32 entry states only (at most 256 (D <= 64: 512)
+ * states of D x D, 16 MiB at D = 128, whatever B, H and N); other shapes and layouts use the
+ * per-chunk states, fla_chunked_workspace_bytes() or, for D_qk in (128, 256] with D_v <= 128,
+ * fla_linear_attn_chunked_workspace_bytes().  All calls on one GPU share that array (it keeps
  * the previous call's contents; the kernels overwrite what they read): calls that overlap in
  * time on one GPU -- different streams, different host threads -- race; calls on one stream do not. */
 #define FLA_STATIC_SCRATCH_BYTES (64 * 1024 * 1024)

@@ -1,0 +1,251 @@
+"""The launch plans of the operators, enumerated and checked on the CPU (tests/launch_plan.py):
+every launch an operator call would make -- from the library's real host code, compiled into a
+trace build that records instead of launching -- against the hardware's limits and against
+lane-level models of the kernels' index arithmetic.
+
+The grids include the random sweep of the normalised operator in which one run once went silent
+(bf16, B 2, H 80, N 300, D_qk = D_v = 72, quadratic evaluation) and every other case of that
+sweep's space: head-dim pairs x (batch, heads) x lengths x both evaluations.
+"""
+
+import ctypes
+import itertools
+
+import pytest
+
+import launch_plan as lp
+
+DIMS = [(64, 64), (32, 32), (48, 64), (64, 40), (128, 128), (96, 128), (128, 72), (104, 120), (256, 64), (160, 96),
+        (72, 72)]
+BHS = [1, 2, 3, 8, 16, 17, 40, 64, 160, 200, 320, 400]
+NS = [129, 257, 300, 513, 640, 1000, 1301, 2048, 2450, 3000, 4100]
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return lp.trace_lib()
+
+
+def _clip_n(bh, n, dqk, dv):
+    """the sweep's size limit (its own loop had no exit for B H = 320, 400 at D_qk = 256: see
+    test_the_silent_sweep_stopped_in_its_own_size_loop)"""
+    while bh * n * max(dqk, dv) > 16 * 4100 * 128 and n > 129:
+        n = max(129, n // 2 + 1)
+    return n
+
+
+def _workspace(arena, name, nbytes):
+    return arena.alloc(name, max(int(nbytes), 16))
+
+
+def trace_normalised(lib, b, h, n, dqk, dv, chunked, dtype=0, layout="contiguous"):
+    """fla_linear_attn_normalised_fwd + _bwd as LinearAttentionNormalised calls them."""
+    arena = lp.Arena()
+    q, k = (lp.make_tensor(arena, nm, b, h, n, dqk, layout) for nm in ("q", "k"))
+    v = lp.make_tensor(arena, "v", b, h, n, dv, layout)
+    o, g = (lp.make_tensor(arena, nm, b, h, n, dv) for nm in ("out", "grad_out"))
+    dq, dk = (lp.make_tensor(arena, nm, b, h, n, dqk) for nm in ("dq", "dk"))
+    dvv = lp.make_tensor(arena, "dv", b, h, n, dv)
+    denom = arena.alloc("denom", 4 * b * h * n)
+    wbytes = lib.fla_normalised_workspace_bytes(b, h, n, dqk, dv, int(chunked))
+    sbytes = lib.fla_linear_attn_chunked_state_bytes(b, h, n, dqk, dv) if chunked else 0
+    state = arena.alloc("state", sbytes) if sbytes else None
+    valid = ctypes.c_int32(0)
+    launches = []
+    work = _workspace(arena, "forward workspace", wbytes)
+    rc = lib.fla_linear_attn_normalised_fwd(q.ptr, k.ptr, v.ptr, o.ptr, denom, b, h, n, dqk, dv, q.strides_arg(),
+                                            k.strides_arg(), v.strides_arg(), o.strides_arg(), 1e-5, dtype, int(chunked),
+                                            state, ctypes.byref(valid), work, wbytes, None)
+    assert rc == 0, rc
+    launches += lp.take_launches(lib)
+    work2 = _workspace(arena, "backward workspace", wbytes)
+    rc = lib.fla_linear_attn_normalised_bwd(g.ptr, q.ptr, k.ptr, v.ptr, o.ptr, denom, dq.ptr, dk.ptr, dvv.ptr, b, h, n,
+                                            dqk, dv, g.strides_arg(), q.strides_arg(), k.strides_arg(), v.strides_arg(),
+                                            o.strides_arg(), dq.strides_arg(), dk.strides_arg(), dvv.strides_arg(), dtype,
+                                            int(chunked), state if valid.value else None, work2, wbytes, None)
+    assert rc == 0, rc
+    launches += lp.take_launches(lib)
+    return arena, launches
+
+
+def trace_plain(lib, b, h, n, dqk, dv, chunked, dtype=0, layout="contiguous", with_state=True):
+    """forward + backward of the plain operator: the quadratic entry points or the chunk-wise ones."""
+    arena = lp.Arena()
+    q, k = (lp.make_tensor(arena, nm, b, h, n, dqk, layout) for nm in ("q", "k"))
+    v = lp.make_tensor(arena, "v", b, h, n, dv, layout)
+    out_layout = "contiguous" if layout == "expanded" else layout  # (results have rows of their own)
+    g = lp.make_tensor(arena, "grad_out", b, h, n, dv, layout)
+    o = lp.make_tensor(arena, "out", b, h, n, dv, out_layout)
+    dq, dk = (lp.make_tensor(arena, nm, b, h, n, dqk, out_layout) for nm in ("dq", "dk"))
+    dvv = lp.make_tensor(arena, "dv", b, h, n, dv, out_layout)
+    launches = []
+    if not chunked:
+        # (the primitive: the small-V forward wrapper keeps the reference's power-of-two rule for D_v)
+        rc = lib.fla_tri_xyt_z(q.ptr, k.ptr, v.ptr, o.ptr, b, h, n, dqk, dv, q.strides_arg(), k.strides_arg(),
+                               v.strides_arg(), o.strides_arg(), 0, dtype, None)
+        assert rc == 0, rc
+        rc = lib.fla_linear_attn_smallv_bwd(g.ptr, q.ptr, k.ptr, v.ptr, dq.ptr, dk.ptr, dvv.ptr, b, h, n, dqk, dv,
+                                            g.strides_arg(), q.strides_arg(), k.strides_arg(), v.strides_arg(),
+                                            dq.strides_arg(), dk.strides_arg(), dvv.strides_arg(), dtype, None)
+        assert rc == 0, rc
+        return arena, lp.take_launches(lib)
+    wbytes = lib.fla_linear_attn_chunked_workspace_bytes(b, h, n, dqk, dv)
+    sbytes = lib.fla_linear_attn_chunked_state_bytes(b, h, n, dqk, dv) if with_state else 0
+    state = arena.alloc("state", sbytes) if sbytes else None
+    valid = ctypes.c_int32(0)
+    work = _workspace(arena, "forward workspace", wbytes)
+    rc = lib.fla_linear_attn_chunked_fwd(q.ptr, k.ptr, v.ptr, o.ptr, b, h, n, dqk, dv, q.strides_arg(), k.strides_arg(),
+                                         v.strides_arg(), o.strides_arg(), dtype, state, ctypes.byref(valid), work, wbytes,
+                                         None)
+    assert rc == 0, rc
+    launches += lp.take_launches(lib)
+    work2 = _workspace(arena, "backward workspace", wbytes)
+    rc = lib.fla_linear_attn_chunked_bwd(g.ptr, q.ptr, k.ptr, v.ptr, dq.ptr, dk.ptr, dvv.ptr, b, h, n, dqk, dv,
+                                         g.strides_arg(), q.strides_arg(), k.strides_arg(), v.strides_arg(),
+                                         dq.strides_arg(), dk.strides_arg(), dvv.strides_arg(), dtype,
+                                         state if valid.value else None, work2, wbytes, None)
+    assert rc == 0, rc
+    launches += lp.take_launches(lib)
+    return arena, launches
+
+
+SWEEP_OUTPUT = """\
+case 0: chunked=False b=2 h=1 n=4100 dqk=64 dv=40
+case 1: chunked=False b=2 h=200 n=129 dqk=128 dv=128
+case 2: chunked=True b=2 h=160 n=258 dqk=48 dv=64
+case 3: chunked=True b=4 h=10 n=129 dqk=104 dv=120
+case 4: chunked=False b=1 h=17 n=1000 dqk=48 dv=64
+case 5: chunked=True b=1 h=400 n=151 dqk=128 dv=72
+case 6: chunked=True b=1 h=1 n=257 dqk=96 dv=128
+case 7: chunked=False b=2 h=32 n=300 dqk=48 dv=64
+case 8: chunked=False b=2 h=80 n=300 dqk=72 dv=72
+"""
+
+
+def test_the_silent_sweep_stopped_in_its_own_size_loop():
+    """What the sweep printed before it went silent, replayed: its generator (random.Random(seed),
+    four choices per case, a loop that halves N while B H N max(D) exceeds a limit, then the choice of
+    the evaluation) reproduces the nine printed lines for exactly one seed below 1000, and that seed's
+    tenth draw is D_qk = 256, B H = 320, N = 129 -- above the limit with N at its floor, so the halving
+    loop `while ...: n = max(129, n // 2 + 1)` never ends.  The sweep stopped on the host, in its own
+    loop, after case 8 had passed and before printing case 9; no kernel was running."""
+    import random
+
+    limit = 16 * 4100 * 128
+    hits = []
+    for seed in range(1000):
+        rng = random.Random(seed)
+        lines, stuck = [], None
+        for i in range(10):
+            dqk, dv = rng.choice(DIMS)
+            bh = rng.choice(BHS)
+            b = rng.choice([d for d in (1, 2, 4) if bh % d == 0])
+            n = rng.choice(NS)
+            while bh * n * max(dqk, dv) > limit:
+                if max(129, n // 2 + 1) == n:
+                    stuck = (i, dqk, dv, bh, n)
+                    break
+                n = max(129, n // 2 + 1)
+            if stuck:
+                break
+            chunked = rng.choice([True, True, False])
+            lines.append(f"case {i}: chunked={chunked} b={b} h={bh // b} n={n} dqk={dqk} dv={dv}")
+        if "\n".join(lines) + "\n" == SWEEP_OUTPUT:
+            hits.append((seed, stuck))
+    assert hits == [(78, (9, 256, 64, 320, 129))]
+    assert 320 * 129 * 256 > limit
+
+
+def test_the_case_that_once_went_silent(lib):
+    """bf16, B 2, H 80, N 300, D_qk = D_v = 72, quadratic evaluation of the normalised operator: the
+    launches it makes, named, with their grids -- and all of them sound."""
+    arena, launches = trace_normalised(lib, 2, 80, 300, 72, 72, chunked=False)
+    got = [(l.kernel, tuple(l.targs), l.grid, l.lds) for l in launches]
+    assert got == [
+        # forward: the product with the normaliser inside (row sums of the masked scores), single-tile mode
+        ("tri_xyt_z_fast_kernel", ("bf16", 128, 128, False, 1), (320, 1, 1), 163840),
+        # backward: dO = g / n and dn; the three gradient products in one launch; chunk sums of k and
+        # dn q (2 chunks of 256 rows); their scan; the normaliser's terms added to dQ and dK
+        ("norm_bwd_pre_kernel", ("bf16", 16, True), (2, 160, 1), 0),
+        ("tri_xyt_z_fast_batch_kernel", ("bf16", 128, 128), (320, 3, 1), 163840),
+        ("norm_chunk_sums_kernel", ("bf16", 16, True, True), (2, 160, 1), 0),
+        ("norm_scan_kernel", (0,), (80, 1, 1), 0),
+        ("norm_bwd_post_kernel", ("bf16", 16, True), (2, 160, 2), 0),
+    ]
+    stats = lp.Stats()
+    lp.check_all(arena, launches, stats)
+    assert stats.workgroups > 0 and stats.lane_accesses > 100000
+
+
+@pytest.mark.parametrize("dims", DIMS, ids=lambda d: f"{d[0]}x{d[1]}")
+def test_normalised_operator_over_the_sweep_space(lib, dims):
+    dqk, dv = dims
+    stats = lp.Stats()
+    cases = 0
+    for bh, n0, chunked in itertools.product(BHS, NS, (False, True)):
+        n = _clip_n(bh, n0, dqk, dv)
+        # (the lane-level model is the slow part: every (B H, N) for the shapes of the silent case,
+        # a thinned grid for the others)
+        if dims != (72, 72) and (bh + n0) % 5 != 0:
+            continue
+        b = 2 if bh % 2 == 0 and bh > 1 else 1
+        arena, launches = trace_normalised(lib, b, bh // b, n, dqk, dv, chunked)
+        lp.check_all(arena, launches, stats)
+        cases += 1
+    assert cases > 25 and stats.launches > cases * 4
+
+
+@pytest.mark.parametrize("dims", DIMS + [(256, 256), (40, 40), (25, 25), (91, 91), (128, 32), (200, 200)],
+                         ids=lambda d: f"{d[0]}x{d[1]}")
+@pytest.mark.parametrize("chunked", (False, True), ids=("quadratic", "chunkwise"))
+def test_plain_operator(lib, dims, chunked):
+    dqk, dv = dims
+    stats = lp.Stats()
+    for (bh, n), dtype, layout in itertools.product(((1, 64), (3, 192), (17, 1000), (64, 2048), (160, 300), (256, 512),
+                                                     (128, 4096)), (0, 1),
+                                                    ("contiguous", "bnhd", "padded", "odd", "expanded")):
+        if layout != "contiguous" and (bh + n + dtype) % 2:
+            continue
+        n = _clip_n(bh, n, dqk, dv)
+        b = 2 if bh % 2 == 0 and bh > 1 else 1
+        for with_state in ((True, False) if chunked else (True,)):
+            arena, launches = trace_plain(lib, b, bh // b, n, dqk, dv, chunked, dtype, layout, with_state)
+            lp.check_all(arena, launches, stats)
+    assert stats.launches > 0
+
+
+def test_rows_expanded_along_the_sequence_take_the_bounds_checked_kernel(lib):
+    """A row stride below the width (stride 0: one row repeated) would defeat the fast kernels' zero fill
+    of the rows beyond N -- the range check of their buffer loads sees offsets inside the one stored
+    row -- so such operands must go to the kernel with element-wise bounds checks."""
+    arena, launches = trace_plain(lib, 1, 2, 300, 64, 64, chunked=False, layout="expanded")
+    assert launches and all(l.kernel == "tri_xyt_z_kernel" for l in launches)
+    arena, launches = trace_plain(lib, 1, 2, 300, 64, 64, chunked=True, layout="expanded")
+    assert launches and all(l.kernel == "tri_xyt_z_kernel" for l in launches)
+
+
+def test_benchmark_shapes(lib):
+    """C2 - C5 of the benchmark, both evaluations, and the normalised operator on C3 and C5."""
+    stats = lp.Stats()
+    for b, h, n, dqk, dv, dtype in ((4, 16, 2048, 64, 64, 1), (4, 32, 4096, 128, 128, 0), (4, 16, 4096, 256, 64, 0),
+                                    (1, 16, 32768, 64, 64, 0)):
+        for chunked in (False, True):
+            arena, launches = trace_plain(lib, b, h, n, dqk, dv, chunked, dtype)
+            lp.check_all(arena, launches, stats)
+            arena, launches = trace_normalised(lib, b, h, n, dqk, dv, chunked, dtype)
+            lp.check_all(arena, launches, stats)
+    assert stats.kernels["tri_xyt_z_fast_batch_kernel"] >= 4 and stats.kernels["walk_bwd_rev_kernel"] >= 1
+
+
+def test_empty_problems_make_no_launch(lib):
+    """B = 0 or H = 0 at a length that has a chunk-wise plan: sizes are 0, calls succeed, nothing is enqueued."""
+    for b, h in ((0, 2), (2, 0)):
+        for dqk, dv in ((64, 64), (128, 128), (256, 64)):
+            assert lib.fla_linear_attn_chunked_workspace_bytes(b, h, 1024, dqk, dv) == 0
+            assert lib.fla_linear_attn_chunked_state_bytes(b, h, 1024, dqk, dv) == 0
+            assert lib.fla_normalised_workspace_bytes(b, h, 1024, dqk, dv, 1) == 0
+            assert lib.fla_linear_attn_prefers_chunked(b, h, 1024, dqk, dv) == 0
+            arena, launches = trace_plain(lib, b, h, 1024, dqk, dv, chunked=True)
+            assert launches == []
+            arena, launches = trace_normalised(lib, b, h, 1024, dqk, dv, chunked=True)
+            assert launches == []

@@ -43,6 +43,12 @@ CASES = [
     (2, 100, 1024, 64, 64),
     (1, 72, 512, 128, 128),  # (three segments per (b, h))
     (2, 80, 330, 128, 128),  # (no room for a second segment per (b, h): one)
+    # fast-path widths that are whole 16-byte chunks but no power of two, many heads, ragged length:
+    # single row tiles per workgroup with chunks of the padded width out of range
+    (2, 80, 300, 72, 72),
+    (1, 200, 513, 104, 120),
+    (2, 32, 300, 48, 64),
+    (1, 160, 257, 120, 72),
 ]
 
 

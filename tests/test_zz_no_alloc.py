@@ -67,15 +67,35 @@ def test_static_scratch_entry_point_matches_the_workspace_one(gpu_device):
 
 
 def test_static_scratch_entry_point_rejects_what_does_not_fit(gpu_device):
+    """Rows that are not 16-byte aligned take the 256-row chunks, whose states (about 200 MB at this
+    size) do not fit the array; the same size with aligned rows needs 16 MiB of entry states and runs
+    (first case of the test above at a smaller size, and the benchmark shape below)."""
     lib = _lib.load()
-    b, h, n, d = 4, 32, 4096, 128  # needs about 200 MB of chunk states
-    assert lib.fla_linear_attn_chunked_workspace_bytes(b, h, n, d, d) > STATIC_BYTES
+    b, h, n, d = 4, 32, 4096, 128
+    assert lib.fla_chunked_workspace_bytes(b, h, n, d, d) > STATIC_BYTES
     q = torch.zeros(1, 1, 64, d, dtype=torch.bfloat16, device=gpu_device)  # never read: the call is refused first
-    s = (ctypes.c_int64 * 4)(h * n * d, n * d, d, 1)
+    rs = d + 1  # row stride in elements: rows start at odd multiples of 2 bytes
+    s = (ctypes.c_int64 * 4)(h * n * rs, n * rs, rs, 1)
     fake = [ctypes.c_void_p(q.data_ptr() + (i << 32)) for i in range(4)]
     rc = lib.fla_linear_attn_chunked_fwd_static(*fake, b, h, n, d, d, s, s, s, s, 0, _stream())
     assert rc == -9, lib.fla_strerror(rc)
     torch.cuda.synchronize()
+
+
+def test_static_scratch_entry_point_at_the_benchmark_shape(gpu_device):
+    """B 4, H 32, N 4096, D 128: two segments per (b, h), 16 MiB of the array."""
+    from helpers import reference_style_inputs
+
+    lib = _lib.load()
+    q, k, v, _ = (t.to(gpu_device) for t in reference_style_inputs(4, 32, 4096, 128, 128, torch.bfloat16, seed=97))
+    want, _ = _with_workspace(lib, q, k, v)
+    out = torch.full_like(v, float("nan"))
+    before = torch.cuda.memory_allocated()
+    rc = _static(lib, q, k, v, out)
+    assert rc == 0, lib.fla_strerror(rc)
+    assert torch.cuda.memory_allocated() == before
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
 
 
 def test_static_scratch_entry_point_at_other_widths(gpu_device):
