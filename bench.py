@@ -59,6 +59,10 @@ PROFILED_TRAFFIC = {
 PROFILED_MFMA_RATIO = {("C3", "quadratic"): (1.008, "profiles/tri_xyt_z_fast_kernels_C3_pmc.md")}
 
 ALGOS = ["quadratic", "chunked", "normalised", "normalised-chunked", "poly", "feature"]
+# how the quadratic backward is evaluated: "products" = dQ, dV, dK as three products in one launch (the
+# library's choice); "fused-dkdv" = dV and dK by one kernel from one stream of (Q, dO) tiles plus dQ's
+# product (fla_linear_attn_bwd_fused_dkdv, the measured alternative)
+BWD_PLAN = "products"
 
 
 def _parse():
@@ -76,6 +80,9 @@ def _parse():
     ap.add_argument("--no-other-workloads", action="store_true",
                     help="skip the short runs of the other workloads that the default run appends")
     ap.add_argument("--other-steps", type=int, default=50, help="timed iterations per entry of other_workloads")
+    ap.add_argument("--bwd-plan", choices=["products", "fused-dkdv"], default="products",
+                    help="evaluation of the quadratic backward (see BWD_PLAN); the default is what the library's "
+                         "operators use")
     ap.add_argument("--algo", default="quadratic", choices=ALGOS,
                     help="quadratic: the tiled O(N^2 D) kernels the headline metric is defined on (default); "
                          "chunked: the O(N) chunk-state path, reported with its own FLOP count and an HBM roofline; "
@@ -201,6 +208,10 @@ def _ops(torch, w, algo, dev):
     fwd = linear_flash_wrapper_fwd_smallv_hd if w.small_v else linear_flash_wrapper_fwd
     bwd = linear_flash_wrapper_bwd_smallv_hd if w.small_v else linear_flash_wrapper_bwd
     op = LinearAttentionSmallVHD if w.small_v else LinearAttention
+    if BWD_PLAN == "fused-dkdv" and algo == "quadratic":
+        from flashy_linear_attention_amd.kernels.linear_attn_kernels import linear_flash_wrapper_bwd_fused_dkdv
+
+        bwd = linear_flash_wrapper_bwd_fused_dkdv
     if algo in ("chunked", "normalised-chunked"):
         from flashy_linear_attention_amd.chunked import linear_attention_chunked_bwd, linear_attention_chunked_fwd
 
@@ -265,6 +276,78 @@ def _other_workload(torch, name, algo, dev, steps):
                     "own_tflops": round((ff + fb) / (ms_step * 1e-3) / 1e12, 1),
                     "bytes": "each operand read once, each result written once"})
     del o
+    torch.cuda.empty_cache()
+    return rec
+
+
+def _other_extension(torch, name, algo, dev, steps):
+    """A short run of one of the operators beyond the reference's two (normaliser inside, feature map on
+    load, polynomial score map) with the caller-side PyTorch recipe it replaces timed beside it."""
+    import argparse
+
+    from flashy_linear_attention_amd.synthetic import WORKLOADS
+
+    w = WORKLOADS[name]
+    short = argparse.Namespace(steps=steps, warmup=10, settle_seconds=0.15)
+    if algo in ("poly", "feature"):
+        full = (_bench_poly if algo == "poly" else _bench_feature)(torch, short, w, dev)
+        c, r = full["config"], full["roofline"]
+        rec = {"workload": name, "algo": algo, "dtype": "bf16", "steps": steps,
+               "shape": f"B={w.batch} H={w.heads} N={w.seq} D_qk={w.d_qk} D_v={w.d_v}", "step_ms": full["ms_per_step"],
+               "bound": r["bound"], "frac_of_peak": r["frac"]}
+        if algo == "poly":
+            rec.update({"own_tflops": full["value"], "flops": "its own causal-counted FLOPs (scores over the 16-wide x)",
+                        "materialised_features_step_ms": c["materialised_features_step_ms"],
+                        "speedup_vs_materialised_features": c["speedup_vs_materialised_features"]})
+        else:
+            rec.update({"gbps_algorithmic": full["value"], "algorithmic_bytes_per_step": c["algorithmic_bytes_per_step"],
+                        "bytes": "the plain operator's tensors (xq, xk for q, k) plus phi(xq), phi(xk) written once",
+                        "autograd_step_ms": c["median_ms"]["autograd_step"],
+                        "pytorch_elu_passes_plus_chunked_operator_autograd_step_ms":
+                            c["pytorch_elu_passes_plus_chunked_operator_autograd_step_ms"],
+                        "speedup_vs_pytorch_elu_passes": c["speedup_vs_pytorch_elu_passes"]})
+        torch.cuda.empty_cache()
+        return rec
+    from flashy_linear_attention_amd import LinearAttention, LinearAttentionSmallVHD
+    from flashy_linear_attention_amd.normalised import linear_attention_normalised_bwd, linear_attention_normalised_fwd
+    from flashy_linear_attention_amd.synthetic import make_inputs
+
+    chunked = algo == "normalised-chunked"
+    q, k, v, do = (t.to(dev) for t in make_inputs(w, seed=0))
+    out, denom, state = linear_attention_normalised_fwd(q, k, v, 1e-5, chunked, want_state=True)
+
+    def step():
+        linear_attention_normalised_fwd(q, k, v, 1e-5, chunked, want_state=chunked)
+        linear_attention_normalised_bwd(do, q, k, v, out, denom, chunked, state)
+
+    def recipe_step():  # README.md:27-30 of the reference around the quadratic operator, through autograd
+        qr, kr, vr = (t.detach().requires_grad_(True) for t in (q, k, v))
+        num = (LinearAttentionSmallVHD if w.small_v else LinearAttention).apply(qr, kr, vr)
+        (num / ((qr * kr.cumsum(-2)).sum(dim=-1, keepdim=True) + 1e-5)).backward(do)
+
+    _settle(torch, step, 0.15)
+    for _ in range(10):
+        step()
+    ms_step = _median_ms(torch, step, steps)
+    for _ in range(3):
+        recipe_step()
+    ms_recipe = _median_ms(torch, recipe_step, max(5, steps // 5))
+    rec = {"workload": name, "algo": algo, "dtype": "bf16", "steps": steps,
+           "shape": f"B={w.batch} H={w.heads} N={w.seq} D_qk={w.d_qk} D_v={w.d_v}", "step_ms": round(ms_step, 4),
+           "pytorch_recipe_step_ms": round(ms_recipe, 4), "speedup_vs_pytorch_recipe": round(ms_recipe / ms_step, 2)}
+    if chunked:
+        e = float(w.batch * w.heads * w.seq)
+        nbytes = w.bytes_fwd + w.bytes_bwd + 4.0 * e + 4.0 * e + 2.0 * e * w.d_v
+        gbs = nbytes / (ms_step * 1e-3) / 1e9
+        rec.update({"bound": "hbm", "gbps_algorithmic": round(gbs, 1), "frac_of_peak": round(gbs / HBM_PEAK_GBS, 4),
+                    "algorithmic_bytes_per_step": nbytes,
+                    "bytes": "the plain operator's (operands read once, results written once) plus n written and read "
+                             "and the saved output read in backward"})
+    else:
+        tf = (w.flops_fwd + w.flops_bwd) / (ms_step * 1e-3) / 1e12
+        rec.update({"bound": "mfma", "tflops": round(tf, 1), "frac_of_peak": round(tf / PEAK_TFLOPS["bf16"], 4),
+                    "flops": "quadratic algorithm, causal-counted (the normaliser's passes add time, no counted FLOPs)"})
+    del q, k, v, do, out, denom, state
     torch.cuda.empty_cache()
     return rec
 
@@ -427,7 +510,7 @@ def _cpu_baseline(torch, w, target_seconds):
     }
 
 
-def _bench_poly(torch, args, w, dev) -> int:
+def _bench_poly(torch, args, w, dev):
     """C4's function, O = tril(phi(xq) phi(xk)^T) V with phi(x) = flatten(x (x) x) / sqrt 2, evaluated
     from the 16-wide x with the polynomial score map f(u) = u^2 / 2, next to the same step on the
     materialised 256-wide features (LinearAttentionSmallVHD's kernels) in the same run."""
@@ -438,7 +521,7 @@ def _bench_poly(torch, args, w, dev) -> int:
 
     if w.features != "taylor2":
         print("bench.py: --algo poly needs a workload whose q, k are Taylor features (C4)", file=sys.stderr)
-        return 2
+        return None
     r = math.isqrt(w.d_qk)
     gen = torch.Generator().manual_seed(0)
     xq = (0.5 * torch.randn(w.batch, w.heads, w.seq, r, generator=gen)).to(w.dtype)
@@ -492,11 +575,10 @@ def _bench_poly(torch, args, w, dev) -> int:
                      "achieved": round(value, 2), "peak": PEAK_TFLOPS["bf16"], "unit": "TFLOP/s",
                      "frac": round(value / PEAK_TFLOPS["bf16"], 4), "traffic": None},
     }
-    print(json.dumps(result))
-    return 0
+    return result
 
 
-def _bench_feature(torch, args, w, dev) -> int:
+def _bench_feature(torch, args, w, dev):
     """The chunk-wise operator from the raw inputs xq, xk (q = elu(xq) + 1, k = elu(xk) + 1 formed while
     the kernels load them, gradients with respect to xq, xk), against the same function built the
     caller's way: elu passes in PyTorch around LinearAttentionChunked, differentiated by autograd."""
@@ -505,7 +587,7 @@ def _bench_feature(torch, args, w, dev) -> int:
 
     if w.features != "elu1" or not w.backward:
         print("bench.py: --algo feature needs a forward + backward workload with elu(x) + 1 features (C3, C5)", file=sys.stderr)
-        return 2
+        return None
     gen = torch.Generator().manual_seed(0)
     xq, xk = (torch.randn(w.batch, w.heads, w.seq, w.d_qk, generator=gen).to(w.dtype).to(dev) for _ in range(2))
     v, do = (torch.randn(w.batch, w.heads, w.seq, w.d_v, generator=gen).to(w.dtype).to(dev) for _ in range(2))
@@ -568,12 +650,13 @@ def _bench_feature(torch, args, w, dev) -> int:
                      "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None, "algorithmic_bytes_per_step": bytes_step},
     }
-    print(json.dumps(result))
-    return 0
+    return result
 
 
 def main() -> int:
+    global BWD_PLAN
     args = _parse()
+    BWD_PLAN = args.bwd_plan
     if args.gpus != 1:
         print("bench.py: this build runs the hot path on ONE GPU only (every (batch, head) slice is independent; "
               "no collective exists on this path). Re-run with --gpus 1.", file=sys.stderr)
@@ -595,10 +678,12 @@ def main() -> int:
         return _sweep(torch, dev, min(args.steps, 30))
     if args.crossover:
         return _crossover(torch, dev, min(args.steps, 30))
-    if args.algo == "poly":
-        return _bench_poly(torch, args, w, dev)
-    if args.algo == "feature":
-        return _bench_feature(torch, args, w, dev)
+    if args.algo in ("poly", "feature"):
+        rec = (_bench_poly if args.algo == "poly" else _bench_feature)(torch, args, w, dev)
+        if rec is None:
+            return 2
+        print(json.dumps(rec))
+        return 0
     normalised = args.algo.startswith("normalised")
     chunked = args.algo in ("chunked", "normalised-chunked")
     o = _ops(torch, w, "chunked" if chunked else "quadratic", dev)
@@ -692,9 +777,14 @@ def main() -> int:
         flops_launch = flops_step / launches
         executed_launch = flops_product * products / launches
         ms_launch = ms_step / launches
+    if BWD_PLAN == "fused-dkdv" and batched_bwd:
+        # two launches: the fused dV + dK kernel and dQ's product; figures below are for the pair of them
+        launches = 3
+        kernel_name = ("fla::tri_pair_upper_kernel (dV and dK from one stream of (Q, dO) tiles) + fla::tri_xyt_z_fast_kernel "
+                       "(dQ): the backward's two launches together")
     achieved = flops_launch / (ms_launch * 1e-3) / 1e12
     executed = executed_launch / (ms_launch * 1e-3) / 1e12
-    traffic, traffic_src = PROFILED_TRAFFIC.get((w.name, "quadratic"), (None, None))
+    traffic, traffic_src = PROFILED_TRAFFIC.get((w.name, "quadratic" if BWD_PLAN == "products" else BWD_PLAN), (None, None))
     mfma_ratio, mfma_src = PROFILED_MFMA_RATIO.get((w.name, "quadratic"), (None, None))
     alg_bytes_launch = (w.bytes_bwd if batched_bwd else (w.bytes_fwd + (w.bytes_bwd if w.backward else 0.0)) / launches)
 
@@ -717,6 +807,7 @@ def main() -> int:
                         f"{'fwd+bwd' if w.backward else 'fwd'}, {dt_name}, B={w.batch} H={w.heads} N={w.seq} "
                         f"D_qk={w.d_qk} D_v={w.d_v}, q/k features {w.features}, v and dO randn, seed 0",
             "flops_per_step": flops_step,
+            "bwd_plan": BWD_PLAN,
             "clock_settle_steps": settle_steps,
             "fwd_ms": round(ms_fwd, 4),
             "bwd_ms": None if ms_bwd is None else round(ms_bwd, 4),
@@ -863,6 +954,11 @@ def main() -> int:
             _other_workload(torch, name, algo, dev, args.other_steps)
             for name, algo in (("C2", "quadratic"), ("C4", "quadratic"), ("C5", "quadratic"),
                                ("C3", "chunked"), ("C4", "chunked"), ("C5", "chunked"))
+        ] + [
+            # the operators beyond the reference's two, each beside the PyTorch recipe it replaces
+            _other_extension(torch, name, algo, dev, min(args.other_steps, 30))
+            for name, algo in (("C3", "normalised"), ("C3", "normalised-chunked"), ("C5", "normalised-chunked"),
+                               ("C3", "feature"), ("C4", "poly"))
         ]
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = _cpu_baseline(torch, w, args.cpu_seconds)

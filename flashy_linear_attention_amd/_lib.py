@@ -12,7 +12,7 @@ import threading
 
 _PKG_DIR = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_PKG_DIR, "libfla_gfx950.so")
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 FLA_DTYPE_BF16 = 0
 FLA_DTYPE_F16 = 1
@@ -29,6 +29,7 @@ SIGNATURES = {
     "fla_linear_attn_bwd": ([_ptr] * 7 + [_i64] * 4 + [_strides] * 7 + [ctypes.c_int, _ptr], ctypes.c_int),
     "fla_linear_attn_smallv_fwd": ([_ptr] * 4 + [_i64] * 5 + [_strides] * 4 + [ctypes.c_int, _ptr], ctypes.c_int),
     "fla_linear_attn_smallv_bwd": ([_ptr] * 7 + [_i64] * 5 + [_strides] * 7 + [ctypes.c_int, _ptr], ctypes.c_int),
+    "fla_linear_attn_bwd_fused_dkdv": ([_ptr] * 7 + [_i64] * 5 + [_strides] * 7 + [ctypes.c_int, _ptr], ctypes.c_int),
     "fla_tri_xyt_z": ([_ptr] * 4 + [_i64] * 5 + [_strides] * 4 + [ctypes.c_int, ctypes.c_int, _ptr], ctypes.c_int),
     "fla_chunked_workspace_bytes": ([_i64] * 5, ctypes.c_int64),
     "fla_tri_xyt_z_chunked": ([_ptr] * 4 + [_i64] * 5 + [_strides] * 4 + [ctypes.c_int, ctypes.c_int, _ptr, _i64, _ptr],

@@ -71,8 +71,12 @@ def build(jobs: int | None = None, verbose: bool = True) -> str:
     _run([_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, "fla_capi.hip"), "-o", capi])
     walk = os.path.join(OBJ_DIR, "fla_walk_inst.o")
     _run([_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, "fla_walk_inst.hip"), "-o", walk])
+    # (this one without the VGPR form of MFMA: see the file's header)
+    pair = os.path.join(OBJ_DIR, "fla_pair_inst.o")
+    pair_flags = [f for f in HIPCC_FLAGS if f not in ("-mllvm", "-amdgpu-mfma-vgpr-form")]
+    _run([_hipcc(), *pair_flags, "-c", os.path.join(CSRC, "fla_pair_inst.hip"), "-o", pair])
     tmp = LIB_PATH + ".tmp"
-    _run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, capi, walk, *objs])
+    _run([_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, capi, walk, pair, *objs])
     os.replace(tmp, LIB_PATH)
     if verbose:
         print(f"built {LIB_PATH} ({os.path.getsize(LIB_PATH) / 1e6:.1f} MB, {len(objs)} kernel objects)")
@@ -101,6 +105,7 @@ def build_trace(jobs: int | None = None) -> str:
              [f"-DFLA_INST_DTYPE={t}", f"-DFLA_INST_DC={dc}", f"-DFLA_INST_DO={do}"])
             for t in (0, 1) for dc in DIMS for do in DIMS]
     work += [("fla_capi.hip", "fla_capi.o", []), ("fla_walk_inst.hip", "fla_walk_inst.o", []),
+             ("fla_pair_inst.hip", "fla_pair_inst.o", []),
              ("fla_trace.cc", "fla_trace.o", ["-x", "c++"])]
     with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as pool:
         objs = list(pool.map(one, work))

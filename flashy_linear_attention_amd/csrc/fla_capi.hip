@@ -1015,6 +1015,29 @@ int backward_products(const View &go, const View &q, const View &k, const View &
     return run_tri(v, go, q, dk, B, H, N, dvw, dqk, 1, dtype, stream);
 }
 
+// The same gradients with dV and dK from one stream of (Q, dO) tiles (fla_tri_pair.h) and dQ as a
+// product of its own: equal padded head dims up to 128, operands on the fast path.
+int backward_fused_dkdv(const View &go, const View &q, const View &k, const View &v, const View &dq, const View &dk,
+                        const View &dv, int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dvw, int dtype,
+                        void *stream) {
+    const View all[] = {go, q, k, v, dq, dk, dv};
+    for (const View &t : all)
+        if (int rc = check_view(t)) return rc;
+    if (int rc = check_alias_bwd(go, q, k, v, nullptr, dq, dk, dv, B, H, N, dqk, dvw)) return rc;
+    if (pad_index(dqk) != pad_index(dvw) || padded(dqk) > 128) return FLA_ERR_UNSUPPORTED;
+    if (B == 0 || H == 0 || N == 0) return FLA_OK;
+    const TriParams pq = make_params(go, v, k, dq, B, H, N, dvw, dqk, 0);
+    const TriParams pv = make_params(k, q, go, dv, B, H, N, dqk, dvw, 1);
+    const TriParams pk = make_params(v, go, q, dk, B, H, N, dvw, dqk, 1);
+    if (!fla::fast_path_ok(pq) || !fla::fast_path_ok(pv) || !fla::fast_path_ok(pk)) return FLA_ERR_UNSUPPORTED;
+    typedef hipError_t (*pair_fn)(const TriParams &, const TriParams &, hipStream_t);
+    static const pair_fn table[3][2] = {{fla::FLA_PAIR_NAME(0, 32), fla::FLA_PAIR_NAME(1, 32)},
+                                        {fla::FLA_PAIR_NAME(0, 64), fla::FLA_PAIR_NAME(1, 64)},
+                                        {fla::FLA_PAIR_NAME(0, 128), fla::FLA_PAIR_NAME(1, 128)}};
+    if (table[pad_index(dqk)][dtype](pv, pk, static_cast<hipStream_t>(stream)) != hipSuccess) return FLA_ERR_LAUNCH;
+    return run_tri(go, v, k, dq, B, H, N, dvw, dqk, 0, dtype, stream);
+}
+
 int backward(const View &go, const View &q, const View &k, const View &v, const View &dq, const View &dk,
              const View &dv, int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dvw, int dtype, void *stream) {
     const View all[] = {go, q, k, v, dq, dk, dv};
@@ -1437,6 +1460,18 @@ int fla_linear_attn_smallv_bwd(const void *grad_out, const void *q, const void *
     if (D_v < 1 || D_v > 256) return FLA_ERR_V_HEAD_DIM;
     return backward({grad_out, go_strides}, {q, q_strides}, {k, k_strides}, {v, v_strides}, {dq, dq_strides},
                     {dk, dk_strides}, {dv, dv_strides}, B, H, N, D_qk, D_v, dtype, stream);
+}
+
+int fla_linear_attn_bwd_fused_dkdv(const void *grad_out, const void *q, const void *k, const void *v, void *dq, void *dk,
+                                   void *dv, int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                                   const int64_t *go_strides, const int64_t *q_strides, const int64_t *k_strides,
+                                   const int64_t *v_strides, const int64_t *dq_strides, const int64_t *dk_strides,
+                                   const int64_t *dv_strides, int dtype, void *stream) {
+    if (int rc = check_common(B, H, N, dtype)) return rc;
+    if (D_qk < 1 || D_qk > 256) return FLA_ERR_HEAD_DIM;
+    if (D_v < 1 || D_v > 256) return FLA_ERR_V_HEAD_DIM;
+    return backward_fused_dkdv({grad_out, go_strides}, {q, q_strides}, {k, k_strides}, {v, v_strides}, {dq, dq_strides},
+                               {dk, dk_strides}, {dv, dv_strides}, B, H, N, D_qk, D_v, dtype, stream);
 }
 
 int fla_tri_xyt_z(const void *x, const void *y, const void *z, void *out, int64_t B, int64_t H, int64_t N,

@@ -22,6 +22,8 @@
 #define FLA_BATCH_NAME(t, d) FLA_BATCH_NAME_(t, d)
 #define FLA_CBATCH_NAME_(t, d) fla_launch_chunked_batch_t##t##_d##d
 #define FLA_CBATCH_NAME(t, d) FLA_CBATCH_NAME_(t, d)
+#define FLA_PAIR_NAME_(t, d) fla_launch_pair_t##t##_d##d
+#define FLA_PAIR_NAME(t, d) FLA_PAIR_NAME_(t, d)
 
 namespace fla {
 #define FLA_DECLARE(dc, dout)                                                               \
@@ -40,6 +42,12 @@ FLA_FOR_EACH_DIM_PAIR(FLA_DECLARE)
     hipError_t FLA_CBATCH_NAME(1, d)(const TriBatch &b, int count, hipStream_t stream);
 FLA_DECLARE_BATCH(32) FLA_DECLARE_BATCH(64) FLA_DECLARE_BATCH(128) FLA_DECLARE_BATCH(256)
 #undef FLA_DECLARE_BATCH
+// two upper products that stream the same tiles (fla_tri_pair.h: the backward's dV and dK), padded head dims up to 128
+#define FLA_DECLARE_PAIR(d)                                                                          \
+    hipError_t FLA_PAIR_NAME(0, d)(const TriParams &a, const TriParams &b, hipStream_t stream);      \
+    hipError_t FLA_PAIR_NAME(1, d)(const TriParams &a, const TriParams &b, hipStream_t stream);
+FLA_DECLARE_PAIR(32) FLA_DECLARE_PAIR(64) FLA_DECLARE_PAIR(128)
+#undef FLA_DECLARE_PAIR
 // walk kernels (fla_chunk_walk.h), dtype 0 bf16 / 1 f16, padded head dim D = 32, 64 or 128
 // (walk_bwd: 32 and 64; walk_dkdv, walk_bwd_rev: 128)
 hipError_t walk_totals(int dtype, int D, const WalkTotalsParams &p, hipStream_t stream);

@@ -2,6 +2,7 @@
 //   -DFLA_INST_DTYPE={0 bf16 | 1 f16} -DFLA_INST_DC=<32|64|128|256> -DFLA_INST_DO=<32|64|128|256>
 #include "fla_dispatch.h"
 #include "fla_tri_fast.h"
+#include "fla_tri_pair.h"
 
 #if !defined(FLA_INST_DTYPE) || !defined(FLA_INST_DC) || !defined(FLA_INST_DO)
 #error "define FLA_INST_DTYPE, FLA_INST_DC and FLA_INST_DO"
@@ -37,6 +38,12 @@ hipError_t FLA_BATCH_NAME(FLA_INST_DTYPE, FLA_INST_DC)(const TriBatch &b, int co
 
 hipError_t FLA_CBATCH_NAME(FLA_INST_DTYPE, FLA_INST_DC)(const TriBatch &b, int count, hipStream_t stream) {
     return launch_tri_fast_chunked_batch<InstT, FLA_INST_DC, FLA_INST_DO>(b, count, stream);
+}
+#endif
+
+#if FLA_INST_DC == FLA_INST_DO && FLA_INST_DC <= 64  // (128: fla_pair_inst.hip)
+hipError_t FLA_PAIR_NAME(FLA_INST_DTYPE, FLA_INST_DC)(const TriParams &a, const TriParams &b, hipStream_t stream) {
+    return launch_tri_pair<InstT, FLA_INST_DC>(a, b, stream);
 }
 #endif
 

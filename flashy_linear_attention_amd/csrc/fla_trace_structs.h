@@ -9,6 +9,7 @@
 #include "fla_chunk_walk.h"
 #include "fla_norm.h"
 #include "fla_tri_kernel.h"
+#include "fla_tri_pair.h"
 
 namespace fla {
 
@@ -27,6 +28,14 @@ FLA_FIELD(single) FLA_FIELD(vec_x) FLA_FIELD(vec_y) FLA_FIELD(vec_z) FLA_FIELD(v
 FLA_FIELD(state_transposed) FLA_FIELD(denom) FLA_FIELD(eps) FLA_FIELD(poly_on) FLA_FIELD(map_x) FLA_FIELD(map_out)
 FLA_FIELD(xmap_out) FLA_FIELD(xo_b) FLA_FIELD(xo_h) FLA_FIELD(xo_n) FLA_FIELD(omap) FLA_FIELD(ms_b) FLA_FIELD(ms_h)
 FLA_FIELD(ms_n)
+FLA_FIELDS_END
+
+FLA_FIELDS_BEGIN(TriPairParams)
+FLA_FIELD(xa) FLA_FIELD(xb) FLA_FIELD(ya) FLA_FIELD(yb) FLA_FIELD(oa) FLA_FIELD(ob)
+FLA_FIELD(xas_b) FLA_FIELD(xas_h) FLA_FIELD(xas_n) FLA_FIELD(xbs_b) FLA_FIELD(xbs_h) FLA_FIELD(xbs_n)
+FLA_FIELD(yas_b) FLA_FIELD(yas_h) FLA_FIELD(yas_n) FLA_FIELD(ybs_b) FLA_FIELD(ybs_h) FLA_FIELD(ybs_n)
+FLA_FIELD(oas_b) FLA_FIELD(oas_h) FLA_FIELD(oas_n) FLA_FIELD(obs_b) FLA_FIELD(obs_h) FLA_FIELD(obs_n)
+FLA_FIELD(H) FLA_FIELD(N) FLA_FIELD(BH) FLA_FIELD(wa) FLA_FIELD(wb) FLA_FIELD(n_tiles) FLA_FIELD(single)
 FLA_FIELDS_END
 
 FLA_FIELDS_BEGIN(NormParams)
@@ -77,6 +86,7 @@ FLA_FIELDS_END
 #undef FLA_FIELDS_END
 
 inline void trace_describe(trace::Record &r, int arg, const TriParams &p) { trace_fields(r, arg, "", p); }
+inline void trace_describe(trace::Record &r, int arg, const TriPairParams &p) { trace_fields(r, arg, "", p); }
 inline void trace_describe(trace::Record &r, int arg, const NormParams &p) { trace_fields(r, arg, "", p); }
 inline void trace_describe(trace::Record &r, int arg, const WalkParams &p) { trace_fields(r, arg, "", p); }
 inline void trace_describe(trace::Record &r, int arg, const WalkTotalsParams &p) { trace_fields(r, arg, "", p); }

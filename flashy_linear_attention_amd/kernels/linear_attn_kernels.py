@@ -72,3 +72,33 @@ def linear_flash_wrapper_bwd(
             dtype_code(q), stream_handle(q.device),
         )
     return dQ, dK, dV
+
+
+def linear_flash_wrapper_bwd_fused_dkdv(
+    grad_output: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(dQ, dK, dV) like :func:`linear_flash_wrapper_bwd`, with dV and dK formed by one kernel from one
+    stream of (Q, dO) tiles -- the loop structure of the reference's backward kernel
+    (flashlinear/kernels/linear_attn_kernels.py:160-227).  Head dims up to 128 (q/k and v may differ
+    within one padded width).  Measured slower than :func:`linear_flash_wrapper_bwd` on MI355X; kept
+    as the measured alternative (``fla_linear_attn_bwd_fused_dkdv``)."""
+    batch, nh, sq, hd = q.shape
+    hd_v = v.shape[-1]
+    assert hd <= 128 and hd_v <= 128, "Only head_dims <= 128 are supported by the fused dK / dV kernel."
+    assert k.shape == q.shape and v.shape[:3] == q.shape[:3] and grad_output.shape == v.shape, \
+        "grad_output must match v; q, k, v must agree in batch, heads and sequence"
+    grad_output, q, k, v = prepare(grad_output, q, k, v)
+    dQ = torch.empty_like(q, memory_format=torch.contiguous_format)
+    dK = torch.empty_like(k, memory_format=torch.contiguous_format)
+    dV = torch.empty_like(v, memory_format=torch.contiguous_format)
+    with torch.cuda.device(q.device):
+        call(
+            "fla_linear_attn_bwd_fused_dkdv",
+            grad_output.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+            dQ.data_ptr(), dK.data_ptr(), dV.data_ptr(),
+            batch, nh, sq, hd, hd_v,
+            _lib.strides_arg(grad_output), _lib.strides_arg(q), _lib.strides_arg(k), _lib.strides_arg(v),
+            _lib.strides_arg(dQ), _lib.strides_arg(dK), _lib.strides_arg(dV),
+            dtype_code(q), stream_handle(q.device),
+        )
+    return dQ, dK, dV

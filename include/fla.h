@@ -12,6 +12,17 @@
  *     element strides (b, h, n, d) and strides[3] must be 1.
  *   - `dtype` selects 16-bit storage: FLA_DTYPE_BF16 or FLA_DTYPE_F16.  Products
  *     run on bf16 / fp16 MFMA with fp32 accumulation; outputs are rounded once.
+ *     Range of FLA_DTYPE_F16: the un-normalised product grows with N (an output element is a sum
+ *     of up to N scores times values) and fp16 ends at 65504.  An output or gradient element
+ *     whose fp32 value lies beyond that leaves as +inf or -inf, exactly as a cast of the fp32
+ *     value would; finite inputs never produce NaN.  The masked scores are rounded to fp16 before
+ *     the second product, so a single score q_i . k_j above 65504 becomes inf there (and inf * 0
+ *     is NaN): keep |q_i . k_j| below that, e.g. by the usual 1/sqrt(D) scaling.  The chunk-wise
+ *     entry points also round the running state (sums of k_j v_j^T over the rows before a chunk)
+ *     to the storage type, so there the state's elements must fit as well.  The normalised
+ *     entry points divide in fp32 before the one rounding: their outputs are averages of v and
+ *     do not grow with N.  FLA_DTYPE_BF16 has fp32's exponent range and no such limit (the
+ *     reference computes in bf16 only, flashlinear/kernels/linear_attn_kernels.py:82,98).
  *   - `stream` is a hipStream_t (NULL = the null stream).  Calls only enqueue
  *     work; they never synchronise, allocate or free.  Outputs must not alias
  *     inputs or each other: the byte range each tensor spans (first to last
@@ -35,7 +46,7 @@
 extern "C" {
 #endif
 
-#define FLA_ABI_VERSION 3
+#define FLA_ABI_VERSION 4
 
 enum fla_dtype { FLA_DTYPE_BF16 = 0, FLA_DTYPE_F16 = 1 };
 
@@ -105,6 +116,25 @@ int fla_linear_attn_smallv_bwd(const void *grad_out, const void *q, const void *
                                const int64_t *dq_strides, const int64_t *dk_strides,
                                const int64_t *dv_strides,
                                int dtype, void *stream);
+
+/* The gradients of fla_linear_attn_bwd / fla_linear_attn_smallv_bwd evaluated the way the reference's
+ * backward kernel does it in its first phase (linear_attn_kernels.py:160-227): a workgroup owns rows
+ * of K and V and forms dV and dK from ONE stream of (Q, dO) tiles; dQ is a product of its own.
+ * Equal padded head dims (32 / 64 / 128) with 16-byte aligned rows only, else FLA_ERR_UNSUPPORTED.
+ * Results agree with fla_linear_attn_bwd (bit for bit up to padded width 64; up to the order of
+ * fp32 sums at 128).  On MI355X this evaluation measured 4 - 16 % SLOWER than the three products in one
+ * launch that fla_linear_attn_bwd makes, at every shape tried (the fused kernel halves the tile traffic
+ * of two products but needs the whole register file of a SIMD for one wave, and the products are not
+ * bound by that traffic), so nothing calls it by default; it is kept, tested and timed
+ * (bench.py --bwd-plan fused-dkdv) as the measured alternative. */
+int fla_linear_attn_bwd_fused_dkdv(const void *grad_out, const void *q, const void *k, const void *v,
+                                   void *dq, void *dk, void *dv,
+                                   int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v,
+                                   const int64_t *go_strides, const int64_t *q_strides,
+                                   const int64_t *k_strides, const int64_t *v_strides,
+                                   const int64_t *dq_strides, const int64_t *dk_strides,
+                                   const int64_t *dv_strides,
+                                   int dtype, void *stream);
 
 /* The one primitive all four calls above are built from:
  *

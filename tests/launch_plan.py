@@ -557,6 +557,94 @@ def model_tri_fast(arena: Arena, l: Launch, p: Dict, T: str, DC: int, DO: int, c
 
 
 # ---------------------------------------------------------------------------------------------
+# model of the fused dV + dK kernel (csrc/fla_tri_pair.h)
+
+def walk_swizzle(CR: int, row):
+    if CR == 4:
+        return (row >> 2) & 3
+    if CR == 8:
+        t = (row >> 1) & 7
+        return ((t & 1) << 2) | (t >> 1)
+    t = row & 15
+    return ((t & 3) << 2) | (t >> 2)
+
+
+def model_tri_pair(arena: Arena, l: Launch, p: Dict, D: int, stats: Stats) -> None:
+    NIB = 2 if D <= 64 else 1
+    BM = 4 * 32 * NIB
+    RB, CR = 2 * D, D // 8
+    TILE = 64 * RB
+    STAGE = 2 * TILE
+    NBUF = min(6, LDS_PER_CU // STAGE)
+    NI = TILE // 4096
+    NT, RPI = 2 * NI, 1024 // RB
+    assert l.lds == NBUF * STAGE and BM // 64 <= NBUF - 1 and BM * (2 * D + 16) <= NBUF * STAGE
+    assert (NBUF - 3) * NT < 64, "wait_tile's vmcnt does not fit its 6-bit field"
+    assert NI == 1 or (4 * RPI) % 16 == 0
+    N, BH, H, wa, wb = p["N"], p["BH"], p["H"], p["wa"], p["wb"]
+    assert 1 <= wa <= D and 1 <= wb <= D and wa % 8 == 0 and wb % 8 == 0
+    n_tiles = -(-N // BM)
+    assert p["n_tiles"] == n_tiles
+    single = p["single"] != 0
+    assert single == run_single_tiles(BH * ((n_tiles + 1) // 2), 1)
+    n_pairs = n_tiles if single else (n_tiles + 1) // 2
+    assert l.grid == (8 * ((BH + 7) // 8) * n_pairs, 1, 1)
+    for nm, ptr, sb, sh, sn, w in (("xa", "xa", "xas_b", "xas_h", "xas_n", wa), ("xb", "xb", "xbs_b", "xbs_h", "xbs_n", wb),
+                                   ("ya", "ya", "yas_b", "yas_h", "yas_n", wa), ("yb", "yb", "ybs_b", "ybs_h", "ybs_n", wb),
+                                   ("oa", "oa", "oas_b", "oas_h", "oas_n", wb), ("ob", "ob", "obs_b", "obs_h", "obs_n", wa)):
+        lo, hi = tensor_extent(p, ptr, sb, sh, sn, H, BH, N, w)
+        arena.require(f"fused dV + dK kernel, {nm}", lo, hi)
+        assert p[ptr] % 16 == 0 and all(p[x] % 8 == 0 for x in (sb, sh, sn)) and p[sn] >= w
+        assert N * p[sn] * 2 <= 0x3fffffff
+    lanes = np.arange(64)
+    seen = set()
+    n_hl = (BH + 7) >> 3
+    for wg in range(l.grid[0]):
+        xcd, slot = wg & 7, wg >> 3
+        hl, rank = (slot % n_hl, slot // n_hl) if single else (slot // n_pairs, slot % n_pairs)
+        bh = hl * 8 + xcd
+        if bh >= BH:
+            continue
+        stats.workgroups += 1
+        tiles = [rank] if single or rank == n_tiles - 1 - rank else [rank, n_tiles - 1 - rank]
+        for t in tiles:
+            assert 0 <= t < n_tiles and (bh, t) not in seen
+            seen.add((bh, t))
+        if bh not in (0, BH - 1) or rank not in {0, 1, n_pairs // 2, n_pairs - 1}:
+            continue
+        for tile in tiles:
+            i0 = tile * BM
+            diag_rows = min(N - i0, BM)
+            rest = N - (i0 + BM)
+            n_full = -(-rest // 64) if rest > 0 else 0
+            n_seq = n_full + -(-diag_rows // 64)
+            for q in sorted({0, 1, n_full - 1, n_full + NBUF - 1} | set(range(n_full, n_seq + 2))):
+                if q < 0:
+                    continue
+                exists = q < n_seq
+                row0 = (i0 + BM + q * 64 if q < n_full else i0 + (q - n_full) * 64) if exists else 0
+                for which, s2, w in ((0, 2 * p["yas_n"], wa), (1, 2 * p["ybs_n"], wb)):
+                    rec = (N - 1) * s2 + w * 2
+                    for wave in range(4):
+                        row_l = wave * RPI + lanes // CR
+                        c = (lanes % CR) ^ walk_swizzle(CR, row_l)
+                        voff = row_l * s2 + c * 16 + np.where(c * 8 < w, 0, K_OOB)
+                        for I in range(NI):
+                            so = (row0 + I * 4 * RPI) * s2 if exists else K_OOB
+                            dst = I * 4096 + wave * 1024 + lanes * 16  # within the operand's tile
+                            lrow, lchunk = dst // RB, (dst % RB) // 16
+                            want_chunk = lchunk ^ walk_swizzle(CR, lrow)
+                            grow = row0 + lrow
+                            if exists:
+                                ok = want_chunk * 8 < w
+                                assert ((voff + so == grow * s2 + want_chunk * 16) | ~ok).all(), \
+                                    "fused kernel tile load: a lane fetches the wrong row or chunk"
+                            _buffer_check("fused kernel tile load", voff + so, exists & (grow < N) & (want_chunk * 8 < w), rec)
+                            stats.lane_accesses += 64
+    assert seen == {(bh, t) for bh in range(BH) for t in range(n_tiles)}
+
+
+# ---------------------------------------------------------------------------------------------
 # model of the generic masked-product kernel (csrc/fla_tri_kernel.h)
 
 def model_tri_generic(arena: Arena, l: Launch, p: Dict, DC: int, DO: int, stats: Stats) -> None:
@@ -749,6 +837,8 @@ def check_all(arena: Arena, launches: List[Launch], stats: Stats) -> None:
                 n_tiles = -(-p["N"] // cfg.BM)
                 arena.require("chunk states", p["state"], p["state"] + p["BH"] * n_tiles * DC * DO * 2)
                 model_tri_fast(arena, l, p, T, DC, DO, True, 0, lds, stats)
+        elif k == "tri_pair_upper_kernel":
+            model_tri_pair(arena, l, l.struct("a0"), t[1], stats)
         elif k == "tri_xyt_z_kernel":
             T, DC, DO = t
             model_tri_generic(arena, l, l.struct("a0"), DC, DO, stats)

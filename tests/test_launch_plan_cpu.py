@@ -224,6 +224,26 @@ def test_rows_expanded_along_the_sequence_take_the_bounds_checked_kernel(lib):
     assert launches and all(l.kernel == "tri_xyt_z_kernel" for l in launches)
 
 
+def test_fused_dkdv_backward(lib):
+    """fla_linear_attn_bwd_fused_dkdv: the fused dV + dK kernel and dQ's product, every padded width."""
+    stats = lp.Stats()
+    for (b, h, n, dqk, dv), dtype in itertools.product(((1, 2, 64, 64, 64), (2, 3, 320, 64, 64), (1, 16, 2048, 64, 64),
+                                                        (1, 5, 1000, 48, 64), (2, 2, 1984, 32, 32), (1, 130, 300, 24, 32),
+                                                        (1, 300, 512, 64, 64), (2, 3, 1000, 128, 128), (1, 130, 384, 96, 128),
+                                                        (4, 32, 4096, 128, 128), (1, 16, 32768, 64, 64)), (0, 1)):
+        arena = lp.Arena()
+        q, k, dq, dk = (lp.make_tensor(arena, nm, b, h, n, dqk) for nm in ("q", "k", "dq", "dk"))
+        v, g, dvv = (lp.make_tensor(arena, nm, b, h, n, dv) for nm in ("v", "grad_out", "dv"))
+        rc = lib.fla_linear_attn_bwd_fused_dkdv(g.ptr, q.ptr, k.ptr, v.ptr, dq.ptr, dk.ptr, dvv.ptr, b, h, n, dqk, dv,
+                                                g.strides_arg(), q.strides_arg(), k.strides_arg(), v.strides_arg(),
+                                                dq.strides_arg(), dk.strides_arg(), dvv.strides_arg(), dtype, None)
+        assert rc == 0, rc
+        launches = lp.take_launches(lib)
+        assert [l.kernel for l in launches] == ["tri_pair_upper_kernel", "tri_xyt_z_fast_kernel"]
+        lp.check_all(arena, launches, stats)
+    assert stats.lane_accesses > 0
+
+
 def test_benchmark_shapes(lib):
     """C2 - C5 of the benchmark, both evaluations, and the normalised operator on C3 and C5."""
     stats = lp.Stats()

@@ -256,3 +256,34 @@ def test_feature_operator_gradients(kind):
             minus[which][idx] -= h
             fd = (scalar(*plus) - scalar(*minus)) / (2 * h)
             assert g[idx].item() == pytest.approx(fd.item(), rel=1e-6, abs=1e-8)
+
+
+@pytest.mark.parametrize("kind", ["elu1", "softplus"])
+def test_feature_recipe_is_a_weighted_average_under_the_map(kind):
+    """feature_linear_attention_normalised by what the mathematics fixes, not by its formula:
+    (i) both maps are positive, so the scores are positive weights and with eps = 0 every output
+    row is a weighted AVERAGE of the value rows so far -- a constant v comes back unchanged, the
+    first row is v_0 itself, and every entry lies between the running minimum and maximum of its
+    column; (ii) the normaliser the recipe divides by equals the row sums of the masked scores of
+    the MAPPED operands, summed by plain loops here; (iii) eps enters as out = O / (n + eps)."""
+    xq, xk, v = _rand((1, 2, 11, 5), 41), _rand((1, 2, 11, 5), 42), _rand((1, 2, 11, 3), 43)
+    const = torch.full_like(v, 0.75)
+    torch.testing.assert_close(naive.feature_linear_attention_normalised(xq, xk, const, kind, eps=0.0), const,
+                               rtol=1e-12, atol=1e-12)
+    out = naive.feature_linear_attention_normalised(xq, xk, v, kind, eps=0.0)
+    torch.testing.assert_close(out[:, :, 0], v[:, :, 0], rtol=1e-12, atol=1e-12)
+    lo, hi = torch.cummin(v, dim=-2).values, torch.cummax(v, dim=-2).values
+    assert (out >= lo - 1e-12).all() and (out <= hi + 1e-12).all()
+    # (ii), (iii): out (n + eps) = unnormalised product, n by explicit loops over the mapped rows
+    eps = 0.37
+    fq, fk = naive.feature_map(xq, kind), naive.feature_map(xk, kind)
+    n = torch.zeros(1, 2, 11, dtype=torch.float64)
+    for h in range(2):
+        for i in range(11):
+            for j in range(i + 1):
+                n[0, h, i] += float((fq[0, h, i] * fk[0, h, j]).sum())
+    got = naive.feature_linear_attention_normalised(xq, xk, v, kind, eps=eps)
+    want = naive.causal_dot_product_recurrent(fq, fk, v) / (n + eps).unsqueeze(-1)
+    torch.testing.assert_close(got, want, rtol=1e-12, atol=1e-12)
+    # the map matters: on operands with negative entries the unmapped recipe gives something else
+    assert not torch.allclose(got, naive.linear_attention_normalised(xq, xk, v, eps=eps))

@@ -38,6 +38,10 @@ EQUAL_D_CASES = [
     (1, 2, 256, 256),
     (1, 3, 448, 200),
     (1, 1, 1024, 17),
+    # head dims above 128 allow sequence lengths that are multiples of 32 only (the reference's
+    # BLOCK_SQ = 32 branch, flashlinear/kernels/linear_attn_kernels.py:317,354-356)
+    (1, 2, 96, 200),
+    (2, 2, 160, 256),
 ]
 
 # (batch, heads, seq, hd_qk, hd_v): reference small-V envelope
@@ -52,6 +56,9 @@ SMALL_V_CASES = [
     (1, 2, 320, 128, 128),
     (1, 2, 192, 100, 8),
 ]
+# forward only: with hd_qk above 128 the forward wrapper allows multiples of 32
+# (flashlinear/kernels/linear_attn_kernels_smallv_hd.py:331,340-342); its backward wants 64 (:376,382-384)
+SMALL_V_FWD_ONLY_CASES = [(1, 2, 96, 256, 64), (1, 3, 160, 200, 32)]
 
 
 def _oracle_fwd(q, k, v):
@@ -88,7 +95,7 @@ def test_attn_bwd(dims, dtype, gpu_device):
         assert_close(name, got, want)
 
 
-@pytest.mark.parametrize("dims", SMALL_V_CASES, ids=lambda d: "x".join(map(str, d)))
+@pytest.mark.parametrize("dims", SMALL_V_CASES + SMALL_V_FWD_ONLY_CASES, ids=lambda d: "x".join(map(str, d)))
 def test_attn_smallv_fwd(dims, gpu_device):
     bs, nh, sq, hd_qk, hd_v = dims
     q, k, v, _ = reference_style_inputs(bs, nh, sq, hd_qk, hd_v, torch.bfloat16, seed=sum(dims))
@@ -225,3 +232,25 @@ def test_end_to_end_with_pytorch_denominator(gpu_device):
                                     ("dV", vg.grad, vo.grad, vr.grad)):
         assert_close(name + " vs fp32 recipe", g, exact, tol_fro=1e-2, tol_max=5e-2)
         assert_close(name + " vs rounded oracle", g, rounded, tol_fro=1e-2, tol_max=5e-2)
+
+
+def test_fp16_output_overflow_is_infinity_never_nan(gpu_device):
+    """The un-normalised product grows with the sequence length, and fp16 ends at 65504: results are
+    accumulated in fp32 and rounded once, so an element beyond the range leaves as +-inf (as a cast
+    of the exact result would) and finite inputs never give NaN.  Constructed so that every partial
+    sum is an integer fp32 holds exactly: q = k = 4, v = +-1 by column, O[i, c] = +-1024 (i + 1)."""
+    n, d = 128, 64
+    q = torch.full((1, 2, n, d), 4.0, dtype=torch.float16)
+    k = torch.full((1, 2, n, d), 4.0, dtype=torch.float16)
+    v = torch.ones(1, 2, n, d, dtype=torch.float16)
+    v[..., 1::2] = -1.0
+    want = naive.causal_dot_product(q.float(), k.float(), v.float()).to(torch.float16)  # overflow -> +-inf here too
+    assert torch.isinf(want).any() and torch.isfinite(want).any() and not torch.isnan(want).any()
+    with torch.no_grad():
+        got = LinearAttention.apply(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device)).cpu()
+    assert not torch.isnan(got).any()
+    assert torch.equal(got, want)  # exact integers: same finite values, same +-inf in the same places
+    # bf16 has fp32's exponent range: the same problem stays finite
+    with torch.no_grad():
+        got_bf = LinearAttention.apply(*(t.to(torch.bfloat16).to(gpu_device) for t in (q, k, v)))
+    assert torch.isfinite(got_bf).all()
