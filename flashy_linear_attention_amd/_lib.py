@@ -102,9 +102,36 @@ def load() -> ctypes.CDLL:
     return _lib
 
 
+_STRIDES = {}
+
+
 def strides_arg(t) -> ctypes.Array:
-    """A tensor's 4 element strides as a C ``int64_t[4]``."""
-    return (ctypes.c_int64 * 4)(*t.stride())
+    """A tensor's 4 element strides as a C ``int64_t[4]``.  The arrays are read-only to the library
+    and kept per distinct stride tuple: building one costs about as much as the rest of a call's
+    argument conversion, and a caller's tensors come in a handful of layouts."""
+    s = t.stride()
+    a = _STRIDES.get(s)
+    if a is None:
+        if len(_STRIDES) > 4096:
+            _STRIDES.clear()
+        a = _STRIDES[s] = (ctypes.c_int64 * 4)(*s)
+    return a
+
+
+_SIZES = {}
+
+
+def query(name: str, *args) -> int:
+    """A size or plan query of the library (``fla_*_bytes``, ``fla_linear_attn_prefers_chunked``): pure
+    host arithmetic on the shape, so the answer is kept per (function, arguments) -- an operator call
+    makes two or three of them, each the cost of a ctypes call."""
+    key = (name,) + args
+    v = _SIZES.get(key)
+    if v is None:
+        if len(_SIZES) > 65536:
+            _SIZES.clear()
+        v = _SIZES[key] = getattr(load(), name)(*args)
+    return v
 
 
 def check(fn: str, status: int) -> None:

@@ -28,7 +28,7 @@ from .kernels import (
 def prefers_chunked(q: torch.Tensor, v: torch.Tensor) -> bool:
     """Whether the chunk-wise kernels are the faster choice for (B, H, N, D_qk) q and (B, H, N, D_v) v."""
     b, h, n, dqk = q.shape
-    return bool(_lib.load().fla_linear_attn_prefers_chunked(b, h, n, dqk, v.shape[-1]))
+    return bool(_lib.query("fla_linear_attn_prefers_chunked", b, h, n, dqk, v.shape[-1]))
 
 
 class LinearAttentionAuto(Function):

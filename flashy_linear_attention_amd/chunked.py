@@ -17,7 +17,7 @@ import torch
 from torch.autograd import Function
 
 from . import _lib
-from .kernels._common import dtype_code, prepare, stream_handle
+from .kernels._common import device_guard, dtype_code, prepare, stream_handle
 
 
 def tri_xyt_z_chunked(x: torch.Tensor, y: torch.Tensor, z: torch.Tensor, upper: bool) -> torch.Tensor:
@@ -28,8 +28,8 @@ def tri_xyt_z_chunked(x: torch.Tensor, y: torch.Tensor, z: torch.Tensor, upper: 
     do = z.shape[-1]
     out = torch.empty_like(z, memory_format=torch.contiguous_format)
     lib = _lib.load()
-    with torch.cuda.device(x.device):
-        nbytes = lib.fla_chunked_workspace_bytes(b, h, n, dc, do)
+    with device_guard(x.device):
+        nbytes = _lib.query("fla_chunked_workspace_bytes", b, h, n, dc, do)
         work = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
         _lib.check(
             "fla_tri_xyt_z_chunked",
@@ -55,10 +55,10 @@ def linear_attention_chunked_fwd(
     dv = v.shape[-1]
     out = torch.empty_like(v, memory_format=torch.contiguous_format)
     lib = _lib.load()
-    with torch.cuda.device(q.device):
-        sbytes = lib.fla_linear_attn_chunked_state_bytes(b, h, n, dqk, dv) if want_state else 0
+    with device_guard(q.device):
+        sbytes = _lib.query("fla_linear_attn_chunked_state_bytes", b, h, n, dqk, dv) if want_state else 0
         state = torch.empty(sbytes, dtype=torch.uint8, device=q.device) if sbytes else None
-        wbytes = lib.fla_linear_attn_chunked_workspace_bytes(b, h, n, dqk, dv)
+        wbytes = _lib.query("fla_linear_attn_chunked_workspace_bytes", b, h, n, dqk, dv)
         work = torch.empty(max(wbytes, 16), dtype=torch.uint8, device=q.device)
         valid = ctypes.c_int32(0)
         _lib.check(
@@ -86,10 +86,10 @@ def linear_attention_chunked_bwd(
     dk = torch.empty_like(k, memory_format=torch.contiguous_format)
     dvv = torch.empty_like(v, memory_format=torch.contiguous_format)
     lib = _lib.load()
-    with torch.cuda.device(q.device):
+    with device_guard(q.device):
         if state is not None:
-            assert state.numel() == lib.fla_linear_attn_chunked_state_bytes(b, h, n, dqk, dv), "state of another shape"
-        wbytes = lib.fla_linear_attn_chunked_workspace_bytes(b, h, n, dqk, dv)
+            assert state.numel() == _lib.query("fla_linear_attn_chunked_state_bytes", b, h, n, dqk, dv), "state of another shape"
+        wbytes = _lib.query("fla_linear_attn_chunked_workspace_bytes", b, h, n, dqk, dv)
         work = torch.empty(max(wbytes, 16), dtype=torch.uint8, device=q.device)
         _lib.check(
             "fla_linear_attn_chunked_bwd",

@@ -422,9 +422,19 @@ WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
 // totals of Y^T Z over the walk's segments into `work`, then the segments' entry states: their sums
 // over the segments before (reverse == 0) or after (reverse != 0), written to `entry` (null: over
 // the totals in `work`).  Returns where the entry states are.
+// `second`: the same for another Y operand of the same layout against the same Z (the other half of a
+// wide q / k) in the same launches -- one totals launch and one scan for the two of them.
+struct EntryHalf {
+    const void *y;  // Y's pointer (Y's strides are the first operand's)
+    int64_t dy;
+    void *work;
+    float *entry;
+    const float **where;
+};
+
 int walk_entry_states(const WalkPlan &w, const View &y, const View &z, int64_t B, int64_t H, int64_t N, int64_t dy,
                       int64_t dz, int dtype, int reverse, void *work, float *entry, const float **where, hipStream_t s,
-                      int map_y = 0, const View *ymap_out = nullptr) {
+                      int map_y = 0, const View *ymap_out = nullptr, const EntryHalf *second = nullptr) {
     fla::WalkTotalsParams tp{};
     if (map_y) {
         tp.map_y = map_y, tp.ymap_out = const_cast<void *>(ymap_out->ptr);
@@ -433,9 +443,11 @@ int walk_entry_states(const WalkPlan &w, const View &y, const View &z, int64_t B
     float *totals = static_cast<float *>(work);
     if (!entry) entry = totals;
     // (two segments: the one total needed is the other segment's entry state; the totals kernel writes it as the
-    // walks read it, two partial sums, and no scan follows)
-    const bool direct = w.n_seg == 2;
-    tp.y = y.ptr, tp.z = z.ptr, tp.totals = direct ? entry : totals, tp.direct = direct;
+    // walks read it, two partial sums, and no scan follows.  A few segments more: the walks add up the totals
+    // themselves as they start -- fla::walk_entries_are_totals -- and no scan follows either)
+    const bool direct = w.n_seg == 2, summed_on_load = fla::walk_entries_are_totals(w.D, (int)w.n_seg);
+    const bool no_scan = direct || summed_on_load;
+    tp.y = y.ptr, tp.z = z.ptr, tp.totals = no_scan ? entry : totals, tp.direct = direct;
     tp.ys_b = y.strides[0], tp.ys_h = y.strides[1], tp.ys_n = y.strides[2];
     tp.zs_b = z.strides[0], tp.zs_h = z.strides[1], tp.zs_n = z.strides[2];
     tp.H = (int32_t)H, tp.N = (int32_t)N, tp.BH = (int32_t)(B * H), tp.dy = (int32_t)dy, tp.dz = (int32_t)dz;
@@ -445,13 +457,37 @@ int walk_entry_states(const WalkPlan &w, const View &y, const View &z, int64_t B
     tp.seg_lo = reverse && !map_y ? 1 : 0;
     tp.seg_hi = (int32_t)(!reverse && !map_y ? w.n_seg - 1 : w.n_seg);
     if (direct) tp.seg_lo = reverse ? 1 : 0, tp.seg_hi = tp.seg_lo + 1;  // (the needed one)
+    float *totals2 = nullptr, *entry2 = nullptr;
+    if (second) {
+        totals2 = static_cast<float *>(second->work);
+        entry2 = second->entry ? second->entry : totals2;
+        tp.y2 = second->y, tp.dy2 = (int32_t)second->dy, tp.totals2 = no_scan ? entry2 : totals2;
+        *second->where = entry2;
+    }
     if (fla::walk_totals(dtype, w.D, tp, s) != hipSuccess) return FLA_ERR_LAUNCH;
     *where = entry;
-    if (direct) return FLA_OK;
+    if (no_scan) return FLA_OK;
     return fla::walk_scan(totals, entry, B * H, (int)w.n_seg, w.D, fla::walk_totals_cols(w.D, (int)dy, (int)dz), reverse,
-                          s) == hipSuccess
+                          s, totals2, entry2) == hipSuccess
                ? FLA_OK
                : FLA_ERR_LAUNCH;
+}
+
+// Entry states of both 128-column halves of a wide q / k (Y = the halves of `y`, against the same Z):
+// one totals launch and one scan for the two when both halves take the same kernel variant, else
+// one after the other.  work[h], entry[h] (null: over work[h]) and where[h] per half.
+int wide_entry_states(const WalkPlan &wp, const View &y, const View &z, int64_t B, int64_t H, int64_t N, int64_t dy_all,
+                      int64_t dz, int dtype, int reverse, void *const (&work)[2], float *const (&entry)[2],
+                      const float *(&where)[2], hipStream_t s) {
+    const View y1{static_cast<const char *>(y.ptr) + 128 * 2, y.strides};
+    const int64_t dy1 = dy_all - 128;
+    if (fla::walk_totals_cols(wp.D, 128, (int)dz) == fla::walk_totals_cols(wp.D, (int)dy1, (int)dz)) {
+        const EntryHalf other{y1.ptr, dy1, work[1], entry[1], &where[1]};
+        return walk_entry_states(wp, y, z, B, H, N, 128, dz, dtype, reverse, work[0], entry[0], &where[0], s, 0, nullptr,
+                                 &other);
+    }
+    if (int rc = walk_entry_states(wp, y, z, B, H, N, 128, dz, dtype, reverse, work[0], entry[0], &where[0], s)) return rc;
+    return walk_entry_states(wp, y1, z, B, H, N, dy1, dz, dtype, reverse, work[1], entry[1], &where[1], s);
 }
 
 // The normaliser's terms handed to the walk kernels (fla_chunk_walk.h, WalkParams::denom ...).
@@ -532,9 +568,9 @@ int64_t shared_state_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t
     return core ? core + walk_vec_bytes(B, H, N, dqk, dv) : 0;
 }
 
-// workspace of the two-halves evaluation: the scratch tensor for dV, then totals and entry states of one
-// half at a time (two sets in backward: Q^T dO, and K^T V when forward's entry states are not given)
-int64_t wide_workspace_bytes(const WidePlan &w) { return w.temp_bytes + 2 * w.wp.work_bytes; }
+// workspace of the two-halves evaluation: the scratch tensor for dV, then totals and entry states of both
+// halves (two sets of them in backward: Q^T dO, and K^T V when forward's entry states are not given)
+int64_t wide_workspace_bytes(const WidePlan &w) { return w.temp_bytes + 4 * w.wp.work_bytes; }
 
 int64_t chunked_op_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     const int64_t shared = shared_state_bytes(B, H, N, dqk, dv);
@@ -575,17 +611,23 @@ int wide_forward(const WidePlan &wide, const View &q, const View &k, const View 
                  int64_t N, int64_t dqk, int64_t dv, int dtype, void *state_out, void *workspace, hipStream_t s) {
     const WalkPlan &wp = wide.wp;
     char *ws = static_cast<char *>(workspace);
+    const float *entry[2] = {nullptr, nullptr};
+    if (wp.n_seg > 1) {
+        // (kept for backward when there is a state buffer: each half's entry states, its final state behind them;
+        // otherwise the two halves' states share the workspace behind the scratch tensor)
+        float *keep[2] = {nullptr, nullptr};
+        void *work[2];
+        for (int h = 0; h < 2; ++h) {
+            if (state_out) keep[h] = reinterpret_cast<float *>(static_cast<char *>(state_out) + h * wp.saved_bytes);
+            work[h] = keep[h] ? static_cast<void *>(keep[h]) : static_cast<void *>(ws + wide.temp_bytes + h * wp.work_bytes);
+        }
+        if (int rc = wide_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, work, keep, entry, s)) return rc;
+    }
     for (int h = 0; h < 2; ++h) {
         const View qh = column_half(q, h), kh = column_half(k, h);
         const int64_t wqk = h == 0 ? 128 : dqk - 128;
-        const float *entry = nullptr;
-        if (wp.n_seg > 1) {
-            float *keep = state_out ? reinterpret_cast<float *>(static_cast<char *>(state_out) + h * wp.saved_bytes) : nullptr;
-            void *work = keep ? static_cast<void *>(keep) : static_cast<void *>(ws + wide.temp_bytes);
-            if (int rc = walk_entry_states(wp, kh, v, B, H, N, wqk, dv, dtype, 0, work, keep, &entry, s)) return rc;
-        }
         // (the second half's walk adds its result to the first one's)
-        fla::WalkParams w = lower_walk_params(wp, qh, kh, v, o, B, H, N, wqk, dv, entry);
+        fla::WalkParams w = lower_walk_params(wp, qh, kh, v, o, B, H, N, wqk, dv, entry[h]);
         w.accumulate = h;
         if (state_out)  // (behind this half's entry states: the state after the last chunk)
             w.total_out = reinterpret_cast<float *>(static_cast<char *>(state_out) + h * wp.saved_bytes + wp.entry_bytes);
@@ -601,19 +643,26 @@ int wide_backward(const WidePlan &wide, const View &go, const View &q, const Vie
     char *ws = static_cast<char *>(workspace);
     const int64_t temp_strides[4] = {H * N * dv, N * dv, dv, 1};
     const View temp{ws, temp_strides};
+    // entry states of both halves up front: Q_h^T dO over the segments after, and -- when forward's are not
+    // at hand -- K_h^T V over the segments before
+    const float *fwd_entries[2] = {nullptr, nullptr}, *entries[2] = {nullptr, nullptr};
+    if (wp.n_seg > 1) {
+        float *const none[2] = {nullptr, nullptr};
+        char *base = ws + wide.temp_bytes;
+        if (state_in) {
+            for (int h = 0; h < 2; ++h)
+                fwd_entries[h] = reinterpret_cast<const float *>(static_cast<const char *>(state_in) + h * wp.saved_bytes);
+        } else {
+            void *const work[2] = {base + 2 * wp.work_bytes, base + 3 * wp.work_bytes};
+            if (int rc = wide_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, work, none, fwd_entries, s)) return rc;
+        }
+        void *const work[2] = {base, base + wp.work_bytes};
+        if (int rc = wide_entry_states(wp, q, go, B, H, N, dqk, dv, dtype, 1, work, none, entries, s)) return rc;
+    }
     for (int h = 0; h < 2; ++h) {
         const View qh = column_half(q, h), kh = column_half(k, h), dqh = column_half(dq, h), dkh = column_half(dk, h);
         const int64_t wqk = h == 0 ? 128 : dqk - 128;
-        const float *fwd_entry = nullptr, *entry = nullptr;
-        if (wp.n_seg > 1) {
-            if (state_in)
-                fwd_entry = reinterpret_cast<const float *>(static_cast<const char *>(state_in) + h * wp.saved_bytes);
-            else if (int rc = walk_entry_states(wp, kh, v, B, H, N, wqk, dv, dtype, 0, ws + wide.temp_bytes + wp.work_bytes,
-                                                nullptr, &fwd_entry, s))
-                return rc;
-            if (int rc = walk_entry_states(wp, qh, go, B, H, N, wqk, dv, dtype, 1, ws + wide.temp_bytes, nullptr, &entry, s))
-                return rc;
-        }
+        const float *fwd_entry = fwd_entries[h], *entry = entries[h];
         const View &dvh = h == 0 ? dvv : temp;
         if (state_in) {  // forward's states at hand: dQ_h, dK_h and this half's part of dV in one reverse walk
             fla::WalkParams r{};

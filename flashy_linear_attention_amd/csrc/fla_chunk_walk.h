@@ -718,11 +718,37 @@ __device__ __forceinline__ void walk_load_state(const float *init, bool transpos
     if (init2) walk_read_state<D, B, true>(init2, transposed, wave, lane, st);
 }
 
-// Entry states in memory: one fp32 [D][D] per segment, [bh][seg] -- except with two segments per
-// (b, h), where the first segment in walking order starts from zero and the other one from the one
-// total the totals kernel forms; its two workgroups of a (b, h) then add up half of that segment
-// each, and the two slots hold their partial sums.
-//
+// Entry states in memory, fp32 [D][D] per segment, [bh][seg], in one of three forms that host and
+// kernels tell apart by the number of segments alone:
+//   * two segments per (b, h): the first segment in walking order starts from zero and the other one
+//     from the one total the totals kernel forms; its two workgroups of a (b, h) add up half of that
+//     segment each, and the two slots hold their partial sums;
+//   * three to walk_sum_on_load_max(D) segments: the slots hold the segments' TOTALS as the totals kernel
+//     wrote them, and a walk adds up the totals of the segments before it (after it, walking in reverse)
+//     as it starts -- a few states of D x D read from L2 per workgroup instead of a scan kernel between
+//     the totals kernel and the walk, whose launch costs more than it computes on plans this small
+//     (B H = 16, N = 1024, D = 64, forward + backward: 40.7 -> 32.8 us, bound by its six -> four launches);
+//   * more segments: the slots hold the entry states themselves (walk_scan_kernel).
+// Padded head dims up to 64 only.  At D = 128 a workgroup has its CU to itself and nothing hides the
+// latency of those reads at its start: with four segments the forward walk gained 10 us and the reverse
+// walk, which starts from two such sums, lost 60 (B 4, H 16, N 4096, D_qk 256 as two halves: 0.333 -> 0.384 ms).
+__host__ __device__ constexpr int walk_sum_on_load_max(int D) { return D <= 64 ? 8 : 0; }
+__host__ __device__ constexpr bool walk_entries_are_totals(int D, int n_seg) {
+    return n_seg >= 3 && n_seg <= walk_sum_on_load_max(D);
+}
+
+// this wave's blocks of the sum of the states buf[f_lo .. f_hi - 1] (zeros for an empty range)
+template <int D, typename B>
+__device__ __forceinline__ void walk_sum_states(const float *buf, int f_lo, int f_hi, bool transposed, int wave, int lane,
+                                                f32x16 (&st)[WalkCfg<D>::NBW]) {
+#pragma unroll
+    for (int i = 0; i < WalkCfg<D>::NBW; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) st[i][v] = 0.f;
+#pragma unroll 1
+    for (int f = f_lo; f < f_hi; ++f) walk_read_state<D, B, true>(buf + (int64_t)f * (D * D), transposed, wave, lane, st);
+}
+
 // this wave's blocks of the entry state of segment sl.seg (zeros without an init buffer) of a walk
 // in ascending (`reverse` false) or descending order of the chunks
 template <int D, typename B = WalkExt<D>>
@@ -732,6 +758,10 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
     if (p.init) {
         if (p.n_seg == 2) {
             if (sl.seg != (reverse ? 1 : 0)) init = p.init + (int64_t)sl.bh * 2 * (D * D), init2 = init + D * D;
+        } else if (walk_entries_are_totals(D, p.n_seg)) {
+            walk_sum_states<D, B>(p.init + (int64_t)sl.bh * p.n_seg * (D * D), reverse ? sl.seg + 1 : 0,
+                                  reverse ? p.n_seg : sl.seg, p.init_transposed != 0, wave, lane, st);
+            return;
         } else {
             init = p.init + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D);
         }
@@ -740,16 +770,20 @@ __device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSl
 }
 
 // the forward state at the end of segment sl.seg from what forward handed over: the entry state of
-// the next segment (xinit, in the layout above) or, for the last one, the final state (xtotal)
+// the next segment (xinit, in the forms above) or, for the last one, the final state (xtotal)
 template <int D, typename B = WalkExt<D>>
 __device__ __forceinline__ void walk_load_end_state(const WalkParams &p, const WalkSlice &sl, int wave, int lane,
                                                     f32x16 (&xs)[WalkCfg<D>::NBW]) {
     const float *x = p.xtotal + (int64_t)sl.bh * (D * D), *x2 = nullptr;
     if (sl.c_hi < p.n_chunks) {
-        if (p.n_seg == 2)
+        if (p.n_seg == 2) {
             x = p.xinit + (int64_t)sl.bh * 2 * (D * D), x2 = x + D * D;
-        else
+        } else if (walk_entries_are_totals(D, p.n_seg)) {
+            walk_sum_states<D, B>(p.xinit + (int64_t)sl.bh * p.n_seg * (D * D), 0, sl.seg + 1, false, wave, lane, xs);
+            return;
+        } else {
             x = p.xinit + ((int64_t)sl.bh * p.n_seg + sl.seg + 1) * (D * D);
+        }
     }
     walk_load_state<D, B>(x, false, wave, lane, xs, x2);
 }
@@ -1362,6 +1396,11 @@ struct WalkTotalsParams {
     int32_t map_y;
     void *ymap_out;
     int64_t yo_b, yo_h, yo_n;
+    // A second Y operand of the same layout against the same Z, in the same launch (grid y = 1): the other
+    // 128-column half of a wide q / k, whose totals go to `totals2`.  Null: none.  (Without a feature map.)
+    const void *y2;
+    int32_t dy2;
+    float *totals2;
 };
 
 constexpr int walk_totals_sets(int D) { return D == 128 ? 4 : 2; }  // sets of (Y, Z) tiles in LDS
@@ -1378,6 +1417,9 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
     const int hl = slot / p.n_seg, bh = hl * 8 + xcd;
     int seg = slot - hl * p.n_seg;
     if (bh >= p.BH) return;
+    const bool second = blockIdx.y != 0;  // (the launch's second Y operand: see WalkTotalsParams::y2)
+    float *const totals = second ? p.totals2 : p.totals;
+    const int dy = second ? p.dy2 : p.dy;
     float *out;
     int c_lo, c_hi;
     if (p.direct) {
@@ -1385,7 +1427,7 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
         // every row has to be visited: the needed segment's workgroup forms its total alone, the other one
         // maps its own segment's rows and hands in zeros)
         const int needed = p.seg_lo, part = seg != needed;
-        out = p.totals + ((int64_t)bh * 2 + part) * (D * D);
+        out = totals + ((int64_t)bh * 2 + part) * (D * D);
         c_lo = seg * p.seg_chunks;
         c_hi = c_lo + p.seg_chunks < p.n_chunks ? c_lo + p.seg_chunks : p.n_chunks;
         if (!p.map_y) {
@@ -1396,7 +1438,7 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
         }
     } else {
         if (seg < p.seg_lo || seg >= p.seg_hi) return;
-        out = p.totals + ((int64_t)bh * p.n_seg + seg) * (D * D);
+        out = totals + ((int64_t)bh * p.n_seg + seg) * (D * D);
         c_lo = seg * p.seg_chunks;
         c_hi = c_lo + p.seg_chunks < p.n_chunks ? c_lo + p.seg_chunks : p.n_chunks;
     }
@@ -1406,10 +1448,10 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
     }
     const bool discard = p.direct && p.map_y && seg != p.seg_lo;  // (visited for the map only)
     const int b = bh / p.H, h = bh - b * p.H, N = p.N;
-    const T *Y = static_cast<const T *>(p.y) + b * p.ys_b + h * p.ys_h;
+    const T *Y = static_cast<const T *>(second ? p.y2 : p.y) + b * p.ys_b + h * p.ys_h;
     const T *Z = static_cast<const T *>(p.z) + b * p.zs_b + h * p.zs_h;
     const int ys2 = (int)p.ys_n * 2, zs2 = (int)p.zs_n * 2;
-    const u32x4 ry = make_rsrc(Y, (uint32_t)((N - 1) * ys2 + p.dy * 2));
+    const u32x4 ry = make_rsrc(Y, (uint32_t)((N - 1) * ys2 + dy * 2));
     const u32x4 rz = make_rsrc(Z, (uint32_t)((N - 1) * zs2 + p.dz * 2));
     using B = WalkExt<D, NQ, NV>;  // (blocks outside it stay unwritten: no walk of the same extent reads them)
     f32x16 st[W::NBW];
@@ -1422,11 +1464,11 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
     // workgroup's own chain load -> barrier -> product bounds its rate): three chunks in flight.
     constexpr int SETS = walk_totals_sets(D);
     auto load_chunk = [&](int c, int set) {
-        walk_load_tile<D>(ry, lds0 + set * 2 * W::TILE, c * W::C, ys2, p.dy, wave, lane);
+        walk_load_tile<D>(ry, lds0 + set * 2 * W::TILE, c * W::C, ys2, dy, wave, lane);
         walk_load_tile<D>(rz, lds0 + set * 2 * W::TILE + W::TILE, c * W::C, zs2, p.dz, wave, lane);
     };
     auto map_tile = [&](unsigned char *ty, int c) {
-        walk_map_tile<T, D>(ty, p.map_y, c * W::C, N, p.dy, static_cast<T *>(p.ymap_out) + b * p.yo_b + h * p.yo_h,
+        walk_map_tile<T, D>(ty, p.map_y, c * W::C, N, dy, static_cast<T *>(p.ymap_out) + b * p.yo_b + h * p.yo_h,
                             p.yo_n, tid);
         __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the rewritten tile is in LDS
         __builtin_amdgcn_s_barrier();
@@ -1503,12 +1545,15 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
 // `cols`: only the first `cols` columns of every row of the D-wide states are summed (the totals
 // kernel built for a narrow v side writes no others, and no walk of that extent reads them).
 // (a template only so that the header can be included by several translation units)
+// grid y = 1 scans a second pair of buffers of the same shape (totals_b, entry_b; the other half of a wide q / k).
 template <int kUnused = 0>
 __global__ __launch_bounds__(256) void walk_scan_kernel(const float *totals, float *entry, int n_seg, int E,
-                                                        int64_t total2, int reverse, int D, int cols) {
+                                                        int64_t total2, int reverse, int D, int cols,
+                                                        const float *totals_b, float *entry_b) {
     typedef float f32x2 __attribute__((ext_vector_type(2)));
     const int64_t i2 = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i2 >= total2) return;
+    if (blockIdx.y != 0) totals = totals_b, entry = entry_b;
     const int half = cols / 2;
     const int64_t per_bh = (int64_t)(E / D) * half, bh = i2 / per_bh, r = i2 - bh * per_bh;
     const int64_t e = (r / half) * D + 2 * (r % half);
@@ -1646,25 +1691,31 @@ hipError_t launch_walk_totals(const WalkTotalsParams &p, hipStream_t stream) {
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     constexpr int smem = walk_totals_sets(D) * 2 * WalkCfg<D>::TILE;
     if (p.direct && (p.n_seg != 2 || p.seg_lo < 0 || p.seg_lo > 1)) return hipErrorInvalidValue;
+    // (a second operand runs the same kernel variant: the caller pairs operands of one kind only)
+    if (p.y2 && (p.map_y || !p.totals2 || walk_totals_cols(D, p.dy2, p.dz) != walk_totals_cols(D, p.dy, p.dz)))
+        return hipErrorInvalidValue;
+    const dim3 g((unsigned)grid, p.y2 ? 2u : 1u);
     if constexpr (D == 128) {
         if (walk_totals_cols(D, p.dy, p.dz) == 64) {  // z of at most 64 true columns: the state's other v blocks hold zeros
             constexpr auto kern = walk_totals_kernel<T, D, 4, 2>;
             if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-            return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), smem, stream, p);
+            return launch_kernel<kern>(g, dim3(256), smem, stream, p);
         }
     }
     constexpr auto kern = walk_totals_kernel<T, D>;
     if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
-    return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), smem, stream, p);
+    return launch_kernel<kern>(g, dim3(256), smem, stream, p);
 }
 
 inline hipError_t launch_walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, int D, int cols,
-                                   int reverse, hipStream_t stream) {
+                                   int reverse, hipStream_t stream, const float *totals_b = nullptr,
+                                   float *entry_b = nullptr) {
     const int E = D * D;
     const int64_t total2 = BH * D * (cols / 2);
-    if (n_seg < 1 || cols < 2 || cols > D || cols % 2) return hipErrorInvalidValue;
-    return launch_kernel<walk_scan_kernel<0>>(dim3((unsigned)((total2 + 255) / 256)), dim3(256), 0, stream, totals, entry,
-                         n_seg, E, total2, reverse, D, cols);
+    if (n_seg < 1 || cols < 2 || cols > D || cols % 2 || (totals_b != nullptr) != (entry_b != nullptr))
+        return hipErrorInvalidValue;
+    return launch_kernel<walk_scan_kernel<0>>(dim3((unsigned)((total2 + 255) / 256), totals_b ? 2u : 1u), dim3(256), 0,
+                                              stream, totals, entry, n_seg, E, total2, reverse, D, cols, totals_b, entry_b);
 }
 
 template <auto kern>

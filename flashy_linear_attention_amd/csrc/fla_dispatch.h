@@ -58,5 +58,5 @@ hipError_t walk_dkdv(int dtype, int D, const WalkParams &p, hipStream_t stream);
 hipError_t walk_vec_sums(int dtype, int D, const WalkVecParams &p, int64_t BH, hipStream_t stream);
 hipError_t walk_vec_scan(float *v, int64_t BH, int n_chunks, int D, int reverse, hipStream_t stream);
 hipError_t walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, int D, int cols, int reverse,
-                     hipStream_t stream);
+                     hipStream_t stream, const float *totals_b = nullptr, float *entry_b = nullptr);
 }  // namespace fla

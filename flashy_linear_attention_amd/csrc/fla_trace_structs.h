@@ -67,7 +67,8 @@ FLA_FIELDS_BEGIN(WalkTotalsParams)
 FLA_FIELD(y) FLA_FIELD(z) FLA_FIELD(ys_b) FLA_FIELD(ys_h) FLA_FIELD(ys_n) FLA_FIELD(zs_b) FLA_FIELD(zs_h)
 FLA_FIELD(zs_n) FLA_FIELD(H) FLA_FIELD(N) FLA_FIELD(BH) FLA_FIELD(dy) FLA_FIELD(dz) FLA_FIELD(n_chunks)
 FLA_FIELD(seg_chunks) FLA_FIELD(n_seg) FLA_FIELD(seg_lo) FLA_FIELD(seg_hi) FLA_FIELD(totals) FLA_FIELD(direct)
-FLA_FIELD(map_y) FLA_FIELD(ymap_out) FLA_FIELD(yo_b) FLA_FIELD(yo_h) FLA_FIELD(yo_n)
+FLA_FIELD(map_y) FLA_FIELD(ymap_out) FLA_FIELD(yo_b) FLA_FIELD(yo_h) FLA_FIELD(yo_n) FLA_FIELD(y2) FLA_FIELD(dy2)
+FLA_FIELD(totals2)
 FLA_FIELDS_END
 
 FLA_FIELDS_BEGIN(WalkVecParams)

@@ -38,8 +38,8 @@ hipError_t walk_vec_scan(float *v, int64_t BH, int n_chunks, int D, int reverse,
     return launch_walk_vec_scan(v, BH, n_chunks, D, reverse, stream);
 }
 hipError_t walk_scan(const float *totals, float *entry, int64_t BH, int n_seg, int D, int cols, int reverse,
-                     hipStream_t stream) {
-    return launch_walk_scan(totals, entry, BH, n_seg, D, cols, reverse, stream);
+                     hipStream_t stream, const float *totals_b, float *entry_b) {
+    return launch_walk_scan(totals, entry, BH, n_seg, D, cols, reverse, stream, totals_b, entry_b);
 }
 
 }  // namespace fla

@@ -26,7 +26,7 @@ import torch
 from torch.autograd import Function
 
 from . import _lib
-from .kernels._common import dtype_code, prepare, stream_handle
+from .kernels._common import device_guard, dtype_code, prepare, stream_handle
 
 FEATURE_MAPS = {"elu1": 1, "softplus": 2}  # enum fla_feature_map
 
@@ -53,10 +53,10 @@ def feature_attention_fwd(xq: torch.Tensor, xk: torch.Tensor, v: torch.Tensor, f
     q = torch.empty_like(xq, memory_format=torch.contiguous_format)
     k = torch.empty_like(xk, memory_format=torch.contiguous_format)
     lib = _lib.load()
-    with torch.cuda.device(xq.device):
-        sbytes = lib.fla_linear_attn_chunked_state_bytes(b, h, n, dqk, dv) if want_state else 0
+    with device_guard(xq.device):
+        sbytes = _lib.query("fla_linear_attn_chunked_state_bytes", b, h, n, dqk, dv) if want_state else 0
         state = torch.empty(sbytes, dtype=torch.uint8, device=xq.device) if sbytes else None
-        wbytes = lib.fla_linear_attn_chunked_workspace_bytes(b, h, n, dqk, dv)
+        wbytes = _lib.query("fla_linear_attn_chunked_workspace_bytes", b, h, n, dqk, dv)
         work = torch.empty(max(wbytes, 16), dtype=torch.uint8, device=xq.device)
         valid = ctypes.c_int32(0)
         _lib.check(
@@ -87,10 +87,10 @@ def feature_attention_bwd(grad_output: torch.Tensor, q: torch.Tensor, k: torch.T
     dxk = torch.empty_like(xk, memory_format=torch.contiguous_format)
     dvv = torch.empty_like(v, memory_format=torch.contiguous_format)
     lib = _lib.load()
-    with torch.cuda.device(xq.device):
+    with device_guard(xq.device):
         if state is not None:
-            assert state.numel() == lib.fla_linear_attn_chunked_state_bytes(b, h, n, dqk, dv), "state of another shape"
-        wbytes = lib.fla_linear_attn_chunked_workspace_bytes(b, h, n, dqk, dv)
+            assert state.numel() == _lib.query("fla_linear_attn_chunked_state_bytes", b, h, n, dqk, dv), "state of another shape"
+        wbytes = _lib.query("fla_linear_attn_chunked_workspace_bytes", b, h, n, dqk, dv)
         work = torch.empty(max(wbytes, 16), dtype=torch.uint8, device=xq.device)
         _lib.check(
             "fla_feature_attn_bwd",
@@ -121,10 +121,10 @@ def feature_attention_normalised_fwd(xq: torch.Tensor, xk: torch.Tensor, v: torc
     k = torch.empty_like(xk, memory_format=torch.contiguous_format)
     denom = torch.empty(b, h, n, dtype=torch.float32, device=xq.device)
     lib = _lib.load()
-    with torch.cuda.device(xq.device):
-        nbytes = lib.fla_normalised_workspace_bytes(b, h, n, dqk, dv, int(chunked))
+    with device_guard(xq.device):
+        nbytes = _lib.query("fla_normalised_workspace_bytes", b, h, n, dqk, dv, int(chunked))
         work = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=xq.device)
-        sbytes = lib.fla_linear_attn_chunked_state_bytes(b, h, n, dqk, dv) if (want_state and chunked) else 0
+        sbytes = _lib.query("fla_linear_attn_chunked_state_bytes", b, h, n, dqk, dv) if (want_state and chunked) else 0
         state = torch.empty(sbytes, dtype=torch.uint8, device=xq.device) if sbytes else None
         valid = ctypes.c_int32(0)
         _lib.check(
@@ -157,8 +157,8 @@ def feature_attention_normalised_bwd(grad_output: torch.Tensor, q: torch.Tensor,
     dxk = torch.empty_like(k, memory_format=torch.contiguous_format)
     dvv = torch.empty_like(v, memory_format=torch.contiguous_format)
     lib = _lib.load()
-    with torch.cuda.device(q.device):
-        nbytes = lib.fla_normalised_workspace_bytes(b, h, n, dqk, dv, int(chunked))
+    with device_guard(q.device):
+        nbytes = _lib.query("fla_normalised_workspace_bytes", b, h, n, dqk, dv, int(chunked))
         work = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=q.device)
         _lib.check(
             "fla_feature_attn_normalised_bwd",

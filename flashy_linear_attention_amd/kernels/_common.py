@@ -28,23 +28,60 @@ def prepare(*tensors: torch.Tensor) -> Tuple[torch.Tensor, ...]:
     first = tensors[0]
     if not first.is_cuda:
         raise RuntimeError("flashy_linear_attention_amd operators need tensors on a ROCm GPU (device 'cuda')")
-    out = []
+    device, dtype = first.device, first.dtype
+    dense = True
     for t in tensors:
         if t.dim() != 4:
             raise ValueError(f"expected (batch, heads, seq, head_dim) tensors, got shape {tuple(t.shape)}")
-        if t.device != first.device:
+        if t.device != device:
             raise RuntimeError("all tensors must be on the same device")
-        if t.dtype != first.dtype:
-            raise TypeError(f"all tensors must share one dtype, got {first.dtype} and {t.dtype}")
-        if t.stride(-1) != 1 and t.shape[-1] > 1:
-            t = t.contiguous()
-        out.append(t)
-    return tuple(out)
+        if t.dtype != dtype:
+            raise TypeError(f"all tensors must share one dtype, got {dtype} and {t.dtype}")
+        dense = dense and t.stride(3) == 1
+    if dense:  # (the usual case: nothing to copy, the caller's tuple goes back as it came)
+        return tensors
+    return tuple(t.contiguous() if (t.stride(3) != 1 and t.shape[3] > 1) else t for t in tensors)
+
+
+try:  # the current stream's handle as a plain integer, without building a torch.cuda.Stream object
+    _raw_stream = torch._C._cuda_getCurrentRawStream
+except AttributeError:  # pragma: no cover - older or differently built torch
+    _raw_stream = None
 
 
 def stream_handle(device: torch.device) -> int:
+    if _raw_stream is not None:
+        return _raw_stream(device.index if device.index is not None else torch.cuda.current_device())
     return torch.cuda.current_stream(device).cuda_stream
 
 
+class _NoGuard:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_GUARD = _NoGuard()
+
+
+def device_guard(device: torch.device):
+    """Context that makes `device` the current one for the call into the library (which launches on
+    the current device).  When it already is -- the usual case -- nothing is switched: entering and
+    leaving torch.cuda.device costs two device exchanges per call."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_GUARD
+    return torch.cuda.device(device)
+
+
+_FUNCS = {}
+
+
 def call(name: str, *args) -> None:
-    _lib.check(name, getattr(_lib.load(), name)(*args))
+    fn = _FUNCS.get(name)
+    if fn is None:
+        fn = _FUNCS[name] = getattr(_lib.load(), name)
+    status = fn(*args)
+    if status != 0:
+        _lib.check(name, status)

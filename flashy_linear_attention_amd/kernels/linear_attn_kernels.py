@@ -16,7 +16,7 @@ from typing import Tuple
 import torch
 
 from .. import _lib
-from ._common import call, dtype_code, next_power_of_2, prepare, stream_handle
+from ._common import call, device_guard, dtype_code, next_power_of_2, prepare, stream_handle
 
 
 def _block_sq(hd: int) -> int:
@@ -34,7 +34,7 @@ def linear_flash_wrapper_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) 
 
     q, k, v = prepare(q, k, v)
     out = torch.empty_like(q, memory_format=torch.contiguous_format)
-    with torch.cuda.device(q.device):
+    with device_guard(q.device):
         call(
             "fla_linear_attn_fwd",
             q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
@@ -61,7 +61,7 @@ def linear_flash_wrapper_bwd(
     dQ = torch.empty_like(q, memory_format=torch.contiguous_format)
     dK = torch.empty_like(k, memory_format=torch.contiguous_format)
     dV = torch.empty_like(v, memory_format=torch.contiguous_format)
-    with torch.cuda.device(q.device):
+    with device_guard(q.device):
         call(
             "fla_linear_attn_bwd",
             grad_output.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),
@@ -91,7 +91,7 @@ def linear_flash_wrapper_bwd_fused_dkdv(
     dQ = torch.empty_like(q, memory_format=torch.contiguous_format)
     dK = torch.empty_like(k, memory_format=torch.contiguous_format)
     dV = torch.empty_like(v, memory_format=torch.contiguous_format)
-    with torch.cuda.device(q.device):
+    with device_guard(q.device):
         call(
             "fla_linear_attn_bwd_fused_dkdv",
             grad_output.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(),

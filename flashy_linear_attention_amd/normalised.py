@@ -21,17 +21,17 @@ import torch
 from torch.autograd import Function
 
 from . import _lib
-from .kernels._common import dtype_code, prepare, stream_handle
+from .kernels._common import device_guard, dtype_code, prepare, stream_handle
 
 
 def _workspace(lib, b: int, h: int, n: int, dqk: int, dv: int, chunked: bool,
                device: torch.device) -> Tuple[torch.Tensor, int]:
-    nbytes = lib.fla_normalised_workspace_bytes(b, h, n, dqk, dv, int(chunked))
+    nbytes = _lib.query("fla_normalised_workspace_bytes", b, h, n, dqk, dv, int(chunked))
     return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=device), nbytes
 
 
 def _state_buffer(lib, b: int, h: int, n: int, dqk: int, dv: int, want: bool, device: torch.device):
-    sbytes = lib.fla_linear_attn_chunked_state_bytes(b, h, n, dqk, dv) if want else 0
+    sbytes = _lib.query("fla_linear_attn_chunked_state_bytes", b, h, n, dqk, dv) if want else 0
     return torch.empty(sbytes, dtype=torch.uint8, device=device) if sbytes else None
 
 
@@ -51,7 +51,7 @@ def linear_attention_normalised_fwd(
     out = torch.empty_like(v, memory_format=torch.contiguous_format)
     denom = torch.empty(b, h, n, dtype=torch.float32, device=q.device)
     lib = _lib.load()
-    with torch.cuda.device(q.device):
+    with device_guard(q.device):
         work, nbytes = _workspace(lib, b, h, n, dqk, dv, chunked, q.device)
         state = _state_buffer(lib, b, h, n, dqk, dv, want_state and chunked, q.device)
         valid = ctypes.c_int32(0)
@@ -83,7 +83,7 @@ def linear_attention_normalised_bwd(
     dk = torch.empty_like(k, memory_format=torch.contiguous_format)
     dvv = torch.empty_like(v, memory_format=torch.contiguous_format)
     lib = _lib.load()
-    with torch.cuda.device(q.device):
+    with device_guard(q.device):
         work, nbytes = _workspace(lib, b, h, n, dqk, dv, chunked, q.device)
         _lib.check(
             "fla_linear_attn_normalised_bwd",

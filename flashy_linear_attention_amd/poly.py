@@ -22,7 +22,7 @@ import torch
 from torch.autograd import Function
 
 from . import _lib
-from .kernels._common import dtype_code, prepare, stream_handle
+from .kernels._common import device_guard, dtype_code, prepare, stream_handle
 
 
 def _coef(c0: float, c1: float, c2: float):
@@ -48,7 +48,7 @@ def poly_attention_fwd(
     out = torch.empty_like(v, memory_format=torch.contiguous_format)
     denom = torch.empty(b, h, n, dtype=torch.float32, device=xq.device) if normalise else None
     lib = _lib.load()
-    with torch.cuda.device(xq.device):
+    with device_guard(xq.device):
         _lib.check(
             "fla_poly_attn_fwd",
             lib.fla_poly_attn_fwd(
@@ -78,8 +78,8 @@ def poly_attention_bwd(
     dxk = torch.empty_like(xk, memory_format=torch.contiguous_format)
     dvv = torch.empty_like(v, memory_format=torch.contiguous_format)
     lib = _lib.load()
-    with torch.cuda.device(xq.device):
-        nbytes = lib.fla_poly_attn_workspace_bytes(b, h, n, r, dv)
+    with device_guard(xq.device):
+        nbytes = _lib.query("fla_poly_attn_workspace_bytes", b, h, n, r, dv)
         work = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=xq.device)
         _lib.check(
             "fla_poly_attn_bwd",

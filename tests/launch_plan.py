@@ -797,7 +797,15 @@ def model_walk_totals(arena: Arena, l: Launch, p: Dict, D: int, stats: Stats) ->
     assert n_chunks == -(-N // rows) and (n_seg - 1) * seg_chunks < n_chunks <= n_seg * seg_chunks
     assert 0 <= p["seg_lo"] <= p["seg_hi"] <= n_seg
     assert l.grid[0] == 8 * ((BH + 7) // 8) * n_seg
-    for nm, ptr, sb, sh, sn, w in (("y", "y", "ys_b", "ys_h", "ys_n", p["dy"]), ("z", "z", "zs_b", "zs_h", "zs_n", p["dz"])):
+    operands = [("y", "y", "ys_b", "ys_h", "ys_n", p["dy"]), ("z", "z", "zs_b", "zs_h", "zs_n", p["dz"])]
+    if p["y2"]:  # a second Y operand (the other half of a wide q / k) in the same launch
+        assert l.grid[1] == 2 and not p["map_y"] and p["totals2"]
+        operands.append(("y2", "y2", "ys_b", "ys_h", "ys_n", p["dy2"]))
+        arena.require("segment totals of the second operand", p["totals2"], p["totals2"] + BH * n_seg * D * D * 4)
+        assert not (p["totals"] <= p["totals2"] < p["totals"] + BH * n_seg * D * D * 4), "the two operands' totals overlap"
+    else:
+        assert l.grid[1] == 1
+    for nm, ptr, sb, sh, sn, w in operands:
         lo, hi = tensor_extent(p, ptr, sb, sh, sn, H, BH, N, w)
         arena.require(f"totals {nm}", lo, hi)
     arena.require("segment totals", p["totals"], p["totals"] + BH * n_seg * D * D * 4)
@@ -854,6 +862,14 @@ def check_all(arena: Arena, launches: List[Launch], stats: Stats) -> None:
                 arena.require("wsum", wsum, wsum + BH * chunks * DP * 4)
         elif k in ("walk_fwd_kernel", "walk_bwd_kernel", "walk_dkdv_kernel", "walk_bwd_rev_kernel"):
             model_walk(arena, l, l.struct("a0"), t[1], stats)
+        elif k == "walk_scan_kernel":
+            totals, entry, n_seg, E, total2 = (l.args[f"a{i}"] for i in range(5))
+            totals_b, entry_b = l.args["a8"], l.args["a9"]
+            BH = total2 // (E // l.args["a6"] * (l.args["a7"] // 2))
+            assert l.grid[1] == (2 if totals_b else 1) and bool(totals_b) == bool(entry_b)
+            for t_, e_ in ((totals, entry),) + (((totals_b, entry_b),) if totals_b else ()):
+                arena.require("segment totals", t_, t_ + BH * n_seg * E * 4)
+                arena.require("entry states", e_, e_ + BH * n_seg * E * 4)
         elif k == "walk_totals_kernel":
             model_walk_totals(arena, l, l.struct("a0"), t[1], stats)
         else:
