@@ -275,7 +275,12 @@ def _other_workload(torch, name, algo, dev, steps):
         ff, fb = _chunked_flops(w)
         rec.update({"gbps_algorithmic": round(gbs, 1), "bound": "hbm", "frac_of_peak": round(gbs / HBM_PEAK_GBS, 4),
                     "own_tflops": round((ff + fb) / (ms_step * 1e-3) / 1e12, 1),
-                    "bytes": "each operand read once, each result written once"})
+                    "bytes": "each operand read once, each result written once",
+                    "algorithmic_bytes_per_step": nbytes})
+        traffic, src = PROFILED_TRAFFIC.get((name, algo), (None, None))
+        if traffic is not None:  # HBM bytes all kernels of a step move (rocprofv3 FETCH_SIZE / WRITE_SIZE, see the file)
+            rec.update({"traffic_bytes_per_step": traffic, "traffic_over_algorithmic_bytes": round(traffic / nbytes, 2),
+                        "traffic_gbps": round(traffic / (ms_step * 1e-3) / 1e9, 1), "traffic_source": src})
     del o
     torch.cuda.empty_cache()
     return rec

@@ -46,10 +46,31 @@ def _hipcc() -> str:
     return exe
 
 
-def _run(cmd: List[str]) -> None:
+def _run(cmd: List[str]) -> str:
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if proc.returncode != 0:
         raise RuntimeError("command failed: " + " ".join(cmd) + "\n" + proc.stdout)
+    return proc.stdout
+
+
+def _check_no_scratch(report: str, kernel: str) -> None:
+    """Fail the build if an instantiation of `kernel` spills registers.  The reverse walk keeps its
+    running sums in accumulation registers through MFMAs issued from inline assembly, with the wait
+    states they need placed by hand; a spill or reload the register allocator put between two of them
+    would get none and read stale values without any error.  `report`: the compiler's
+    -Rpass-analysis=kernel-resource-usage remarks."""
+    name, seen = None, 0
+    for line in report.splitlines():
+        if "Function Name:" in line:
+            name = line.split("Function Name:")[1].split()[0]
+        elif "ScratchSize" in line and name and kernel in name:
+            seen += 1
+            size = int(line.split("ScratchSize [bytes/lane]:")[1].split()[0])
+            if size != 0:
+                raise RuntimeError(f"{name} uses {size} bytes of scratch per lane: its hand-placed MFMA wait states "
+                                   "assume that no spill code sits between its MFMAs")
+    if seen == 0:
+        raise RuntimeError(f"no resource report for {kernel}: the spill check did not run")
 
 
 def _compile_inst(args) -> str:
@@ -70,7 +91,9 @@ def build(jobs: int | None = None, verbose: bool = True) -> str:
     capi = os.path.join(OBJ_DIR, "fla_capi.o")
     _run([_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, "fla_capi.hip"), "-o", capi])
     walk = os.path.join(OBJ_DIR, "fla_walk_inst.o")
-    _run([_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, "fla_walk_inst.hip"), "-o", walk])
+    report = _run([_hipcc(), *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", "-c",
+                   os.path.join(CSRC, "fla_walk_inst.hip"), "-o", walk])
+    _check_no_scratch(report, "walk_bwd_rev_kernel")
     # (this one without the VGPR form of MFMA: see the file's header)
     pair = os.path.join(OBJ_DIR, "fla_pair_inst.o")
     pair_flags = [f for f in HIPCC_FLAGS if f not in ("-mllvm", "-amdgpu-mfma-vgpr-form")]

@@ -39,10 +39,13 @@ def _cases(seed: int, count: int):
     return out
 
 
+# (every third case in fp16: both storage types of the walk kernels, whose reverse walk issues its state
+# MFMAs from per-type inline assembly)
 @pytest.mark.parametrize("case", _cases(20240607, 48), ids=lambda c: "x".join(map(str, c[:5])))
 def test_chunked_random_shapes_vs_fp32_formula(case, gpu_device):
     b, h, n, dqk, dv, seed = case
-    q, k, v, dy = (t.to(gpu_device) for t in reference_style_inputs(b, h, n, dqk, dv, torch.bfloat16, seed=seed))
+    dtype = torch.float16 if seed % 3 == 0 else torch.bfloat16
+    q, k, v, dy = (t.to(gpu_device) for t in reference_style_inputs(b, h, n, dqk, dv, dtype, seed=seed))
     want_o, want_g = gpu_fp32_reference(q, k, v, dy, True)
     qg, kg, vg = (t.clone().requires_grad_(True) for t in (q, k, v))
     out = LinearAttentionChunked.apply(qg, kg, vg)
@@ -56,7 +59,7 @@ def test_chunked_random_shapes_vs_fp32_formula(case, gpu_device):
                          ids=lambda c: "x".join(map(str, c[:5])))
 def test_normalised_chunked_random_shapes_vs_oracle(case, gpu_device):
     b, h, n, dqk, dv, seed = case
-    q, k, v, dy = reference_style_inputs(b, h, n, dqk, dv, torch.bfloat16, seed=seed)
+    q, k, v, dy = reference_style_inputs(b, h, n, dqk, dv, torch.float16 if seed % 3 == 0 else torch.bfloat16, seed=seed)
     qo, ko, vo = (t.to(gpu_device).float().requires_grad_(True) for t in (q, k, v))
     want = naive.linear_attention_normalised(qo, ko, vo, eps=1e-5)
     want.backward(dy.to(gpu_device).float())
