@@ -186,7 +186,7 @@ def test_normalised_operator_over_the_sweep_space(lib, dims):
         n = _clip_n(bh, n0, dqk, dv)
         # (the lane-level model is the slow part: every (B H, N) for the shapes of the silent case,
         # a thinned grid for the others)
-        if dims != (72, 72) and (bh + n0) % 5 != 0:
+        if (bh + n0) % (2 if dims == (72, 72) else 5) != 0 and not (dims == (72, 72) and (bh, n0) == (160, 300)):
             continue
         b = 2 if bh % 2 == 0 and bh > 1 else 1
         arena, launches = trace_normalised(lib, b, bh // b, n, dqk, dv, chunked)
@@ -201,10 +201,11 @@ def test_normalised_operator_over_the_sweep_space(lib, dims):
 def test_plain_operator(lib, dims, chunked):
     dqk, dv = dims
     stats = lp.Stats()
-    for (bh, n), dtype, layout in itertools.product(((1, 64), (3, 192), (17, 1000), (64, 2048), (160, 300), (256, 512),
-                                                     (128, 4096)), (0, 1),
+    for (bh, n), dtype, layout in itertools.product(((1, 64), (3, 192), (17, 1000), (160, 300), (256, 512), (128, 4096)),
+                                                    (0, 1),
                                                     ("contiguous", "bnhd", "padded", "odd", "expanded")):
-        if layout != "contiguous" and (bh + n + dtype) % 2:
+        # (other layouts: bf16, three of the sizes; the two storage types share all host code but the kernel table)
+        if layout != "contiguous" and (dtype or (bh, n) not in ((3, 192), (160, 300), (128, 4096))):
             continue
         n = _clip_n(bh, n, dqk, dv)
         b = 2 if bh % 2 == 0 and bh > 1 else 1
