@@ -1019,7 +1019,10 @@ inline bool fast_path_ok(const TriParams &p) {
 // workgroups each) runs as single tiles, heaviest first: pairs would leave slots idle (measured
 // 7-20 % faster there).  Exactly one pair per CU stays paired: every CU then has the same work
 // (1-4 % faster than single tiles; also for the kernels that could run two workgroups per CU:
-// fp16 B 4, H 16, N 2048, D 64 forward takes 34.4 us paired, 35.7 us as 512 unequal single tiles).
+// fp16 B 4, H 16, N 2048, D 64 forward takes 34.0 - 34.6 us paired, 35.7 us as 512 single tiles heaviest
+// first, 33.7 us with the tiles ordered so that workgroups g and g + 256, which share a CU, add up to
+// equal work -- within the spread between runs, not kept --, 37.6 us with neighbours in the grid
+// complementary).
 constexpr int kCuCount = 256;
 inline int run_single_tiles(int64_t pairs, int workgroups_per_cu) {
     return pairs < (int64_t)kCuCount * workgroups_per_cu && pairs % kCuCount != 0;
