@@ -623,17 +623,14 @@ int wide_forward(const WidePlan &wide, const View &q, const View &k, const View 
         }
         if (int rc = wide_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, work, keep, entry, s)) return rc;
     }
-    for (int h = 0; h < 2; ++h) {
-        const View qh = column_half(q, h), kh = column_half(k, h);
-        const int64_t wqk = h == 0 ? 128 : dqk - 128;
-        // (the second half's walk adds its result to the first one's)
-        fla::WalkParams w = lower_walk_params(wp, qh, kh, v, o, B, H, N, wqk, dv, entry[h]);
-        w.accumulate = h;
-        if (state_out)  // (behind this half's entry states: the state after the last chunk)
-            w.total_out = reinterpret_cast<float *>(static_cast<char *>(state_out) + h * wp.saved_bytes + wp.entry_bytes);
-        if (fla::walk_fwd(dtype, wp.D, w, s) != hipSuccess) return FLA_ERR_LAUNCH;
+    // one walk over both halves (the second one's columns start 128 elements into q's and k's rows)
+    fla::WalkParams w = lower_walk_params(wp, q, k, v, o, B, H, N, 128, dv, entry[0]);
+    w.wqk2 = (int32_t)(dqk - 128), w.init2 = wp.n_seg > 1 ? entry[1] : nullptr;
+    if (state_out) {  // (behind each half's entry states: its state after the last chunk)
+        w.total_out = reinterpret_cast<float *>(static_cast<char *>(state_out) + wp.entry_bytes);
+        w.total_out2 = reinterpret_cast<float *>(static_cast<char *>(state_out) + wp.saved_bytes + wp.entry_bytes);
     }
-    return FLA_OK;
+    return fla::walk_fwd_wide(dtype, w, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
 }
 
 int wide_backward(const WidePlan &wide, const View &go, const View &q, const View &k, const View &v, const View &dq,

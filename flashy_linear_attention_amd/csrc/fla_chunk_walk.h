@@ -122,6 +122,13 @@ struct WalkParams {
     // D = 128, plain: the result (forward: o; walk_bwd_rev_kernel: dv) is added to what its place in
     // memory holds already -- the second of two walks whose results sum up (halves of a wide q / k)
     int32_t accumulate;
+    // The wide walks (walk_fwd_wide_kernel, walk_bwd_rev_wide_kernel): q and k (dq and dk) have 129 .. 256
+    // columns.  Columns 128 .. are the second half, of true width wqk2 (wqk = 128 is the first half's), with
+    // entry and final states of its own in the layouts of init, total_out, xinit and xtotal.
+    int32_t wqk2;
+    const float *init2;
+    float *total_out2;
+    const float *xinit2, *xtotal2;
 };
 
 template <int D>
@@ -339,8 +346,9 @@ __device__ __forceinline__ void walk_pipe(Read &&read, Use &&use) {
 }
 
 // KCL: 16-wide k chunks of the contraction X Y^T that hold anything; NOB: output blocks that do.
-template <typename T, int D, bool UPPER, int EX = 0, int KCL = WalkCfg<D>::KC, int NOB = WalkCfg<D>::DB, typename SFrag,
-          typename YRows = WalkNoRows>
+// KEEP: the product is added to what acc holds.
+template <typename T, int D, bool UPPER, int EX = 0, int KCL = WalkCfg<D>::KC, int NOB = WalkCfg<D>::DB, bool KEEP = false,
+          typename SFrag, typename YRows = WalkNoRows>
 __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsigned char *yt, const unsigned char *zt,
                                              int wave, int lane, bool has_state, SFrag &&sfrag,
                                              f32x16 (&acc)[WalkCfg<D>::DBW], float *ex = nullptr,
@@ -365,10 +373,12 @@ __device__ __forceinline__ void walk_product(const unsigned char *xt, const unsi
                 for (int b = 0; b < 4; ++b) rsum += static_cast<float>(xf[kc][4 * a + b]) * z[b];
             }
     }
+    if constexpr (!KEEP) {
 #pragma unroll
-    for (int i = 0; i < W::DBW; ++i)
+        for (int i = 0; i < W::DBW; ++i)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+            for (int v = 0; v < 16; ++v) acc[i][v] = 0.f;
+    }
     // One 32-row block s of Y and Z: scores, mask and rounding, second product.  ST: the state product's
     // MFMAs are issued in between -- PER / 2 of them after every score MFMA (they share its X fragment
     // and fill the gaps of the dependent chain), the rest after the last one, where the rounding of the
@@ -749,43 +759,54 @@ __device__ __forceinline__ void walk_sum_states(const float *buf, int f_lo, int 
     for (int f = f_lo; f < f_hi; ++f) walk_read_state<D, B, true>(buf + (int64_t)f * (D * D), transposed, wave, lane, st);
 }
 
-// this wave's blocks of the entry state of segment sl.seg (zeros without an init buffer) of a walk
-// in ascending (`reverse` false) or descending order of the chunks
+// this wave's blocks of the entry state of segment sl.seg (zeros without a buffer) of a walk in
+// ascending (`reverse` false) or descending order of the chunks; `buf`: the entry states of one operand
 template <int D, typename B = WalkExt<D>>
-__device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSlice &sl, int wave, int lane,
-                                               f32x16 (&st)[WalkCfg<D>::NBW], bool reverse) {
+__device__ __forceinline__ void walk_load_init_from(const float *buf, const WalkParams &p, const WalkSlice &sl, int wave,
+                                                    int lane, f32x16 (&st)[WalkCfg<D>::NBW], bool reverse) {
     const float *init = nullptr, *init2 = nullptr;
-    if (p.init) {
+    if (buf) {
         if (p.n_seg == 2) {
-            if (sl.seg != (reverse ? 1 : 0)) init = p.init + (int64_t)sl.bh * 2 * (D * D), init2 = init + D * D;
+            if (sl.seg != (reverse ? 1 : 0)) init = buf + (int64_t)sl.bh * 2 * (D * D), init2 = init + D * D;
         } else if (walk_entries_are_totals(D, p.n_seg)) {
-            walk_sum_states<D, B>(p.init + (int64_t)sl.bh * p.n_seg * (D * D), reverse ? sl.seg + 1 : 0,
+            walk_sum_states<D, B>(buf + (int64_t)sl.bh * p.n_seg * (D * D), reverse ? sl.seg + 1 : 0,
                                   reverse ? p.n_seg : sl.seg, p.init_transposed != 0, wave, lane, st);
             return;
         } else {
-            init = p.init + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D);
+            init = buf + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D);
         }
     }
     walk_load_state<D, B>(init, p.init_transposed != 0, wave, lane, st, init2);
+}
+template <int D, typename B = WalkExt<D>>
+__device__ __forceinline__ void walk_load_init(const WalkParams &p, const WalkSlice &sl, int wave, int lane,
+                                               f32x16 (&st)[WalkCfg<D>::NBW], bool reverse) {
+    walk_load_init_from<D, B>(p.init, p, sl, wave, lane, st, reverse);
 }
 
 // the forward state at the end of segment sl.seg from what forward handed over: the entry state of
 // the next segment (xinit, in the forms above) or, for the last one, the final state (xtotal)
 template <int D, typename B = WalkExt<D>>
-__device__ __forceinline__ void walk_load_end_state(const WalkParams &p, const WalkSlice &sl, int wave, int lane,
-                                                    f32x16 (&xs)[WalkCfg<D>::NBW]) {
-    const float *x = p.xtotal + (int64_t)sl.bh * (D * D), *x2 = nullptr;
+__device__ __forceinline__ void walk_load_end_state_from(const float *xinit, const float *xtotal, const WalkParams &p,
+                                                         const WalkSlice &sl, int wave, int lane,
+                                                         f32x16 (&xs)[WalkCfg<D>::NBW]) {
+    const float *x = xtotal + (int64_t)sl.bh * (D * D), *x2 = nullptr;
     if (sl.c_hi < p.n_chunks) {
         if (p.n_seg == 2) {
-            x = p.xinit + (int64_t)sl.bh * 2 * (D * D), x2 = x + D * D;
+            x = xinit + (int64_t)sl.bh * 2 * (D * D), x2 = x + D * D;
         } else if (walk_entries_are_totals(D, p.n_seg)) {
-            walk_sum_states<D, B>(p.xinit + (int64_t)sl.bh * p.n_seg * (D * D), 0, sl.seg + 1, false, wave, lane, xs);
+            walk_sum_states<D, B>(xinit + (int64_t)sl.bh * p.n_seg * (D * D), 0, sl.seg + 1, false, wave, lane, xs);
             return;
         } else {
-            x = p.xinit + ((int64_t)sl.bh * p.n_seg + sl.seg + 1) * (D * D);
+            x = xinit + ((int64_t)sl.bh * p.n_seg + sl.seg + 1) * (D * D);
         }
     }
     walk_load_state<D, B>(x, false, wave, lane, xs, x2);
+}
+template <int D, typename B = WalkExt<D>>
+__device__ __forceinline__ void walk_load_end_state(const WalkParams &p, const WalkSlice &sl, int wave, int lane,
+                                                    f32x16 (&xs)[WalkCfg<D>::NBW]) {
+    walk_load_end_state_from<D, B>(p.xinit, p.xtotal, p, sl, wave, lane, xs);
 }
 
 // ---- one product with its running state, chunks ascending:
@@ -968,6 +989,128 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
         if constexpr (NQ < W::DB) {
             for (int e = tid; e < D * D; e += 256)
                 if (e / D >= 32 * NQ || e % D >= 32 * NV) out[e] = 0.f;
+        }
+    }
+#else
+    (void)p;
+#endif
+}
+
+// this wave's blocks of a state to an fp32 buffer [D][D] ([q/k index][v index]); blocks outside B stay unwritten
+template <int D, typename B>
+__device__ __forceinline__ void walk_write_state(float *out, int wave, int lane, const f32x16 (&st)[WalkCfg<D>::NBW]) {
+    const int l32 = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < B::SLOTS; ++i)
+        if (B::valid(wave, i)) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                out[(32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * B::eb(wave) + l32] = st[i][v];
+        }
+}
+
+// ---- forward for q and k of 129 .. 256 columns (v of at most 128), one walk over both 128-column halves:
+//   O_c = sum over the halves h of lower(Q_h,c K_h,c^T) V_c + Q_h,c S_h,   then S_h += K_h,c^T V_c
+// Each half is the D = 128 product of walk_fwd_kernel with a state of its own; the chunk's result stays in
+// its fp32 accumulators from the first half to the second and is rounded and stored once, and V is loaded
+// once per chunk -- where two walks of walk_fwd_kernel, the second adding to the first one's result, load V
+// twice, write O twice and read it back once.
+// LDS: a set of (Q_h, K_h) tiles per half -- while half h of a chunk is multiplied, the loads of the next
+// half-chunk go to the other set -- two V tiles (chunk parity), and ONE 16-bit state: a half's state is
+// needed in LDS only for that half's product, so at the end of a half-chunk the other half's state (in
+// registers throughout, updated one half-chunk earlier) is rounded into the buffer.
+// NV: the state's v blocks that hold anything (2: v of at most 64 columns).
+template <typename T, int NV>
+__global__ __launch_bounds__(256, 1) void walk_fwd_wide_kernel(const WalkParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int D = 128;
+    using W = WalkCfg<D>;
+    using V8 = typename Mma<T>::V8;
+    using B = WalkExt<D, D / 32, NV>;
+    using OB = WalkOut<D, NV>;  // the result is as wide as v
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    unsigned char *tl = smem + 6 * W::TILE;
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rb = wave % W::NRB, db0 = OB::db0(wave);
+    const WalkSlice sl = walk_slice(p);
+    if (!sl.valid) return;
+    const int b = sl.bh / p.H, h = sl.bh - b * p.H, N = p.N;
+    const T *Q = static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h;
+    const T *K = static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h;
+    const T *V = static_cast<const T *>(p.v) + b * p.vs_b + h * p.vs_h;
+    T *O = static_cast<T *>(p.o) + b * p.os_b + h * p.os_h;
+    const int qs2 = (int)p.qs_n * 2, ks2 = (int)p.ks_n * 2, vs2 = (int)p.vs_n * 2, os2 = (int)p.os_n * 2;
+    const u32x4 rq0 = make_rsrc(Q, (uint32_t)((N - 1) * qs2 + p.wqk * 2));
+    const u32x4 rk0 = make_rsrc(K, (uint32_t)((N - 1) * ks2 + p.wqk * 2));
+    const u32x4 rq1 = make_rsrc(Q + D, (uint32_t)((N - 1) * qs2 + p.wqk2 * 2));
+    const u32x4 rk1 = make_rsrc(K + D, (uint32_t)((N - 1) * ks2 + p.wqk2 * 2));
+    const u32x4 rv = make_rsrc(V, (uint32_t)((N - 1) * vs2 + p.wv * 2));
+    const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(O, 0, (N - 1) * os2 + p.wv * 2, 0x00020000);
+
+    f32x16 st0[W::NBW], st1[W::NBW];
+    walk_load_init_from<D, B>(p.init, p, sl, wave, lane, st0, false);
+    walk_load_init_from<D, B>(p.init2, p, sl, wave, lane, st1, false);
+    walk_state_to_lds<T, D, B>(tl, wave, lane, st0);
+
+    auto load_half = [&](int c, auto half) {  // Q_h, K_h of chunk c to set h
+        constexpr int HF = decltype(half)::value;
+        const uint32_t base = lds0 + HF * 2 * W::TILE;
+        walk_load_tile<D>(HF ? rq1 : rq0, base, c * W::C, qs2, HF ? p.wqk2 : p.wqk, wave, lane);
+        walk_load_tile<D>(HF ? rk1 : rk0, base + W::TILE, c * W::C, ks2, HF ? p.wqk2 : p.wqk, wave, lane);
+    };
+    auto v_slot = [&](int c) { return 4 + ((c - sl.c_lo) & 1); };
+    auto load_v = [&](int c) { walk_load_tile<D>(rv, lds0 + v_slot(c) * W::TILE, c * W::C, vs2, p.wv, wave, lane); };
+    auto sync = [&]() {  // this wave's LDS accesses are done; then every wave's
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+    auto sfrag = [&](int db, int kc) -> V8 { return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g); };
+    load_half(sl.c_lo, std::integral_constant<int, 0>{});
+    load_v(sl.c_lo);
+#pragma unroll 1
+    for (int c = sl.c_lo; c < sl.c_hi; ++c) {
+        unsigned char *tq0 = smem, *tk0 = smem + W::TILE, *tq1 = smem + 2 * W::TILE, *tk1 = smem + 3 * W::TILE;
+        unsigned char *tv = smem + v_slot(c) * W::TILE;
+        const int row = c * W::C + 32 * rb + l32;
+        f32x16 acc[W::DBW];
+        // first half.  (Every wave has left the barrier that ended the reads of the set loaded next, one
+        // half-chunk ago.)  This wave's loads of the half-chunk have landed when at most the loads issued
+        // after them are outstanding; the stores of the chunk before were issued before those.
+        load_half(c, std::integral_constant<int, 1>{});
+        wait_vm<2 * W::NI>();
+        sync();  // the tiles have landed, S_0 is in LDS
+        walk_product<T, D, false, 0, B::KQ, NV>(tq0, tk0, tv, wave, lane, c > 0, sfrag, acc);
+        walk_update<T, D, B>(tk0, tv, wave, lane, st0);
+        sync();  // every wave has read S_0 and this half's tiles
+        walk_state_to_lds<T, D, B>(tl, wave, lane, st1);
+        // second half
+        const bool more = c + 1 < sl.c_hi;
+        if (more) {
+            load_half(c + 1, std::integral_constant<int, 0>{});
+            load_v(c + 1);  // (to the slot of the chunk before this one)
+            wait_vm<3 * W::NI>();
+        } else {
+            wait_vm<0>();
+        }
+        sync();  // the tiles have landed, S_1 is in LDS
+        walk_product<T, D, false, 0, B::KQ, NV, true>(tq1, tk1, tv, wave, lane, c > 0, sfrag, acc);
+        walk_store<T, D, OB::PER>(ro, os2, p.wv, row, g, db0, acc);
+        walk_update<T, D, B>(tk1, tv, wave, lane, st1);
+        sync();  // every wave has read S_1, this half's tiles and V
+        walk_state_to_lds<T, D, B>(tl, wave, lane, st0);
+    }
+    if (p.total_out && sl.c_hi == p.n_chunks) {  // the states after the last chunk, for the backward walk
+        walk_write_state<D, B>(p.total_out + (int64_t)sl.bh * (D * D), wave, lane, st0);
+        walk_write_state<D, B>(p.total_out2 + (int64_t)sl.bh * (D * D), wave, lane, st1);
+        // (a reader that takes the second half for a narrow q / k against a full-width v reads every block)
+        if (NV < W::DB && p.wqk2 <= 64) {
+            float *out = p.total_out2 + (int64_t)sl.bh * (D * D);
+            for (int e = tid; e < D * D; e += 256)
+                if (e % D >= 32 * NV) out[e] = 0.f;
         }
     }
 #else
@@ -1754,6 +1897,19 @@ hipError_t launch_walk_fwd(const WalkParams &p, hipStream_t stream) {
     }
     if (p.accumulate) return hipErrorNotSupported;
     return launch_walk_kernel<walk_fwd_kernel<T, D, kDouble, 0, false>>(grid, smem, p, stream);
+}
+
+template <typename T>
+hipError_t launch_walk_fwd_wide(const WalkParams &p, hipStream_t stream) {
+    using W = WalkCfg<128>;
+    const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
+    if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    if (p.wqk != 128 || p.wqk2 < 1 || p.wqk2 > 128 || p.wv < 1 || p.wv > 128 || p.fmap || p.slope_y || p.denom || p.dn ||
+        p.accumulate || p.init_transposed || (p.n_seg > 1 && (!p.init || !p.init2)) || (p.total_out && !p.total_out2))
+        return hipErrorInvalidValue;
+    constexpr int smem = 6 * W::TILE + W::STATE;  // two sets of (Q_h, K_h), two V tiles, one state
+    if (p.wv <= 64) return launch_walk_kernel<walk_fwd_wide_kernel<T, 2>>(grid, smem, p, stream);
+    return launch_walk_kernel<walk_fwd_wide_kernel<T, 4>>(grid, smem, p, stream);
 }
 
 template <typename T, int D>

@@ -31,6 +31,9 @@ hipError_t walk_totals(int dtype, int D, const WalkTotalsParams &p, hipStream_t 
 hipError_t walk_fwd(int dtype, int D, const WalkParams &p, hipStream_t stream) {
     FLA_WALK_DISPATCH3(launch_walk_fwd, p, stream);
 }
+hipError_t walk_fwd_wide(int dtype, const WalkParams &p, hipStream_t stream) {
+    return dtype == 0 ? launch_walk_fwd_wide<__bf16>(p, stream) : launch_walk_fwd_wide<_Float16>(p, stream);
+}
 hipError_t walk_vec_sums(int dtype, int D, const WalkVecParams &p, int64_t BH, hipStream_t stream) {
     FLA_WALK_DISPATCH3(launch_walk_vec_sums, p, BH, stream);
 }

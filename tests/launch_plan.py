@@ -790,6 +790,27 @@ def model_walk(arena: Arena, l: Launch, p: Dict, D: int, stats: Stats) -> None:
     stats.workgroups += BH * n_seg
 
 
+def model_walk_wide(arena: Arena, l: Launch, p: Dict, stats: Stats) -> None:
+    """One walk over both 128-column halves of a q / k of 129 .. 256 columns: the plan of a D = 128 walk
+    whose q, k (dq, dk) rows are 128 + wqk2 wide, with a second set of states for the second half."""
+    D, E = 128, 128 * 128 * 4
+    assert p["wqk"] == 128 and 1 <= p["wqk2"] <= 128 and p["wqk2"] % 8 == 0 and not p["accumulate"]
+    assert not p["init_transposed"] and not p["fmap"] and not p["denom"] and not p["dn"] and not p["saved"]
+    whole = dict(p)
+    whole["wqk"] = 128 + p["wqk2"]
+    model_walk(arena, l, whole, D, stats)
+    BH, n_seg = p["BH"], p["n_seg"]
+    tiles = 6 if l.kernel == "walk_fwd_wide_kernel" else 8
+    assert l.lds == tiles * 64 * 256 + 128 * 256, f"{l.kernel}: {l.lds} bytes of LDS"
+    for first, second, count in (("init", "init2", BH * n_seg), ("xinit", "xinit2", BH * n_seg),
+                                 ("total_out", "total_out2", BH), ("xtotal", "xtotal2", BH)):
+        assert bool(p[first]) == bool(p[second]), f"{l.kernel}: {first} without {second} or the reverse"
+        if p[second]:
+            arena.require(f"{second} (second half)", p[second], p[second] + count * E)
+            assert not (p[first] <= p[second] < p[first] + count * E) and \
+                not (p[second] <= p[first] < p[second] + count * E), f"{l.kernel}: {first} and {second} overlap"
+
+
 def model_walk_totals(arena: Arena, l: Launch, p: Dict, D: int, stats: Stats) -> None:
     rows = 128 if D <= 64 else 64
     N, BH, H = p["N"], p["BH"], p["H"]
@@ -862,6 +883,8 @@ def check_all(arena: Arena, launches: List[Launch], stats: Stats) -> None:
                 arena.require("wsum", wsum, wsum + BH * chunks * DP * 4)
         elif k in ("walk_fwd_kernel", "walk_bwd_kernel", "walk_dkdv_kernel", "walk_bwd_rev_kernel"):
             model_walk(arena, l, l.struct("a0"), t[1], stats)
+        elif k in ("walk_fwd_wide_kernel", "walk_bwd_rev_wide_kernel"):
+            model_walk_wide(arena, l, l.struct("a0"), stats)
         elif k == "walk_scan_kernel":
             totals, entry, n_seg, E, total2 = (l.args[f"a{i}"] for i in range(5))
             totals_b, entry_b = l.args["a8"], l.args["a9"]
