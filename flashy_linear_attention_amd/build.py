@@ -94,6 +94,7 @@ def build(jobs: int | None = None, verbose: bool = True) -> str:
     report = _run([_hipcc(), *HIPCC_FLAGS, "-Rpass-analysis=kernel-resource-usage", "-c",
                    os.path.join(CSRC, "fla_walk_inst.hip"), "-o", walk])
     _check_no_scratch(report, "walk_bwd_rev_kernel")
+    _check_no_scratch(report, "walk_bwd_rev_wide_kernel")
     # (this one without the VGPR form of MFMA: see the file's header)
     pair = os.path.join(OBJ_DIR, "fla_pair_inst.o")
     pair_flags = [f for f in HIPCC_FLAGS if f not in ("-mllvm", "-amdgpu-mfma-vgpr-form")]

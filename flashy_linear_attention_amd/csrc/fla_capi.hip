@@ -656,6 +656,27 @@ int wide_backward(const WidePlan &wide, const View &go, const View &q, const Vie
         void *const work[2] = {base, base + wp.work_bytes};
         if (int rc = wide_entry_states(wp, q, go, B, H, N, dqk, dv, dtype, 1, work, none, entries, s)) return rc;
     }
+    if (state_in && dv <= 64) {  // forward's states at hand, narrow v: one reverse walk over both halves
+        fla::WalkParams r{};
+        r.q = q.ptr, r.k = k.ptr, r.v = v.ptr, r.go = go.ptr;
+        r.dq = const_cast<void *>(dq.ptr), r.dk = const_cast<void *>(dk.ptr), r.dv = const_cast<void *>(dvv.ptr);
+        r.qs_b = q.strides[0], r.qs_h = q.strides[1], r.qs_n = q.strides[2];
+        r.ks_b = k.strides[0], r.ks_h = k.strides[1], r.ks_n = k.strides[2];
+        r.vs_b = v.strides[0], r.vs_h = v.strides[1], r.vs_n = v.strides[2];
+        r.gs_b = go.strides[0], r.gs_h = go.strides[1], r.gs_n = go.strides[2];
+        r.dqs_b = dq.strides[0], r.dqs_h = dq.strides[1], r.dqs_n = dq.strides[2];
+        r.dks_b = dk.strides[0], r.dks_h = dk.strides[1], r.dks_n = dk.strides[2];
+        r.dvs_b = dvv.strides[0], r.dvs_h = dvv.strides[1], r.dvs_n = dvv.strides[2];
+        r.H = (int32_t)H, r.N = (int32_t)N, r.BH = (int32_t)(B * H), r.wqk = 128, r.wqk2 = (int32_t)(dqk - 128);
+        r.wv = (int32_t)dv;
+        r.n_chunks = (int32_t)wp.n_chunks, r.seg_chunks = (int32_t)wp.seg_chunks, r.n_seg = (int32_t)wp.n_seg;
+        r.init = entries[0], r.init2 = entries[1];
+        const char *half0 = static_cast<const char *>(state_in), *half1 = half0 + wp.saved_bytes;
+        r.xinit = reinterpret_cast<const float *>(half0), r.xinit2 = reinterpret_cast<const float *>(half1);
+        r.xtotal = reinterpret_cast<const float *>(half0 + wp.entry_bytes);
+        r.xtotal2 = reinterpret_cast<const float *>(half1 + wp.entry_bytes);
+        return fla::walk_bwd_rev_wide(dtype, r, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;
+    }
     for (int h = 0; h < 2; ++h) {
         const View qh = column_half(q, h), kh = column_half(k, h), dqh = column_half(dq, h), dkh = column_half(dk, h);
         const int64_t wqk = h == 0 ? 128 : dqk - 128;

@@ -1106,12 +1106,7 @@ __global__ __launch_bounds__(256, 1) void walk_fwd_wide_kernel(const WalkParams 
     if (p.total_out && sl.c_hi == p.n_chunks) {  // the states after the last chunk, for the backward walk
         walk_write_state<D, B>(p.total_out + (int64_t)sl.bh * (D * D), wave, lane, st0);
         walk_write_state<D, B>(p.total_out2 + (int64_t)sl.bh * (D * D), wave, lane, st1);
-        // (a reader that takes the second half for a narrow q / k against a full-width v reads every block)
-        if (NV < W::DB && p.wqk2 <= 64) {
-            float *out = p.total_out2 + (int64_t)sl.bh * (D * D);
-            for (int e = tid; e < D * D; e += 256)
-                if (e % D >= 32 * NV) out[e] = 0.f;
-        }
+        // (NV = 2: the v blocks beyond stay unwritten -- walk_bwd_rev_wide_kernel, the reader, is built for the same extent)
     }
 #else
     (void)p;
@@ -1516,6 +1511,138 @@ __global__ __launch_bounds__(256, 1) void walk_bwd_rev_kernel(const WalkParams p
         if (!(kSplitUpdate && rb == 1)) walk_update<T, D, B, false, true>(tq, tg, wave, lane, st);
         sync();  // every wave has read X and is done with the tiles
         walk_state_to_lds<T, D, B>(tl, wave, lane, st);
+    }
+#else
+    (void)p;
+#endif
+}
+
+// ---- walk_bwd_rev_kernel for q and k of 129 .. 256 columns against a v of at most 64: one reverse walk over
+// both 128-column halves.  Per chunk and half h, with R_h and X_h the states of walk_bwd_rev_kernel for the half:
+//   dV  += upper(K_h Q_h^T) dO + K_h R_h        (fp32 accumulators from the first half to the second, stored once)
+//   dK_h = upper(V dO^T) Q_h + V R_h^T          dQ_h = lower(dO V^T) K_h + dO X_h^T
+// V and dO are loaded once per chunk, where two walks of walk_bwd_rev_kernel, the second adding its part of dV to
+// the first one's, load them twice, write dV twice and read it back once.
+// LDS as in walk_fwd_wide_kernel: a set of (Q_h, K_h) tiles per half, two (V, dO) pairs by chunk parity, and ONE
+// 16-bit state that holds R_h, then X_h, of the half at work; at the end of a half-chunk the other half's R (in
+// registers throughout) is rounded into it.  Four states in registers: built for v blocks NV = 2 only.
+template <typename T, int NV>
+__global__ __launch_bounds__(256, 1) void walk_bwd_rev_wide_kernel(const WalkParams p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int D = 128, NQ = D / 32;
+    static_assert(NV == 2, "R and X of both halves live in registers: two blocks per wave and state");
+    using W = WalkCfg<D>;
+    using V8 = typename Mma<T>::V8;
+    using B = WalkExt<D, NQ, NV>;   // R, X [q/k index][v index]
+    using OV = WalkOut<D, NV>;      // dV is as wide as v,
+    using OQ = WalkOut<D, NQ>;      // dK and dQ as q and k
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
+    unsigned char *tl = smem + 8 * W::TILE;
+    const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int rb = wave % W::NRB;
+    const WalkSlice sl = walk_slice(p);
+    if (!sl.valid) return;
+    const int b = sl.bh / p.H, h = sl.bh - b * p.H, N = p.N;
+    const T *Q = static_cast<const T *>(p.q) + b * p.qs_b + h * p.qs_h;
+    const T *K = static_cast<const T *>(p.k) + b * p.ks_b + h * p.ks_h;
+    const T *V = static_cast<const T *>(p.v) + b * p.vs_b + h * p.vs_h;
+    const T *G = static_cast<const T *>(p.go) + b * p.gs_b + h * p.gs_h;
+    T *DQ = static_cast<T *>(p.dq) + b * p.dqs_b + h * p.dqs_h;
+    T *DK = static_cast<T *>(p.dk) + b * p.dks_b + h * p.dks_h;
+    T *DV = static_cast<T *>(p.dv) + b * p.dvs_b + h * p.dvs_h;
+    const int qs2 = (int)p.qs_n * 2, ks2 = (int)p.ks_n * 2, vs2 = (int)p.vs_n * 2, gs2 = (int)p.gs_n * 2;
+    const int dqs2 = (int)p.dqs_n * 2, dks2 = (int)p.dks_n * 2, dvs2 = (int)p.dvs_n * 2;
+    const u32x4 rq0 = make_rsrc(Q, (uint32_t)((N - 1) * qs2 + p.wqk * 2));
+    const u32x4 rk0 = make_rsrc(K, (uint32_t)((N - 1) * ks2 + p.wqk * 2));
+    const u32x4 rq1 = make_rsrc(Q + D, (uint32_t)((N - 1) * qs2 + p.wqk2 * 2));
+    const u32x4 rk1 = make_rsrc(K + D, (uint32_t)((N - 1) * ks2 + p.wqk2 * 2));
+    const u32x4 rv = make_rsrc(V, (uint32_t)((N - 1) * vs2 + p.wv * 2));
+    const u32x4 rg = make_rsrc(G, (uint32_t)((N - 1) * gs2 + p.wv * 2));
+    const __amdgpu_buffer_rsrc_t rdq0 = __builtin_amdgcn_make_buffer_rsrc(DQ, 0, (N - 1) * dqs2 + p.wqk * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rdk0 = __builtin_amdgcn_make_buffer_rsrc(DK, 0, (N - 1) * dks2 + p.wqk * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rdq1 = __builtin_amdgcn_make_buffer_rsrc(DQ + D, 0, (N - 1) * dqs2 + p.wqk2 * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rdk1 = __builtin_amdgcn_make_buffer_rsrc(DK + D, 0, (N - 1) * dks2 + p.wqk2 * 2, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rdv = __builtin_amdgcn_make_buffer_rsrc(DV, 0, (N - 1) * dvs2 + p.wv * 2, 0x00020000);
+
+    f32x16 st0[W::NBW], st1[W::NBW];  // R_0, R_1
+    f32x16 xs0[W::NBW], xs1[W::NBW];  // X_0, X_1
+    walk_load_init_from<D, B>(p.init, p, sl, wave, lane, st0, true);
+    walk_load_init_from<D, B>(p.init2, p, sl, wave, lane, st1, true);
+    walk_load_end_state_from<D, B>(p.xinit, p.xtotal, p, sl, wave, lane, xs0);
+    walk_load_end_state_from<D, B>(p.xinit2, p.xtotal2, p, sl, wave, lane, xs1);
+    walk_state_to_lds<T, D, B>(tl, wave, lane, st0);
+
+    auto load_half = [&](int c, auto half) {  // Q_h, K_h of chunk c to set h
+        constexpr int HF = decltype(half)::value;
+        const uint32_t base = lds0 + HF * 2 * W::TILE;
+        walk_load_tile<D>(HF ? rq1 : rq0, base, c * W::C, qs2, HF ? p.wqk2 : p.wqk, wave, lane);
+        walk_load_tile<D>(HF ? rk1 : rk0, base + W::TILE, c * W::C, ks2, HF ? p.wqk2 : p.wqk, wave, lane);
+    };
+    auto vg_slot = [&](int c) { return 4 + 2 * ((sl.c_hi - 1 - c) & 1); };
+    auto load_vg = [&](int c) {
+        const uint32_t base = lds0 + vg_slot(c) * W::TILE;
+        walk_load_tile<D>(rv, base, c * W::C, vs2, p.wv, wave, lane);
+        walk_load_tile<D>(rg, base + W::TILE, c * W::C, gs2, p.wv, wave, lane);
+    };
+    auto sync = [&]() {  // this wave's LDS accesses are done; then every wave's
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0xc07f);
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+    // A operands of the state products: R^T[v index][q/k index] is the LDS copy as it is (dV); R and X
+    // [q/k index][v index] are the copy read transposed (dK, dQ)
+    auto rows_of_state = [&](int db, int kc) -> V8 { return walk_row_frag<T, D>(tl, 32 * db + walk_e_lane(l32), kc, g); };
+    auto cols_of_state = [&](int db, int kc) -> V8 { return walk_col_frag_perm<T, D>(tl, 16 * kc, db, lane, true); };
+    load_half(sl.c_hi - 1, std::integral_constant<int, 0>{});
+    load_vg(sl.c_hi - 1);
+#pragma unroll 1
+    for (int c = sl.c_hi - 1; c >= sl.c_lo; --c) {
+        unsigned char *tv = smem + vg_slot(c) * W::TILE, *tg = tv + W::TILE;
+        const int row = c * W::C + 32 * rb + l32;
+        const bool later = c + 1 < p.n_chunks;  // chunks after this one exist: R is not identically zero
+        f32x16 dvacc[W::DBW];
+        auto half_chunk = [&](auto half, f32x16 (&st)[W::NBW], f32x16 (&xs)[W::NBW], f32x16 (&st_next)[W::NBW]) {
+            constexpr int HF = decltype(half)::value;
+            unsigned char *tq = smem + HF * 2 * W::TILE, *tk = tq + W::TILE;
+            // (every wave has left the barrier that ended the reads of the set loaded next, one half-chunk ago.)
+            // This wave's loads of the half-chunk have landed when at most the loads issued after them are
+            // outstanding; the stores of the half-chunk before were issued before those.
+            if constexpr (HF == 0) {
+                load_half(c, std::integral_constant<int, 1>{});
+                wait_vm<2 * W::NI>();
+            } else {
+                if (c > sl.c_lo) {
+                    load_half(c - 1, std::integral_constant<int, 0>{});
+                    load_vg(c - 1);  // (to the slots of the chunk after this one)
+                    wait_vm<4 * W::NI>();
+                } else {
+                    wait_vm<0>();
+                }
+            }
+            sync();  // the tiles have landed, R_h is in LDS
+            walk_update<T, D, B, true, true>(tk, tv, wave, lane, xs);  // X_h: now the sum over the chunks before this one
+            walk_product<T, D, true, 0, B::KQ, NV, HF != 0>(tk, tq, tg, wave, lane, later, rows_of_state, dvacc);
+            f32x16 acc[W::DBW];
+            walk_product<T, D, true, 0, B::KV, NQ>(tv, tg, tq, wave, lane, later, cols_of_state, acc);
+            walk_store<T, D, OQ::PER>(HF ? rdk1 : rdk0, dks2, HF ? p.wqk2 : p.wqk, row, g, OQ::db0(wave), acc);
+            sync();  // every wave has read R_h
+            // (X stays in its accumulation registers up to here: without this the copies that the rounding
+            // below reads are made right after the update and occupy registers through both products)
+            asm volatile("" : "+a"(xs[0]), "+a"(xs[1]));
+            walk_state_to_lds<T, D, B>(tl, wave, lane, xs);
+            sync();  // X_h is in LDS
+            walk_product<T, D, false, 0, B::KV, NQ>(tg, tv, tk, wave, lane, c > 0, cols_of_state, acc);
+            walk_store<T, D, OQ::PER>(HF ? rdq1 : rdq0, dqs2, HF ? p.wqk2 : p.wqk, row, g, OQ::db0(wave), acc);
+            if constexpr (HF != 0) walk_store<T, D, OV::PER>(rdv, dvs2, p.wv, row, g, OV::db0(wave), dvacc);
+            walk_update<T, D, B, false, true>(tq, tg, wave, lane, st);  // R_h += Q_h^T dO
+            sync();  // every wave has read X_h and is done with this half's tiles
+            walk_state_to_lds<T, D, B>(tl, wave, lane, st_next);
+        };
+        half_chunk(std::integral_constant<int, 0>{}, st0, xs0, st1);
+        half_chunk(std::integral_constant<int, 1>{}, st1, xs1, st0);
     }
 #else
     (void)p;
@@ -1974,5 +2101,20 @@ hipError_t launch_walk_bwd_rev(const WalkParams &p, hipStream_t stream) {
     if (p.accumulate) return launch_walk_kernel<walk_bwd_rev_kernel<T, D, D / 32, D / 32, true>>(grid, smem, p, stream);
     return launch_walk_kernel<walk_bwd_rev_kernel<T, D>>(grid, smem, p, stream);
 }
+
+template <typename T>
+hipError_t launch_walk_bwd_rev_wide(const WalkParams &p, hipStream_t stream) {
+    using W = WalkCfg<128>;
+    const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
+    if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
+    if (p.wqk != 128 || p.wqk2 < 1 || p.wqk2 > 128 || p.wv < 1 || p.wv > 64) return hipErrorNotSupported;
+    if (p.fmap || p.dn || p.accumulate || p.init_transposed || !p.xtotal || !p.xtotal2 ||
+        (p.n_seg > 1 && (!p.init || !p.init2 || !p.xinit || !p.xinit2)))
+        return hipErrorInvalidValue;
+    constexpr int smem = 8 * W::TILE + W::STATE;  // two sets of (Q_h, K_h), two of (V, dO), one state
+    static_assert(smem <= 160 * 1024, "the tiles and the state must fit the LDS of a CU");
+    return launch_walk_kernel<walk_bwd_rev_wide_kernel<T, 2>>(grid, smem, p, stream);
+}
+
 
 }  // namespace fla

@@ -53,6 +53,7 @@ FLA_DECLARE_PAIR(32) FLA_DECLARE_PAIR(64) FLA_DECLARE_PAIR(128)
 hipError_t walk_totals(int dtype, int D, const WalkTotalsParams &p, hipStream_t stream);
 hipError_t walk_fwd(int dtype, int D, const WalkParams &p, hipStream_t stream);
 hipError_t walk_fwd_wide(int dtype, const WalkParams &p, hipStream_t stream);  // (q, k of 129 .. 256 columns)
+hipError_t walk_bwd_rev_wide(int dtype, const WalkParams &p, hipStream_t stream);  // (... and v of at most 64)
 hipError_t walk_bwd_rev(int dtype, int D, const WalkParams &p, hipStream_t stream);
 hipError_t walk_bwd(int dtype, int D, const WalkParams &p, hipStream_t stream);
 hipError_t walk_dkdv(int dtype, int D, const WalkParams &p, hipStream_t stream);

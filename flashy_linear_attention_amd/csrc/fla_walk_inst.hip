@@ -34,6 +34,9 @@ hipError_t walk_fwd(int dtype, int D, const WalkParams &p, hipStream_t stream) {
 hipError_t walk_fwd_wide(int dtype, const WalkParams &p, hipStream_t stream) {
     return dtype == 0 ? launch_walk_fwd_wide<__bf16>(p, stream) : launch_walk_fwd_wide<_Float16>(p, stream);
 }
+hipError_t walk_bwd_rev_wide(int dtype, const WalkParams &p, hipStream_t stream) {
+    return dtype == 0 ? launch_walk_bwd_rev_wide<__bf16>(p, stream) : launch_walk_bwd_rev_wide<_Float16>(p, stream);
+}
 hipError_t walk_vec_sums(int dtype, int D, const WalkVecParams &p, int64_t BH, hipStream_t stream) {
     FLA_WALK_DISPATCH3(launch_walk_vec_sums, p, BH, stream);
 }

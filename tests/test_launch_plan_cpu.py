@@ -256,7 +256,8 @@ def test_benchmark_shapes(lib):
             arena, launches = trace_normalised(lib, b, h, n, dqk, dv, chunked, dtype)
             lp.check_all(arena, launches, stats)
     assert stats.kernels["tri_xyt_z_fast_batch_kernel"] >= 4 and stats.kernels["walk_bwd_rev_kernel"] >= 1
-    assert stats.kernels["walk_fwd_wide_kernel"] >= 1  # (C4: one walk over both halves of q / k)
+    # (C4: one walk over both halves of q / k, forward and backward)
+    assert stats.kernels["walk_fwd_wide_kernel"] >= 1 and stats.kernels["walk_bwd_rev_wide_kernel"] >= 1
 
 
 def test_empty_problems_make_no_launch(lib):
