@@ -434,7 +434,8 @@ struct EntryHalf {
 
 int walk_entry_states(const WalkPlan &w, const View &y, const View &z, int64_t B, int64_t H, int64_t N, int64_t dy,
                       int64_t dz, int dtype, int reverse, void *work, float *entry, const float **where, hipStream_t s,
-                      int map_y = 0, const View *ymap_out = nullptr, const EntryHalf *second = nullptr) {
+                      int map_y = 0, const View *ymap_out = nullptr, const EntryHalf *second = nullptr,
+                      bool totals_only = false) {
     fla::WalkTotalsParams tp{};
     if (map_y) {
         tp.map_y = map_y, tp.ymap_out = const_cast<void *>(ymap_out->ptr);
@@ -445,7 +446,9 @@ int walk_entry_states(const WalkPlan &w, const View &y, const View &z, int64_t B
     // (two segments: the one total needed is the other segment's entry state; the totals kernel writes it as the
     // walks read it, two partial sums, and no scan follows.  A few segments more: the walks add up the totals
     // themselves as they start -- fla::walk_entries_are_totals -- and no scan follows either)
-    const bool direct = w.n_seg == 2, summed_on_load = fla::walk_entries_are_totals(w.D, (int)w.n_seg);
+    // (totals_only: the caller's walk adds them up itself -- WalkParams::init_is_totals; not with two segments)
+    const bool direct = w.n_seg == 2;
+    const bool summed_on_load = fla::walk_entries_are_totals(w.D, (int)w.n_seg) || (totals_only && !direct);
     const bool no_scan = direct || summed_on_load;
     tp.y = y.ptr, tp.z = z.ptr, tp.totals = no_scan ? entry : totals, tp.direct = direct;
     tp.ys_b = y.strides[0], tp.ys_h = y.strides[1], tp.ys_n = y.strides[2];
@@ -478,16 +481,19 @@ int walk_entry_states(const WalkPlan &w, const View &y, const View &z, int64_t B
 // one after the other.  work[h], entry[h] (null: over work[h]) and where[h] per half.
 int wide_entry_states(const WalkPlan &wp, const View &y, const View &z, int64_t B, int64_t H, int64_t N, int64_t dy_all,
                       int64_t dz, int dtype, int reverse, void *const (&work)[2], float *const (&entry)[2],
-                      const float *(&where)[2], hipStream_t s) {
+                      const float *(&where)[2], hipStream_t s, bool totals_only = false) {
     const View y1{static_cast<const char *>(y.ptr) + 128 * 2, y.strides};
     const int64_t dy1 = dy_all - 128;
     if (fla::walk_totals_cols(wp.D, 128, (int)dz) == fla::walk_totals_cols(wp.D, (int)dy1, (int)dz)) {
         const EntryHalf other{y1.ptr, dy1, work[1], entry[1], &where[1]};
         return walk_entry_states(wp, y, z, B, H, N, 128, dz, dtype, reverse, work[0], entry[0], &where[0], s, 0, nullptr,
-                                 &other);
+                                 &other, totals_only);
     }
-    if (int rc = walk_entry_states(wp, y, z, B, H, N, 128, dz, dtype, reverse, work[0], entry[0], &where[0], s)) return rc;
-    return walk_entry_states(wp, y1, z, B, H, N, dy1, dz, dtype, reverse, work[1], entry[1], &where[1], s);
+    if (int rc = walk_entry_states(wp, y, z, B, H, N, 128, dz, dtype, reverse, work[0], entry[0], &where[0], s, 0, nullptr,
+                                   nullptr, totals_only))
+        return rc;
+    return walk_entry_states(wp, y1, z, B, H, N, dy1, dz, dtype, reverse, work[1], entry[1], &where[1], s, 0, nullptr,
+                             nullptr, totals_only);
 }
 
 // The normaliser's terms handed to the walk kernels (fla_chunk_walk.h, WalkParams::denom ...).
@@ -612,20 +618,29 @@ int wide_forward(const WidePlan &wide, const View &q, const View &k, const View 
     const WalkPlan &wp = wide.wp;
     char *ws = static_cast<char *>(workspace);
     const float *entry[2] = {nullptr, nullptr};
+    // A few segments more than two: no scan -- the walk adds up the totals of the segments before its own as it
+    // starts (three of each half in flight together) and writes the entry state it formed for backward
+    // (B 4, H 16, N 4096, D_qk 256, D_v 64, four segments: see the measurements beside WalkParams::init_is_totals).
+    const bool sum_on_load = wp.n_seg >= 3 && wp.n_seg <= 7;
+    float *keep[2] = {nullptr, nullptr};
     if (wp.n_seg > 1) {
         // (kept for backward when there is a state buffer: each half's entry states, its final state behind them;
-        // otherwise the two halves' states share the workspace behind the scratch tensor)
-        float *keep[2] = {nullptr, nullptr};
+        // otherwise, and the totals that the walk adds up, in the workspace behind the scratch tensor)
         void *work[2];
         for (int h = 0; h < 2; ++h) {
             if (state_out) keep[h] = reinterpret_cast<float *>(static_cast<char *>(state_out) + h * wp.saved_bytes);
-            work[h] = keep[h] ? static_cast<void *>(keep[h]) : static_cast<void *>(ws + wide.temp_bytes + h * wp.work_bytes);
+            work[h] = keep[h] && !sum_on_load ? static_cast<void *>(keep[h])
+                                              : static_cast<void *>(ws + wide.temp_bytes + h * wp.work_bytes);
         }
-        if (int rc = wide_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, work, keep, entry, s)) return rc;
+        float *const none[2] = {nullptr, nullptr};
+        if (int rc = wide_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, work, sum_on_load ? none : keep, entry, s,
+                                       sum_on_load))
+            return rc;
     }
     // one walk over both halves (the second one's columns start 128 elements into q's and k's rows)
     fla::WalkParams w = lower_walk_params(wp, q, k, v, o, B, H, N, 128, dv, entry[0]);
     w.wqk2 = (int32_t)(dqk - 128), w.init2 = wp.n_seg > 1 ? entry[1] : nullptr;
+    if (sum_on_load) w.init_is_totals = 1, w.entry_out = keep[0], w.entry_out2 = keep[1];
     if (state_out) {  // (behind each half's entry states: its state after the last chunk)
         w.total_out = reinterpret_cast<float *>(static_cast<char *>(state_out) + wp.entry_bytes);
         w.total_out2 = reinterpret_cast<float *>(static_cast<char *>(state_out) + wp.saved_bytes + wp.entry_bytes);

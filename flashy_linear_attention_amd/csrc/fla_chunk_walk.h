@@ -129,6 +129,12 @@ struct WalkParams {
     const float *init2;
     float *total_out2;
     const float *xinit2, *xtotal2;
+    // init_is_totals: init and init2 hold the segments' TOTALS as the totals kernel wrote them, and a workgroup adds
+    // up those of the segments before its own (after it, walking in reverse) as it starts, all loads in flight together
+    // (walk_sum_two) -- no scan launch between the totals kernel and the walk.  The forward walk then writes the
+    // entry state it formed to entry_out / entry_out2 (the layout of init; null: nowhere), for the backward walk.
+    int32_t init_is_totals;
+    float *entry_out, *entry_out2;
 };
 
 template <int D>
@@ -759,6 +765,40 @@ __device__ __forceinline__ void walk_sum_states(const float *buf, int f_lo, int 
     for (int f = f_lo; f < f_hi; ++f) walk_read_state<D, B, true>(buf + (int64_t)f * (D * D), transposed, wave, lane, st);
 }
 
+// st_a, st_b = this wave's blocks of the sums of the states a[f_lo .. f_hi - 1], b[f_lo .. f_hi - 1], the loads of
+// up to three states of each in flight together (a chain of dependent loads costs a memory latency per state)
+template <int D, typename B>
+__device__ __forceinline__ void walk_sum_two(const float *a, const float *b, int f_lo, int f_hi, int wave, int lane,
+                                             f32x16 (&st_a)[WalkCfg<D>::NBW], f32x16 (&st_b)[WalkCfg<D>::NBW]) {
+    using W = WalkCfg<D>;
+    constexpr int E = D * D, GROUP = 3;
+#pragma unroll
+    for (int i = 0; i < W::NBW; ++i)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) st_a[i][v] = 0.f, st_b[i][v] = 0.f;
+#pragma unroll 1
+    for (int f0 = f_lo; f0 < f_hi; f0 += GROUP) {
+        f32x16 ta[GROUP][W::NBW], tb[GROUP][W::NBW];
+#pragma unroll
+        for (int u = 0; u < GROUP; ++u) {
+            // (past the range: the last state once more, not added)
+            const int f = f0 + u < f_hi ? f0 + u : f_hi - 1;
+            walk_read_state<D, B, false>(a + (int64_t)f * E, false, wave, lane, ta[u]);
+            walk_read_state<D, B, false>(b + (int64_t)f * E, false, wave, lane, tb[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < GROUP; ++u) {
+            const float keep = f0 + u < f_hi ? 1.f : 0.f;
+#pragma unroll
+            for (int i = 0; i < B::SLOTS; ++i)
+                if (B::valid(wave, i)) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) st_a[i][v] += keep * ta[u][i][v], st_b[i][v] += keep * tb[u][i][v];
+                }
+        }
+    }
+}
+
 // this wave's blocks of the entry state of segment sl.seg (zeros without a buffer) of a walk in
 // ascending (`reverse` false) or descending order of the chunks; `buf`: the entry states of one operand
 template <int D, typename B = WalkExt<D>>
@@ -1050,8 +1090,17 @@ __global__ __launch_bounds__(256, 1) void walk_fwd_wide_kernel(const WalkParams 
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(O, 0, (N - 1) * os2 + p.wv * 2, 0x00020000);
 
     f32x16 st0[W::NBW], st1[W::NBW];
-    walk_load_init_from<D, B>(p.init, p, sl, wave, lane, st0, false);
-    walk_load_init_from<D, B>(p.init2, p, sl, wave, lane, st1, false);
+    if (p.init_is_totals) {
+        const int64_t at = (int64_t)sl.bh * p.n_seg * (D * D);
+        walk_sum_two<D, B>(p.init + at, p.init2 + at, 0, sl.seg, wave, lane, st0, st1);
+        if (p.entry_out && sl.seg > 0) {  // (the first segment's entry state, zero, is read by nobody)
+            walk_write_state<D, B>(p.entry_out + at + (int64_t)sl.seg * (D * D), wave, lane, st0);
+            walk_write_state<D, B>(p.entry_out2 + at + (int64_t)sl.seg * (D * D), wave, lane, st1);
+        }
+    } else {
+        walk_load_init_from<D, B>(p.init, p, sl, wave, lane, st0, false);
+        walk_load_init_from<D, B>(p.init2, p, sl, wave, lane, st1, false);
+    }
     walk_state_to_lds<T, D, B>(tl, wave, lane, st0);
 
     auto load_half = [&](int c, auto half) {  // Q_h, K_h of chunk c to set h
@@ -1666,8 +1715,9 @@ struct WalkTotalsParams {
     int32_t map_y;
     void *ymap_out;
     int64_t yo_b, yo_h, yo_n;
-    // A second Y operand of the same layout against the same Z, in the same launch (grid y = 1): the other
-    // 128-column half of a wide q / k, whose totals go to `totals2`.  Null: none.  (Without a feature map.)
+    // A second Y operand of the same layout against the same Z, in the same launch: the other 128-column half
+    // of a wide q / k, whose totals go to `totals2`.  Null: none.  (Without a feature map.)  Grid y = 1 takes
+    // it, or -- the kernel variant with BOTH -- every workgroup takes both operands.
     const void *y2;
     int32_t dy2;
     float *totals2;
@@ -1675,10 +1725,13 @@ struct WalkTotalsParams {
 
 constexpr int walk_totals_sets(int D) { return D == 128 ? 4 : 2; }  // sets of (Y, Z) tiles in LDS
 
-template <typename T, int D, int NQ = D / 32, int NV = D / 32>
-__global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsParams p) {
+// BOTH (D = 128, NV = 2): the launch's two Y operands (WalkTotalsParams::y2) in ONE workgroup -- three sets of
+// (Y, Y2, Z) tiles, a state per operand -- so that Z is loaded once for the two; otherwise grid y picks the operand.
+template <typename T, int D, int NQ = D / 32, int NV = D / 32, bool BOTH = false>
+__global__ __launch_bounds__(256, BOTH ? 1 : 2) void walk_totals_kernel(const WalkTotalsParams p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     using W = WalkCfg<D>;
+    static_assert(!BOTH || (D == 128 && NV == 2), "two states per wave: built for the narrow v side of D = 128");
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)smem;
     const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, g = lane >> 5;
@@ -1687,17 +1740,16 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
     const int hl = slot / p.n_seg, bh = hl * 8 + xcd;
     int seg = slot - hl * p.n_seg;
     if (bh >= p.BH) return;
-    const bool second = blockIdx.y != 0;  // (the launch's second Y operand: see WalkTotalsParams::y2)
-    float *const totals = second ? p.totals2 : p.totals;
+    const bool second = !BOTH && blockIdx.y != 0;  // (the launch's second Y operand: see WalkTotalsParams::y2)
     const int dy = second ? p.dy2 : p.dy;
-    float *out;
+    int64_t out_at;
     int c_lo, c_hi;
     if (p.direct) {
         // both workgroups of a (b, h) at work: half of the needed segment's chunks each (with a feature map
         // every row has to be visited: the needed segment's workgroup forms its total alone, the other one
         // maps its own segment's rows and hands in zeros)
         const int needed = p.seg_lo, part = seg != needed;
-        out = totals + ((int64_t)bh * 2 + part) * (D * D);
+        out_at = ((int64_t)bh * 2 + part) * (D * D);
         c_lo = seg * p.seg_chunks;
         c_hi = c_lo + p.seg_chunks < p.n_chunks ? c_lo + p.seg_chunks : p.n_chunks;
         if (!p.map_y) {
@@ -1708,34 +1760,43 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
         }
     } else {
         if (seg < p.seg_lo || seg >= p.seg_hi) return;
-        out = totals + ((int64_t)bh * p.n_seg + seg) * (D * D);
+        out_at = ((int64_t)bh * p.n_seg + seg) * (D * D);
         c_lo = seg * p.seg_chunks;
         c_hi = c_lo + p.seg_chunks < p.n_chunks ? c_lo + p.seg_chunks : p.n_chunks;
     }
+    float *const out = (second ? p.totals2 : p.totals) + out_at;
+    float *const out2 = BOTH ? p.totals2 + out_at : nullptr;
     if (c_lo >= c_hi) {  // nothing to add up (a segment beyond the end of the sequence, the second half of one chunk)
-        for (int i = tid; i < D * D; i += 256) out[i] = 0.f;
+        for (int i = tid; i < D * D; i += 256) {
+            out[i] = 0.f;
+            if constexpr (BOTH) out2[i] = 0.f;
+        }
         return;
     }
     const bool discard = p.direct && p.map_y && seg != p.seg_lo;  // (visited for the map only)
     const int b = bh / p.H, h = bh - b * p.H, N = p.N;
     const T *Y = static_cast<const T *>(second ? p.y2 : p.y) + b * p.ys_b + h * p.ys_h;
+    const T *Y2 = static_cast<const T *>(BOTH ? p.y2 : p.y) + b * p.ys_b + h * p.ys_h;
     const T *Z = static_cast<const T *>(p.z) + b * p.zs_b + h * p.zs_h;
     const int ys2 = (int)p.ys_n * 2, zs2 = (int)p.zs_n * 2;
     const u32x4 ry = make_rsrc(Y, (uint32_t)((N - 1) * ys2 + dy * 2));
+    const u32x4 ry2 = make_rsrc(Y2, (uint32_t)((N - 1) * ys2 + (BOTH ? p.dy2 : dy) * 2));
     const u32x4 rz = make_rsrc(Z, (uint32_t)((N - 1) * zs2 + p.dz * 2));
     using B = WalkExt<D, NQ, NV>;  // (blocks outside it stay unwritten: no walk of the same extent reads them)
-    f32x16 st[W::NBW];
+    f32x16 st[W::NBW], st2[W::NBW];
 #pragma unroll
     for (int i = 0; i < W::NBW; ++i)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) st[i][v] = 0.f;
+        for (int v = 0; v < 16; ++v) st[i][v] = 0.f, st2[i][v] = 0.f;
     // SETS sets of tiles.  Two (two workgroups per CU): the loads of chunk c + 1 are in flight while
-    // chunk c is multiplied.  Four (D = 128, where the grid has at most one workgroup per CU and a
-    // workgroup's own chain load -> barrier -> product bounds its rate): three chunks in flight.
-    constexpr int SETS = walk_totals_sets(D);
+    // chunk c is multiplied.  More (D = 128, where the grid has at most one workgroup per CU and a
+    // workgroup's own chain load -> barrier -> product bounds its rate): SETS - 1 chunks in flight.
+    constexpr int SETS = BOTH ? 3 : walk_totals_sets(D), TPS = BOTH ? 3 : 2;  // tiles per set: Y, (Y2,) Z
     auto load_chunk = [&](int c, int set) {
-        walk_load_tile<D>(ry, lds0 + set * 2 * W::TILE, c * W::C, ys2, dy, wave, lane);
-        walk_load_tile<D>(rz, lds0 + set * 2 * W::TILE + W::TILE, c * W::C, zs2, p.dz, wave, lane);
+        const uint32_t base = lds0 + set * TPS * W::TILE;
+        walk_load_tile<D>(ry, base, c * W::C, ys2, dy, wave, lane);
+        if constexpr (BOTH) walk_load_tile<D>(ry2, base + W::TILE, c * W::C, ys2, p.dy2, wave, lane);
+        walk_load_tile<D>(rz, base + (TPS - 1) * W::TILE, c * W::C, zs2, p.dz, wave, lane);
     };
     auto map_tile = [&](unsigned char *ty, int c) {
         walk_map_tile<T, D>(ty, p.map_y, c * W::C, N, dy, static_cast<T *>(p.ymap_out) + b * p.yo_b + h * p.yo_h,
@@ -1767,29 +1828,30 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
             __builtin_amdgcn_s_barrier();
         }
     } else {
-        static_assert(SETS == 4, "the waits below count two chunks behind the awaited one");
+        static_assert(SETS == 3 || SETS == 4, "the waits below count up to two chunks behind the awaited one");
 #pragma unroll
         for (int i = 0; i < SETS - 1; ++i)
             if (c_lo + i < c_hi) load_chunk(c_lo + i, i);
         int set = 0;
 #pragma unroll 1
         for (int c = c_lo; c < c_hi; ++c) {
-            unsigned char *ty = smem + set * 2 * W::TILE, *tz = ty + W::TILE;
-            // this wave's loads of chunk c have landed: those of up to two later chunks may still be in
+            unsigned char *ty = smem + set * TPS * W::TILE, *tz = ty + (TPS - 1) * W::TILE;
+            // this wave's loads of chunk c have landed: those of up to SETS - 2 later chunks may still be in
             // flight (the mapped rows' stores of a feature map share the counter: then everything is awaited)
             const int behind = c_hi - 1 - c;
             if (p.map_y || behind == 0)
                 wait_vm<0>();
-            else if (behind == 1)
-                wait_vm<2 * W::NI>();
+            else if (behind == 1 || SETS == 3)
+                wait_vm<TPS * W::NI>();
             else
-                wait_vm<4 * W::NI>();
+                wait_vm<2 * TPS * W::NI>();
             __builtin_amdgcn_s_waitcnt(0xc07f);  // this wave's LDS reads of the chunk before are done
             __builtin_amdgcn_s_barrier();        // ... and so are every wave's: its set can be loaded over
             asm volatile("" ::: "memory");
             if (c + SETS - 1 < c_hi) load_chunk(c + SETS - 1, (set + SETS - 1) % SETS);
             if (p.map_y) map_tile(ty, c);
             walk_update<T, D, B>(ty, tz, wave, lane, st);
+            if constexpr (BOTH) walk_update<T, D, B>(ty + W::TILE, tz, wave, lane, st2);
             asm volatile("" ::: "memory");
             set = (set + 1) % SETS;
         }
@@ -1798,9 +1860,11 @@ __global__ __launch_bounds__(256, 2) void walk_totals_kernel(const WalkTotalsPar
     for (int i = 0; i < B::SLOTS; ++i)
         if (B::valid(wave, i)) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v)
-                out[(32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * B::eb(wave) + l32] =
-                    discard ? 0.f : st[i][v];
+            for (int v = 0; v < 16; ++v) {
+                const int at = (32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * B::eb(wave) + l32;
+                out[at] = discard ? 0.f : st[i][v];
+                if constexpr (BOTH) out2[at] = st2[i][v];
+            }
         }
 #else
     (void)p;
@@ -1966,6 +2030,12 @@ hipError_t launch_walk_totals(const WalkTotalsParams &p, hipStream_t stream) {
         return hipErrorInvalidValue;
     const dim3 g((unsigned)grid, p.y2 ? 2u : 1u);
     if constexpr (D == 128) {
+        if (p.y2 && walk_totals_cols(D, p.dy, p.dz) == 64) {  // ... and both operands in one workgroup: z loaded once
+            constexpr auto kern = walk_totals_kernel<T, D, 4, 2, true>;
+            constexpr int smem_both = 3 * 3 * WalkCfg<D>::TILE;
+            if (hipError_t e = ensure_dynamic_lds<kern>(smem_both)) return e;
+            return launch_kernel<kern>(dim3((unsigned)grid), dim3(256), smem_both, stream, p);
+        }
         if (walk_totals_cols(D, p.dy, p.dz) == 64) {  // z of at most 64 true columns: the state's other v blocks hold zeros
             constexpr auto kern = walk_totals_kernel<T, D, 4, 2>;
             if (hipError_t e = ensure_dynamic_lds<kern>(smem)) return e;
@@ -2032,7 +2102,8 @@ hipError_t launch_walk_fwd_wide(const WalkParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     if (p.wqk != 128 || p.wqk2 < 1 || p.wqk2 > 128 || p.wv < 1 || p.wv > 128 || p.fmap || p.slope_y || p.denom || p.dn ||
-        p.accumulate || p.init_transposed || (p.n_seg > 1 && (!p.init || !p.init2)) || (p.total_out && !p.total_out2))
+        p.accumulate || p.init_transposed || (p.n_seg > 1 && (!p.init || !p.init2)) || (p.total_out && !p.total_out2) ||
+        (p.init_is_totals && (p.n_seg < 3 || !p.init || !p.init2)) || (p.entry_out != nullptr) != (p.entry_out2 != nullptr))
         return hipErrorInvalidValue;
     constexpr int smem = 6 * W::TILE + W::STATE;  // two sets of (Q_h, K_h), two V tiles, one state
     if (p.wv <= 64) return launch_walk_kernel<walk_fwd_wide_kernel<T, 2>>(grid, smem, p, stream);

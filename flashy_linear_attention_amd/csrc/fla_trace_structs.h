@@ -62,6 +62,7 @@ FLA_FIELD(qo_b) FLA_FIELD(qo_h) FLA_FIELD(qo_n) FLA_FIELD(slope_y) FLA_FIELD(sy_
 FLA_FIELD(denom) FLA_FIELD(eps) FLA_FIELD(zc) FLA_FIELD(dn) FLA_FIELD(rc) FLA_FIELD(total_out) FLA_FIELD(xinit)
 FLA_FIELD(xtotal) FLA_FIELD(accumulate)
     FLA_FIELD(wqk2) FLA_FIELD(init2) FLA_FIELD(total_out2) FLA_FIELD(xinit2) FLA_FIELD(xtotal2)
+    FLA_FIELD(init_is_totals) FLA_FIELD(entry_out) FLA_FIELD(entry_out2)
 FLA_FIELDS_END
 
 FLA_FIELDS_BEGIN(WalkTotalsParams)

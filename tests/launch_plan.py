@@ -796,6 +796,13 @@ def model_walk_wide(arena: Arena, l: Launch, p: Dict, stats: Stats) -> None:
     D, E = 128, 128 * 128 * 4
     assert p["wqk"] == 128 and 1 <= p["wqk2"] <= 128 and p["wqk2"] % 8 == 0 and not p["accumulate"]
     assert not p["init_transposed"] and not p["fmap"] and not p["denom"] and not p["dn"] and not p["saved"]
+    if p["init_is_totals"]:  # (the walk adds up the segments' totals itself; what it forms goes to entry_out)
+        assert 3 <= p["n_seg"] <= 7 and p["init"] and l.kernel == "walk_fwd_wide_kernel"
+        if p["entry_out"]:
+            arena.require("entry_out", p["entry_out"], p["entry_out"] + p["BH"] * p["n_seg"] * E)
+            assert not (p["init"] <= p["entry_out"] < p["init"] + p["BH"] * p["n_seg"] * E), "entry states over the totals"
+    else:
+        assert not p["entry_out"]
     whole = dict(p)
     whole["wqk"] = 128 + p["wqk2"]
     model_walk(arena, l, whole, D, stats)
@@ -803,7 +810,8 @@ def model_walk_wide(arena: Arena, l: Launch, p: Dict, stats: Stats) -> None:
     tiles = 6 if l.kernel == "walk_fwd_wide_kernel" else 8
     assert l.lds == tiles * 64 * 256 + 128 * 256, f"{l.kernel}: {l.lds} bytes of LDS"
     for first, second, count in (("init", "init2", BH * n_seg), ("xinit", "xinit2", BH * n_seg),
-                                 ("total_out", "total_out2", BH), ("xtotal", "xtotal2", BH)):
+                                 ("total_out", "total_out2", BH), ("xtotal", "xtotal2", BH),
+                                 ("entry_out", "entry_out2", BH * n_seg)):
         assert bool(p[first]) == bool(p[second]), f"{l.kernel}: {first} without {second} or the reverse"
         if p[second]:
             arena.require(f"{second} (second half)", p[second], p[second] + count * E)
@@ -811,7 +819,7 @@ def model_walk_wide(arena: Arena, l: Launch, p: Dict, stats: Stats) -> None:
                 not (p[second] <= p[first] < p[second] + count * E), f"{l.kernel}: {first} and {second} overlap"
 
 
-def model_walk_totals(arena: Arena, l: Launch, p: Dict, D: int, stats: Stats) -> None:
+def model_walk_totals(arena: Arena, l: Launch, p: Dict, D: int, stats: Stats, both: bool = False) -> None:
     rows = 128 if D <= 64 else 64
     N, BH, H = p["N"], p["BH"], p["H"]
     n_chunks, seg_chunks, n_seg = p["n_chunks"], p["seg_chunks"], p["n_seg"]
@@ -820,12 +828,14 @@ def model_walk_totals(arena: Arena, l: Launch, p: Dict, D: int, stats: Stats) ->
     assert l.grid[0] == 8 * ((BH + 7) // 8) * n_seg
     operands = [("y", "y", "ys_b", "ys_h", "ys_n", p["dy"]), ("z", "z", "zs_b", "zs_h", "zs_n", p["dz"])]
     if p["y2"]:  # a second Y operand (the other half of a wide q / k) in the same launch
-        assert l.grid[1] == 2 and not p["map_y"] and p["totals2"]
+        # (grid y picks the operand, or -- the kernel built for it -- every workgroup takes both: three sets of three tiles)
+        assert l.grid[1] == (1 if both else 2) and not p["map_y"] and p["totals2"]
+        assert not both or (D == 128 and p["dz"] <= 64 and l.lds == 9 * 64 * 256)
         operands.append(("y2", "y2", "ys_b", "ys_h", "ys_n", p["dy2"]))
         arena.require("segment totals of the second operand", p["totals2"], p["totals2"] + BH * n_seg * D * D * 4)
         assert not (p["totals"] <= p["totals2"] < p["totals"] + BH * n_seg * D * D * 4), "the two operands' totals overlap"
     else:
-        assert l.grid[1] == 1
+        assert l.grid[1] == 1 and not both
     for nm, ptr, sb, sh, sn, w in operands:
         lo, hi = tensor_extent(p, ptr, sb, sh, sn, H, BH, N, w)
         arena.require(f"totals {nm}", lo, hi)
@@ -894,7 +904,7 @@ def check_all(arena: Arena, launches: List[Launch], stats: Stats) -> None:
                 arena.require("segment totals", t_, t_ + BH * n_seg * E * 4)
                 arena.require("entry states", e_, e_ + BH * n_seg * E * 4)
         elif k == "walk_totals_kernel":
-            model_walk_totals(arena, l, l.struct("a0"), t[1], stats)
+            model_walk_totals(arena, l, l.struct("a0"), t[1], stats, both=len(t) > 4 and bool(t[4]))
         else:
             # remaining kernels (scans, vector sums, element-wise passes, chunk states): limits above,
             # and every pointer argument inside a tensor or the workspace
