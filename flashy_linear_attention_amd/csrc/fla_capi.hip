@@ -658,6 +658,8 @@ int wide_backward(const WidePlan &wide, const View &go, const View &q, const Vie
     // entry states of both halves up front: Q_h^T dO over the segments after, and -- when forward's are not
     // at hand -- K_h^T V over the segments before
     const float *fwd_entries[2] = {nullptr, nullptr}, *entries[2] = {nullptr, nullptr};
+    // (the one reverse walk over both halves adds up the totals of the segments after its own itself, as forward does)
+    const bool rev_sums_on_load = state_in && dv <= 64 && wp.n_seg >= 3 && wp.n_seg <= 7;
     if (wp.n_seg > 1) {
         float *const none[2] = {nullptr, nullptr};
         char *base = ws + wide.temp_bytes;
@@ -669,7 +671,8 @@ int wide_backward(const WidePlan &wide, const View &go, const View &q, const Vie
             if (int rc = wide_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, work, none, fwd_entries, s)) return rc;
         }
         void *const work[2] = {base, base + wp.work_bytes};
-        if (int rc = wide_entry_states(wp, q, go, B, H, N, dqk, dv, dtype, 1, work, none, entries, s)) return rc;
+        if (int rc = wide_entry_states(wp, q, go, B, H, N, dqk, dv, dtype, 1, work, none, entries, s, rev_sums_on_load))
+            return rc;
     }
     if (state_in && dv <= 64) {  // forward's states at hand, narrow v: one reverse walk over both halves
         fla::WalkParams r{};
@@ -685,7 +688,7 @@ int wide_backward(const WidePlan &wide, const View &go, const View &q, const Vie
         r.H = (int32_t)H, r.N = (int32_t)N, r.BH = (int32_t)(B * H), r.wqk = 128, r.wqk2 = (int32_t)(dqk - 128);
         r.wv = (int32_t)dv;
         r.n_chunks = (int32_t)wp.n_chunks, r.seg_chunks = (int32_t)wp.seg_chunks, r.n_seg = (int32_t)wp.n_seg;
-        r.init = entries[0], r.init2 = entries[1];
+        r.init = entries[0], r.init2 = entries[1], r.init_is_totals = rev_sums_on_load;
         const char *half0 = static_cast<const char *>(state_in), *half1 = half0 + wp.saved_bytes;
         r.xinit = reinterpret_cast<const float *>(half0), r.xinit2 = reinterpret_cast<const float *>(half1);
         r.xtotal = reinterpret_cast<const float *>(half0 + wp.entry_bytes);

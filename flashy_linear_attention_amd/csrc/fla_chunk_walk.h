@@ -1617,8 +1617,13 @@ __global__ __launch_bounds__(256, 1) void walk_bwd_rev_wide_kernel(const WalkPar
 
     f32x16 st0[W::NBW], st1[W::NBW];  // R_0, R_1
     f32x16 xs0[W::NBW], xs1[W::NBW];  // X_0, X_1
-    walk_load_init_from<D, B>(p.init, p, sl, wave, lane, st0, true);
-    walk_load_init_from<D, B>(p.init2, p, sl, wave, lane, st1, true);
+    if (p.init_is_totals) {
+        const int64_t at = (int64_t)sl.bh * p.n_seg * (D * D);
+        walk_sum_two<D, B>(p.init + at, p.init2 + at, sl.seg + 1, p.n_seg, wave, lane, st0, st1);
+    } else {
+        walk_load_init_from<D, B>(p.init, p, sl, wave, lane, st0, true);
+        walk_load_init_from<D, B>(p.init2, p, sl, wave, lane, st1, true);
+    }
     walk_load_end_state_from<D, B>(p.xinit, p.xtotal, p, sl, wave, lane, xs0);
     walk_load_end_state_from<D, B>(p.xinit2, p.xtotal2, p, sl, wave, lane, xs1);
     walk_state_to_lds<T, D, B>(tl, wave, lane, st0);
@@ -2179,8 +2184,8 @@ hipError_t launch_walk_bwd_rev_wide(const WalkParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     if (p.wqk != 128 || p.wqk2 < 1 || p.wqk2 > 128 || p.wv < 1 || p.wv > 64) return hipErrorNotSupported;
-    if (p.fmap || p.dn || p.accumulate || p.init_transposed || !p.xtotal || !p.xtotal2 ||
-        (p.n_seg > 1 && (!p.init || !p.init2 || !p.xinit || !p.xinit2)))
+    if (p.fmap || p.dn || p.accumulate || p.init_transposed || !p.xtotal || !p.xtotal2 || p.entry_out || p.entry_out2 ||
+        (p.n_seg > 1 && (!p.init || !p.init2 || !p.xinit || !p.xinit2)) || (p.init_is_totals && p.n_seg < 3))
         return hipErrorInvalidValue;
     constexpr int smem = 8 * W::TILE + W::STATE;  // two sets of (Q_h, K_h), two of (V, dO), one state
     static_assert(smem <= 160 * 1024, "the tiles and the state must fit the LDS of a CU");

@@ -797,8 +797,9 @@ def model_walk_wide(arena: Arena, l: Launch, p: Dict, stats: Stats) -> None:
     assert p["wqk"] == 128 and 1 <= p["wqk2"] <= 128 and p["wqk2"] % 8 == 0 and not p["accumulate"]
     assert not p["init_transposed"] and not p["fmap"] and not p["denom"] and not p["dn"] and not p["saved"]
     if p["init_is_totals"]:  # (the walk adds up the segments' totals itself; what it forms goes to entry_out)
-        assert 3 <= p["n_seg"] <= 7 and p["init"] and l.kernel == "walk_fwd_wide_kernel"
+        assert 3 <= p["n_seg"] <= 7 and p["init"]
         if p["entry_out"]:
+            assert l.kernel == "walk_fwd_wide_kernel"
             arena.require("entry_out", p["entry_out"], p["entry_out"] + p["BH"] * p["n_seg"] * E)
             assert not (p["init"] <= p["entry_out"] < p["init"] + p["BH"] * p["n_seg"] * E), "entry states over the totals"
     else:
