@@ -52,7 +52,7 @@ PROFILED_TRAFFIC = {
     ("C3", "quadratic"): (2.426e9, "profiles/tri_xyt_z_fast_kernels_C3_pmc.md"),
     # chunk-wise: all kernels of a step
     ("C3", "chunked"): (1.847e9, "profiles/chunked_C3_C5_kernel_trace_pmc.md"),
-    ("C4", "chunked"): (1.650e9, "profiles/chunked_C4_kernel_trace_pmc.md"),
+    ("C4", "chunked"): (1.310e9, "profiles/chunked_C4_kernel_trace_pmc.md"),
     ("C5", "chunked"): (1.074e9, "profiles/chunked_C3_C5_kernel_trace_pmc.md"),
 }
 # MFMA operations the dominant kernel issues over those of its product-units (rocprofv3

@@ -56,6 +56,12 @@ CASES = [
     (1, 64, 1024, 128, 128),
     (1, 72, 512, 256, 64),
     (1, 160, 1500, 64, 64),
+    # a wide q / k in one walk over both halves, with segment totals that the walks add up themselves: six segments
+    # (two groups of loads for the late ones), four with a second half of 32 columns, and a v wider than 64
+    # (one forward walk, two reverse walks)
+    (1, 40, 700, 200, 48),
+    (3, 20, 900, 160, 64),
+    (1, 40, 700, 256, 96),
 ]
 
 
@@ -134,7 +140,8 @@ def test_chunked_workspace_errors(gpu_device):
 
 
 @pytest.mark.parametrize("dims", [(2, 3, 1280, 128, 128), (1, 100, 330, 128, 128), (1, 100, 330, 256, 64), (1, 72, 512, 128, 128),
-                                  (2, 100, 900, 64, 64)], ids=lambda d: "x".join(map(str, d)))
+                                  (2, 100, 900, 64, 64), (1, 40, 700, 200, 48), (1, 40, 700, 256, 96)],
+                         ids=lambda d: "x".join(map(str, d)))
 def test_chunked_backward_with_and_without_the_forward_state(dims, gpu_device):
     """Backward given what the forward pass saved, and backward without it (D = 128: two walks from entry
     states it forms again; below: the 256-row chunks with states of their own), both match the oracle -- on
@@ -258,7 +265,7 @@ def test_chunked_small_v_state_hand_over(gpu_device):
     want = naive.causal_dot_product_grads(q.float().cpu(), k.float().cpu(), v.float().cpu(), dy.float().cpu())
     with_state = linear_attention_chunked_bwd(dy, q, k, v, state)
     without = linear_attention_chunked_bwd(dy, q, k, v, None)
-    # (with the states: one reverse walk per half; without: dQ's forward-direction walk and the dK / dV walk)
+    # (with the states: one reverse walk over both halves; without: per half, dQ's forward-direction walk and the dK / dV walk)
     for name, a, b, w in zip(("dQ", "dK", "dV"), with_state, without, want):
         assert_close(name, a, w)
         assert_close(name + " (no saved state)", b, w)
