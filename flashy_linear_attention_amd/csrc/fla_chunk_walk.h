@@ -753,16 +753,37 @@ __host__ __device__ constexpr bool walk_entries_are_totals(int D, int n_seg) {
     return n_seg >= 3 && n_seg <= walk_sum_on_load_max(D);
 }
 
-// this wave's blocks of the sum of the states buf[f_lo .. f_hi - 1] (zeros for an empty range)
+// this wave's blocks of the sum of the states buf[f_lo .. f_hi - 1] (zeros for an empty range), added in
+// ascending order, the loads of up to four states in flight together (one state at a time is a chain of
+// dependent loads: a memory latency per state at the start of every workgroup)
 template <int D, typename B>
 __device__ __forceinline__ void walk_sum_states(const float *buf, int f_lo, int f_hi, bool transposed, int wave, int lane,
                                                 f32x16 (&st)[WalkCfg<D>::NBW]) {
+    using W = WalkCfg<D>;
+    constexpr int GROUP = 4;
 #pragma unroll
-    for (int i = 0; i < WalkCfg<D>::NBW; ++i)
+    for (int i = 0; i < W::NBW; ++i)
 #pragma unroll
         for (int v = 0; v < 16; ++v) st[i][v] = 0.f;
 #pragma unroll 1
-    for (int f = f_lo; f < f_hi; ++f) walk_read_state<D, B, true>(buf + (int64_t)f * (D * D), transposed, wave, lane, st);
+    for (int f0 = f_lo; f0 < f_hi; f0 += GROUP) {
+        f32x16 t[GROUP][W::NBW];
+#pragma unroll
+        for (int u = 0; u < GROUP; ++u) {
+            const int f = f0 + u < f_hi ? f0 + u : f_hi - 1;  // (past the range: the last state once more, not added)
+            walk_read_state<D, B, false>(buf + (int64_t)f * (D * D), transposed, wave, lane, t[u]);
+        }
+#pragma unroll
+        for (int u = 0; u < GROUP; ++u) {
+            const float keep = f0 + u < f_hi ? 1.f : 0.f;
+#pragma unroll
+            for (int i = 0; i < B::SLOTS; ++i)
+                if (B::valid(wave, i)) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) st[i][v] += keep * t[u][i][v];
+                }
+        }
+    }
 }
 
 // st_a, st_b = this wave's blocks of the sums of the states a[f_lo .. f_hi - 1], b[f_lo .. f_hi - 1], the loads of
@@ -772,6 +793,7 @@ __device__ __forceinline__ void walk_sum_two(const float *a, const float *b, int
                                              f32x16 (&st_a)[WalkCfg<D>::NBW], f32x16 (&st_b)[WalkCfg<D>::NBW]) {
     using W = WalkCfg<D>;
     constexpr int E = D * D, GROUP = 3;
+    static_assert(B::SLOTS <= 2, "2 x GROUP x SLOTS x 16 registers beside the two sums: for states of two blocks per wave");
 #pragma unroll
     for (int i = 0; i < W::NBW; ++i)
 #pragma unroll
@@ -1090,14 +1112,19 @@ __global__ __launch_bounds__(256, 1) void walk_fwd_wide_kernel(const WalkParams 
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(O, 0, (N - 1) * os2 + p.wv * 2, 0x00020000);
 
     f32x16 st0[W::NBW], st1[W::NBW];
-    if (p.init_is_totals) {
-        const int64_t at = (int64_t)sl.bh * p.n_seg * (D * D);
-        walk_sum_two<D, B>(p.init + at, p.init2 + at, 0, sl.seg, wave, lane, st0, st1);
-        if (p.entry_out && sl.seg > 0) {  // (the first segment's entry state, zero, is read by nobody)
-            walk_write_state<D, B>(p.entry_out + at + (int64_t)sl.seg * (D * D), wave, lane, st0);
-            walk_write_state<D, B>(p.entry_out2 + at + (int64_t)sl.seg * (D * D), wave, lane, st1);
+    bool summed = false;
+    if constexpr (NV == 2) {  // (init_is_totals: with a narrow v only -- the launcher refuses it otherwise)
+        if (p.init_is_totals) {
+            const int64_t at = (int64_t)sl.bh * p.n_seg * (D * D);
+            walk_sum_two<D, B>(p.init + at, p.init2 + at, 0, sl.seg, wave, lane, st0, st1);
+            if (p.entry_out && sl.seg > 0) {  // (the first segment's entry state, zero, is read by nobody)
+                walk_write_state<D, B>(p.entry_out + at + (int64_t)sl.seg * (D * D), wave, lane, st0);
+                walk_write_state<D, B>(p.entry_out2 + at + (int64_t)sl.seg * (D * D), wave, lane, st1);
+            }
+            summed = true;
         }
-    } else {
+    }
+    if (!summed) {
         walk_load_init_from<D, B>(p.init, p, sl, wave, lane, st0, false);
         walk_load_init_from<D, B>(p.init2, p, sl, wave, lane, st1, false);
     }
@@ -2108,7 +2135,8 @@ hipError_t launch_walk_fwd_wide(const WalkParams &p, hipStream_t stream) {
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     if (p.wqk != 128 || p.wqk2 < 1 || p.wqk2 > 128 || p.wv < 1 || p.wv > 128 || p.fmap || p.slope_y || p.denom || p.dn ||
         p.accumulate || p.init_transposed || (p.n_seg > 1 && (!p.init || !p.init2)) || (p.total_out && !p.total_out2) ||
-        (p.init_is_totals && (p.n_seg < 3 || !p.init || !p.init2)) || (p.entry_out != nullptr) != (p.entry_out2 != nullptr))
+        (p.init_is_totals && (p.n_seg < 3 || !p.init || !p.init2 || p.wv > 64)) ||
+        (p.entry_out != nullptr) != (p.entry_out2 != nullptr) || (p.entry_out && !p.init_is_totals))
         return hipErrorInvalidValue;
     constexpr int smem = 6 * W::TILE + W::STATE;  // two sets of (Q_h, K_h), two V tiles, one state
     if (p.wv <= 64) return launch_walk_kernel<walk_fwd_wide_kernel<T, 2>>(grid, smem, p, stream);
