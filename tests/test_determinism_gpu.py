@@ -31,3 +31,23 @@ def test_repeated_launches_are_bit_identical(name, gpu_device):
     for it in range(8):
         for i, (a, b) in enumerate(zip(run(), ref)):
             assert torch.equal(a, b), f"{name}: output {i} differs on repeat {it}"
+
+
+@pytest.mark.parametrize("dims", [(4, 16, 4096, 256, 64), (1, 40, 1400, 200, 48), (2, 8, 2100, 256, 96)],
+                         ids=lambda d: "x".join(map(str, d)))
+def test_repeated_wide_walks_are_bit_identical(dims, gpu_device):
+    """q and k wider than 128 columns, chunk-wise: one walk over both 128-column halves whose states take turns in
+    one LDS buffer and whose V (V, dO) tiles alternate between two slots -- four, six and many segments per (b, h)
+    (segment totals added up by the walks themselves, or entry states from the scan), a v of 64, 48 and 96 columns."""
+    from helpers import reference_style_inputs
+
+    q, k, v, do = (t.to(gpu_device) for t in reference_style_inputs(*dims, torch.bfloat16, seed=5))
+
+    def run():
+        out, state = linear_attention_chunked_fwd(q, k, v, True)
+        return (out, *linear_attention_chunked_bwd(do, q, k, v, state), *linear_attention_chunked_bwd(do, q, k, v, None))
+
+    ref = run()
+    for it in range(8):
+        for i, (a, b) in enumerate(zip(run(), ref)):
+            assert torch.equal(a, b), f"output {i} differs on repeat {it}"

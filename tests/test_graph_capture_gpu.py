@@ -57,8 +57,9 @@ def test_replayed_graph_equals_eager(dims, fwd, bwd, gpu_device):
 
 
 @pytest.mark.parametrize("dims,normalised", [((2, 4, 2048, 64, 64), False), ((1, 8, 2048, 128, 128), False),
-                                             ((2, 4, 2048, 64, 64), True), ((1, 8, 2048, 128, 128), True)],
-                         ids=["d64", "d128", "d64-normalised", "d128-normalised"])
+                                             ((2, 4, 2048, 64, 64), True), ((1, 8, 2048, 128, 128), True),
+                                             ((1, 64, 1024, 256, 64), False), ((1, 8, 2048, 256, 64), False)],
+                         ids=["d64", "d128", "d64-normalised", "d128-normalised", "wide-4-segments", "wide-scan"])
 def test_replayed_graph_of_the_chunkwise_operators_equals_eager(dims, normalised, gpu_device):
     """The chunk-wise walk kernels (totals, scan, walks; with the normaliser also the vector sums and
     the dO pass), forward handing its state to backward: captured once, replayed on fresh inputs."""
