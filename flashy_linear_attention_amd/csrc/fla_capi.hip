@@ -1595,14 +1595,14 @@ int fla_tri_xyt_z_chunked(const void *x, const void *y, const void *z, void *out
 // Which evaluation of forward + backward is faster on MI355X, from timings of both over grids of
 // (head dims, B H, N) (bench.py --crossover): the quadratic kernels' time grows with
 // W = B H N^2 D (D: the larger padded head dim), the chunk-wise kernels' with B H N D above a floor
-// of launches (four to six for the walk kernels, twice that for a wide q / k as two halves), so each
+// of launches (four to six for the walk kernels, also for a wide q / k against a narrow v), so each
 // of these classes of shapes has one threshold on W.
 int fla_linear_attn_prefers_chunked(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v) {
     if (B < 1 || H < 1 || N < 1 || D_qk < 1 || D_qk > 256 || D_v < 1 || D_v > 256) return 0;
     const double w = (double)B * (double)H * (double)N * (double)N * (double)padded(D_qk > D_v ? D_qk : D_v);
     const WalkPlan wp = walk_plan(B, H, N, D_qk, D_v);
     if (wp.ok) return w >= (wp.D <= 64 ? 4e9 : 8e9);                              // equal padded head dims up to 128
-    if (wide_plan(B, H, N, D_qk, D_v).ok) return w >= (D_v <= 64 ? 1e9 : 3e10);  // D_qk in (128, 256], D_v <= 128
+    if (wide_plan(B, H, N, D_qk, D_v).ok) return w >= (D_v <= 64 ? 1e9 : 1.5e10);  // D_qk in (128, 256], D_v <= 128
     return N >= 4096;  // chunk states in memory, a launch per product and state (measured at 256 / 256)
 }
 
