@@ -959,7 +959,7 @@ def main() -> int:
         result["config"]["other_workloads"] = [
             _other_workload(torch, name, algo, dev, args.other_steps)
             for name, algo in (("C2", "quadratic"), ("C4", "quadratic"), ("C5", "quadratic"),
-                               ("C3", "chunked"), ("C4", "chunked"), ("C5", "chunked"))
+                               ("C2", "chunked"), ("C3", "chunked"), ("C4", "chunked"), ("C5", "chunked"))
         ] + [
             # the operators beyond the reference's two, each beside the PyTorch recipe it replaces
             _other_extension(torch, name, algo, dev, min(args.other_steps, 30))
