@@ -28,12 +28,14 @@ def prepare(*tensors: torch.Tensor) -> Tuple[torch.Tensor, ...]:
     first = tensors[0]
     if not first.is_cuda:
         raise RuntimeError("flashy_linear_attention_amd operators need tensors on a ROCm GPU (device 'cuda')")
-    device, dtype = first.device, first.dtype
+    # (get_device() is the device index, -1 on the CPU: an integer comparison per tensor where comparing
+    # torch.device objects costs several times as much)
+    index, dtype = first.get_device(), first.dtype
     dense = True
     for t in tensors:
         if t.dim() != 4:
             raise ValueError(f"expected (batch, heads, seq, head_dim) tensors, got shape {tuple(t.shape)}")
-        if t.device != device:
+        if t.get_device() != index:
             raise RuntimeError("all tensors must be on the same device")
         if t.dtype != dtype:
             raise TypeError(f"all tensors must share one dtype, got {dtype} and {t.dtype}")
@@ -66,11 +68,19 @@ class _NoGuard:
 _NO_GUARD = _NoGuard()
 
 
+try:  # the current device's index without the checks of torch.cuda.current_device (lazy initialisation, a Python frame)
+    _current_device = torch._C._cuda_getDevice
+except AttributeError:  # pragma: no cover - older or differently built torch
+    _current_device = torch.cuda.current_device
+
+
 def device_guard(device: torch.device):
     """Context that makes `device` the current one for the call into the library (which launches on
     the current device).  When it already is -- the usual case -- nothing is switched: entering and
-    leaving torch.cuda.device costs two device exchanges per call."""
-    if device.index is None or device.index == torch.cuda.current_device():
+    leaving torch.cuda.device costs two device exchanges per call.  (The callers hold a tensor on
+    `device`, so the GPU runtime is initialised.)"""
+    index = device.index
+    if index is None or index == _current_device():
         return _NO_GUARD
     return torch.cuda.device(device)
 
