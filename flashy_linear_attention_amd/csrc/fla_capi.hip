@@ -555,7 +555,44 @@ WidePlan wide_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
 
 View column_half(const View &t, int h) { return View{static_cast<const char *>(t.ptr) + h * 128 * 2, t.strides}; }
 
+// ---- D_v in (128, 256] with D_qk in (64, 256].  O and dV are column by column in v's (dO's) columns, and dQ, dK
+// are sums over them: the two column halves of v (128 and D_v - 128 columns) each run the plan of a
+// (D_qk, at most 128) problem -- the walk kernels at D = 128, or the walks over a wide q / k -- on column views
+// of v, O, dO, dV; the second half's dQ and dK go to scratch tensors that one element-wise pass each adds to the
+// first half's.  (q and k are read once per half; the 256-row chunk kernels with their per-chunk states in
+// memory, which these shapes took before, measured 2.4x slower at 256 / 256.)
+struct VSplit {
+    bool ok;
+    int64_t dv1;         // columns of the second half
+    int64_t state0;      // bytes of the first half's state (the second half's follows it)
+    int64_t temp_bytes;  // one scratch tensor, contiguous (B, H, N, D_qk)
+};
+
+int64_t shared_state_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv);
+int64_t chunked_op_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv);
+
+VSplit vsplit_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
+    VSplit s{};
+    if (dv <= 128 || dv > 256 || dqk <= 64 || dqk > 256 || B <= 0 || H <= 0) return s;
+    s.dv1 = dv - 128;
+    auto planned = [&](int64_t d) { return walk_plan(B, H, N, dqk, d).ok || wide_plan(B, H, N, dqk, d).ok; };
+    s.ok = planned(128) && planned(s.dv1);
+    if (!s.ok) return s;
+    s.state0 = (shared_state_bytes(B, H, N, dqk, 128) + 255) / 256 * 256;
+    s.temp_bytes = (B * H * N * dqk * 2 + 255) / 256 * 256;
+    return s;
+}
+
+View v_half(const View &t, int j) { return View{static_cast<const char *>(t.ptr) + j * 128 * 2, t.strides}; }
+
+// what the halves' own calls use of the workspace (the scratch tensors follow it)
+int64_t vsplit_inner_bytes(const VSplit &vs, int64_t B, int64_t H, int64_t N, int64_t dqk) {
+    const int64_t a = chunked_op_workspace_bytes(B, H, N, dqk, 128), b = chunked_op_workspace_bytes(B, H, N, dqk, vs.dv1);
+    return ((a > b ? a : b) + 255) / 256 * 256;
+}
+
 int64_t state_core_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
+    if (const VSplit vs = vsplit_plan(B, H, N, dqk, dv); vs.ok) return vs.state0 + shared_state_bytes(B, H, N, dqk, vs.dv1);
     const WalkPlan w = walk_plan(B, H, N, dqk, dv);
     if (w.ok && !w.split) return w.saved_bytes;  // one state per 128-row chunk (also room for the 256-row chunks' states)
     if (!states_shareable(dqk, dv, N)) {
@@ -589,6 +626,10 @@ int64_t chunked_op_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk,
     if (t > m) m = t;
     const WidePlan wide = wide_plan(B, H, N, dqk, dv);
     if (wide.ok && wide_workspace_bytes(wide) > m) m = wide_workspace_bytes(wide);
+    if (const VSplit vs = vsplit_plan(B, H, N, dqk, dv); vs.ok) {
+        const int64_t need = vsplit_inner_bytes(vs, B, H, N, dqk) + 2 * vs.temp_bytes;
+        if (need > m) m = need;
+    }
     return m;
 }
 
@@ -744,6 +785,26 @@ int wide_backward(const WidePlan &wide, const View &go, const View &q, const Vie
     return state_in ? FLA_OK : launch_feature_pass(3, 0, temp, dvv, B, H, N, dv, dtype, s);
 }
 
+// both column halves of (x4, o4) = (v, O) / (dO, dV) with (a, b) = (q, k) / (dQ, dK) qualify for their plans' kernels
+bool vsplit_fast_path(const VSplit &vs, const View &a, const View &b, const View &x4, const View &o4, int64_t B, int64_t H,
+                      int64_t N, int64_t dqk) {
+    for (int j = 0; j < 2; ++j) {
+        const int64_t d = j == 0 ? 128 : vs.dv1;
+        const View xj = v_half(x4, j), oj = v_half(o4, j);
+        const bool ok = dqk > 128 ? wide_fast_path(a, b, xj, oj, B, H, N, dqk, d)
+                                  : fla::fast_path_ok(make_params(a, b, xj, oj, B, H, N, dqk, d, 0));
+        if (!ok) return false;
+    }
+    return true;
+}
+
+int chunked_forward(const View &q, const View &k, const View &v, const View &o, int64_t B, int64_t H, int64_t N,
+                    int64_t dqk, int64_t dv, int dtype, void *state_out, int32_t *state_valid, void *workspace,
+                    int64_t workspace_bytes, void *stream, int fmap, const View *mapped, bool *mapped_done, WalkNorm *nx);
+int chunked_backward(const View &go, const View &q, const View &k, const View &v, const View &dq, const View &dk,
+                     const View &dvv, int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv, int dtype,
+                     const void *state_in, void *workspace, int64_t workspace_bytes, void *stream, int fmap, WalkNorm *nx);
+
 // fmap != 0 (feature_forward below): q and k hold the arguments xq, xk of the feature map phi, and
 // `mapped` = {phi(xq), phi(xk)} are outputs: the state kernel maps xk as it loads it and writes
 // phi(xk), which the main kernel then reads as its Y operand; the main kernel maps its X rows xq
@@ -760,6 +821,23 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
     if (int rc = check_alias_fwd(q, k, v, o, B, H, N, dqk, dv)) return rc;
     if (B == 0 || H == 0 || N == 0) return FLA_OK;
     if (!fmap && !nx) {
+        // a v wider than 128 columns: its two column halves, one after the other (the second half's state behind the first's)
+        const VSplit vs = vsplit_plan(B, H, N, dqk, dv);
+        if (vs.ok && vsplit_fast_path(vs, q, k, v, o, B, H, N, dqk)) {
+            if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 ||
+                workspace_bytes < vsplit_inner_bytes(vs, B, H, N, dqk))
+                return FLA_ERR_WORKSPACE;
+            if (state_out && reinterpret_cast<uintptr_t>(state_out) % 16 != 0) return FLA_ERR_WORKSPACE;
+            int32_t valid[2] = {0, 0};
+            for (int j = 0; j < 2; ++j) {
+                void *st = state_out ? static_cast<char *>(state_out) + j * vs.state0 : nullptr;
+                if (int rc = chunked_forward(q, k, v_half(v, j), v_half(o, j), B, H, N, dqk, j == 0 ? 128 : vs.dv1, dtype, st,
+                                             &valid[j], workspace, workspace_bytes, stream, 0, nullptr, nullptr, nullptr))
+                    return rc;
+            }
+            if (state_out && state_valid) *state_valid = valid[0] && valid[1];
+            return FLA_OK;
+        }
         const WidePlan wide = wide_plan(B, H, N, dqk, dv);
         if (wide.ok && wide_fast_path(q, k, v, o, B, H, N, dqk, dv)) {
             if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wide_workspace_bytes(wide))
@@ -866,6 +944,26 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
     TriParams pv = make_params(k, q, go, dvv, B, H, N, dqk, dv, 1);  // dV = upper(K Q^T) dO
     TriParams pk = make_params(v, go, q, dk, B, H, N, dv, dqk, 1);   // dK = upper(V dO^T) Q
     if (!fmap && !nx) {
+        // a v wider than 128 columns: dV of each column half; dQ and dK of the second half to scratch tensors, then added
+        const VSplit vs = vsplit_plan(B, H, N, dqk, dv);
+        if (vs.ok && vsplit_fast_path(vs, q, k, v, go, B, H, N, dqk) && vsplit_fast_path(vs, dq, dk, dvv, dvv, B, H, N, dqk)) {
+            const int64_t inner = vsplit_inner_bytes(vs, B, H, N, dqk);
+            if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < inner + 2 * vs.temp_bytes)
+                return FLA_ERR_WORKSPACE;
+            if (state_in && reinterpret_cast<uintptr_t>(state_in) % 16 != 0) return FLA_ERR_WORKSPACE;
+            const int64_t temp_strides[4] = {H * N * dqk, N * dqk, dqk, 1};
+            const View tq{static_cast<char *>(workspace) + inner, temp_strides};
+            const View tk{static_cast<char *>(workspace) + inner + vs.temp_bytes, temp_strides};
+            for (int j = 0; j < 2; ++j) {
+                const void *st = state_in ? static_cast<const char *>(state_in) + j * vs.state0 : nullptr;
+                if (int rc = chunked_backward(v_half(go, j), q, k, v_half(v, j), j == 0 ? dq : tq, j == 0 ? dk : tk,
+                                              v_half(dvv, j), B, H, N, dqk, j == 0 ? 128 : vs.dv1, dtype, st, workspace, inner,
+                                              stream, 0, nullptr))
+                    return rc;
+            }
+            if (int rc = launch_feature_pass(3, 0, tq, dq, B, H, N, dqk, dtype, stream)) return rc;
+            return launch_feature_pass(3, 0, tk, dk, B, H, N, dqk, dtype, stream);
+        }
         const WidePlan wide = wide_plan(B, H, N, dqk, dv);
         if (wide.ok && wide_fast_path(q, k, v, go, B, H, N, dqk, dv) && wide_fast_path(dq, dk, dvv, dvv, B, H, N, dqk, dv)) {
             if (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wide_workspace_bytes(wide))
@@ -1603,6 +1701,7 @@ int fla_linear_attn_prefers_chunked(int64_t B, int64_t H, int64_t N, int64_t D_q
     const WalkPlan wp = walk_plan(B, H, N, D_qk, D_v);
     if (wp.ok) return w >= (wp.D <= 64 ? 4e9 : 8e9);                              // equal padded head dims up to 128
     if (wide_plan(B, H, N, D_qk, D_v).ok) return w >= (D_v <= 64 ? 1e9 : 1.5e10);  // D_qk in (128, 256], D_v <= 128
+    if (vsplit_plan(B, H, N, D_qk, D_v).ok) return w >= 3e10;  // D_v in (128, 256] as two column halves of v
     return N >= 4096;  // chunk states in memory, a launch per product and state (measured at 256 / 256)
 }
 

@@ -62,6 +62,13 @@ CASES = [
     (1, 40, 700, 200, 48),
     (3, 20, 900, 160, 64),
     (1, 40, 700, 256, 96),
+    # a v wider than 128 columns as two column halves: over the walks for a wide q / k (256 / 256, a second half of
+    # 8 columns, 200 / 200) and over the D = 128 walks (128 / 256, 96 / 200)
+    (2, 8, 1300, 256, 256),
+    (1, 5, 900, 256, 136),
+    (1, 64, 640, 200, 200),
+    (1, 3, 1100, 128, 256),
+    (1, 40, 700, 96, 200),
 ]
 
 
@@ -140,7 +147,8 @@ def test_chunked_workspace_errors(gpu_device):
 
 
 @pytest.mark.parametrize("dims", [(2, 3, 1280, 128, 128), (1, 100, 330, 128, 128), (1, 100, 330, 256, 64), (1, 72, 512, 128, 128),
-                                  (2, 100, 900, 64, 64), (1, 40, 700, 200, 48), (1, 40, 700, 256, 96)],
+                                  (2, 100, 900, 64, 64), (1, 40, 700, 200, 48), (1, 40, 700, 256, 96),
+                                  (2, 8, 1300, 256, 256), (1, 3, 1100, 128, 256)],
                          ids=lambda d: "x".join(map(str, d)))
 def test_chunked_backward_with_and_without_the_forward_state(dims, gpu_device):
     """Backward given what the forward pass saved, and backward without it (D = 128: two walks from entry
