@@ -387,11 +387,16 @@ struct WalkPlan {
                                           // up to 64, the 16-bit state of every chunk (room for the larger of the two)
 };
 
-WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
+// `mixed`: also for head dims whose padded widths differ (128 / 64, 64 / 32, 64 / 128 ...), at the larger one: the tiles
+// are padded with zeros as they land in LDS, and at D = 128 the kernels built for at most 64 true columns on one side
+// leave the padding's MFMAs out.  The plain operator only (the normaliser's and the feature maps' variants of the
+// kernels are built for equal padded widths).
+WalkPlan walk_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv, bool mixed = false) {
     WalkPlan w{};
     if (B <= 0 || H <= 0 || N <= 0) return w;  // (an empty problem has no plan; the callers return before any launch)
-    if (pad_index(dqk) != pad_index(dv) || padded(dqk) > 128) return w;
-    w.D = (int)padded(dqk);
+    const int64_t wider = padded(dqk) > padded(dv) ? padded(dqk) : padded(dv);
+    if (wider > 128 || (!mixed && pad_index(dqk) != pad_index(dv))) return w;
+    w.D = (int)wider;
     w.rows = fla::walk_rows(w.D);
     w.split = w.D > 64;
     w.ok = N > (w.split ? 256 : w.rows);  // (D = 128: up to 256 rows one diagonal block of the quadratic kernel does it)
@@ -555,7 +560,7 @@ WidePlan wide_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
 
 View column_half(const View &t, int h) { return View{static_cast<const char *>(t.ptr) + h * 128 * 2, t.strides}; }
 
-// ---- D_v in (128, 256] with D_qk in (64, 256].  O and dV are column by column in v's (dO's) columns, and dQ, dK
+// ---- D_v in (128, 256].  O and dV are column by column in v's (dO's) columns, and dQ, dK
 // are sums over them: the two column halves of v (128 and D_v - 128 columns) each run the plan of a
 // (D_qk, at most 128) problem -- the walk kernels at D = 128, or the walks over a wide q / k -- on column views
 // of v, O, dO, dV; the second half's dQ and dK go to scratch tensors that one element-wise pass each adds to the
@@ -573,9 +578,9 @@ int64_t chunked_op_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk,
 
 VSplit vsplit_plan(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     VSplit s{};
-    if (dv <= 128 || dv > 256 || dqk <= 64 || dqk > 256 || B <= 0 || H <= 0) return s;
+    if (dv <= 128 || dv > 256 || dqk < 1 || dqk > 256 || B <= 0 || H <= 0) return s;
     s.dv1 = dv - 128;
-    auto planned = [&](int64_t d) { return walk_plan(B, H, N, dqk, d).ok || wide_plan(B, H, N, dqk, d).ok; };
+    auto planned = [&](int64_t d) { return walk_plan(B, H, N, dqk, d, true).ok || wide_plan(B, H, N, dqk, d).ok; };
     s.ok = planned(128) && planned(s.dv1);
     if (!s.ok) return s;
     s.state0 = (shared_state_bytes(B, H, N, dqk, 128) + 255) / 256 * 256;
@@ -593,7 +598,7 @@ int64_t vsplit_inner_bytes(const VSplit &vs, int64_t B, int64_t H, int64_t N, in
 
 int64_t state_core_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     if (const VSplit vs = vsplit_plan(B, H, N, dqk, dv); vs.ok) return vs.state0 + shared_state_bytes(B, H, N, dqk, vs.dv1);
-    const WalkPlan w = walk_plan(B, H, N, dqk, dv);
+    const WalkPlan w = walk_plan(B, H, N, dqk, dv, true);
     if (w.ok && !w.split) return w.saved_bytes;  // one state per 128-row chunk (also room for the 256-row chunks' states)
     if (!states_shareable(dqk, dv, N)) {
         const WidePlan wide = wide_plan(B, H, N, dqk, dv);
@@ -618,8 +623,15 @@ int64_t wide_workspace_bytes(const WidePlan &w) { return w.temp_bytes + 4 * w.wp
 int64_t chunked_op_workspace_bytes(int64_t B, int64_t H, int64_t N, int64_t dqk, int64_t dv) {
     const int64_t shared = shared_state_bytes(B, H, N, dqk, dv);
     if (shared) {  // fp32 chunk states (2x) + two rounded states (backward without a saved one); the walk's totals
-        const WalkPlan w = walk_plan(B, H, N, dqk, dv);
-        if (w.ok || states_shareable(dqk, dv, N)) return w.ok && w.work_bytes * 2 > shared * 4 ? w.work_bytes * 2 : shared * 4;
+        const WalkPlan w = walk_plan(B, H, N, dqk, dv, true);
+        if (w.ok || states_shareable(dqk, dv, N)) {
+            int64_t m = w.ok && w.work_bytes * 2 > shared * 4 ? w.work_bytes * 2 : shared * 4;
+            if (pad_index(dqk) != pad_index(dv)) {  // (off the walks these shapes evaluate product by product)
+                const int64_t a = chunked_bytes(B, H, N, dqk, dv), b = chunked_bytes(B, H, N, dv, dqk);
+                m = a > m ? a : m, m = b > m ? b : m;
+            }
+            return m;
+        }
     }
     int64_t m = chunked_bytes(B, H, N, dqk, dv);
     const int64_t t = chunked_bytes(B, H, N, dv, dqk);
@@ -850,7 +862,7 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
             return FLA_OK;
         }
     }
-    const WalkPlan wp = walk_plan(B, H, N, dqk, dv);
+    const WalkPlan wp = walk_plan(B, H, N, dqk, dv, !fmap && !nx);
     if (wp.ok && fla::fast_path_ok(make_params(q, k, v, o, B, H, N, dqk, dv, 0)) &&
         (!fmap || fla::fast_path_ok(make_params(mapped[0], mapped[1], v, o, B, H, N, dqk, dv, 0)))) {
         // the segments' entry states; with a feature map the same kernel maps xk as it loads it and
@@ -975,7 +987,13 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
     }
     // (with the normaliser's terms still to be added by the caller, so is the slope)
     const int fmap_late = nx ? 0 : fmap;
-    if (!states_shareable(dqk, dv, N) || !fla::fast_path_ok(pq) || !fla::fast_path_ok(pv) || !fla::fast_path_ok(pk)) {
+    const WalkPlan wp = walk_plan(B, H, N, dqk, dv, !fmap && !nx);
+    // (what forward saved is in the walks' format; at D = 128 the entry states are cheap to recompute)
+    const bool walk = wp.ok && (state_in || wp.split);
+    // (padded widths that differ: the walks or product by product -- the 256-row chunks share states between equal ones only)
+    const bool mixed_walk = walk && pad_index(dqk) != pad_index(dv);
+    if ((!states_shareable(dqk, dv, N) && !mixed_walk) || !fla::fast_path_ok(pq) || !fla::fast_path_ok(pv) ||
+        !fla::fast_path_ok(pk)) {
         if (int rc = run_tri_chunked(go, v, k, dq, B, H, N, dv, dqk, 0, dtype, workspace, workspace_bytes, stream))
             return rc;
         if (int rc = run_tri_chunked(k, q, go, dvv, B, H, N, dqk, dv, 1, dtype, workspace, workspace_bytes, stream))
@@ -986,9 +1004,6 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         if (int rc = launch_feature_pass(2, fmap, q, dq, B, H, N, dqk, dtype, stream)) return rc;
         return launch_feature_pass(2, fmap, k, dk, B, H, N, dqk, dtype, stream);
     }
-    const WalkPlan wp = walk_plan(B, H, N, dqk, dv);
-    // (what forward saved is in this path's format; the split path's entry states are cheap to recompute)
-    const bool walk = wp.ok && (state_in || wp.split);
     // the normalised forward left zc behind its state
     const float *zc_saved = nx && state_in ? reinterpret_cast<const float *>(static_cast<const char *>(state_in) +
                                                                            state_core_bytes(B, H, N, dqk, dv))
@@ -1698,8 +1713,8 @@ int fla_tri_xyt_z_chunked(const void *x, const void *y, const void *z, void *out
 int fla_linear_attn_prefers_chunked(int64_t B, int64_t H, int64_t N, int64_t D_qk, int64_t D_v) {
     if (B < 1 || H < 1 || N < 1 || D_qk < 1 || D_qk > 256 || D_v < 1 || D_v > 256) return 0;
     const double w = (double)B * (double)H * (double)N * (double)N * (double)padded(D_qk > D_v ? D_qk : D_v);
-    const WalkPlan wp = walk_plan(B, H, N, D_qk, D_v);
-    if (wp.ok) return w >= (wp.D <= 64 ? 4e9 : 8e9);                              // equal padded head dims up to 128
+    const WalkPlan wp = walk_plan(B, H, N, D_qk, D_v, true);
+    if (wp.ok) return w >= (wp.D <= 64 ? 4e9 : 8e9);                              // padded head dims up to 128
     if (wide_plan(B, H, N, D_qk, D_v).ok) return w >= (D_v <= 64 ? 1e9 : 1.5e10);  // D_qk in (128, 256], D_v <= 128
     if (vsplit_plan(B, H, N, D_qk, D_v).ok) return w >= 3e10;  // D_v in (128, 256] as two column halves of v
     return N >= 4096;  // chunk states in memory, a launch per product and state (measured at 256 / 256)
@@ -1740,7 +1755,7 @@ int fla_linear_attn_chunked_fwd_static(const void *q, const void *k, const void 
     const View all[] = {vq, vk, vv, vo};
     for (const View &t : all)
         if (int rc = check_view(t)) return rc;
-    const WalkPlan wp = walk_plan(B, H, N, D_qk, D_v);
+    const WalkPlan wp = walk_plan(B, H, N, D_qk, D_v, true);
     int64_t need = chunked_op_workspace_bytes(B, H, N, D_qk, D_v);
     if (wp.ok)
         need = fla::fast_path_ok(make_params(vq, vk, vv, vo, B, H, N, D_qk, D_v, 0)) ? wp.work_bytes

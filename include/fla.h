@@ -176,11 +176,11 @@ int fla_tri_xyt_z_chunked(const void *x, const void *y, const void *z, void *out
 /* The whole operator evaluated chunk-wise, forward and backward, with the running states
  * shared between products: O and dQ use the same state (sum of K_c^T V_c over earlier chunks),
  * dV and dK the same one (sum of Q_c^T dO_c over later chunks), so a forward + backward pair
- * computes two states instead of four.  Sharing needs equal padded head dims (next of 32 / 64 /
- * 128) up to 128 -- or a D_qk up to 256, taken as two 128-column halves, and a D_v up to 256 with
- * D_qk > 64, taken as two column halves of v -- operands that meet the speed-path alignment rules
- * and more than one chunk; every other case evaluates each product with fla_tri_xyt_z_chunked's
- * method, same results.
+ * computes two states instead of four.  Sharing needs operands that meet the speed-path alignment
+ * rules and more than one chunk (more than 256 rows at padded head dims above 64); head dims are
+ * padded to the next of 32 / 64 / 128, a D_qk up to 256 is taken as two 128-column halves and a D_v
+ * up to 256 as two column halves of v.  Every other case evaluates each product with
+ * fla_tri_xyt_z_chunked's method, same results.
  *
  * forward:  `state_out` (optional, fla_linear_attn_chunked_state_bytes() bytes, 16-byte aligned)
  *           receives what a later backward call can reuse of the running state (the fp32 state at

@@ -219,8 +219,12 @@ def test_chunkwise_state_and_workspace_sizes():
     # D_qk = 256, D_v = 64: the fp32 entry states of both 128-column halves, 4 walk segments per (b, h), and their
     # states after the last chunk
     assert sb(4, 16, 4096, 256, 64) == 2 * 64 * 5 * 128 * 128 * 4
-    # nothing to hand over: a value head dim wider than the query / key one, a single chunk
-    assert sb(4, 16, 4096, 64, 256) == 0 and sb(1, 2, 256, 128, 128) == 0 and sb(1, 2, 128, 64, 64) == 0
+    # D_v = 256 against D_qk = 64: the two column halves of v, each a 64 / 128 problem on the D = 128 walks (4 segments)
+    assert sb(4, 16, 4096, 64, 256) == 2 * 64 * 5 * 128 * 128 * 4
+    # padded widths that differ run at the larger one: 128 / 64 as D = 128, 64 / 32 as D = 64 (room for 32 chunk states)
+    assert sb(4, 16, 4096, 128, 64) == 64 * 5 * 128 * 128 * 4 and sb(4, 16, 4096, 64, 32) == 64 * 32 * 64 * 64 * 2
+    # nothing to hand over: a single chunk
+    assert sb(1, 2, 256, 128, 128) == 0 and sb(1, 2, 128, 64, 64) == 0 and sb(1, 2, 256, 64, 256) == 0
     ws = lib.fla_linear_attn_chunked_workspace_bytes
     for shape in [(4, 32, 4096, 128, 128), (1, 16, 32768, 64, 64), (2, 8, 2450, 128, 128), (1, 4, 1500, 104, 120)]:
         assert ws(*shape) >= 4 * (sb(*shape) - shape[0] * shape[1] * 4)  # room for the 256-row path's four buffers

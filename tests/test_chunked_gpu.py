@@ -69,6 +69,14 @@ CASES = [
     (1, 64, 640, 200, 200),
     (1, 3, 1100, 128, 256),
     (1, 40, 700, 96, 200),
+    # padded widths that differ, on the walk kernels at the larger one (the small-V operator's shapes among them)
+    (2, 8, 1300, 128, 64),
+    (1, 40, 700, 128, 32),
+    (1, 5, 900, 64, 128),
+    (2, 8, 1300, 64, 32),
+    (1, 70, 600, 32, 64),
+    (1, 3, 1100, 24, 128),
+    (1, 6, 1000, 64, 256),
 ]
 
 
@@ -148,7 +156,8 @@ def test_chunked_workspace_errors(gpu_device):
 
 @pytest.mark.parametrize("dims", [(2, 3, 1280, 128, 128), (1, 100, 330, 128, 128), (1, 100, 330, 256, 64), (1, 72, 512, 128, 128),
                                   (2, 100, 900, 64, 64), (1, 40, 700, 200, 48), (1, 40, 700, 256, 96),
-                                  (2, 8, 1300, 256, 256), (1, 3, 1100, 128, 256)],
+                                  (2, 8, 1300, 256, 256), (1, 3, 1100, 128, 256), (2, 8, 1300, 128, 64), (2, 8, 1300, 64, 32),
+                                  (1, 5, 900, 64, 128)],
                          ids=lambda d: "x".join(map(str, d)))
 def test_chunked_backward_with_and_without_the_forward_state(dims, gpu_device):
     """Backward given what the forward pass saved, and backward without it (D = 128: two walks from entry
@@ -169,9 +178,10 @@ def test_chunked_backward_with_and_without_the_forward_state(dims, gpu_device):
         assert_close(name + " (no saved state)", other, w)
     if dims != (2, 3, 1280, 128, 128):
         return
-    # a value head dim wider than the query / key one, and a single chunk: no shared state
-    q2, k2, v2, _ = (t.to(gpu_device) for t in reference_style_inputs(1, 2, 1024, 64, 256, torch.bfloat16, seed=32))
-    assert linear_attention_chunked_fwd(q2, k2, v2, want_state=True)[1] is None
+    # rows that do not meet the alignment rules of the walk kernels (product by product then), and a single chunk:
+    # no shared state
+    q2, k2, v2, _ = (t.to(gpu_device) for t in reference_style_inputs(1, 2, 1024, 64, 264, torch.bfloat16, seed=32))
+    assert linear_attention_chunked_fwd(q2, k2, v2[..., 4:260], want_state=True)[1] is None
     assert linear_attention_chunked_fwd(q[:, :, :256], k[:, :, :256], v[:, :, :256], want_state=True)[1] is None
 
 

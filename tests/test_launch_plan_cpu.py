@@ -195,9 +195,10 @@ def test_normalised_operator_over_the_sweep_space(lib, dims):
     assert cases > 25 and stats.launches > cases * 4
 
 
-# (the last three: a v wider than 128 columns as two column halves, over the D = 128 walks and over the wide ones)
+# (a v wider than 128 columns as two column halves, over the D = 128 walks and over the wide ones; padded widths that differ)
 @pytest.mark.parametrize("dims", DIMS + [(256, 256), (40, 40), (25, 25), (91, 91), (128, 32), (200, 200), (128, 256),
-                                         (96, 200), (256, 136)],
+                                         (96, 200), (256, 136), (128, 64), (64, 128), (64, 32), (32, 64), (24, 128),
+                                         (64, 256), (32, 200)],
                          ids=lambda d: f"{d[0]}x{d[1]}")
 @pytest.mark.parametrize("chunked", (False, True), ids=("quadratic", "chunkwise"))
 def test_plain_operator(lib, dims, chunked):
