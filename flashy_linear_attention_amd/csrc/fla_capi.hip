@@ -1714,7 +1714,9 @@ int fla_linear_attn_prefers_chunked(int64_t B, int64_t H, int64_t N, int64_t D_q
     if (B < 1 || H < 1 || N < 1 || D_qk < 1 || D_qk > 256 || D_v < 1 || D_v > 256) return 0;
     const double w = (double)B * (double)H * (double)N * (double)N * (double)padded(D_qk > D_v ? D_qk : D_v);
     const WalkPlan wp = walk_plan(B, H, N, D_qk, D_v, true);
-    if (wp.ok) return w >= (wp.D <= 64 ? 4e9 : 8e9);                              // padded head dims up to 128
+    // (padded widths that differ: the quadratic side is the small-V operator, whose wide products are two launches)
+    if (wp.ok && pad_index(D_qk) != pad_index(D_v)) return w >= (wp.D <= 64 ? 1e9 : 5e8);
+    if (wp.ok) return w >= (wp.D <= 64 ? 4e9 : 8e9);                              // equal padded head dims up to 128
     if (wide_plan(B, H, N, D_qk, D_v).ok) return w >= (D_v <= 64 ? 1e9 : 1.5e10);  // D_qk in (128, 256], D_v <= 128
     if (vsplit_plan(B, H, N, D_qk, D_v).ok) return w >= 3e10;  // D_v in (128, 256] as two column halves of v
     return N >= 4096;  // chunk states in memory, a launch per product and state (measured at 256 / 256)

@@ -242,6 +242,7 @@ def test_algorithm_table():
     assert pick(1, 128, 1024, 128, 128) == 1 and pick(1, 512, 512, 64, 64) == 1
     assert pick(1, 16, 256, 256, 64) == 0 and pick(1, 64, 512, 256, 64) == 1 and pick(1, 64, 2048, 256, 64) == 1
     assert pick(1, 16, 2048, 256, 256) == 0 and pick(1, 16, 4096, 256, 256) == 1 and pick(1, 64, 2048, 256, 256) == 1
+    assert pick(1, 16, 512, 128, 64) == 1 and pick(1, 16, 512, 64, 32) == 0 and pick(1, 16, 1024, 64, 32) == 1
     assert pick(1, 16, 1024, 192, 128) == 0 and pick(1, 16, 2048, 192, 128) == 1 and pick(1, 128, 512, 192, 128) == 0
     assert pick(0, 4, 4096, 64, 64) == 0 and pick(1, 4, 4096, 300, 64) == 0
     for shape in [(1, 16, 64, 64), (2, 8, 128, 128), (1, 64, 256, 64), (1, 4, 192, 128), (1, 8, 256, 256)]:
