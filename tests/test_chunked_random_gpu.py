@@ -26,10 +26,10 @@ def _cases(seed: int, count: int):
             dqk, dv = rng.choice([(64, 64), (32, 32), (48, 64), (64, 40), (16, 24)])
         elif kind == 1:  # padded to 128
             dqk, dv = rng.choice([(128, 128), (96, 128), (128, 72), (104, 120)])
-        elif kind == 2:  # wide query / key, narrow value
-            dqk, dv = rng.choice([(256, 64), (192, 64), (256, 128), (136, 32), (200, 8)])
-        else:            # shapes without walk kernels
-            dqk, dv = rng.choice([(64, 256), (256, 256), (64, 128), (32, 96)])
+        elif kind == 2:  # wide query / key, narrow value; padded widths that differ
+            dqk, dv = rng.choice([(256, 64), (192, 64), (256, 128), (136, 32), (200, 8), (128, 64), (128, 24), (64, 32)])
+        else:            # a value wider than the query / key; a v of more than 128 columns; widths that are no multiples of 8
+            dqk, dv = rng.choice([(64, 256), (256, 256), (64, 128), (32, 96), (100, 250), (20, 100)])
         bh = rng.choice([1, 3, 8, 17, 40, 96])
         b = rng.choice([d for d in (1, 2, 3, 4) if bh % d == 0])
         n = rng.choice([129, 257, 300, 513, 640, 777, 1000, 1301, 2049, 2450, 3000, 4100, 6000])
