@@ -712,8 +712,8 @@ int wide_backward(const WidePlan &wide, const View &go, const View &q, const Vie
     // entry states of both halves up front: Q_h^T dO over the segments after, and -- when forward's are not
     // at hand -- K_h^T V over the segments before
     const float *fwd_entries[2] = {nullptr, nullptr}, *entries[2] = {nullptr, nullptr};
-    // (the one reverse walk over both halves adds up the totals of the segments after its own itself, as forward does)
-    const bool rev_sums_on_load = state_in && dv <= 64 && wp.n_seg >= 3 && wp.n_seg <= 7;
+    // (the reverse walks add up the totals of the segments after their own themselves, as forward does)
+    const bool rev_sums_on_load = state_in && wp.n_seg >= 3 && wp.n_seg <= 7;
     if (wp.n_seg > 1) {
         float *const none[2] = {nullptr, nullptr};
         char *base = ws + wide.temp_bytes;
@@ -768,7 +768,7 @@ int wide_backward(const WidePlan &wide, const View &go, const View &q, const Vie
             r.dvs_b = dvv.strides[0], r.dvs_h = dvv.strides[1], r.dvs_n = dvv.strides[2];
             r.H = (int32_t)H, r.N = (int32_t)N, r.BH = (int32_t)(B * H), r.wqk = (int32_t)wqk, r.wv = (int32_t)dv;
             r.n_chunks = (int32_t)wp.n_chunks, r.seg_chunks = (int32_t)wp.seg_chunks, r.n_seg = (int32_t)wp.n_seg;
-            r.init = entry;
+            r.init = entry, r.init_is_totals = rev_sums_on_load;
             const char *half = static_cast<const char *>(state_in) + h * wp.saved_bytes;
             r.xinit = reinterpret_cast<const float *>(half);
             r.xtotal = reinterpret_cast<const float *>(half + wp.entry_bytes);
@@ -872,16 +872,20 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         // them to state_out (the totals themselves are computed there, and no workspace is used);
         // the normalised operator at padded head dims up to 64 hands over the 16-bit state of every chunk instead
         const bool in_state = state_out && (wp.split || !nx);
-        if (need_totals && !in_state &&
+        // D = 128, a few segments more than two: the totals go to the workspace, the walk adds them up itself as it starts
+        // and writes the entry states it formed to state_out -- no scan launch (B H 64, N 4096: see wide_forward)
+        const bool sum_on_load = wp.split && !fmap && !nx && wp.n_seg >= 3 && wp.n_seg <= 7;
+        if (need_totals && (!in_state || sum_on_load) &&
             (!workspace || reinterpret_cast<uintptr_t>(workspace) % 16 != 0 || workspace_bytes < wp.work_bytes))
             return FLA_ERR_WORKSPACE;
         if (state_out && reinterpret_cast<uintptr_t>(state_out) % 16 != 0) return FLA_ERR_WORKSPACE;
         hipStream_t s = static_cast<hipStream_t>(stream);
         const float *entry = nullptr;
         if (need_totals)
-            if (int rc = walk_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0, in_state ? state_out : workspace,
-                                           in_state ? static_cast<float *>(state_out) : nullptr, &entry, s, fmap,
-                                           fmap ? &mapped[1] : nullptr))
+            if (int rc = walk_entry_states(wp, k, v, B, H, N, dqk, dv, dtype, 0,
+                                           in_state && !sum_on_load ? state_out : workspace,
+                                           in_state && !sum_on_load ? static_cast<float *>(state_out) : nullptr, &entry, s,
+                                           fmap, fmap ? &mapped[1] : nullptr, nullptr, sum_on_load))
                 return rc;
         const View &kk = fmap ? mapped[1] : k;
         fla::WalkParams w{};
@@ -897,6 +901,7 @@ int chunked_forward(const View &q, const View &k, const View &v, const View &o, 
         w.H = (int32_t)H, w.N = (int32_t)N, w.BH = (int32_t)(B * H), w.wqk = (int32_t)dqk, w.wv = (int32_t)dv;
         w.n_chunks = (int32_t)wp.n_chunks, w.seg_chunks = (int32_t)wp.seg_chunks, w.n_seg = (int32_t)wp.n_seg;
         w.init = wp.n_seg > 1 ? entry : nullptr, w.saved = in_state ? nullptr : state_out;
+        if (sum_on_load) w.init_is_totals = 1, w.entry_out = in_state ? static_cast<float *>(state_out) : nullptr;
         if (in_state) w.total_out = reinterpret_cast<float *>(static_cast<char *>(state_out) + wp.entry_bytes);
         if (nx) {  // the normaliser inside the walk: zc = running sum of k at the entry of every chunk
             // (kept behind the state, when there is one, for backward)
@@ -1018,6 +1023,8 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
         const float *entry = nullptr;
         // with forward's states at hand (and without the normaliser): one reverse walk
         const bool one_walk = state_in && !nx;
+        // (... which adds up the totals of the segments after its own itself, as forward does)
+        const bool rev_sums_on_load = one_walk && wp.n_seg >= 3 && wp.n_seg <= 7;
         if (wp.n_seg > 1) {
             if (!state_in) {
                 const float *fwd_entry = nullptr;
@@ -1026,7 +1033,9 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
                     return rc;
                 state_in = fwd_entry;
             }
-            if (int rc = walk_entry_states(wp, q, go, B, H, N, dqk, dv, dtype, 1, workspace, nullptr, &entry, s)) return rc;
+            if (int rc = walk_entry_states(wp, q, go, B, H, N, dqk, dv, dtype, 1, workspace, nullptr, &entry, s, 0, nullptr,
+                                           nullptr, rev_sums_on_load))
+                return rc;
         }
         float *zc = nullptr, *rcv = nullptr;
         if (nx) {  // zc: running sum of k at the entry of every chunk; rc: sum of dn_i q_i over the rows after it
@@ -1050,6 +1059,7 @@ int chunked_backward(const View &go, const View &q, const View &k, const View &v
             r.H = (int32_t)H, r.N = (int32_t)N, r.BH = (int32_t)(B * H), r.wqk = (int32_t)dqk, r.wv = (int32_t)dv;
             r.n_chunks = (int32_t)wp.n_chunks, r.seg_chunks = (int32_t)wp.seg_chunks, r.n_seg = (int32_t)wp.n_seg;
             r.init = entry, r.fmap = fmap;  // (dQ, dK: the slopes from phi(xq), phi(xk) in the Q and K tiles)
+            r.init_is_totals = rev_sums_on_load;
             r.xinit = static_cast<const float *>(state_in);
             r.xtotal = reinterpret_cast<const float *>(static_cast<const char *>(state_in) + wp.entry_bytes);
             return fla::walk_bwd_rev(dtype, wp.D, r, s) == hipSuccess ? FLA_OK : FLA_ERR_LAUNCH;

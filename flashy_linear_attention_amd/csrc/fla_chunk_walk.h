@@ -129,10 +129,11 @@ struct WalkParams {
     const float *init2;
     float *total_out2;
     const float *xinit2, *xtotal2;
-    // init_is_totals: init and init2 hold the segments' TOTALS as the totals kernel wrote them, and a workgroup adds
-    // up those of the segments before its own (after it, walking in reverse) as it starts, all loads in flight together
-    // (walk_sum_two) -- no scan launch between the totals kernel and the walk.  The forward walk then writes the
-    // entry state it formed to entry_out / entry_out2 (the layout of init; null: nowhere), for the backward walk.
+    // init_is_totals (every D = 128 walk; three segments or more): init (and init2) hold the segments' TOTALS as the
+    // totals kernel wrote them, and a workgroup adds up those of the segments before its own (after it, walking in
+    // reverse) as it starts, several loads in flight together -- no scan launch between the totals kernel and the
+    // walk.  The forward walks (walk_fwd_kernel's plain D = 128 variant, walk_fwd_wide_kernel) then write the entry
+    // state they formed to entry_out / entry_out2 (the layout of init; null: nowhere), for the backward walk.
     int32_t init_is_totals;
     float *entry_out, *entry_out2;
 };
@@ -754,13 +755,13 @@ __host__ __device__ constexpr bool walk_entries_are_totals(int D, int n_seg) {
 }
 
 // this wave's blocks of the sum of the states buf[f_lo .. f_hi - 1] (zeros for an empty range), added in
-// ascending order, the loads of up to four states in flight together (one state at a time is a chain of
+// ascending order, the loads of up to four states (two of four blocks per wave) in flight together (one state at a time is a chain of
 // dependent loads: a memory latency per state at the start of every workgroup)
 template <int D, typename B>
 __device__ __forceinline__ void walk_sum_states(const float *buf, int f_lo, int f_hi, bool transposed, int wave, int lane,
                                                 f32x16 (&st)[WalkCfg<D>::NBW]) {
     using W = WalkCfg<D>;
-    constexpr int GROUP = 4;
+    constexpr int GROUP = B::SLOTS > 2 ? 2 : 4;  // (GROUP x SLOTS x 16 registers beside the sum)
 #pragma unroll
     for (int i = 0; i < W::NBW; ++i)
 #pragma unroll
@@ -830,7 +831,7 @@ __device__ __forceinline__ void walk_load_init_from(const float *buf, const Walk
     if (buf) {
         if (p.n_seg == 2) {
             if (sl.seg != (reverse ? 1 : 0)) init = buf + (int64_t)sl.bh * 2 * (D * D), init2 = init + D * D;
-        } else if (walk_entries_are_totals(D, p.n_seg)) {
+        } else if (walk_entries_are_totals(D, p.n_seg) || p.init_is_totals) {
             walk_sum_states<D, B>(buf + (int64_t)sl.bh * p.n_seg * (D * D), reverse ? sl.seg + 1 : 0,
                                   reverse ? p.n_seg : sl.seg, p.init_transposed != 0, wave, lane, st);
             return;
@@ -869,6 +870,19 @@ template <int D, typename B = WalkExt<D>>
 __device__ __forceinline__ void walk_load_end_state(const WalkParams &p, const WalkSlice &sl, int wave, int lane,
                                                     f32x16 (&xs)[WalkCfg<D>::NBW]) {
     walk_load_end_state_from<D, B>(p.xinit, p.xtotal, p, sl, wave, lane, xs);
+}
+
+// this wave's blocks of a state to an fp32 buffer [D][D] ([q/k index][v index]); blocks outside B stay unwritten
+template <int D, typename B>
+__device__ __forceinline__ void walk_write_state(float *out, int wave, int lane, const f32x16 (&st)[WalkCfg<D>::NBW]) {
+    const int l32 = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < B::SLOTS; ++i)
+        if (B::valid(wave, i)) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                out[(32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * B::eb(wave) + l32] = st[i][v];
+        }
 }
 
 // ---- one product with its running state, chunks ascending:
@@ -918,6 +932,10 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
 
     f32x16 st[W::NBW];
     walk_load_init<D, B>(p, sl, wave, lane, st, false);
+    if constexpr (DOUBLE && NORM == 0 && !FM) {  // (the entry state this walk formed from the segments' totals, for backward)
+        if (p.init_is_totals && p.entry_out && sl.seg > 0)
+            walk_write_state<D, B>(p.entry_out + ((int64_t)sl.bh * p.n_seg + sl.seg) * (D * D), wave, lane, st);
+    }
     walk_state_to_lds<T, D, B>(tl, wave, lane, st);
 
     auto load_chunk = [&](int c, int buf) {
@@ -1056,19 +1074,6 @@ __global__ __launch_bounds__(256, DOUBLE ? 1 : 2) void walk_fwd_kernel(const Wal
 #else
     (void)p;
 #endif
-}
-
-// this wave's blocks of a state to an fp32 buffer [D][D] ([q/k index][v index]); blocks outside B stay unwritten
-template <int D, typename B>
-__device__ __forceinline__ void walk_write_state(float *out, int wave, int lane, const f32x16 (&st)[WalkCfg<D>::NBW]) {
-    const int l32 = lane & 31, g = lane >> 5;
-#pragma unroll
-    for (int i = 0; i < B::SLOTS; ++i)
-        if (B::valid(wave, i)) {
-#pragma unroll
-            for (int v = 0; v < 16; ++v)
-                out[(32 * B::dbk(wave, i) + 8 * (v / 4) + 4 * g + (v % 4)) * D + 32 * B::eb(wave) + l32] = st[i][v];
-        }
 }
 
 // ---- forward for q and k of 129 .. 256 columns (v of at most 128), one walk over both 128-column halves:
@@ -2103,6 +2108,9 @@ hipError_t launch_walk_fwd(const WalkParams &p, hipStream_t stream) {
     constexpr bool kDouble = D > 64;  // (the plan's workgroup count must match: one per CU when double)
     constexpr int smem = (kDouble ? 6 : 3) * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
     const bool fm = p.fmap || p.slope_y;
+    // (segment totals in place of entry states: the D = 128 walks, by the flag; below that by the number of segments)
+    if (p.init_is_totals && (D != 128 || p.n_seg < 3 || !p.init)) return hipErrorInvalidValue;
+    if (p.entry_out && (!p.init_is_totals || fm || p.denom || p.dn)) return hipErrorInvalidValue;
     if (p.denom || p.dn) {  // the normaliser's terms: its vectors live behind the state
         if (!p.zc || p.accumulate) return hipErrorInvalidValue;
         constexpr int smem_n = smem + (kDouble ? 2 : 1) * WalkCfg<D>::VEC;
@@ -2191,6 +2199,7 @@ hipError_t launch_walk_bwd_rev(const WalkParams &p, hipStream_t stream) {
     const int64_t grid = (int64_t)8 * ((p.BH + 7) / 8) * p.n_seg;
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     if (!p.xtotal || (p.n_seg > 1 && !p.xinit)) return hipErrorInvalidValue;
+    if (p.entry_out || (p.init_is_totals && (p.n_seg < 3 || !p.init))) return hipErrorInvalidValue;
     constexpr int smem = 8 * WalkCfg<D>::TILE + WalkCfg<D>::STATE;
     static_assert(smem <= 160 * 1024, "two sets of tiles and the state must fit the LDS of a CU");
     if constexpr (D == 128) {  // a half of a wide q / k against a narrow v: without the blocks of padding

@@ -773,6 +773,12 @@ def model_walk(arena: Arena, l: Launch, p: Dict, D: int, stats: Stats) -> None:
         arena.require("entry states", p["init"], p["init"] + BH * n_seg * E)
     else:
         assert n_seg == 1 or l.kernel == "walk_bwd_kernel" and False, f"{l.kernel}: {n_seg} segments without entry states"
+    if p["init_is_totals"]:  # (the walk adds up the segments' totals itself; a forward walk writes what it formed)
+        assert D == 128 and n_seg >= 3 and p["init"], f"{l.kernel}: segment totals in place of entry states"
+    if p["entry_out"]:
+        assert p["init_is_totals"] and l.kernel in ("walk_fwd_kernel", "walk_fwd_wide_kernel")
+        arena.require("entry states written by the walk", p["entry_out"], p["entry_out"] + BH * n_seg * E)
+        assert not (p["init"] <= p["entry_out"] < p["init"] + BH * n_seg * E), "entry states over the totals"
     if p["xinit"]:
         arena.require("forward's entry states", p["xinit"], p["xinit"] + BH * n_seg * E)
     if p["xtotal"]:
