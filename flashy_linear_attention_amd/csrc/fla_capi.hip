@@ -671,11 +671,11 @@ int wide_forward(const WidePlan &wide, const View &q, const View &k, const View 
     const WalkPlan &wp = wide.wp;
     char *ws = static_cast<char *>(workspace);
     const float *entry[2] = {nullptr, nullptr};
-    // A few segments more than two and a narrow v: no scan -- the walk adds up the totals of the segments before its own as it
+    // A few segments more than two: no scan -- the walk adds up the totals of the segments before its own as it
     // starts (three of each half in flight together) and writes the entry state it formed for backward
     // (B 4, H 16, N 4096, D_qk 256, D_v 64, four segments: 0.273 -> 0.267 ms per forward + backward, and 0.264 with
     // the reverse walk doing the same).
-    const bool sum_on_load = wp.n_seg >= 3 && wp.n_seg <= 7 && dv <= 64;
+    const bool sum_on_load = wp.n_seg >= 3 && wp.n_seg <= 7;
     float *keep[2] = {nullptr, nullptr};
     if (wp.n_seg > 1) {
         // (kept for backward when there is a state buffer: each half's entry states, its final state behind them;

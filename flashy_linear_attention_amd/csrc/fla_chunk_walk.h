@@ -1117,19 +1117,19 @@ __global__ __launch_bounds__(256, 1) void walk_fwd_wide_kernel(const WalkParams 
     const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(O, 0, (N - 1) * os2 + p.wv * 2, 0x00020000);
 
     f32x16 st0[W::NBW], st1[W::NBW];
-    bool summed = false;
-    if constexpr (NV == 2) {  // (init_is_totals: with a narrow v only -- the launcher refuses it otherwise)
-        if (p.init_is_totals) {
-            const int64_t at = (int64_t)sl.bh * p.n_seg * (D * D);
+    if (p.init_is_totals) {
+        const int64_t at = (int64_t)sl.bh * p.n_seg * (D * D);
+        if constexpr (NV == 2) {  // (both halves' loads in flight together; with four blocks per wave and state, one half's)
             walk_sum_two<D, B>(p.init + at, p.init2 + at, 0, sl.seg, wave, lane, st0, st1);
-            if (p.entry_out && sl.seg > 0) {  // (the first segment's entry state, zero, is read by nobody)
-                walk_write_state<D, B>(p.entry_out + at + (int64_t)sl.seg * (D * D), wave, lane, st0);
-                walk_write_state<D, B>(p.entry_out2 + at + (int64_t)sl.seg * (D * D), wave, lane, st1);
-            }
-            summed = true;
+        } else {
+            walk_sum_states<D, B>(p.init + at, 0, sl.seg, false, wave, lane, st0);
+            walk_sum_states<D, B>(p.init2 + at, 0, sl.seg, false, wave, lane, st1);
         }
-    }
-    if (!summed) {
+        if (p.entry_out && sl.seg > 0) {  // (the first segment's entry state, zero, is read by nobody)
+            walk_write_state<D, B>(p.entry_out + at + (int64_t)sl.seg * (D * D), wave, lane, st0);
+            walk_write_state<D, B>(p.entry_out2 + at + (int64_t)sl.seg * (D * D), wave, lane, st1);
+        }
+    } else {
         walk_load_init_from<D, B>(p.init, p, sl, wave, lane, st0, false);
         walk_load_init_from<D, B>(p.init2, p, sl, wave, lane, st1, false);
     }
@@ -2143,7 +2143,7 @@ hipError_t launch_walk_fwd_wide(const WalkParams &p, hipStream_t stream) {
     if (grid > 0x7fffffffLL) return hipErrorInvalidConfiguration;
     if (p.wqk != 128 || p.wqk2 < 1 || p.wqk2 > 128 || p.wv < 1 || p.wv > 128 || p.fmap || p.slope_y || p.denom || p.dn ||
         p.accumulate || p.init_transposed || (p.n_seg > 1 && (!p.init || !p.init2)) || (p.total_out && !p.total_out2) ||
-        (p.init_is_totals && (p.n_seg < 3 || !p.init || !p.init2 || p.wv > 64)) ||
+        (p.init_is_totals && (p.n_seg < 3 || !p.init || !p.init2)) ||
         (p.entry_out != nullptr) != (p.entry_out2 != nullptr) || (p.entry_out && !p.init_is_totals))
         return hipErrorInvalidValue;
     constexpr int smem = 6 * W::TILE + W::STATE;  // two sets of (Q_h, K_h), two V tiles, one state
